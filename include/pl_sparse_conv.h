@@ -1,0 +1,189 @@
+/*
+ * C ABI of the MI355X (gfx950) sparse 1x1 convolution.
+ *
+ * This is the boundary a Paddle-Lite HIP-target kernel binds to: plain
+ * pointers, sizes and POD structs only, every function returns a status and
+ * never throws or aborts.  The math entry points take exactly what the ARM
+ * math functions of the reference take (compressed weights, merged
+ * per-channel scale and bias, activation constants) so that a kernel class
+ * written like lite/kernels/arm/sparse_conv_compute.cc can call them from
+ * PrepareForRun() / Run().
+ *
+ * Thread compatibility: functions may be called from any thread; a handle
+ * must not be used by two threads at once.
+ */
+#ifndef PL_SPARSE_CONV_H_
+#define PL_SPARSE_CONV_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PL_SPARSE_CONV_ABI_VERSION 1
+
+/* status codes (negative = failure; HIP errors are reported as
+ * PL_ERR_HIP with the text available from pl_last_error()) */
+enum {
+  PL_OK = 0,
+  PL_ERR_BAD_ARG = -1,
+  PL_ERR_BAD_LAYOUT = -2,   /* OcNonZeros / Diffs do not describe a matrix */
+  PL_ERR_UNSUPPORTED = -3,
+  PL_ERR_HIP = -4,
+  PL_ERR_NO_DEVICE = -5
+};
+
+/* Kernel variants = the registrations of the reference
+ * (lite/kernels/arm/sparse_conv_compute.cc:369-430): fp32 "def",
+ * "int8_fp32_out" and "int8_int8_out".  PL_KIND_INT8_ACC32 additionally
+ * exposes the raw int32 accumulators of the int8 path for verification. */
+enum {
+  PL_KIND_FP32 = 0,
+  PL_KIND_INT8_FP32 = 1,
+  PL_KIND_INT8_INT8 = 2,
+  PL_KIND_INT8_ACC32 = 3
+};
+
+/* lite_api::ActivationType values the sparse kernels implement
+ * (lite/api/paddle_place.h:122-149; selection as in
+ * lite/backends/arm/math/sparse_conv_impl.cc:1197-1215: any other value
+ * means "no activation"). */
+enum {
+  PL_ACT_NONE = 0,
+  PL_ACT_RELU = 1,
+  PL_ACT_RELU6 = 2,
+  PL_ACT_LEAKY_RELU = 4,
+  PL_ACT_HARD_SWISH = 10
+};
+
+/* How the SpMM is executed.
+ *   PL_ALGO_AUTO      library picks (see pl_sparse_conv_info.algo)
+ *   PL_ALGO_ROW_WALK  one wavefront per output channel (pair) walks its
+ *                     nonzero list over an activation tile held in LDS
+ *   PL_ALGO_BLOCK_MFMA int8 only: 32x32 blocks of the weight matrix that
+ *                     hold at least one nonzero are multiplied on the matrix
+ *                     cores, empty blocks are skipped */
+enum { PL_ALGO_AUTO = 0, PL_ALGO_ROW_WALK = 1, PL_ALGO_BLOCK_MFMA = 2 };
+
+/* Activation constants, used as given (replaces the fields of
+ * ActivationParam the math functions read,
+ * lite/operators/op_params.h:331-362). */
+typedef struct pl_activation {
+  int32_t type;        /* PL_ACT_*                                          */
+  float relu6_coef;    /* Relu_clipped_coef                                 */
+  float leaky_alpha;   /* Leaky_relu_alpha                                  */
+  float hs_scale;      /* hard_swish_scale; the kernel multiplies by
+                          (float)(1.0 / hs_scale)                           */
+  float hs_offset;     /* hard_swish_offset                                 */
+  float hs_threshold;  /* hard_swish_threshold                              */
+} pl_activation;
+
+/* Everything PrepareForRun() knows.  All pointers are HOST pointers and are
+ * only read during pl_sparse_conv_prepare(). Replaces the argument list of
+ * sparse_conv_*_pipelined (lite/backends/arm/math/sparse_conv_impl.h:38-73,
+ * sparse_semi_conv_impl.h:30-68) minus the activation/output pointers. */
+typedef struct pl_sparse_conv_desc {
+  uint32_t struct_size;          /* sizeof(pl_sparse_conv_desc)             */
+  int32_t kind;                  /* PL_KIND_*                               */
+  int32_t flag_semi;             /* SparseConvParam::flag_semi              */
+  int32_t first_ic;              /* SparseConvParam::first_ic               */
+  int32_t oc;                    /* M: output channels                      */
+  int32_t ic;                    /* K: input channels                       */
+  int32_t im_size;               /* H*W the Diffs tensor was baked for      */
+  int32_t algo;                  /* PL_ALGO_*                               */
+  const void* nonzero_weights;   /* float or int8_t, n_weights elements     */
+  int64_t n_weights;
+  const uint32_t* oc_nonzeros;   /* oc entries (semi: oc/2 + oc%2 are read) */
+  const int32_t* diffs;          /* n_diffs entries, byte offsets           */
+  int64_t n_diffs;
+  const float* scale;            /* oc merged scales; int8 kinds only       */
+  const float* bias;             /* oc merged biases or NULL                */
+  pl_activation act;
+} pl_sparse_conv_desc;
+
+typedef struct pl_sparse_conv_info {
+  int32_t algo;          /* the algorithm run() will use                    */
+  int32_t oc, ic;
+  int64_t nnz;           /* nonzero weights actually present in the layout  */
+  int64_t stored_weights;/* weights stored in the layout (semi keeps zeros) */
+  int64_t index_entries; /* Diffs entries describing real weights           */
+  int64_t device_bytes;  /* device memory held by the handle                */
+  int64_t mfma_blocks;   /* 32x32 weight blocks with a nonzero (int8)       */
+  int64_t mfma_blocks_total;
+} pl_sparse_conv_info;
+
+typedef struct pl_sparse_conv_handle pl_sparse_conv_handle;
+
+/* Library / device ------------------------------------------------------- */
+int pl_sparse_conv_abi_version(void);
+/* Text of the last failure on the calling thread ("" if none). */
+const char* pl_last_error(void);
+/* Number of usable gfx950 devices (0 on a machine without one). */
+int pl_device_count(void);
+
+/* The op's hot path ------------------------------------------------------ */
+
+/* Replaces SparseConvCompute::PrepareForRun's device-side part: validates the
+ * layout, converts the byte offsets to channel indices and uploads the
+ * GPU-side form to the current HIP device. */
+int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc,
+                           pl_sparse_conv_handle** out_handle);
+
+/* Replaces sparse_conv_{fp32,int8_fp32,int8_int8}_pipelined and their
+ * sparse_semi_ twins, called from SparseConvCompute::Run
+ * (lite/kernels/arm/sparse_conv_compute.cc:104-267).
+ *   x_dev   : device pointer, NCHW [batch, ic, im_size] float or int8_t
+ *   out_dev : device pointer, NCHW [batch, oc, im_size] float / int8_t /
+ *             int32_t per kind
+ *   im_size : H*W of this call (may differ from the baked one)
+ *   stream  : hipStream_t (NULL = default stream); the call only enqueues. */
+int pl_sparse_conv_run(pl_sparse_conv_handle* handle, const void* x_dev,
+                       void* out_dev, int32_t batch, int32_t im_size,
+                       void* stream);
+
+int pl_sparse_conv_get_info(const pl_sparse_conv_handle* handle,
+                            pl_sparse_conv_info* info);
+
+/* Replace scale / bias / activation without re-uploading weights (what a
+ * second PrepareForRun with new quantisation parameters would do). Either
+ * pointer may be NULL to keep the current values. */
+int pl_sparse_conv_set_epilogue(pl_sparse_conv_handle* handle,
+                                const float* scale, const float* bias,
+                                const pl_activation* act);
+
+void pl_sparse_conv_destroy(pl_sparse_conv_handle* handle);
+
+/* Opt-time packers (host only) -------------------------------------------
+ * dtype: 0 = fp32 weights, 1 = int8 weights.  Dense weights are [oc x ic]
+ * row major. */
+
+/* Replaces SparseConvDetectPass::ComputeSemiSparseZeros
+ * (lite/core/optimizer/mir/sparse_conv_detect_pass.cc:303-368). Returns the
+ * zero count the pass compares with sparse_threshold. */
+int pl_sparse_count_semi(int32_t dtype, const void* dense, int32_t oc,
+                         int32_t ic, int32_t* count_nonzeroes,
+                         int32_t* count_channels, int32_t* count_blocks,
+                         int32_t* flag_semi);
+
+/* Replaces SparseConvDetectPass::ComputeSparseZeros
+ * (sparse_conv_detect_pass.cc:480-517). */
+int pl_sparse_count_zeros(int32_t dtype, const void* dense, int32_t oc,
+                          int32_t ic, int32_t* num_build_nonzeroes);
+
+/* Replaces ComputeSparseWeight (both overloads) and ComputeSemiSparseWeight
+ * (sparse_conv_detect_pass.cc:35-301) with the pass's own choice between
+ * them (:732-780): semi layout when flag_semi, else rows padded to four for
+ * fp32 and unpadded for int8.  Output arrays must hold n_weights / oc /
+ * n_diffs elements as computed by the two counting functions. Returns
+ * first_ic (>= 0) or a negative status. */
+int pl_sparse_pack(int32_t dtype, int32_t flag_semi, const void* dense,
+                   int32_t oc, int32_t ic, int32_t im_size,
+                   void* nonzero_weights, int64_t n_weights,
+                   uint32_t* oc_nonzeros, int32_t* diffs, int64_t n_diffs);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PL_SPARSE_CONV_H_ */

@@ -1,0 +1,511 @@
+// C ABI of the gfx950 sparse 1x1 convolution: layout validation, one-time
+// conversion of the compressed weights into the device-side forms, launch
+// selection.  No CPU compute path exists here: without a device
+// pl_sparse_conv_prepare() fails with PL_ERR_NO_DEVICE.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "../../include/pl_sparse_conv.h"
+#include "sparse_conv_kernels.h"
+#include "sparse_layout.h"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int Fail(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return code;
+}
+
+int FailHip(hipError_t e, const char* what) {
+  return Fail(PL_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+// Owning device allocation.
+struct DevBuf {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+  DevBuf() = default;
+  DevBuf(const DevBuf&) = delete;
+  DevBuf& operator=(const DevBuf&) = delete;
+  ~DevBuf() { Reset(); }
+  void Reset() {
+    if (ptr) (void)hipFree(ptr);
+    ptr = nullptr;
+    bytes = 0;
+  }
+  hipError_t Upload(const void* host, size_t n) {
+    Reset();
+    if (n == 0) n = 16;  // keep kernels' pointer arguments valid
+    hipError_t e = hipMalloc(&ptr, n);
+    if (e != hipSuccess) {
+      ptr = nullptr;
+      return e;
+    }
+    bytes = n;
+    if (host) e = hipMemcpy(ptr, host, n, hipMemcpyHostToDevice);
+    return e;
+  }
+};
+
+pl::DevAct ToDevAct(const pl_activation& a) {
+  pl::DevAct d{};
+  d.type = a.type;
+  d.relu6_coef = a.relu6_coef;
+  d.leaky_alpha = a.leaky_alpha;
+  // the math functions form 1.0 / scale in double and narrow it
+  // (lite/backends/arm/math/sparse_conv_impl.cc:1211)
+  d.hs_inv_scale = a.type == PL_ACT_HARD_SWISH ? static_cast<float>(1.0 / a.hs_scale) : 0.0f;
+  d.hs_offset = a.hs_offset;
+  d.hs_threshold = a.hs_threshold;
+  return d;
+}
+
+int CeilDiv(int a, int b) { return (a + b - 1) / b; }
+
+}  // namespace
+
+struct pl_sparse_conv_handle {
+  int device = 0;
+  int kind = PL_KIND_FP32;
+  int algo = PL_ALGO_ROW_WALK;
+  int oc = 0, ic = 0;
+  bool int8 = false;
+  bool semi = false;
+  bool has_bias = false;
+  pl::DevAct act{};
+  int64_t nnz = 0, stored = 0, entries = 0;
+  // row walk
+  int n_groups = 0;
+  int kd = 0;
+  int64_t walk_entries = 0;
+  DevBuf groups, kidx, wts;
+  // block MFMA
+  int row_blocks = 0, ksteps = 0;
+  int64_t blocks_present = 0;
+  DevBuf wblocks, kmask;
+  // epilogue
+  DevBuf scale, bias;
+  int padded_rows = 0;
+
+  int64_t DeviceBytes() const {
+    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + wblocks.bytes + kmask.bytes + scale.bytes + bias.bytes);
+  }
+};
+
+namespace {
+
+int OutKind(int kind) {
+  switch (kind) {
+    case PL_KIND_INT8_INT8:
+      return pl::kOutI8;
+    case PL_KIND_INT8_ACC32:
+      return pl::kOutAcc32;
+    default:
+      return pl::kOutF32;
+  }
+}
+
+// Device-side form for the row walk: per group an index list; int8 weights
+// of one channel quad are merged into one dword so that one v_dot4 consumes
+// them.
+int BuildRowWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
+  const int nr = L.semi ? 2 : 1;
+  std::vector<pl::DevGroup> groups;
+  std::vector<uint32_t> kidx, wts;
+  groups.reserve(L.groups.size());
+  for (const pl::RowGroup& g : L.groups) {
+    pl::DevGroup d;
+    d.row0 = g.row0;
+    d.nrows = g.nrows;
+    d.first = static_cast<uint32_t>(kidx.size());
+    if (!h->int8) {
+      for (uint32_t j = 0; j < g.count; ++j) {
+        kidx.push_back(L.ic_index[g.first + j]);
+        wts.push_back(L.w0[g.first + j]);
+        if (nr == 2) wts.push_back(L.w1[g.first + j]);
+      }
+    } else {
+      uint32_t j = 0;
+      while (j < g.count) {
+        const uint32_t q = L.ic_index[g.first + j] >> 2;
+        uint32_t p0 = 0, p1 = 0;
+        while (j < g.count && (L.ic_index[g.first + j] >> 2) == q) {
+          const int sh = 8 * (L.ic_index[g.first + j] & 3u);
+          p0 |= (L.w0[g.first + j] & 0xffu) << sh;
+          p1 |= (L.w1[g.first + j] & 0xffu) << sh;
+          ++j;
+        }
+        kidx.push_back(q);
+        wts.push_back(p0);
+        if (nr == 2) wts.push_back(p1);
+      }
+    }
+    d.count = static_cast<uint32_t>(kidx.size()) - d.first;
+    groups.push_back(d);
+  }
+  h->n_groups = static_cast<int>(groups.size());
+  h->kd = h->int8 ? CeilDiv(L.ic, 4) : L.ic;
+  h->walk_entries = static_cast<int64_t>(kidx.size());
+  hipError_t e = h->groups.Upload(groups.data(), groups.size() * sizeof(pl::DevGroup));
+  if (e == hipSuccess) e = h->kidx.Upload(kidx.data(), kidx.size() * sizeof(uint32_t));
+  if (e == hipSuccess) e = h->wts.Upload(wts.data(), wts.size() * sizeof(uint32_t));
+  if (e != hipSuccess) return FailHip(e, "uploading the row-walk index");
+  return PL_OK;
+}
+
+// Device-side form for the block MFMA path: the weight matrix as dense
+// 32x32 int8 blocks in matrix-core operand order, plus the mask of blocks
+// that hold a nonzero.
+int BuildBlockMfma(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
+  const int rbs = CeilDiv(L.oc, 32), kss = CeilDiv(L.ic, 32);
+  std::vector<int8_t> blocks(static_cast<size_t>(rbs) * kss * 64 * 16, 0);
+  std::vector<uint32_t> mask(rbs, 0u);
+  auto put = [&](int row, uint32_t c, uint32_t wbits) {
+    const int8_t w = static_cast<int8_t>(wbits & 0xffu);
+    if (w == 0) return;
+    const int rb = row >> 5, i = row & 31;
+    const int ks = c >> 5, kk = c & 31;
+    const int lane = i + 32 * (kk >> 4), t = kk & 15;
+    blocks[((static_cast<size_t>(rb) * kss + ks) * 64 + lane) * 16 + t] = w;
+    mask[rb] |= 1u << ks;
+  };
+  for (const pl::RowGroup& g : L.groups) {
+    for (uint32_t j = 0; j < g.count; ++j) {
+      put(g.row0, L.ic_index[g.first + j], L.w0[g.first + j]);
+      if (g.nrows == 2) put(g.row0 + 1, L.ic_index[g.first + j], L.w1[g.first + j]);
+    }
+  }
+  h->row_blocks = rbs;
+  h->ksteps = kss;
+  h->blocks_present = 0;
+  for (uint32_t m : mask) h->blocks_present += __builtin_popcount(m);
+  hipError_t e = h->wblocks.Upload(blocks.data(), blocks.size());
+  if (e == hipSuccess) e = h->kmask.Upload(mask.data(), mask.size() * sizeof(uint32_t));
+  if (e != hipSuccess) return FailHip(e, "uploading the weight blocks");
+  return PL_OK;
+}
+
+int UploadEpilogue(pl_sparse_conv_handle* h, const float* scale, const float* bias) {
+  const size_t n = static_cast<size_t>(h->padded_rows);
+  if (scale) {
+    std::vector<float> s(n, 0.0f);
+    std::copy(scale, scale + h->oc, s.begin());
+    hipError_t e = h->scale.Upload(s.data(), n * sizeof(float));
+    if (e != hipSuccess) return FailHip(e, "uploading scales");
+  }
+  if (bias) {
+    std::vector<float> b(n, 0.0f);
+    std::copy(bias, bias + h->oc, b.begin());
+    hipError_t e = h->bias.Upload(b.data(), n * sizeof(float));
+    if (e != hipSuccess) return FailHip(e, "uploading biases");
+    h->has_bias = true;
+  }
+  return PL_OK;
+}
+
+// Tile shape of the row walk for a given problem.
+pl::WalkConfig ChooseWalk(const pl_sparse_conv_handle* h, uint32_t P) {
+  pl::WalkConfig c{};
+  c.int8 = h->int8;
+  c.out_kind = OutKind(h->kind);
+  c.nrows = h->semi ? 2 : 1;
+  const size_t row_bytes = static_cast<size_t>(h->kd) * 4;
+  // prefer tiles of at most 64 KB (two workgroups per CU), never below one
+  // wavefront of positions unless the channel count forces it
+  int tp = 256;
+  while (tp > 64 && row_bytes * tp > 64 * 1024) tp >>= 1;
+  while (tp > 16 && row_bytes * tp > static_cast<size_t>(pl::kMaxLdsBytes)) tp >>= 1;
+  while (tp > 64 && P <= static_cast<uint32_t>(tp) * 64) tp >>= 1;  // small problems: more tiles
+  c.tile_pos = tp;
+  const size_t lds = row_bytes * tp;
+  c.threads = lds > 80 * 1024 ? 1024 : (lds > 40 * 1024 ? 512 : 256);
+  if (c.threads < tp) c.threads = tp;
+  const int nwaves = c.threads / 64;
+  const uint32_t tiles = (P + tp - 1) / tp;
+  int slices = static_cast<int>((1024 + tiles - 1) / tiles);
+  slices = std::min(slices, std::max(1, h->n_groups / nwaves));
+  slices = std::max(1, std::min(slices, 65535));
+  c.slices = slices;
+  return c;
+}
+
+}  // namespace
+
+extern "C" {
+
+int pl_sparse_conv_abi_version(void) { return PL_SPARSE_CONV_ABI_VERSION; }
+
+const char* pl_last_error(void) { return g_last_error.c_str(); }
+
+int pl_device_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  int usable = 0;
+  for (int d = 0; d < n; ++d) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, d) == hipSuccess && std::strstr(prop.gcnArchName, "gfx950")) ++usable;
+  }
+  return usable;
+}
+
+int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handle** out_handle) {
+  if (!desc || !out_handle) return Fail(PL_ERR_BAD_ARG, "null argument");
+  *out_handle = nullptr;
+  if (desc->struct_size != sizeof(pl_sparse_conv_desc)) return Fail(PL_ERR_BAD_ARG, "pl_sparse_conv_desc size mismatch (%u vs %zu)", desc->struct_size, sizeof(pl_sparse_conv_desc));
+  if (desc->kind < PL_KIND_FP32 || desc->kind > PL_KIND_INT8_ACC32) return Fail(PL_ERR_BAD_ARG, "unknown kind %d", desc->kind);
+  if (desc->algo < PL_ALGO_AUTO || desc->algo > PL_ALGO_BLOCK_MFMA) return Fail(PL_ERR_BAD_ARG, "unknown algo %d", desc->algo);
+  if (desc->oc <= 0 || desc->ic <= 0 || desc->im_size <= 0) return Fail(PL_ERR_BAD_ARG, "oc, ic and im_size must be positive");
+  if (!desc->oc_nonzeros || (desc->n_weights > 0 && (!desc->nonzero_weights || !desc->diffs))) return Fail(PL_ERR_BAD_ARG, "null weight tensors");
+  const bool int8 = desc->kind != PL_KIND_FP32;
+  if (int8 && desc->kind != PL_KIND_INT8_ACC32 && !desc->scale) return Fail(PL_ERR_BAD_ARG, "int8 kinds need per-channel scales");
+  if (desc->algo == PL_ALGO_BLOCK_MFMA && !int8) return Fail(PL_ERR_UNSUPPORTED, "the block MFMA algorithm exists for int8 only");
+
+  int ndev = 0;
+  if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
+    (void)hipGetLastError();
+    return Fail(PL_ERR_NO_DEVICE, "no HIP device: this library has no CPU path");
+  }
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return FailHip(e, "hipGetDevice");
+  hipDeviceProp_t prop;
+  e = hipGetDeviceProperties(&prop, dev);
+  if (e != hipSuccess) return FailHip(e, "hipGetDeviceProperties");
+  if (!std::strstr(prop.gcnArchName, "gfx950")) return Fail(PL_ERR_NO_DEVICE, "device %d is %s; the kernels are built for gfx950 only", dev, prop.gcnArchName);
+
+  pl::DecodedLayout L;
+  std::string why;
+  if (!pl::DecodeLayout(int8 ? pl::WeightType::kInt8 : pl::WeightType::kFloat, desc->flag_semi != 0, desc->nonzero_weights, desc->n_weights, desc->oc_nonzeros, desc->diffs, desc->n_diffs, desc->first_ic, desc->oc, desc->ic,
+                        desc->im_size, &L, &why)) {
+    return Fail(PL_ERR_BAD_LAYOUT, "%s", why.c_str());
+  }
+
+  pl_sparse_conv_handle* h = new (std::nothrow) pl_sparse_conv_handle();
+  if (!h) return Fail(PL_ERR_BAD_ARG, "out of host memory");
+  h->device = dev;
+  h->kind = desc->kind;
+  h->oc = desc->oc;
+  h->ic = desc->ic;
+  h->int8 = int8;
+  h->semi = desc->flag_semi != 0;
+  h->act = ToDevAct(desc->act);
+  h->nnz = L.nnz;
+  h->stored = L.stored_weights;
+  h->entries = static_cast<int64_t>(L.ic_index.size());
+  h->padded_rows = CeilDiv(desc->oc, 32) * 32;
+
+  int algo = desc->algo;
+  const bool mfma_ok = int8 && CeilDiv(desc->ic, 32) <= 32;
+  if (algo == PL_ALGO_BLOCK_MFMA && !mfma_ok) {
+    delete h;
+    return Fail(PL_ERR_UNSUPPORTED, "block MFMA needs ic <= 1024 (got %d)", desc->ic);
+  }
+  if (algo == PL_ALGO_AUTO) algo = mfma_ok ? PL_ALGO_BLOCK_MFMA : PL_ALGO_ROW_WALK;
+  if (algo == PL_ALGO_ROW_WALK) {
+    const size_t row_bytes = static_cast<size_t>(int8 ? CeilDiv(desc->ic, 4) : desc->ic) * 4;
+    if (row_bytes * 16 > static_cast<size_t>(pl::kMaxLdsBytes)) {
+      delete h;
+      return Fail(PL_ERR_UNSUPPORTED, "ic = %d does not fit an LDS tile", desc->ic);
+    }
+  }
+  h->algo = algo;
+
+  int rc = algo == PL_ALGO_BLOCK_MFMA ? BuildBlockMfma(L, h) : BuildRowWalk(L, h);
+  if (rc == PL_OK) {
+    // the MFMA epilogue always reads a bias; give it zeros when the op has none
+    std::vector<float> zeros;
+    const float* bias = desc->bias;
+    if (!bias && algo == PL_ALGO_BLOCK_MFMA) {
+      zeros.assign(h->oc, 0.0f);
+      bias = zeros.data();
+    }
+    std::vector<float> ones;
+    const float* scale = desc->scale;
+    if (!scale && int8) {
+      ones.assign(h->oc, 1.0f);
+      scale = ones.data();
+    }
+    rc = UploadEpilogue(h, int8 ? scale : nullptr, bias);
+    h->has_bias = desc->bias != nullptr || algo == PL_ALGO_BLOCK_MFMA;
+  }
+  if (rc != PL_OK) {
+    delete h;
+    return rc;
+  }
+  *out_handle = h;
+  return PL_OK;
+}
+
+int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_dev, int32_t batch, int32_t im_size, void* stream) {
+  if (!h) return Fail(PL_ERR_BAD_ARG, "null handle");
+  if (batch < 0 || im_size <= 0) return Fail(PL_ERR_BAD_ARG, "batch must be >= 0 and im_size > 0");
+  if (batch == 0) return PL_OK;
+  if (!x_dev || !out_dev) return Fail(PL_ERR_BAD_ARG, "null device pointer");
+  const int64_t P64 = static_cast<int64_t>(batch) * im_size;
+  if (P64 >= (1ll << 31) - 512) return Fail(PL_ERR_UNSUPPORTED, "batch * im_size = %lld exceeds 2^31", static_cast<long long>(P64));
+  const uint32_t P = static_cast<uint32_t>(P64);
+  const int vec = (im_size % 4 == 0) && (reinterpret_cast<uintptr_t>(x_dev) % 16 == 0) && (reinterpret_cast<uintptr_t>(out_dev) % 16 == 0);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipError_t e;
+  if (h->algo == PL_ALGO_BLOCK_MFMA) {
+    pl::MfmaParams p{};
+    p.x = static_cast<const int8_t*>(x_dev);
+    p.out = out_dev;
+    p.wblocks = h->wblocks.ptr;
+    p.kmask = static_cast<const uint32_t*>(h->kmask.ptr);
+    p.scale = static_cast<const float*>(h->scale.ptr);
+    p.bias = static_cast<const float*>(h->bias.ptr);
+    p.row_blocks = h->row_blocks;
+    p.ksteps = h->ksteps;
+    p.M = h->oc;
+    p.K = h->ic;
+    p.hw = im_size;
+    p.P = P;
+    p.vec = vec;
+    p.act = h->act;
+    pl::MfmaConfig c{};
+    c.out_kind = OutKind(h->kind);
+    c.ks_max = 2;
+    while (c.ks_max < h->ksteps) c.ks_max <<= 1;
+    c.waves = c.ks_max >= 32 ? 4 : std::min(4, h->row_blocks);
+    if (c.waves < 1) c.waves = 1;
+    e = pl::LaunchBlockMfma(c, p, s);
+  } else {
+    pl::WalkParams p{};
+    p.x = x_dev;
+    p.out = out_dev;
+    p.groups = static_cast<const pl::DevGroup*>(h->groups.ptr);
+    p.kidx = static_cast<const uint32_t*>(h->kidx.ptr);
+    p.wts = static_cast<const uint32_t*>(h->wts.ptr);
+    p.scale = static_cast<const float*>(h->scale.ptr);
+    p.bias = h->has_bias ? static_cast<const float*>(h->bias.ptr) : nullptr;
+    p.n_groups = h->n_groups;
+    p.M = h->oc;
+    p.K = h->ic;
+    p.kd = h->kd;
+    p.hw = im_size;
+    p.P = P;
+    p.vec = vec;
+    p.act = h->act;
+    pl::WalkConfig c = ChooseWalk(h, P);
+    p.groups_per_slice = CeilDiv(h->n_groups, c.slices);
+    c.slices = CeilDiv(h->n_groups, p.groups_per_slice);
+    e = pl::LaunchRowWalk(c, p, s);
+  }
+  if (e != hipSuccess) return FailHip(e, "kernel launch");
+  return PL_OK;
+}
+
+int pl_sparse_conv_get_info(const pl_sparse_conv_handle* h, pl_sparse_conv_info* info) {
+  if (!h || !info) return Fail(PL_ERR_BAD_ARG, "null argument");
+  std::memset(info, 0, sizeof(*info));
+  info->algo = h->algo;
+  info->oc = h->oc;
+  info->ic = h->ic;
+  info->nnz = h->nnz;
+  info->stored_weights = h->stored;
+  info->index_entries = h->entries;
+  info->device_bytes = h->DeviceBytes();
+  info->mfma_blocks = h->blocks_present;
+  info->mfma_blocks_total = static_cast<int64_t>(h->row_blocks) * h->ksteps;
+  return PL_OK;
+}
+
+int pl_sparse_conv_set_epilogue(pl_sparse_conv_handle* h, const float* scale, const float* bias, const pl_activation* act) {
+  if (!h) return Fail(PL_ERR_BAD_ARG, "null handle");
+  if (scale && !h->int8) return Fail(PL_ERR_BAD_ARG, "fp32 kernels take no scales");
+  int rc = UploadEpilogue(h, scale, bias);
+  if (rc != PL_OK) return rc;
+  if (act) h->act = ToDevAct(*act);
+  return PL_OK;
+}
+
+void pl_sparse_conv_destroy(pl_sparse_conv_handle* h) { delete h; }
+
+// ------------------------------------------------------------ host packers
+int pl_sparse_count_semi(int32_t dtype, const void* dense, int32_t oc, int32_t ic, int32_t* count_nonzeroes, int32_t* count_channels, int32_t* count_blocks, int32_t* flag_semi) {
+  if (!dense || oc <= 0 || ic <= 0 || (dtype != 0 && dtype != 1)) return Fail(PL_ERR_BAD_ARG, "bad argument");
+  pl::SemiCounts c = dtype == 0 ? pl::CountSemi(static_cast<const float*>(dense), oc, ic) : pl::CountSemi(static_cast<const int8_t*>(dense), oc, ic);
+  if (count_nonzeroes) *count_nonzeroes = c.count_nonzeroes;
+  if (count_channels) *count_channels = c.count_channels;
+  if (count_blocks) *count_blocks = c.count_blocks;
+  if (flag_semi) *flag_semi = c.flag_semi;
+  return c.zeros;
+}
+
+int pl_sparse_count_zeros(int32_t dtype, const void* dense, int32_t oc, int32_t ic, int32_t* num_build_nonzeroes) {
+  if (!dense || oc <= 0 || ic <= 0 || (dtype != 0 && dtype != 1)) return Fail(PL_ERR_BAD_ARG, "bad argument");
+  int nb = 0;
+  int z = dtype == 0 ? pl::CountZerosPad4(static_cast<const float*>(dense), oc, ic, &nb) : pl::CountZerosPad4(static_cast<const int8_t*>(dense), oc, ic, &nb);
+  if (num_build_nonzeroes) *num_build_nonzeroes = nb;
+  return z;
+}
+
+int pl_sparse_pack(int32_t dtype, int32_t flag_semi, const void* dense, int32_t oc, int32_t ic, int32_t im_size, void* nonzero_weights, int64_t n_weights, uint32_t* oc_nonzeros, int32_t* diffs, int64_t n_diffs) {
+  if (!dense || !oc_nonzeros || oc <= 0 || ic <= 0 || im_size <= 0 || (dtype != 0 && dtype != 1)) return Fail(PL_ERR_BAD_ARG, "bad argument");
+  // the arrays must have exactly the sizes the counting passes report
+  int64_t need_w = 0, need_d = 0;
+  if (flag_semi) {
+    pl::SemiCounts c = dtype == 0 ? pl::CountSemi(static_cast<const float*>(dense), oc, ic) : pl::CountSemi(static_cast<const int8_t*>(dense), oc, ic);
+    if (!c.flag_semi) {
+      // caller forces the paired layout on a matrix the rule would not pick:
+      // count its blocks directly
+      int64_t blocks = 0, tail = 0;
+      const int even = oc - (oc & 1);
+      for (int r = 0; r < even; r += 2)
+        for (int k = 0; k < ic; ++k) {
+          bool a, b;
+          if (dtype == 0) {
+            const float* w = static_cast<const float*>(dense);
+            a = w[(size_t)r * ic + k] != 0.f;
+            b = w[(size_t)(r + 1) * ic + k] != 0.f;
+          } else {
+            const int8_t* w = static_cast<const int8_t*>(dense);
+            a = w[(size_t)r * ic + k] != 0;
+            b = w[(size_t)(r + 1) * ic + k] != 0;
+          }
+          blocks += (a || b);
+        }
+      for (int r = even; r < oc; ++r)
+        for (int k = 0; k < ic; ++k) tail += dtype == 0 ? (static_cast<const float*>(dense)[(size_t)r * ic + k] != 0.f) : (static_cast<const int8_t*>(dense)[(size_t)r * ic + k] != 0);
+      need_w = 2 * blocks + tail;
+      need_d = blocks + tail;
+    } else {
+      need_w = c.count_nonzeroes;
+      need_d = c.count_blocks;
+    }
+  } else if (dtype == 0) {
+    int nb = 0;
+    pl::CountZerosPad4(static_cast<const float*>(dense), oc, ic, &nb);
+    need_w = need_d = nb;
+  } else {
+    int nb = 0;
+    int z = pl::CountZerosPad4(static_cast<const int8_t*>(dense), oc, ic, &nb);
+    need_w = need_d = static_cast<int64_t>(oc) * ic - z;
+  }
+  if (n_weights != need_w || n_diffs != need_d) return Fail(PL_ERR_BAD_ARG, "output arrays must hold %lld weights and %lld diffs", static_cast<long long>(need_w), static_cast<long long>(need_d));
+  if (need_w > 0 && (!nonzero_weights || !diffs)) return Fail(PL_ERR_BAD_ARG, "null output array");
+  std::memset(oc_nonzeros, 0, sizeof(uint32_t) * oc);  // semi writes only oc/2 + oc%2 entries
+  if (dtype == 0) return pl::PackWeights(static_cast<const float*>(dense), oc, ic, im_size, flag_semi != 0, static_cast<float*>(nonzero_weights), oc_nonzeros, diffs);
+  return pl::PackWeights(static_cast<const int8_t*>(dense), oc, ic, im_size, flag_semi != 0, static_cast<int8_t*>(nonzero_weights), oc_nonzeros, diffs);
+}
+
+}  // extern "C"

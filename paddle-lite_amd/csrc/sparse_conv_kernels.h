@@ -1,0 +1,90 @@
+// Launch interface of the gfx950 sparse 1x1 convolution kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace pl {
+
+// Output kinds of the kernels.
+enum : int { kOutF32 = 0, kOutI8 = 1, kOutAcc32 = 2 };
+
+struct DevAct {
+  int type;  // lite_api::ActivationType value: 1 relu, 2 relu6, 4 leaky, 10 hard_swish
+  float relu6_coef;
+  float leaky_alpha;
+  float hs_inv_scale;
+  float hs_offset;
+  float hs_threshold;
+};
+
+// One output row, or two rows that share an index list.
+struct DevGroup {
+  int row0;
+  int nrows;
+  uint32_t first;
+  uint32_t count;
+};
+
+// Row-walk SpMM: arguments common to all instantiations.
+struct WalkParams {
+  const void* x;
+  void* out;
+  const DevGroup* groups;
+  const uint32_t* kidx;  // per entry: input channel (fp32) or channel quad (int8)
+  const uint32_t* wts;   // per entry: 1 or 2 dwords (float bits / 4 packed int8)
+  const float* scale;    // int8 only
+  const float* bias;     // may be null
+  int n_groups;
+  int groups_per_slice;
+  int M, K;
+  int kd;                // LDS tile rows: K (fp32) or ceil(K/4) (int8)
+  int hw;
+  uint32_t P;            // batch * hw
+  int vec;               // 1: hw % 4 == 0 and pointers 16-byte aligned
+  DevAct act;
+};
+
+struct WalkConfig {
+  bool int8;       // activations / weights are int8
+  int out_kind;    // kOutF32 / kOutI8 / kOutAcc32
+  int nrows;       // 1 unstructured, 2 semi
+  int tile_pos;    // positions per workgroup tile: 16, 32, 64, 128 or 256
+  int threads;     // 256, 512 or 1024
+  int slices;      // grid.y
+};
+
+hipError_t LaunchRowWalk(const WalkConfig& cfg, const WalkParams& p, hipStream_t stream);
+
+// Block MFMA SpMM (int8): dense 32x32 weight blocks pre-arranged in operand
+// order, empty blocks skipped through a per-row-block bit mask.
+struct MfmaParams {
+  const int8_t* x;
+  void* out;
+  const void* wblocks;     // [row_blocks][ksteps][64 lanes][16 bytes]
+  const uint32_t* kmask;   // [row_blocks] bit ks set = block (rb, ks) has a nonzero
+  const float* scale;      // padded to 32 * row_blocks
+  const float* bias;       // padded likewise (zeros when the op has no bias)
+  int row_blocks;
+  int ksteps;              // ceil(K / 32)
+  int M, K;
+  int hw;
+  uint32_t P;
+  int vec;
+  DevAct act;
+};
+
+struct MfmaConfig {
+  int out_kind;
+  int ks_max;   // 2, 4, 8, 16 or 32 (>= ksteps)
+  int waves;    // row blocks per workgroup: 4, 8 or 16
+};
+
+hipError_t LaunchBlockMfma(const MfmaConfig& cfg, const MfmaParams& p, hipStream_t stream);
+
+// Largest dynamic LDS size a kernel of this library may be given.
+constexpr int kMaxLdsBytes = 160 * 1024;
+constexpr int kMfmaTilePos = 128;
+
+}  // namespace pl

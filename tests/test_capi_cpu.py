@@ -1,0 +1,134 @@
+"""CPU-side checks of the shipped library: it loads, exports every symbol the
+header declares, its host packers agree with the oracle bit for bit, and it
+refuses to compute without a device (no CPU fallback)."""
+import ctypes as C
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+
+from helpers import capi, pla, workloads
+from oracle import oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "pl_sparse_conv.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pl_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_functions()
+    assert len(names) >= 11
+    L = capi.lib()
+    for n in names:
+        assert hasattr(L, n), "libpl_sparse_conv.so does not export %s" % n
+    assert sorted(capi.EXPORTS) == names
+    assert L.pl_sparse_conv_abi_version() == capi.ABI_VERSION
+
+
+def test_struct_layout_matches_header():
+    # pl_sparse_conv_desc: 8 x int32, then pointers / int64, then the 24-byte activation
+    assert C.sizeof(capi.Activation) == 24
+    assert C.sizeof(capi.Desc) == 8 * 4 + 7 * 8 + 24
+    assert C.sizeof(capi.Info) == 4 * 4 + 6 * 8 or C.sizeof(capi.Info) == 3 * 4 + 4 + 6 * 8
+
+
+def _rand(rng, oc, ic, density, dtype, paired):
+    if paired:
+        m = np.repeat(rng.random_sample(((oc + 1) // 2, ic)) < density, 2, axis=0)[:oc]
+    else:
+        m = rng.random_sample((oc, ic)) < density
+    v = rng.randint(1, 100, size=(oc, ic))
+    return (v * m).astype(dtype)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.int8])
+def test_host_packers_equal_oracle_packers(dtype):
+    rng = np.random.RandomState(17)
+    for trial in range(120):
+        oc, ic, n = int(rng.randint(1, 20)), int(rng.randint(1, 30)), int(rng.randint(1, 60))
+        w = _rand(rng, oc, ic, rng.choice([0.0, 0.1, 0.4, 1.0]), dtype, paired=bool(trial % 2))
+        if oc > 2:
+            w[rng.randint(0, oc)] = 0
+        for force in (None, True, False):
+            got = pla.detect_and_pack(w, n, force_semi=force)
+            if force is None:
+                want = O.pack_like_pass(w, n)
+            elif force:
+                want = O.pack(w, n, O.LAYOUT_SEMI)
+            else:
+                want = O.pack(w, n, O.LAYOUT_PADDED if dtype == np.float32 else O.LAYOUT_UNPADDED)
+            assert got.flag_semi == want.flag_semi and got.first_ic == want.first_ic
+            assert np.array_equal(got.nonzero_weights, want.nonzero_weights)
+            assert np.array_equal(got.oc_nonzeros, want.oc_nonzeros)
+            assert np.array_equal(got.diffs, want.diffs)
+
+
+def test_host_packers_known_answers():
+    kat = json.load(open(os.path.join(ROOT, "tests", "golden", "packer_kat.json")))
+    for case in kat["cases"]:
+        w = np.array(case["dense"], dtype=case["dtype"]).reshape(case["rows"], case["cols"])
+        got = pla.detect_and_pack(w, kat["im_size"])
+        assert got.flag_semi == case["flag_semi"] and got.first_ic == case["first_ic"]
+        assert got.nonzero_weights.tolist() == case["nonzero_weights"]
+        assert got.diffs.tolist() == case["diffs"]
+        used = case.get("oc_nonzeros", case.get("oc_nonzeros_used"))
+        assert got.oc_nonzeros[:len(used)].tolist() == used
+
+
+def test_sparse_threshold_gate():
+    # the pass skips a conv whose zero fraction is below the threshold
+    # (sparse_conv_detect_pass.cc:684-692); for the semi layout the stored
+    # zero partners count as nonzeros
+    w = np.zeros((4, 10), np.float32)
+    w[:, :3] = 1.0  # 70 % zeros
+    assert pla.detect_and_pack(w, 9, sparse_threshold=0.71) is None
+    assert pla.detect_and_pack(w, 9, sparse_threshold=0.70) is not None
+    with pytest.raises(ValueError):
+        pla.detect_and_pack(w, 9, sparse_threshold=1.5)
+    assert pla.detect_and_pack(np.ones((4, 10, 3, 3), np.float32), 9) is None  # not a 1x1 kernel
+
+
+def test_unknown_activation_is_fatal():
+    with pytest.raises(ValueError):
+        pla.ActivationParam("sigmoid")
+
+
+def test_weight_scale_size_is_checked():
+    w = pla.detect_and_pack(_rand(np.random.RandomState(0), 6, 8, 0.5, np.int8, False), 4)
+    p = pla.SparseConvParam(w, enable_int8=True, weight_scale=[0.1, 0.2])
+    with pytest.raises(ValueError, match="weights scale size"):
+        pla.SparseConvKernel(p, "int8", "float32").PrepareForRun()
+
+
+def test_no_device_no_compute():
+    """Without a gfx950 device the library must fail loudly, never compute on
+    the CPU."""
+    import torch
+
+    if torch.cuda.is_available():
+        pytest.skip("a device is present")
+    assert capi.lib().pl_device_count() == 0
+    case = workloads.make_int8("t", 1, 8, 4, 2, 2, 0.5, False, pla.ActivationParam(), False, seed=0)
+    w = pla.detect_and_pack(case.dense, 4)
+    p = pla.SparseConvParam(w, enable_int8=True, weight_scale=case.weight_scale, input_scale=0.01)
+    with pytest.raises(capi.SparseConvError) as e:
+        pla.SparseConvKernel(p, "int8", "float32").PrepareForRun()
+    assert e.value.code == capi.PL_ERR_NO_DEVICE
+
+
+def test_workloads_are_seeded_and_shaped():
+    a, b = workloads.config3(batch=2), workloads.config3(batch=2)
+    assert np.array_equal(a.x, b.x) and np.array_equal(a.dense, b.dense)
+    assert a.dense.shape == (512, 512) and a.x.shape == (2, 512, 14, 14)
+    assert abs(1 - a.nnz / (512 * 512.0) - 0.85) < 0.01
+    c4 = workloads.config4(batch=1)
+    assert O.count_semi(c4.dense)["flag_semi"] == 1 and O.count_semi(a.dense)["flag_semi"] == 0
+    c2 = workloads.config2(batch=1)
+    assert O.count_semi(c2.dense)["flag_semi"] == 1 and c2.dense.dtype == np.float32
+    assert len(workloads.MOBILENET_V1_POINTWISE) == 13

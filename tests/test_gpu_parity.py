@@ -1,0 +1,203 @@
+"""Parity of the HIP kernels (called through the C ABI) with the CPU oracle on
+identical seeded inputs: int8 paths bit-exact, fp32 within 1e-5 relative."""
+import sys
+
+import numpy as np
+import pytest
+
+from helpers import capi, workloads, pla, make_kernel, run_hip, run_oracle, oracle_pack, assert_same, merged_for_oracle
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+AP = pla.ActivationParam
+ACTS = {
+    "none": AP(),
+    "relu": AP("relu"),
+    "relu6": AP("relu6", Relu_clipped_coef=6.0),
+    "leaky": AP("leaky_relu", Leaky_relu_alpha=0.1),
+    "hswish": AP("hard_swish"),
+}
+ALGOS = {"walk": capi.ALGO_ROW_WALK, "mfma": capi.ALGO_BLOCK_MFMA}
+
+
+def announce(*what):
+    print("CASE", *what, file=sys.stderr, flush=True)
+
+
+def small_case(kind, batch, ic, oc, h, w, sparsity, paired, act, seed, output_scale=1.0):
+    if kind == capi.KIND_FP32:
+        return workloads.make_fp32("t", batch, ic, oc, h, w, sparsity, paired, act, seed=seed)
+    c = workloads.make_int8("t", batch, ic, oc, h, w, sparsity, paired, act, out_int8=(kind == capi.KIND_INT8_INT8), seed=seed, output_scale=output_scale)
+    c.kind = kind
+    return c
+
+
+def test_library_sees_the_device():
+    assert capi.lib().pl_device_count() >= 1
+
+
+# (batch, ic, oc, h, w): aligned and ragged spatial sizes, channel counts off
+# the 4 / 32 grids, odd output channels, single pixel, single channel
+SHAPES = [(2, 64, 64, 4, 4), (3, 37, 29, 7, 7), (1, 96, 48, 8, 6), (2, 130, 67, 5, 3), (1, 1, 1, 1, 1), (5, 8, 33, 1, 1), (1, 512, 40, 14, 14)]
+
+
+@pytest.mark.parametrize("algo", ["walk", "mfma"])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
+def test_int32_accumulators_bit_exact(shape, paired, algo):
+    announce("acc", shape, paired, algo)
+    batch, ic, oc, h, w = shape
+    case = small_case(capi.KIND_INT8_ACC32, batch, ic, oc, h, w, 0.7, paired, AP(), seed=ic * 7 + oc)
+    got = run_hip(case, ALGOS[algo], force_semi=paired)
+    want = run_oracle(case, oracle_pack(case, force_semi=paired))
+    assert_same(case, got, want, "int32 accumulators")
+    # independent of both: plain integer matmul
+    ref = np.einsum("mk,bkp->bmp", case.dense.astype(np.int64), case.x.reshape(batch, ic, -1).astype(np.int64)).reshape(got.shape)
+    assert np.array_equal(got.astype(np.int64), ref)
+
+
+@pytest.mark.parametrize("algo", ["walk", "mfma"])
+@pytest.mark.parametrize("act", sorted(ACTS))
+@pytest.mark.parametrize("out_int8", [False, True], ids=["fp32out", "int8out"])
+@pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
+def test_int8_outputs_bit_exact(paired, out_int8, act, algo):
+    announce("int8", paired, out_int8, act, algo)
+    kind = capi.KIND_INT8_INT8 if out_int8 else capi.KIND_INT8_FP32
+    for shape in [(2, 72, 45, 6, 6), (2, 50, 31, 5, 5)]:
+        batch, ic, oc, h, w = shape
+        case = small_case(kind, batch, ic, oc, h, w, 0.8, paired, ACTS[act], seed=11 + ic, output_scale=0.05 if out_int8 else 1.0)
+        got = run_hip(case, ALGOS[algo], force_semi=paired)
+        want = run_oracle(case, oracle_pack(case, force_semi=paired))
+        assert_same(case, got, want, "int8 %s %s" % (act, shape))
+        if out_int8:
+            assert np.abs(got.astype(int)).max() <= 127
+
+
+@pytest.mark.parametrize("act", sorted(ACTS))
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
+def test_fp32_within_tolerance(shape, paired, act):
+    announce("fp32", shape, paired, act)
+    batch, ic, oc, h, w = shape
+    case = small_case(capi.KIND_FP32, batch, ic, oc, h, w, 0.8, paired, ACTS[act], seed=ic + 3 * oc)
+    got = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired)
+    want = run_oracle(case, oracle_pack(case, force_semi=paired))
+    assert_same(case, got, want, "fp32 %s" % act)
+    # and against the dense naive reference formula in float64
+    if act == "none":
+        ref = np.einsum("mk,bkp->bmp", case.dense.astype(np.float64), case.x.reshape(batch, ic, -1).astype(np.float64)) + case.bias[None, :, None]
+        np.testing.assert_allclose(got.reshape(batch, oc, -1), ref, rtol=1e-4, atol=1e-5)
+
+
+def test_no_bias_and_single_scale():
+    announce("nobias")
+    for kind in (capi.KIND_FP32, capi.KIND_INT8_FP32, capi.KIND_INT8_INT8):
+        case = small_case(kind, 2, 40, 24, 4, 4, 0.6, False, ACTS["relu"], seed=5, output_scale=0.04 if kind == capi.KIND_INT8_INT8 else 1.0)
+        case.bias = None
+        if kind != capi.KIND_FP32:
+            case.weight_scale = np.array([0.01], np.float32)
+        for algo in ([capi.ALGO_ROW_WALK] if kind == capi.KIND_FP32 else [capi.ALGO_ROW_WALK, capi.ALGO_BLOCK_MFMA]):
+            assert_same(case, run_hip(case, algo), run_oracle(case), "kind %d algo %d" % (kind, algo))
+
+
+def test_empty_rows_all_zero_and_dense():
+    announce("empty/dense")
+    rng = np.random.RandomState(3)
+    for kind in (capi.KIND_FP32, capi.KIND_INT8_FP32):
+        case = small_case(kind, 2, 36, 20, 4, 4, 0.7, False, ACTS["leaky"], seed=9)
+        case.dense[[0, 3, 19]] = 0  # empty first, middle and last rows
+        for algo in ([capi.ALGO_ROW_WALK] if kind == capi.KIND_FP32 else [capi.ALGO_ROW_WALK, capi.ALGO_BLOCK_MFMA]):
+            assert_same(case, run_hip(case, algo), run_oracle(case), "empty rows")
+        zero = small_case(kind, 1, 12, 6, 4, 4, 0.5, False, ACTS["none"], seed=1)
+        zero.dense[:] = 0
+        for algo in ([capi.ALGO_ROW_WALK] if kind == capi.KIND_FP32 else [capi.ALGO_ROW_WALK, capi.ALGO_BLOCK_MFMA]):
+            got = run_hip(zero, algo)
+            assert_same(zero, got, run_oracle(zero), "all-zero weights")
+        full = small_case(kind, 1, 16, 8, 4, 4, 0.0, False, ACTS["none"], seed=2)
+        assert np.count_nonzero(full.dense) == full.dense.size
+        assert_same(full, run_hip(full, capi.ALGO_ROW_WALK), run_oracle(full), "fully dense weights")
+    del rng
+
+
+def test_runtime_spatial_size_may_differ_from_baked_one():
+    """Diffs are byte offsets baked for one H*W; the library converts them to
+    channel indices once, so a handle serves any spatial size and batch."""
+    announce("respatial")
+    case = small_case(capi.KIND_INT8_FP32, 1, 48, 32, 4, 4, 0.75, False, ACTS["relu"], seed=21)
+    kernel, _ = make_kernel(case)
+    for (b, h, w) in [(1, 4, 4), (3, 7, 5), (2, 8, 8), (4, 1, 3)]:
+        x = np.random.RandomState(b * 100 + h).randint(-127, 128, size=(b, 48, h, w)).astype(np.int8)
+        got = run_hip(case, kernel=kernel, x=x)
+        pk = O.pack_like_pass(case.dense, h * w)  # the oracle needs Diffs for this size
+        want = run_oracle(case, pk, x=x)
+        assert_same(case, got, want, "spatial %dx%d batch %d" % (h, w, b))
+
+
+def test_set_epilogue_replaces_scales():
+    import ctypes as C
+
+    announce("set_epilogue")
+    case = small_case(capi.KIND_INT8_FP32, 2, 32, 16, 4, 4, 0.7, False, ACTS["relu"], seed=4)
+    kernel, _ = make_kernel(case)
+    new_ws = np.linspace(0.002, 0.01, 16).astype(np.float32)
+    merged = (new_ws * np.float32(case.input_scale)).astype(np.float32)
+    capi.check(capi.lib().pl_sparse_conv_set_epilogue(kernel._handle, merged.ctypes.data, None, None))
+    case.weight_scale = new_ws
+    assert_same(case, run_hip(case, kernel=kernel), run_oracle(case), "after set_epilogue")
+    del C
+
+
+@pytest.mark.parametrize("quirks", [True, False], ids=["reference_quirks", "scaled_once"])
+@pytest.mark.parametrize("act", ["relu6", "leaky", "hswish"])
+def test_kernel_class_parameter_merging(act, quirks):
+    """SparseConvKernel.PrepareForRun against the merging written out with
+    numpy in helpers.merged_for_oracle (int8 -> int8, where it matters)."""
+    announce("merge", act, quirks)
+    case = small_case(capi.KIND_INT8_INT8, 2, 64, 32, 4, 4, 0.7, False, ACTS[act], seed=31, output_scale=0.05)
+    got = run_hip(case, quirks=quirks)
+    want = run_oracle(case, quirks=quirks)
+    assert_same(case, got, want, "merged %s" % act)
+    # the oracle's own restatement of PrepareForRun agrees on scale and bias
+    ms, mb, _ = O.merge_params(2, 32, case.weight_scale, case.input_scale, case.output_scale, case.bias, None)
+    s, b, _ = merged_for_oracle(case, quirks)
+    assert np.array_equal(ms, s) and np.array_equal(mb, b)
+
+
+def test_error_paths_return_codes():
+    import ctypes as C
+
+    announce("errors")
+    L = capi.lib()
+    case = small_case(capi.KIND_INT8_FP32, 1, 16, 8, 2, 2, 0.5, False, ACTS["none"], seed=1)
+    w = pla.detect_and_pack(case.dense, 4)
+    d = capi.Desc()
+    d.struct_size = C.sizeof(capi.Desc)
+    d.kind, d.flag_semi, d.first_ic, d.oc, d.ic, d.im_size = capi.KIND_INT8_FP32, 0, w.first_ic, 8, 16, 4
+    d.nonzero_weights, d.n_weights = w.nonzero_weights.ctypes.data, w.nonzero_weights.size
+    d.oc_nonzeros, d.diffs, d.n_diffs = w.oc_nonzeros.ctypes.data, w.diffs.ctypes.data, w.diffs.size
+    scale = np.ones(8, np.float32)
+    d.scale = scale.ctypes.data
+    h = C.c_void_p()
+    # corrupt index: walk leaves the channels
+    bad = w.diffs.copy()
+    bad[0] = 4 * 1000
+    d.diffs = bad.ctypes.data
+    assert L.pl_sparse_conv_prepare(C.byref(d), C.byref(h)) == capi.PL_ERR_BAD_LAYOUT and not h.value
+    assert "channels" in capi.last_error()
+    bad[0] = 3  # not a multiple of im_size
+    assert L.pl_sparse_conv_prepare(C.byref(d), C.byref(h)) == capi.PL_ERR_BAD_LAYOUT
+    d.diffs = w.diffs.ctypes.data
+    d.scale = None
+    assert L.pl_sparse_conv_prepare(C.byref(d), C.byref(h)) == capi.PL_ERR_BAD_ARG
+    d.scale = scale.ctypes.data
+    d.struct_size = 8
+    assert L.pl_sparse_conv_prepare(C.byref(d), C.byref(h)) == capi.PL_ERR_BAD_ARG
+    d.struct_size = C.sizeof(capi.Desc)
+    d.kind, d.algo = capi.KIND_FP32, capi.ALGO_BLOCK_MFMA
+    assert L.pl_sparse_conv_prepare(C.byref(d), C.byref(h)) == capi.PL_ERR_UNSUPPORTED
+    d.kind, d.algo = capi.KIND_INT8_FP32, capi.ALGO_AUTO
+    assert L.pl_sparse_conv_prepare(C.byref(d), C.byref(h)) == capi.PL_OK and h.value
+    assert L.pl_sparse_conv_run(h, None, None, 1, 4, None) == capi.PL_ERR_BAD_ARG
+    assert L.pl_sparse_conv_run(h, None, None, 0, 4, None) == capi.PL_OK  # empty batch
+    L.pl_sparse_conv_destroy(h)
