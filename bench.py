@@ -1,0 +1,211 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse_conv2d hot path on one MI355X.
+
+A step is one pass of the sparse 1x1 convolution over one batch of synthetic
+input that already lives in HBM.  The default workload is the metric
+configuration: int8 activations and weights, fp32 output, N=64, 512 -> 512
+channels at 14x14, 85 % unstructured zeros, per-channel scales, bias and
+leaky_relu.  Prints ONE JSON line.
+"""
+import argparse
+import ctypes as C
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+LLC_BYTES = 256 << 20  # last-level (Infinity) cache the rotation must exceed
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4"])
+    ap.add_argument("--algo", default="auto", choices=["auto", "walk", "mfma"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cache-resident", action="store_true", help="reuse one buffer set (reported, never the headline)")
+    return ap.parse_args()
+
+
+def cpu_baseline(case, packed, budget_s=12.0):
+    """The reference's CPU path on this host: its naive test reference (the
+    real header when oracle/_ref was built, else the restatement), and the
+    dense per-image GEMM that Paddle-Lite's x86 conv2d 1x1 performs."""
+    import numpy as np
+    from oracle import oracle as O
+    import helpers
+
+    cores = os.cpu_count() or 1
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except Exception:
+        pass
+    threads = int(os.environ.get("OMP_NUM_THREADS", cores))
+    oc, ic = case.dense.shape
+    hw = case.im_size
+    ops_img = 2.0 * case.nnz * hw
+    scale, bias, act = helpers.merged_for_oracle(case)
+    int8 = case.dense.dtype == np.int8
+    # naive path as the unit test runs it: dequantise, dense basic_gemm per image
+    if int8:
+        wf = O.int8_to_fp32(case.dense, 1.0)
+    else:
+        wf = case.dense
+    use_ref = O.have_ref()
+    gemm = (lambda a, b: O.ref_basic_gemm_f32(a, b, bias, act, omp=True)) if use_ref else (lambda a, b: O.basic_gemm_f32(a, b, bias, act))
+    xf0 = (O.int8_to_fp32(case.x[0], 1.0) if int8 else case.x[0]).reshape(ic, hw)
+    t = time.perf_counter()
+    gemm(wf, xf0)
+    one = time.perf_counter() - t
+    n_img = int(max(1, min(case.batch, budget_s / max(one, 1e-6))))
+    t = time.perf_counter()
+    for i in range(n_img):
+        xf = (O.int8_to_fp32(case.x[i], 1.0) if int8 else case.x[i]).reshape(ic, hw)
+        gemm(wf, xf)
+    naive_s = time.perf_counter() - t
+    naive = {
+        "value": ops_img * n_img / naive_s / 1e9,
+        "unit": "nnz-GOP/s",
+        "cores": threads if use_ref else 1,
+        "kind": "reference" if use_ref else "port",
+        "sample": "%d of %d images through the unit test's naive path (dequantise + dense basic_gemm per image, %s), %.2f s" % (n_img, case.batch, "reference header built with its own OpenMP pragmas" if use_ref else "restated, 1 thread", naive_s),
+        "dense_GOPs": 2.0 * oc * ic * hw * n_img / naive_s / 1e9,
+    }
+    # dense per-image GEMM over the batch, all cores (port of the x86 conv2d 1x1 structure)
+    kind = {helpers.capi.KIND_FP32: 0, helpers.capi.KIND_INT8_FP32: 1, helpers.capi.KIND_INT8_INT8: 2}[case.kind]
+    O.dense_conv1x1(kind, case.dense, case.x[:1], scale, bias, act, threads)
+    best, reps = None, 0
+    t_all = time.perf_counter()
+    while reps < 5 or (time.perf_counter() - t_all < 3.0 and reps < 50):
+        t = time.perf_counter()
+        _, used = O.dense_conv1x1(kind, case.dense, case.x, scale, bias, act, threads)
+        dt = time.perf_counter() - t
+        best = dt if best is None else min(best, dt)
+        reps += 1
+    naive["dense_port"] = {
+        "value": ops_img * case.batch / best / 1e9,
+        "unit": "nnz-GOP/s",
+        "dense_GOPs": 2.0 * oc * ic * hw * case.batch / best / 1e9,
+        "cores": used,
+        "kind": "port",
+        "ms": best * 1e3,
+        "sample": "full batch, best of %d, exact-accumulating blocked per-image GEMM with OpenMP" % reps,
+    }
+    del packed
+    return naive
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        sys.stderr.write("bench.py measures one GPU; --gpus %d is not supported (this path shards over images with no exchange, see DESIGN.md)\n" % args.gpus)
+        return 2
+    import numpy as np
+    import torch
+
+    import helpers
+
+    capi, wl = helpers.capi, helpers.workloads
+    if not torch.cuda.is_available():
+        sys.stderr.write("bench.py needs a GPU\n")
+        return 2
+    torch.cuda.set_device(0)
+    case = wl.CONFIGS[args.config]()
+    algo = {"auto": capi.ALGO_AUTO, "walk": capi.ALGO_ROW_WALK, "mfma": capi.ALGO_BLOCK_MFMA}[args.algo]
+    kernel, weights = helpers.make_kernel(case, algo=algo)
+    info = kernel.info()
+    ops = case.algorithmic_ops()
+    nbytes = case.algorithmic_bytes(weights)
+
+    # rotating buffer sets: footprint above the last-level cache
+    out_dtype = {capi.KIND_FP32: torch.float32, capi.KIND_INT8_FP32: torch.float32, capi.KIND_INT8_INT8: torch.int8}[case.kind]
+    oc = case.dense.shape[0]
+    set_bytes = case.x.nbytes + case.batch * oc * case.im_size * (1 if out_dtype == torch.int8 else 4)
+    n_sets = 1 if args.cache_resident else int(LLC_BYTES * 1.25 // set_bytes) + 1
+    x0 = torch.from_numpy(case.x).cuda()
+    xs = [x0] + [x0.clone() for _ in range(n_sets - 1)]
+    outs = [torch.empty((case.batch, oc) + tuple(case.x.shape[2:]), dtype=out_dtype, device="cuda") for _ in range(n_sets)]
+    xp = (C.c_void_p * n_sets)(*[t.data_ptr() for t in xs])
+    op = (C.c_void_p * n_sets)(*[t.data_ptr() for t in outs])
+    stream = torch.cuda.current_stream().cuda_stream
+    L = capi.lib()
+
+    def sequence(steps, timed):
+        ms = C.c_float(0.0)
+        capi.check(L.pl_sparse_conv_run_sequence(kernel._handle, xp, op, n_sets, case.batch, case.im_size, steps, C.c_void_p(stream), C.byref(ms) if timed else None))
+        return ms.value
+
+    # parity of what is being timed (first set) against the oracle on a slice
+    sequence(min(n_sets, 2), False)
+    torch.cuda.synchronize()
+    nchk = min(case.batch, 2)
+    want = helpers.run_oracle(case, x=case.x[:nchk])
+    got = outs[0][:nchk].cpu().numpy()
+    if case.kind == capi.KIND_FP32:
+        np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
+    else:
+        assert np.array_equal(got, want), "timed kernel output differs from the oracle"
+
+    sequence(args.warmup, False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev_ms = sequence(args.steps, True)  # events on the launch stream bracket exactly the timed steps
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    ms_per_step = wall * 1e3 / args.steps
+    kernel_ms = ev_ms / args.steps
+    achieved = nbytes / (kernel_ms * 1e-3) / 1e9
+    line = {
+        "metric": "sparse 1x1 conv nnz-GOP/s + % HBM roofline (int8, N=64, 512->512@14x14, 85%)",
+        "value": ops * args.steps / wall / 1e9,
+        "unit": "nnz-GOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32" if case.kind == capi.KIND_FP32 else "int8",
+        "data": "synthetic",
+        "config": {
+            "workload": case.name,
+            "shape": "N=%d %d->%d @%dx%d" % (case.batch, case.dense.shape[1], oc, case.x.shape[2], case.x.shape[3]),
+            "nnz": case.nnz,
+            "sparsity": 1.0 - case.nnz / float(case.dense.size),
+            "flag_semi": weights.flag_semi,
+            "algo": {capi.ALGO_ROW_WALK: "row_walk", capi.ALGO_BLOCK_MFMA: "block_mfma"}[info["algo"]],
+            "weight_blocks_present": [info["mfma_blocks"], info["mfma_blocks_total"]],
+            "buffer_sets": n_sets,
+            "rotation_MB": n_sets * set_bytes / 1e6,
+            "parity_checked": True,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": None,
+            "algorithmic_bytes_per_launch": nbytes,
+            "kernel_us": kernel_ms * 1e3,
+            "nnz_TOPs_kernel": ops / (kernel_ms * 1e-3) / 1e12,
+        },
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(case, weights)
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

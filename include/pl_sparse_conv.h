@@ -143,6 +143,20 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* handle, const void* x_dev,
                        void* out_dev, int32_t batch, int32_t im_size,
                        void* stream);
 
+/* The repeat loop of the reference's unit-test benchmark
+ * (lite/tests/math/sparse_conv_int8_compute_test.cc:285-360: warm-up, then
+ * `repeats` timed calls) as one call: enqueues `steps` runs back to back on
+ * `stream`, run i reading x_dev[i % n_sets] and writing out_dev[i % n_sets]
+ * (rotating buffers keep the working set out of the last-level cache).
+ * With elapsed_ms != NULL the runs are bracketed by two HIP events on
+ * `stream`, the call waits for the second one and stores the time between
+ * them in milliseconds. */
+int pl_sparse_conv_run_sequence(pl_sparse_conv_handle* handle,
+                                const void* const* x_dev, void* const* out_dev,
+                                int32_t n_sets, int32_t batch, int32_t im_size,
+                                int32_t steps, void* stream,
+                                float* elapsed_ms);
+
 int pl_sparse_conv_get_info(const pl_sparse_conv_handle* handle,
                             pl_sparse_conv_info* info);
 

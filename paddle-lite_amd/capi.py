@@ -18,6 +18,7 @@ EXPORTS = [
     "pl_device_count",
     "pl_sparse_conv_prepare",
     "pl_sparse_conv_run",
+    "pl_sparse_conv_run_sequence",
     "pl_sparse_conv_get_info",
     "pl_sparse_conv_set_epilogue",
     "pl_sparse_conv_destroy",
@@ -103,6 +104,8 @@ def lib():
     L.pl_sparse_conv_prepare.restype = C.c_int
     L.pl_sparse_conv_run.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]
     L.pl_sparse_conv_run.restype = C.c_int
+    L.pl_sparse_conv_run_sequence.argtypes = [C.c_void_p, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.POINTER(C.c_float)]
+    L.pl_sparse_conv_run_sequence.restype = C.c_int
     L.pl_sparse_conv_get_info.argtypes = [C.c_void_p, C.POINTER(Info)]
     L.pl_sparse_conv_get_info.restype = C.c_int
     L.pl_sparse_conv_set_epilogue.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Activation)]

@@ -380,13 +380,13 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.hw = im_size;
     p.P = P;
     p.vec = vec;
+    p.small = (P64 * h->ic < (1ll << 31)) && (P64 * h->oc * 4 < (1ll << 31));
     p.act = h->act;
     pl::MfmaConfig c{};
     c.out_kind = OutKind(h->kind);
     c.ks_max = 2;
     while (c.ks_max < h->ksteps) c.ks_max <<= 1;
-    c.waves = c.ks_max >= 32 ? 4 : std::min(4, h->row_blocks);
-    if (c.waves < 1) c.waves = 1;
+    c.waves = 4;  // the kernel's thread mapping is written for 256 threads
     e = pl::LaunchBlockMfma(c, p, s);
   } else {
     pl::WalkParams p{};
@@ -412,6 +412,33 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
   }
   if (e != hipSuccess) return FailHip(e, "kernel launch");
   return PL_OK;
+}
+
+int pl_sparse_conv_run_sequence(pl_sparse_conv_handle* h, const void* const* x_dev, void* const* out_dev, int32_t n_sets, int32_t batch, int32_t im_size, int32_t steps, void* stream, float* elapsed_ms) {
+  if (!h || !x_dev || !out_dev || n_sets <= 0 || steps < 0) return Fail(PL_ERR_BAD_ARG, "bad sequence arguments");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipEvent_t t0 = nullptr, t1 = nullptr;
+  if (elapsed_ms) {
+    hipError_t e = hipEventCreate(&t0);
+    if (e == hipSuccess) e = hipEventCreate(&t1);
+    if (e == hipSuccess) e = hipEventRecord(t0, s);
+    if (e != hipSuccess) {
+      if (t0) (void)hipEventDestroy(t0);
+      if (t1) (void)hipEventDestroy(t1);
+      return FailHip(e, "creating timing events");
+    }
+  }
+  int rc = PL_OK;
+  for (int i = 0; i < steps && rc == PL_OK; ++i) rc = pl_sparse_conv_run(h, x_dev[i % n_sets], out_dev[i % n_sets], batch, im_size, stream);
+  if (elapsed_ms) {
+    hipError_t e = hipEventRecord(t1, s);
+    if (e == hipSuccess) e = hipEventSynchronize(t1);
+    if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    if (rc == PL_OK && e != hipSuccess) rc = FailHip(e, "timing the sequence");
+  }
+  return rc;
 }
 
 int pl_sparse_conv_get_info(const pl_sparse_conv_handle* h, pl_sparse_conv_info* info) {

@@ -72,6 +72,9 @@ struct MfmaParams {
   int hw;
   uint32_t P;
   int vec;
+  int small;               // 1: input and output tensors are each below 2 GB
+  int tiles;               // filled in by the launcher: position tiles
+  int row_groups;          // and groups of four row blocks
   DevAct act;
 };
 

@@ -24,12 +24,30 @@
 #include "sparse_conv_kernels.h"
 
 #include <atomic>
+#include <type_traits>
+
+// Phase marks for tuning builds; compiled out of the library.
+#ifndef PL_PHASE_MARK
+#define PL_PHASE_MARK(i)
+#endif
 
 namespace pl {
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// Outputs are written once and never read back by the kernel: store them
+// non-temporally so that they stream to memory instead of sitting dirty in
+// L2 until the end-of-kernel write-back.
+__device__ __forceinline__ void StreamStore(float4 v, void* dst) {
+  __builtin_nontemporal_store(v4f{v.x, v.y, v.z, v.w}, static_cast<v4f*>(dst));
+}
+__device__ __forceinline__ void StreamStore(int4 v, void* dst) {
+  __builtin_nontemporal_store(v4i{v.x, v.y, v.z, v.w}, static_cast<v4i*>(dst));
+}
+__device__ __forceinline__ void StreamStore(uint32_t v, void* dst) { __builtin_nontemporal_store(v, static_cast<uint32_t*>(dst)); }
 
 // ---------------------------------------------------------------- epilogue
 __device__ __forceinline__ float Activate(float v, const DevAct& a) {
@@ -46,6 +64,41 @@ __device__ __forceinline__ float Activate(float v, const DevAct& a) {
     }
     default:
       return v;
+  }
+}
+
+// Same, with the activation fixed at compile time; DispatchAct turns the
+// run-time type into that constant once per kernel instead of once per value.
+template <int ACT>
+__device__ __forceinline__ float ActivateT(float v, const DevAct& a) {
+  if (ACT == 1) return fmaxf(v, 0.0f);
+  if (ACT == 2) return fminf(fmaxf(v, 0.0f), a.relu6_coef);
+  if (ACT == 4) return (v >= 0.0f) ? v : v * a.leaky_alpha;
+  if (ACT == 10) {
+    float gate = fminf(fmaxf(v + a.hs_offset, 0.0f), a.hs_threshold);
+    return (v * a.hs_inv_scale) * gate;
+  }
+  return v;
+}
+
+template <typename F>
+__device__ __forceinline__ void DispatchAct(int type, F&& f) {
+  switch (type) {
+    case 1:
+      f(std::integral_constant<int, 1>());
+      break;
+    case 2:
+      f(std::integral_constant<int, 2>());
+      break;
+    case 4:
+      f(std::integral_constant<int, 4>());
+      break;
+    case 10:
+      f(std::integral_constant<int, 10>());
+      break;
+    default:
+      f(std::integral_constant<int, 0>());
+      break;
   }
 }
 
@@ -285,79 +338,222 @@ __global__ void __launch_bounds__(1024) RowWalkKernel(const WalkParams p) {
 // slot = c*32 + j holds position 4*j + c of the 128-position tile, so that
 // MFMA column j of the four accumulators c = 0..3 are four consecutive
 // positions of one output row (one 16-byte fp32 store, one dword int8 store).
-template <int KSMAX, int OUT>
-__global__ void __launch_bounds__(KSMAX >= 32 ? 256 : 512) BlockMfmaKernel(const MfmaParams p) {
-  extern __shared__ uint4 xt[];
-  const int tid = threadIdx.x;
-  const int nthreads = blockDim.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int nwaves = nthreads >> 6;
-  const uint32_t tile0 = blockIdx.x * (uint32_t)kMfmaTilePos;
-  const int rb = blockIdx.y * nwaves + wave;
-  const bool wave_on = rb < p.row_blocks;
 
-  // weight blocks of this wavefront's 32 rows -> registers
-  const uint32_t kmask = wave_on ? p.kmask[rb] : 0u;
-  v4i a[KSMAX];
+// Stage with aligned dword loads (hw % 4 == 0).  Every load is unconditional
+// so that all loads of a batch are in flight together.  FAST: all channel
+// groups of the batch are complete, the tile lies inside the tensor and the
+// tensor is below 2 GB, so an address is a uniform base plus one 32-bit
+// per-lane offset (no per-load address arithmetic on the vector ALU).
+// Otherwise addresses are clamped and the results masked.
+template <int UNITS, bool FAST>
+__device__ __forceinline__ void StageMfmaVec(uint4* xt, const MfmaParams& p, uint32_t tile0, int kg_base, int kg_lane, int j) {
+  const int n_kg = 2 * p.ksteps;
+  const uint32_t g = tile0 + 4u * j;
+  const bool live = FAST || g < p.P;
+  const uint32_t gs = live ? g : 0u;
+  const uint32_t n = gs / (uint32_t)p.hw, pp = gs % (uint32_t)p.hw;
+  uint32_t r[UNITS][16];
+  if (FAST) {
+    const uint32_t voff = (n * (uint32_t)p.K + 16u * (uint32_t)kg_lane) * (uint32_t)p.hw + pp;
 #pragma unroll
-  for (int ks = 0; ks < KSMAX; ++ks) {
-    a[ks] = v4i{0, 0, 0, 0};
-    if (kmask & (1u << ks)) {
-      a[ks] = static_cast<const v4i*>(p.wblocks)[((size_t)rb * p.ksteps + ks) * 64 + lane];
+    for (int u = 0; u < UNITS; ++u) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int8_t* sbase = p.x + (size_t)(16 * (kg_base + 8 * u) + i) * (size_t)p.hw;  // uniform
+        r[u][i] = *reinterpret_cast<const uint32_t*>(sbase + voff);
+      }
+    }
+  } else {
+    const int8_t* col = p.x + (size_t)n * p.K * p.hw + pp;
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u) {
+      const int kg = kg_base + kg_lane + 8 * u;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int ch = min(16 * kg + i, p.K - 1);
+        r[u][i] = *reinterpret_cast<const uint32_t*>(col + (size_t)ch * p.hw);
+      }
     }
   }
+#pragma unroll
+  for (int u = 0; u < UNITS; ++u) {
+    const int kg = kg_base + kg_lane + 8 * u;
+    if (!FAST) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) r[u][i] = (live && 16 * kg + i < p.K) ? r[u][i] : 0u;
+    }
+#pragma unroll
+    for (int b = 0; b < 4; ++b) Transpose4x4(r[u][4 * b], r[u][4 * b + 1], r[u][4 * b + 2], r[u][4 * b + 3]);
+    // now r[u][4b + c] = channels 16kg+4b..+3 of position 4j+c
+    if (FAST || kg < n_kg) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) xt[(size_t)kg * kMfmaTilePos + c * 32 + j] = make_uint4(r[u][c], r[u][4 + c], r[u][8 + c], r[u][12 + c]);
+    }
+  }
+}
 
-  // ---- stage 128 positions x (32*ksteps) channels, transposed to
-  //      channel-innermost
-  {
-    const int j = tid & 31;               // position quad of the tile
-    const int kg0 = tid >> 5;             // first channel group of this thread
-    const int kg_step = nthreads >> 5;
-    const int n_kg = 2 * p.ksteps;
-    const uint32_t g = tile0 + 4u * j;
-    if (p.vec) {
-      const bool live = g < p.P;
-      const uint32_t n = live ? g / (uint32_t)p.hw : 0u;
-      const uint32_t pp = live ? g % (uint32_t)p.hw : 0u;
-      const int8_t* col = p.x + (size_t)n * p.K * p.hw + pp;
-      for (int kg = kg0; kg < n_kg; kg += kg_step) {
-        uint32_t r[16];
+// Any hw: byte loads.
+__device__ __forceinline__ void StageMfmaBytes(uint4* xt, const MfmaParams& p, uint32_t tile0, int kg0, int kg_step, int j) {
+  const int n_kg = 2 * p.ksteps;
+  const uint32_t g = tile0 + 4u * j;
+  for (int kg = kg0; kg < n_kg; kg += kg_step) {
+    for (int c = 0; c < 4; ++c) {
+      const uint32_t gc = g + c;
+      uint32_t d[4] = {0, 0, 0, 0};
+      if (gc < p.P) {
+        const uint32_t n = gc / (uint32_t)p.hw, pp = gc % (uint32_t)p.hw;
+        const int8_t* col = p.x + (size_t)n * p.K * p.hw + pp;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const int ch = 16 * kg + i;
-          r[i] = (live && ch < p.K) ? *reinterpret_cast<const uint32_t*>(col + (size_t)ch * p.hw) : 0u;
-        }
-#pragma unroll
-        for (int b = 0; b < 4; ++b) Transpose4x4(r[4 * b], r[4 * b + 1], r[4 * b + 2], r[4 * b + 3]);
-        // after the transposes r[4b + c] = channels 16kg+4b..+3 of position 4j+c
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          xt[(size_t)kg * kMfmaTilePos + c * 32 + j] = make_uint4(r[c], r[4 + c], r[8 + c], r[12 + c]);
+          const uint32_t b = (ch < p.K) ? (uint32_t)(uint8_t)col[(size_t)ch * p.hw] : 0u;
+          d[i >> 2] |= b << (8 * (i & 3));
         }
       }
+      xt[(size_t)kg * kMfmaTilePos + c * 32 + j] = make_uint4(d[0], d[1], d[2], d[3]);
+    }
+  }
+}
+
+// Accumulator register r of lane l is output row 8*(r/4) + 4*(l/32) + r%4 of
+// the 32-row block, column l%32; the four accumulators are four consecutive
+// positions.
+template <int OUT, int ACT, bool VEC>
+__device__ __forceinline__ void MfmaEpilogue(const MfmaParams& p, const v16i (&acc)[4], int rb, int lane, uint32_t tile0) {
+  const uint32_t g = tile0 + 4u * (lane & 31);
+  if (g >= p.P) return;
+  const uint32_t n = g / (uint32_t)p.hw, pp = g % (uint32_t)p.hw;
+  const int row_base = rb * 32 + 4 * (lane >> 5);
+  if (VEC && p.small && rb * 32 + 32 <= p.M) {
+    // all 32 rows exist and byte offsets fit 32 bits: uniform row base plus
+    // one per-lane offset
+    constexpr uint32_t kElem = OUT == kOutI8 ? 1u : 4u;
+    const uint32_t voff = ((n * (uint32_t)p.M + (uint32_t)row_base) * (uint32_t)p.hw + pp) * kElem;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int ro = 8 * (r >> 2) + (r & 3);
+      char* dst = static_cast<char*>(p.out) + (size_t)ro * (size_t)p.hw * kElem + voff;
+      int q[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) q[c] = acc[c][r];
+      if (OUT == kOutAcc32) {
+        StreamStore(make_int4(q[0], q[1], q[2], q[3]), dst);
+      } else {
+        const float s = p.scale[row_base + ro], b = p.bias[row_base + ro];
+        float v[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) v[c] = ActivateT<ACT>(__builtin_fmaf((float)q[c], s, b), p.act);
+        if (OUT == kOutF32) {
+          StreamStore(make_float4(v[0], v[1], v[2], v[3]), dst);
+        } else {
+          uint32_t w = (uint32_t)(QuantizeI8(v[0]) & 0xff) | ((uint32_t)(QuantizeI8(v[1]) & 0xff) << 8) |
+                       ((uint32_t)(QuantizeI8(v[2]) & 0xff) << 16) | ((uint32_t)(QuantizeI8(v[3]) & 0xff) << 24);
+          StreamStore(w, dst);
+        }
+      }
+    }
+    return;
+  }
+  float sc[16], bi[16];
+  if (OUT != kOutAcc32) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = row_base + 8 * (r >> 2) + (r & 3);  // scale / bias are padded to 32 rows per block
+      sc[r] = p.scale[row];
+      bi[r] = p.bias[row];
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int row = row_base + 8 * (r >> 2) + (r & 3);
+    if (row >= p.M) continue;
+    float v[4];
+    int q[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) q[c] = acc[c][r];
+    if (OUT != kOutAcc32) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) v[c] = ActivateT<ACT>(__builtin_fmaf((float)q[c], sc[r], bi[r]), p.act);
+    }
+    if (VEC) {
+      const size_t idx = ((size_t)n * p.M + row) * p.hw + pp;
+      if (OUT == kOutF32) {
+        *reinterpret_cast<float4*>(static_cast<float*>(p.out) + idx) = make_float4(v[0], v[1], v[2], v[3]);
+      } else if (OUT == kOutI8) {
+        uint32_t w = (uint32_t)(QuantizeI8(v[0]) & 0xff) | ((uint32_t)(QuantizeI8(v[1]) & 0xff) << 8) |
+                     ((uint32_t)(QuantizeI8(v[2]) & 0xff) << 16) | ((uint32_t)(QuantizeI8(v[3]) & 0xff) << 24);
+        *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(p.out) + idx) = w;
+      } else {
+        *reinterpret_cast<int4*>(static_cast<int*>(p.out) + idx) = make_int4(q[0], q[1], q[2], q[3]);
+      }
     } else {
-      for (int kg = kg0; kg < n_kg; kg += kg_step) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const uint32_t gc = g + c;
-          uint32_t d[4] = {0, 0, 0, 0};
-          if (gc < p.P) {
-            const uint32_t n = gc / (uint32_t)p.hw, pp = gc % (uint32_t)p.hw;
-            const int8_t* col = p.x + (size_t)n * p.K * p.hw + pp;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const int ch = 16 * kg + i;
-              const uint32_t b = (ch < p.K) ? (uint32_t)(uint8_t)col[(size_t)ch * p.hw] : 0u;
-              d[i >> 2] |= b << (8 * (i & 3));
-            }
-          }
-          xt[(size_t)kg * kMfmaTilePos + c * 32 + j] = make_uint4(d[0], d[1], d[2], d[3]);
+      for (int c = 0; c < 4; ++c) {
+        const uint32_t gc = g + c;
+        if (gc < p.P) {
+          const uint32_t nc = gc / (uint32_t)p.hw, pc = gc % (uint32_t)p.hw;
+          StoreOne<OUT>(p.out, ((size_t)nc * p.M + row) * p.hw + pc, v[c], q[c]);
         }
       }
     }
   }
+}
+
+template <int KSMAX, int OUT>
+__global__ void __launch_bounds__(256) BlockMfmaKernel(const MfmaParams p) {
+  extern __shared__ uint4 xt[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // Workgroups are handed to the 8 XCDs round robin.  Map the linear id so
+  // that the workgroups sharing one activation tile (all row-block groups)
+  // run on the same XCD one after the other: the tile is then fetched into
+  // that XCD's L2 once.
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int tile = (slot / p.row_groups) * 8 + xcd;
+  if (tile >= p.tiles) return;
+  const uint32_t tile0 = (uint32_t)tile * (uint32_t)kMfmaTilePos;
+  const int rb = (slot % p.row_groups) * 4 + wave;
+  const bool wave_on = rb < p.row_blocks;
+  const int rbc = wave_on ? rb : p.row_blocks - 1;
+  PL_PHASE_MARK(0);
+
+  // weight blocks of this wavefront's 32 rows -> registers (blocks of absent
+  // k-steps are never multiplied; their loads are clamped to a valid block)
+  const uint32_t kmask = wave_on ? p.kmask[rbc] : 0u;
+  v4i a[KSMAX];
+#pragma unroll
+  for (int ks = 0; ks < KSMAX; ++ks) {
+    const int ksc = min(ks, p.ksteps - 1);
+    a[ks] = static_cast<const v4i*>(p.wblocks)[((size_t)rbc * p.ksteps + ksc) * 64 + lane];
+  }
+
+  PL_PHASE_MARK(1);
+  // ---- stage 128 positions x (32*ksteps) channels, channel-innermost
+  {
+    const int j = tid & 31;    // position quad of the tile
+    const int kg0 = tid >> 5;  // 8 channel groups per pass of the workgroup
+    if (p.vec) {
+      constexpr int kPasses = (2 * KSMAX + 7) / 8;  // passes that cover 2*KSMAX groups
+      constexpr int kBatch = kPasses < 4 ? kPasses : 4;
+      const bool inside = p.small && tile0 + (uint32_t)kMfmaTilePos <= p.P;
+#pragma unroll
+      for (int pass = 0; pass < kPasses; pass += kBatch) {
+        if (8 * pass < 2 * p.ksteps) {
+          if (inside && 16 * 8 * (pass + kBatch) <= p.K) {
+            StageMfmaVec<kBatch, true>(xt, p, tile0, 8 * pass, kg0, j);
+          } else {
+            StageMfmaVec<kBatch, false>(xt, p, tile0, 8 * pass, kg0, j);
+          }
+        }
+      }
+    } else {
+      StageMfmaBytes(xt, p, tile0, kg0, 8, j);
+    }
+  }
+  PL_PHASE_MARK(2);
   __syncthreads();
+  PL_PHASE_MARK(3);
   if (!wave_on) return;
 
   // ---- multiply: D[32 rows][32 cols] += A[32 x 32k] * B[32k x 32], four
@@ -381,47 +577,16 @@ __global__ void __launch_bounds__(KSMAX >= 32 ? 256 : 512) BlockMfmaKernel(const
     }
   }
 
-  // ---- epilogue: accumulator register r of lane l is output row
-  //      8*(r/4) + 4*(l/32) + r%4 of the block, column l%32
-  const uint32_t g = tile0 + 4u * (lane & 31);
-  if (g >= p.P) return;
-  const uint32_t n = g / (uint32_t)p.hw, pp = g % (uint32_t)p.hw;
-#pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int row = rb * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-    if (row >= p.M) continue;
-    float v[4];
-    int q[4];
-#pragma unroll
-    for (int c = 0; c < 4; ++c) q[c] = acc[c][r];
-    if (OUT != kOutAcc32) {
-      const float s = p.scale[row];
-      const float b = p.bias[row];
-#pragma unroll
-      for (int c = 0; c < 4; ++c) v[c] = Activate(__builtin_fmaf((float)q[c], s, b), p.act);
-    }
+  PL_PHASE_MARK(4);
+  DispatchAct(OUT == kOutAcc32 ? 0 : p.act.type, [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
     if (p.vec) {
-      const size_t idx = ((size_t)n * p.M + row) * p.hw + pp;
-      if (OUT == kOutF32) {
-        *reinterpret_cast<float4*>(static_cast<float*>(p.out) + idx) = make_float4(v[0], v[1], v[2], v[3]);
-      } else if (OUT == kOutI8) {
-        uint32_t w = (uint32_t)(QuantizeI8(v[0]) & 0xff) | ((uint32_t)(QuantizeI8(v[1]) & 0xff) << 8) |
-                     ((uint32_t)(QuantizeI8(v[2]) & 0xff) << 16) | ((uint32_t)(QuantizeI8(v[3]) & 0xff) << 24);
-        *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(p.out) + idx) = w;
-      } else {
-        *reinterpret_cast<int4*>(static_cast<int*>(p.out) + idx) = make_int4(q[0], q[1], q[2], q[3]);
-      }
+      MfmaEpilogue<OUT, ACT, true>(p, acc, rb, lane, tile0);
     } else {
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const uint32_t gc = g + c;
-        if (gc < p.P) {
-          const uint32_t nc = gc / (uint32_t)p.hw, pc = gc % (uint32_t)p.hw;
-          StoreOne<OUT>(p.out, ((size_t)nc * p.M + row) * p.hw + pc, v[c], q[c]);
-        }
-      }
+      MfmaEpilogue<OUT, ACT, false>(p, acc, rb, lane, tile0);
     }
-  }
+  });
+  PL_PHASE_MARK(5);
 }
 
 // ------------------------------------------------------------- launch glue
@@ -519,14 +684,18 @@ hipError_t LaunchBlockMfma(const MfmaConfig& cfg, const MfmaParams& p, hipStream
   const size_t lds = (size_t)2 * p.ksteps * kMfmaTilePos * 16;
   if (lds > (size_t)kMaxLdsBytes) return hipErrorInvalidValue;
   const uint32_t tiles = (p.P + kMfmaTilePos - 1) / kMfmaTilePos;
-  dim3 grid(tiles, (p.row_blocks + cfg.waves - 1) / cfg.waves), block(cfg.waves * 64);
+  if (cfg.waves != 4) return hipErrorInvalidValue;
+  MfmaParams q = p;
+  q.tiles = (int)tiles;
+  q.row_groups = (p.row_blocks + 3) / 4;
+  dim3 grid(8u * q.row_groups * ((tiles + 7) / 8)), block(256);
   switch (cfg.out_kind) {
     case kOutF32:
-      return MfmaByKs<kOutF32>(cfg, p, grid, block, lds, stream);
+      return MfmaByKs<kOutF32>(cfg, q, grid, block, lds, stream);
     case kOutI8:
-      return MfmaByKs<kOutI8>(cfg, p, grid, block, lds, stream);
+      return MfmaByKs<kOutI8>(cfg, q, grid, block, lds, stream);
     case kOutAcc32:
-      return MfmaByKs<kOutAcc32>(cfg, p, grid, block, lds, stream);
+      return MfmaByKs<kOutAcc32>(cfg, q, grid, block, lds, stream);
     default:
       return hipErrorInvalidValue;
   }
