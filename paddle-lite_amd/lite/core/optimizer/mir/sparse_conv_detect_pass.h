@@ -1,0 +1,38 @@
+// sparse_conv_detect_pass on a linear op list: rewrites every eligible
+// conv2d (1x1, stride 1, pad 0, group 1, fp32 or int8 weights, enough zeros)
+// into sparse_conv2d and creates its three weight tensors
+// (reference: lite/core/optimizer/mir/sparse_conv_detect_pass.{h,cc}; there
+// the same rewrite runs on the SSA graph and is bound to TARGET(kARM) only).
+#pragma once
+
+#include <string>
+#include <vector>
+
+#include "lite/api/paddle_place.h"
+#include "lite/core/op_desc.h"
+#include "lite/core/scope.h"
+
+namespace paddle {
+namespace lite {
+namespace mir {
+
+class SparseConvDetectPass {
+ public:
+  // reference default 0.6 (lite/api/paddle_api.h:473-474); the predictor
+  // passes 1.5 to disable the pass (lite/api/cxx_api_impl.cc:112-123)
+  void SetSparseThreshold(float t) { sparse_threshold_ = t; }
+  float sparse_threshold() const { return sparse_threshold_; }
+
+  // Targets the pass runs for; the reference binds kARM, this build adds kHIP.
+  static bool BoundTo(lite_api::TargetType t) { return t == lite_api::TargetType::kARM || t == lite_api::TargetType::kHIP; }
+
+  // Rewrites ops in place; returns how many conv2d ops were replaced.
+  int Apply(std::vector<OpInfo>* ops, Scope* scope) const;
+
+ private:
+  float sparse_threshold_{0.6f};
+};
+
+}  // namespace mir
+}  // namespace lite
+}  // namespace paddle

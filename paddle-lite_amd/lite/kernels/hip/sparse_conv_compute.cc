@@ -1,0 +1,180 @@
+#include "lite/kernels/hip/sparse_conv_compute.h"
+
+#include "pl_sparse_conv.h"
+#include "lite/core/op_registry.h"
+
+namespace paddle {
+namespace lite {
+namespace kernels {
+namespace hip {
+
+namespace {
+bool g_reference_quirks = true;
+
+pl_activation ToAbi(const operators::ActivationParam& a) {
+  pl_activation p;
+  p.type = a.has_active ? static_cast<int32_t>(a.active_type) : PL_ACT_NONE;
+  p.relu6_coef = a.Relu_clipped_coef;
+  p.leaky_alpha = a.Leaky_relu_alpha;
+  p.hs_scale = a.hard_swish_scale;
+  p.hs_offset = a.hard_swish_offset;
+  p.hs_threshold = a.hard_swish_threshold;
+  return p;
+}
+
+// weight_scale broadcast to one value per output channel
+// (lite/kernels/arm/sparse_conv_compute.cc:36-46)
+std::vector<float> PerChannelScales(const operators::SparseConvParam& param) {
+  std::vector<float> s = param.weight_scale;
+  const size_t oc = static_cast<size_t>(param.oc_nonzeros->dims()[0]);
+  if (s.size() != 1 && s.size() != oc) {
+    LOG(FATAL) << "weights scale size " << s.size() << " must equal to filter size " << oc;
+  }
+  if (s.size() == 1) s.resize(oc, s[0]);
+  return s;
+}
+}  // namespace
+
+void SetSparseConvReferenceQuirks(bool on) { g_reference_quirks = on; }
+bool SparseConvReferenceQuirks() { return g_reference_quirks; }
+
+template <PrecisionType P, PrecisionType O>
+SparseConvCompute<P, O>::~SparseConvCompute() {
+  if (handle_) pl_sparse_conv_destroy(handle_);
+}
+
+template <PrecisionType P, PrecisionType O>
+void SparseConvCompute<P, O>::Upload(int kind) {
+  auto& param = this->template Param<param_t>();
+  CHECK(param.x && param.nonzero_weights && param.oc_nonzeros && param.diffs) << "sparse_conv2d: unset input";
+  const DDim& xd = param.x->dims();
+  pl_sparse_conv_desc d{};
+  d.struct_size = sizeof(d);
+  d.kind = kind;
+  d.flag_semi = param.flag_semi;
+  d.first_ic = param.first_ic;
+  d.oc = static_cast<int32_t>(param.oc_nonzeros->dims()[0]);
+  d.ic = static_cast<int32_t>(xd[1]);
+  d.im_size = static_cast<int32_t>(xd[2] * xd[3]);
+  d.algo = PL_ALGO_AUTO;
+  d.nonzero_weights = param.nonzero_weights->raw_data();
+  d.n_weights = param.nonzero_weights->numel();
+  d.oc_nonzeros = param.oc_nonzeros->template data<uint32_t>();
+  d.diffs = param.diffs->template data<int32_t>();
+  d.n_diffs = param.diffs->numel();
+  d.scale = w_scale_.empty() ? nullptr : w_scale_.data();
+  const Tensor* bias = flag_trans_bias_ ? &bias_ : param.bias;
+  d.bias = bias ? bias->template data<float>() : nullptr;
+  d.act = ToAbi(param.activation_param);
+  if (kind == PL_KIND_INT8_INT8 && g_reference_quirks && d.act.type == PL_ACT_HARD_SWISH) {
+    // second division, done inside the reference's math function
+    d.act.hs_offset = d.act.hs_offset / param.output_scale;
+    d.act.hs_threshold = d.act.hs_threshold / param.output_scale;
+  }
+  if (handle_) {
+    pl_sparse_conv_destroy(handle_);
+    handle_ = nullptr;
+  }
+  const int rc = pl_sparse_conv_prepare(&d, &handle_);
+  if (rc != PL_OK) LOG(FATAL) << "pl_sparse_conv_prepare failed (" << rc << "): " << pl_last_error();
+}
+
+template <>
+void SparseConvCompute<PRECISION(kFloat), PRECISION(kFloat)>::PrepareForRun() {
+  Upload(PL_KIND_FP32);
+}
+
+template <>
+void SparseConvCompute<PRECISION(kInt8), PRECISION(kFloat)>::PrepareForRun() {
+  auto& param = this->Param<param_t>();
+  w_scale_ = PerChannelScales(param);
+  for (float& s : w_scale_) s *= param.input_scale;
+  Upload(PL_KIND_INT8_FP32);
+}
+
+template <>
+void SparseConvCompute<PRECISION(kInt8), PRECISION(kInt8)>::PrepareForRun() {
+  auto& param = this->Param<param_t>();
+  w_scale_ = PerChannelScales(param);
+  const float in_scale = param.input_scale, out_scale = param.output_scale;
+  for (float& s : w_scale_) s = s * in_scale / out_scale;
+  if (param.bias) {
+    bias_.Resize(param.bias->dims());
+    float* dst = bias_.mutable_data<float>(TargetType::kHost);
+    const float* src = param.bias->data<float>();
+    for (int64_t i = 0; i < bias_.numel(); ++i) dst[i] = src[i] / out_scale;
+    flag_trans_bias_ = true;
+  }
+  // the activation constants move to the output's quantised domain, in the
+  // kernel's own copy of the parameters
+  auto& act = param.activation_param;
+  using AT = lite_api::ActivationType;
+  if (act.active_type == AT::kRelu6) act.Relu_clipped_coef /= out_scale;
+  if (act.active_type == AT::kLeakyRelu && g_reference_quirks) act.Leaky_relu_alpha /= out_scale;
+  if (act.active_type == AT::kHardSwish) {
+    act.hard_swish_scale /= out_scale;
+    act.hard_swish_offset /= out_scale;
+    act.hard_swish_threshold /= out_scale;
+  }
+  Upload(PL_KIND_INT8_INT8);
+}
+
+template <PrecisionType P, PrecisionType O>
+void SparseConvCompute<P, O>::Run() {
+  auto& param = this->template Param<param_t>();
+  auto& ctx = this->ctx_->template As<HIPContext>();
+  CHECK(handle_ != nullptr) << "PrepareForRun was not called";
+  CHECK(param.x->target() == TargetType::kHIP) << "sparse_conv2d(kHIP): Input must live on the device (io_copy missing?)";
+  const DDim& xd = param.x->dims();
+  const DDim& od = param.output->dims();
+  const int batch = static_cast<int>(xd[0]);
+  const int im_size = static_cast<int>(od[2] * od[3]);
+  void* out = (O == PRECISION(kFloat)) ? static_cast<void*>(param.output->template mutable_data<float>(TargetType::kHIP))
+                                       : static_cast<void*>(param.output->template mutable_data<int8_t>(TargetType::kHIP));
+  const int rc = pl_sparse_conv_run(handle_, param.x->raw_data(), out, batch, im_size, ctx.stream());
+  if (rc != PL_OK) LOG(FATAL) << "pl_sparse_conv_run failed (" << rc << "): " << pl_last_error();
+}
+
+template class SparseConvCompute<PRECISION(kFloat), PRECISION(kFloat)>;
+template class SparseConvCompute<PRECISION(kInt8), PRECISION(kFloat)>;
+template class SparseConvCompute<PRECISION(kInt8), PRECISION(kInt8)>;
+
+}  // namespace hip
+}  // namespace kernels
+}  // namespace lite
+}  // namespace paddle
+
+// Same op type, argument names and aliases as the ARM registrations
+// (lite/kernels/arm/sparse_conv_compute.cc:369-430).  Activations live on the
+// device; the three weight tensors and the bias are read on the host once, in
+// PrepareForRun.
+typedef paddle::lite::kernels::hip::SparseConvCompute<PRECISION(kFloat), PRECISION(kFloat)> SparseConvHipFp32;
+typedef paddle::lite::kernels::hip::SparseConvCompute<PRECISION(kInt8), PRECISION(kFloat)> SparseConvHipInt8Fp32;
+typedef paddle::lite::kernels::hip::SparseConvCompute<PRECISION(kInt8), PRECISION(kInt8)> SparseConvHipInt8Int8;
+
+REGISTER_LITE_KERNEL(sparse_conv2d, kHIP, kFloat, kNCHW, SparseConvHipFp32, def)
+    .BindInput("Input", {paddle::lite::LiteType::GetTensorTy(TARGET(kHIP))})
+    .BindInput("NonZeroWeights", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost))})
+    .BindInput("OcNonZeros", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost), PRECISION(kInt32))})
+    .BindInput("Diffs", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost), PRECISION(kInt32))})
+    .BindInput("Bias", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost))})
+    .BindOutput("Output", {paddle::lite::LiteType::GetTensorTy(TARGET(kHIP))})
+    .Finalize();
+
+REGISTER_LITE_KERNEL(sparse_conv2d, kHIP, kInt8, kNCHW, SparseConvHipInt8Fp32, int8_fp32_out)
+    .BindInput("Input", {paddle::lite::LiteType::GetTensorTy(TARGET(kHIP), PRECISION(kInt8))})
+    .BindInput("NonZeroWeights", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost), PRECISION(kInt8))})
+    .BindInput("OcNonZeros", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost), PRECISION(kInt32))})
+    .BindInput("Diffs", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost), PRECISION(kInt32))})
+    .BindInput("Bias", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost), PRECISION(kFloat))})
+    .BindOutput("Output", {paddle::lite::LiteType::GetTensorTy(TARGET(kHIP), PRECISION(kFloat))})
+    .Finalize();
+
+REGISTER_LITE_KERNEL(sparse_conv2d, kHIP, kInt8, kNCHW, SparseConvHipInt8Int8, int8_int8_out)
+    .BindInput("Input", {paddle::lite::LiteType::GetTensorTy(TARGET(kHIP), PRECISION(kInt8))})
+    .BindInput("NonZeroWeights", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost), PRECISION(kInt8))})
+    .BindInput("OcNonZeros", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost), PRECISION(kInt32))})
+    .BindInput("Diffs", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost), PRECISION(kInt32))})
+    .BindInput("Bias", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost), PRECISION(kFloat))})
+    .BindOutput("Output", {paddle::lite::LiteType::GetTensorTy(TARGET(kHIP), PRECISION(kInt8))})
+    .Finalize();

@@ -1,0 +1,52 @@
+// sparse_conv2d kernels of TARGET(kHIP): the class the reference has for
+// TARGET(kARM) (lite/kernels/arm/sparse_conv_compute.h:25-50), with the
+// gfx950 library behind Run().
+#pragma once
+
+#include <vector>
+
+#include "lite/core/kernel.h"
+#include "lite/operators/op_params.h"
+
+struct pl_sparse_conv_handle;
+
+namespace paddle {
+namespace lite {
+namespace kernels {
+namespace hip {
+
+template <PrecisionType Ptype, PrecisionType OutType>
+class SparseConvCompute : public KernelLite<TARGET(kHIP), Ptype> {
+ public:
+  using param_t = operators::SparseConvParam;
+  ~SparseConvCompute() override;
+
+  void PrepareForRun() override;
+  // Nothing to redo when shapes change: the library keeps channel indices,
+  // not byte offsets, so any batch and spatial size can follow.
+  void ReInitWhenNeeded() override {}
+  void Run() override;
+
+  const std::vector<float>& merged_scales() const { return w_scale_; }
+
+ private:
+  void Upload(int kind);
+
+  Tensor bias_;
+  bool flag_trans_bias_{false};
+  std::vector<float> w_scale_;
+  pl_sparse_conv_handle* handle_{nullptr};
+};
+
+// The reference divides the int8-output leaky_relu slope by the output scale
+// (lite/kernels/arm/sparse_conv_compute.cc:86-90) and scales the hard_swish
+// offset / threshold twice (:91-100 and again in
+// lite/backends/arm/math/sparse_conv_impl.cc:3713-3720).  true (default)
+// reproduces that; false scales once and leaves the slope alone.
+void SetSparseConvReferenceQuirks(bool on);
+bool SparseConvReferenceQuirks();
+
+}  // namespace hip
+}  // namespace kernels
+}  // namespace lite
+}  // namespace paddle

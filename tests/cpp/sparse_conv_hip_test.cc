@@ -1,0 +1,355 @@
+// Host-side test of the Lite surface for sparse_conv2d on TARGET(kHIP), in the
+// shape of the reference's math tests (lite/tests/math/
+// sparse_conv_{f32,int8}_compute_test.cc: fill, mask, pack, run, compare with
+// the naive dense reference) but through the whole op path the reference never
+// tests: detect pass -> SparseConvOp::Attach/InferShape -> registered kernel
+// -> Launch.  Seeds are fixed.
+//
+//   sparse_conv_hip_test --cpu   registry, op, pass and error paths (no device)
+//   sparse_conv_hip_test --gpu   the above plus execution on the device
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "lite/core/op_registry.h"
+#include "lite/core/optimizer/mir/sparse_conv_detect_pass.h"
+#include "lite/kernels/hip/sparse_conv_compute.h"
+#include "lite/operators/sparse_conv_op.h"
+#include "pl_sparse_conv.h"
+#include "sparse_conv_oracle.h"
+
+using namespace paddle::lite;  // NOLINT
+
+static int g_failures = 0;
+#define EXPECT(cond)                                                   \
+  do {                                                                 \
+    if (!(cond)) {                                                     \
+      std::printf("  FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond); \
+      ++g_failures;                                                    \
+    }                                                                  \
+  } while (0)
+
+template <typename F>
+static bool Throws(F f) {
+  try {
+    f();
+  } catch (const FatalError&) {
+    return true;
+  }
+  return false;
+}
+
+struct Problem {
+  int batch, ic, oc, h, w;
+  float sparsity;
+  bool paired, int8, out_int8, bias;
+  std::string act;  // "", relu, relu6, leaky_relu, hard_swish
+  unsigned seed;
+};
+
+// Builds a scope holding a conv2d (Input, Filter, Bias) and its op description.
+static OpInfo MakeConv(const Problem& p, Scope* scope, std::vector<float>* ws, float* in_scale, float* out_scale) {
+  std::mt19937 gen(p.seed);
+  std::uniform_real_distribution<float> uni(0.f, 1.f);
+  std::normal_distribution<float> nrm(0.f, 1.f);
+  Tensor* x = scope->NewTensor("x");
+  Tensor* w = scope->NewTensor("conv_w");
+  x->Resize({p.batch, p.ic, p.h, p.w});
+  w->Resize({p.oc, p.ic, 1, 1});
+  std::vector<char> keep(static_cast<size_t>(p.oc) * p.ic);
+  for (int r = 0; r < p.oc; ++r)
+    for (int c = 0; c < p.ic; ++c) {
+      if (p.paired && (r & 1)) {
+        keep[r * p.ic + c] = keep[(r - 1) * p.ic + c];
+      } else {
+        keep[r * p.ic + c] = uni(gen) >= p.sparsity;
+      }
+    }
+  if (p.int8) {
+    int8_t* xd = x->mutable_data<int8_t>(TargetType::kHost);
+    for (int64_t i = 0; i < x->numel(); ++i) xd[i] = static_cast<int8_t>(static_cast<int>(uni(gen) * 255.f) - 127);
+    int8_t* wd = w->mutable_data<int8_t>(TargetType::kHost);
+    for (int64_t i = 0; i < w->numel(); ++i) {
+      int v = static_cast<int>(uni(gen) * 127.f) + 1;
+      if (uni(gen) < 0.5f) v = -v;
+      wd[i] = keep[i] ? static_cast<int8_t>(v) : 0;
+    }
+  } else {
+    float* xd = x->mutable_data<float>(TargetType::kHost);
+    for (int64_t i = 0; i < x->numel(); ++i) xd[i] = uni(gen) * 2.f - 1.f;
+    float* wd = w->mutable_data<float>(TargetType::kHost);
+    for (int64_t i = 0; i < w->numel(); ++i) {
+      float v = nrm(gen) * 0.1f;
+      wd[i] = keep[i] ? (v == 0.f ? 0.1f : v) : 0.f;
+    }
+  }
+  OpInfo conv("conv2d");
+  conv.SetInput("Input", {"x"});
+  conv.SetInput("Filter", {"conv_w"});
+  if (p.bias) {
+    Tensor* b = scope->NewTensor("conv_b");
+    b->Resize({p.oc});
+    float* bd = b->mutable_data<float>(TargetType::kHost);
+    for (int i = 0; i < p.oc; ++i) bd[i] = nrm(gen) * 0.1f;
+    conv.SetInput("Bias", {"conv_b"});
+  }
+  conv.SetOutput("Output", {"y"});
+  scope->NewTensor("y");
+  conv.SetAttr<std::vector<int>>("strides", {1, 1});
+  conv.SetAttr<std::vector<int>>("paddings", {0, 0});
+  conv.SetAttr<std::vector<int>>("dilations", {1, 1});
+  conv.SetAttr<int>("groups", 1);
+  if (!p.act.empty()) {
+    conv.SetAttr<bool>("with_act", true);
+    conv.SetAttr<std::string>("act_type", p.act);
+    conv.SetAttr<float>("fuse_brelu_threshold", 6.f);
+    conv.SetAttr<float>("leaky_relu_alpha", 0.1f);
+    conv.SetAttr<float>("hard_swish_threshold", 6.f);
+    conv.SetAttr<float>("hard_swish_scale", 6.f);
+    conv.SetAttr<float>("hard_swish_offset", 3.f);
+  }
+  if (p.int8) {
+    ws->resize(p.oc);
+    for (float& s : *ws) s = 0.001f + 0.019f * uni(gen);
+    *in_scale = 0.01f;
+    *out_scale = p.out_int8 ? 0.05f : 1.f;
+    conv.SetAttr<bool>("enable_int8", true);
+    conv.SetInputScale("Input0_scale", {*in_scale}, true);
+    conv.SetInputScale("Filter0_scale", *ws, true);
+    conv.SetOutputScale("Output0_scale", {*out_scale}, true);
+  }
+  return conv;
+}
+
+static int ActCode(const std::string& a) { return a == "relu" ? 1 : a == "relu6" ? 2 : a == "leaky_relu" ? 4 : a == "hard_swish" ? 10 : 0; }
+
+// Whole op path on one problem. With run_on_device false stops before Launch.
+static void RunProblem(const Problem& p, bool run_on_device) {
+  std::printf("case ic=%d oc=%d n=%d %dx%d sparsity=%.2f %s %s%s act=%s bias=%d\n", p.ic, p.oc, p.batch, p.h, p.w, p.sparsity, p.paired ? "semi" : "unstructured", p.int8 ? "int8" : "fp32",
+              p.out_int8 ? "->int8" : "", p.act.c_str(), p.bias);
+  std::fflush(stdout);
+  Scope scope;
+  std::vector<float> ws;
+  float in_scale = 1.f, out_scale = 1.f;
+  std::vector<OpInfo> ops{MakeConv(p, &scope, &ws, &in_scale, &out_scale)};
+  // keep dense copies for the reference
+  const int64_t wn = static_cast<int64_t>(p.oc) * p.ic;
+  std::vector<int8_t> w8;
+  std::vector<float> wf;
+  if (p.int8) {
+    w8.assign(scope.FindMutableTensor("conv_w")->data<int8_t>(), scope.FindMutableTensor("conv_w")->data<int8_t>() + wn);
+  } else {
+    wf.assign(scope.FindMutableTensor("conv_w")->data<float>(), scope.FindMutableTensor("conv_w")->data<float>() + wn);
+  }
+
+  mir::SparseConvDetectPass pass;
+  pass.SetSparseThreshold(0.5f);
+  EXPECT(mir::SparseConvDetectPass::BoundTo(TARGET(kHIP)));
+  const int replaced = pass.Apply(&ops, &scope);
+  EXPECT(replaced == 1);
+  EXPECT(ops[0].Type() == "sparse_conv2d");
+  EXPECT(scope.FindVar("conv_w") == nullptr);
+  EXPECT(ops[0].GetAttr<int>("flag_semi") == (p.paired ? 1 : 0));
+  Tensor* ocn = scope.FindMutableTensor("conv_w_oc_nonzeros");
+  EXPECT(ocn != nullptr && ocn->dims()[0] == p.oc && ocn->persistable());
+
+  auto op = LiteOpRegistry::Global().Create("sparse_conv2d");
+  EXPECT(op != nullptr);
+  EXPECT(op->Attach(ops[0], &scope));
+  EXPECT(op->CheckShape());
+  EXPECT(op->InferShape());
+  Tensor* y = scope.FindMutableTensor("y");
+  EXPECT(y->dims() == DDim({p.batch, p.oc, p.h, p.w}));
+
+  const PrecisionType prec = p.int8 ? PRECISION(kInt8) : PRECISION(kFloat);
+  const std::string alias = !p.int8 ? "def" : (p.out_int8 ? "int8_int8_out" : "int8_fp32_out");
+  if (!run_on_device) {
+    auto all = KernelRegistry::Global().Create("sparse_conv2d", TARGET(kHIP), prec, DATALAYOUT(kNCHW));
+    EXPECT(all.size() == (p.int8 ? 2u : 1u));
+    return;
+  }
+  // the io_copy an optimiser would insert in front of a kHIP kernel
+  OpInfo h2d("io_copy");
+  h2d.SetInput("Input", {"x"});
+  h2d.SetOutput("Out", {"x_dev"});
+  auto copy_op = LiteOpRegistry::Global().Create("io_copy");
+  EXPECT(copy_op->Attach(h2d, &scope) && copy_op->InferShape());
+  auto copy_kernels = copy_op->CreateKernels({paddle::lite_api::Place(TARGET(kHIP), PRECISION(kAny), DATALAYOUT(kAny))}, "io_copy/host_to_device");
+  EXPECT(copy_kernels.size() == 1);
+  copy_kernels[0]->Launch();
+  ops[0].SetInput("Input", {"x_dev"});
+  EXPECT(op->Attach(ops[0], &scope) && op->InferShape());
+
+  auto kernels = op->CreateKernels({paddle::lite_api::Place(TARGET(kHIP), prec, DATALAYOUT(kNCHW))}, "sparse_conv2d/" + alias);
+  EXPECT(kernels.size() == 1);
+  KernelBase* k = kernels[0].get();
+  EXPECT(k->alias() == alias && k->target() == TARGET(kHIP));
+  k->Launch();
+  k->Launch();  // second epoch: no PrepareForRun
+  k->mutable_context_as<HIPContext>()->Sync();
+  EXPECT(y->target() == TARGET(kHIP));
+  Tensor y_host;
+  y_host.CopyDataFrom(*y, TargetType::kHost);
+
+  // reference: the oracle's dense per-image GEMM with the merged parameters
+  // (the kernel class scales the activation once here)
+  const int hw = p.h * p.w;
+  plo_act act{ActCode(p.act), 6.f, 0.1f, 6.f, 3.f, 6.f};
+  const float* bias = p.bias ? scope.FindMutableTensor("conv_b")->data<float>() : nullptr;
+  std::vector<float> ms(p.oc), mb(p.oc);
+  const int kind = !p.int8 ? 0 : (p.out_int8 ? 2 : 1);
+  EXPECT(plo_merge_params(kind, p.oc, ws.data(), static_cast<int>(ws.size()), in_scale, out_scale, bias, ms.data(), bias ? mb.data() : nullptr, &act) == 0);
+  if (kind == 2 && act.type == 4) act.leaky_alpha = 0.1f;  // slope left alone
+  const Tensor* xt = scope.FindMutableTensor("x");
+  if (!p.int8) {
+    std::vector<float> want(static_cast<size_t>(p.batch) * p.oc * hw);
+    plo_dense_conv1x1(0, wf.data(), xt->data<float>(), bias, nullptr, want.data(), p.batch, p.oc, p.ic, hw, &act, 1);
+    double max_ratio = 0, max_diff = 0;
+    for (size_t i = 0; i < want.size(); ++i) {
+      const double d = std::fabs(want[i] - y_host.data<float>()[i]);
+      const double r = d / (std::fabs(want[i]) + 1e-6);
+      if (r > max_ratio) {
+        max_ratio = r;
+        max_diff = d;
+      }
+    }
+    // the reference test's criterion (sparse_conv_f32_compute_test.cc:336-361)
+    EXPECT(!(max_ratio > 1e-4 && max_diff > 5e-5));
+  } else if (!p.out_int8) {
+    std::vector<float> want(static_cast<size_t>(p.batch) * p.oc * hw);
+    plo_dense_conv1x1(1, w8.data(), xt->data<int8_t>(), bias, ms.data(), want.data(), p.batch, p.oc, p.ic, hw, &act, 1);
+    EXPECT(std::memcmp(want.data(), y_host.raw_data(), want.size() * 4) == 0);
+  } else {
+    std::vector<int8_t> want(static_cast<size_t>(p.batch) * p.oc * hw);
+    plo_dense_conv1x1(2, w8.data(), xt->data<int8_t>(), bias ? mb.data() : nullptr, ms.data(), want.data(), p.batch, p.oc, p.ic, hw, &act, 1);
+    EXPECT(std::memcmp(want.data(), y_host.raw_data(), want.size()) == 0);
+  }
+}
+
+static void RegistryAndErrorPaths() {
+  std::printf("registry and error paths\n");
+  // the three registrations beside the ARM ones, same aliases
+  auto fp32 = KernelRegistry::Global().Create("sparse_conv2d", TARGET(kHIP), PRECISION(kFloat), DATALAYOUT(kNCHW));
+  auto int8 = KernelRegistry::Global().Create("sparse_conv2d", TARGET(kHIP), PRECISION(kInt8), DATALAYOUT(kNCHW));
+  EXPECT(fp32.size() == 1 && fp32.front()->alias() == "def");
+  EXPECT(int8.size() == 2);
+  bool a = false, b = false;
+  for (auto& k : int8) {
+    a |= k->alias() == "int8_fp32_out";
+    b |= k->alias() == "int8_int8_out";
+  }
+  EXPECT(a && b);
+  EXPECT(KernelRegistry::Global().Create("sparse_conv2d", TARGET(kARM), PRECISION(kFloat), DATALAYOUT(kNCHW)).empty());
+  const auto* types = ParamTypeRegistry::Global().Retrieve("sparse_conv2d/int8_int8_out", paddle::lite_api::Place(TARGET(kHIP), PRECISION(kInt8), DATALAYOUT(kNCHW)));
+  EXPECT(types != nullptr && types->size() == 6);
+  if (types) {
+    for (auto& e : *types) {
+      if (e.arg == "Input" || e.arg == "Output") EXPECT(e.type.target == TARGET(kHIP) && e.type.precision == PRECISION(kInt8));
+      if (e.arg == "OcNonZeros" || e.arg == "Diffs") EXPECT(e.type.target == TARGET(kHost) && e.type.precision == PRECISION(kInt32));
+    }
+  }
+  EXPECT(static_cast<int>(TARGET(kHIP)) == 19 && static_cast<int>(TARGET(kNNAdapter)) == 18);
+
+  // unknown fused activation and bad paddings are fatal in the op
+  Scope scope;
+  std::vector<float> ws;
+  float is, os;
+  Problem p{1, 8, 4, 2, 2, 0.6f, false, false, false, true, "relu", 1};
+  std::vector<OpInfo> ops{MakeConv(p, &scope, &ws, &is, &os)};
+  mir::SparseConvDetectPass pass;
+  pass.SetSparseThreshold(0.0f);
+  EXPECT(pass.Apply(&ops, &scope) == 1);
+  auto op = LiteOpRegistry::Global().Create("sparse_conv2d");
+  OpInfo bad = ops[0];
+  bad.SetAttr<std::string>("act_type", "sigmoid");
+  EXPECT(Throws([&] { op->Attach(bad, &scope); }));
+  bad = ops[0];
+  bad.SetAttr<std::vector<int>>("paddings", {0, 0, 0});
+  EXPECT(Throws([&] { op->Attach(bad, &scope); }));
+  bad = ops[0];
+  bad.SetAttr<std::vector<int>>("paddings", {0, 0, 0, 0});
+  EXPECT(op->Attach(bad, &scope));
+  // hard_sigmoid is accepted by the op (no kernel implements it)
+  bad = ops[0];
+  bad.SetAttr<std::string>("act_type", "hard_sigmoid");
+  bad.SetAttr<float>("slope", 0.2f);
+  bad.SetAttr<float>("offset", 0.5f);
+  EXPECT(op->Attach(bad, &scope));
+
+  // the pass leaves ineligible convs alone: 3x3, stride 2, groups, threshold
+  auto untouched = [&](const char* what, std::function<void(OpInfo*, Scope*)> edit) {
+    Scope s;
+    std::vector<float> w2;
+    Problem q{1, 8, 4, 4, 4, 0.7f, false, false, false, false, "", 2};
+    std::vector<OpInfo> o{MakeConv(q, &s, &w2, &is, &os)};
+    edit(&o[0], &s);
+    mir::SparseConvDetectPass ps;
+    ps.SetSparseThreshold(0.5f);
+    const int n = ps.Apply(&o, &s);
+    if (n != 0 || o[0].Type() != "conv2d") {
+      std::printf("  FAILED: pass rewrote a conv it must skip (%s)\n", what);
+      ++g_failures;
+    }
+  };
+  untouched("stride 2", [](OpInfo* o, Scope*) { o->SetAttr<std::vector<int>>("strides", {2, 2}); });
+  untouched("padding 1", [](OpInfo* o, Scope*) { o->SetAttr<std::vector<int>>("paddings", {1, 1}); });
+  untouched("groups 2", [](OpInfo* o, Scope*) { o->SetAttr<int>("groups", 2); });
+  untouched("3x3", [](OpInfo*, Scope* s) { s->FindMutableTensor("conv_w")->Resize({4, 8, 3, 3}); });
+  untouched("dense weights", [](OpInfo*, Scope* s) {
+    Tensor* w = s->FindMutableTensor("conv_w");
+    float* d = w->mutable_data<float>(TargetType::kHost);
+    for (int64_t i = 0; i < w->numel(); ++i) d[i] = 1.f;
+  });
+  // threshold 1.5 is how the predictor switches the pass off
+  {
+    Scope s;
+    std::vector<float> w2;
+    Problem q{1, 8, 4, 4, 4, 0.9f, false, false, false, false, "", 3};
+    std::vector<OpInfo> o{MakeConv(q, &s, &w2, &is, &os)};
+    mir::SparseConvDetectPass ps;
+    ps.SetSparseThreshold(1.5f);
+    EXPECT(ps.Apply(&o, &s) == 0);
+  }
+  // weight_scale of the wrong size is fatal in PrepareForRun, before any device work
+  {
+    Scope s;
+    std::vector<float> w2;
+    Problem q{1, 8, 4, 2, 2, 0.6f, false, true, false, false, "", 4};
+    std::vector<OpInfo> o{MakeConv(q, &s, &w2, &is, &os)};
+    o[0].SetInputScale("Filter0_scale", {0.1f, 0.2f}, true);
+    mir::SparseConvDetectPass ps;
+    ps.SetSparseThreshold(0.0f);
+    EXPECT(ps.Apply(&o, &s) == 1);
+    auto sp = LiteOpRegistry::Global().Create("sparse_conv2d");
+    EXPECT(sp->Attach(o[0], &s) && sp->InferShape());
+    auto ks = sp->CreateKernels({paddle::lite_api::Place(TARGET(kHIP), PRECISION(kInt8), DATALAYOUT(kNCHW))}, "sparse_conv2d/int8_fp32_out");
+    EXPECT(ks.size() == 1);
+    EXPECT(Throws([&] { ks[0]->Launch(); }));
+  }
+}
+
+int main(int argc, char** argv) {
+  const bool gpu = argc > 1 && std::string(argv[1]) == "--gpu";
+  RegistryAndErrorPaths();
+  const std::vector<Problem> problems = {
+      {2, 64, 48, 8, 8, 0.8f, false, false, false, true, "relu", 11},
+      {2, 57, 31, 7, 7, 0.8f, true, false, false, true, "relu6", 12},
+      {1, 109, 16, 4, 8, 0.7f, false, false, false, false, "hard_swish", 13},
+      {3, 128, 64, 14, 14, 0.85f, false, true, false, true, "leaky_relu", 14},
+      {2, 96, 40, 7, 7, 0.75f, true, true, false, true, "", 15},
+      {2, 128, 64, 8, 8, 0.75f, true, true, true, true, "hard_swish", 16},
+      {2, 70, 33, 5, 5, 0.8f, false, true, true, true, "relu6", 17},
+      {1, 512, 32, 14, 14, 0.85f, false, true, true, false, "leaky_relu", 18},
+  };
+  paddle::lite::kernels::hip::SetSparseConvReferenceQuirks(false);
+  if (gpu && pl_device_count() < 1) {
+    std::printf("no gfx950 device\n");
+    return 2;
+  }
+  for (const Problem& p : problems) RunProblem(p, gpu);
+  std::printf("%s: %d failure(s)\n", gpu ? "gpu" : "cpu", g_failures);
+  return g_failures ? 1 : 0;
+}
