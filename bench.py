@@ -28,7 +28,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4"])
+    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--algo", default="auto", choices=["auto", "walk", "mfma"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cache-resident", action="store_true", help="reuse one buffer set (reported, never the headline)")
@@ -106,6 +106,86 @@ def cpu_baseline(case, packed, budget_s=12.0):
     return naive
 
 
+def run_c5(args):
+    """MobileNetV1-1.0 pointwise stack (13 layers, batch 64, int8 -> int8, 90 %
+    unstructured zeros, relu) timed as one sequence of 13 launches per step.
+    Layer i+1 consumes layer i's int8 output where the shapes chain (2->3,
+    4->5, 6->7..11, 12->13); at the four spatial breaks (stride-2 depthwise
+    layers of the real network, not part of this path) a fresh random tensor
+    is fed.  Not the headline metric: printed as its own JSON line."""
+    import numpy as np
+    import torch
+
+    import helpers
+
+    capi, wl = helpers.capi, helpers.workloads
+    L = capi.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    layers = []
+    prev_out = None
+    total_ops = total_bytes = 0.0
+    for i in range(13):
+        case = wl.config5_layer(i)
+        kernel, weights = helpers.make_kernel(case, algo={"auto": capi.ALGO_AUTO, "walk": capi.ALGO_ROW_WALK, "mfma": capi.ALGO_BLOCK_MFMA}[args.algo])
+        ic, oc, hw = wl.MOBILENET_V1_POINTWISE[i]
+        chained = prev_out is not None and tuple(prev_out.shape[1:]) == (ic, hw, hw)
+        x = prev_out if chained else torch.from_numpy(case.x).cuda()
+        out = torch.empty((case.batch, oc, hw, hw), dtype=torch.int8, device="cuda")
+        # parity of this layer on its actual input (first two images)
+        capi.check(L.pl_sparse_conv_run(kernel._handle, x.data_ptr(), out.data_ptr(), case.batch, hw * hw, C.c_void_p(stream)))
+        torch.cuda.synchronize()
+        want = helpers.run_oracle(case, x=x[:2].cpu().numpy())
+        assert np.array_equal(out[:2].cpu().numpy(), want), "layer %d differs from the oracle" % (i + 1)
+        layers.append((case, kernel, x, out))
+        prev_out = out
+        total_ops += case.algorithmic_ops()
+        total_bytes += case.algorithmic_bytes(weights)
+
+    def sequence():
+        for case, kernel, x, out in layers:
+            capi.check(L.pl_sparse_conv_run(kernel._handle, x.data_ptr(), out.data_ptr(), case.batch, case.im_size, C.c_void_p(stream)))
+
+    # per-layer kernel time (events around repeated launches of one layer)
+    per_layer = []
+    for case, kernel, x, out in layers:
+        xp = (C.c_void_p * 1)(x.data_ptr())
+        op = (C.c_void_p * 1)(out.data_ptr())
+        ms = C.c_float(0.0)
+        capi.check(L.pl_sparse_conv_run_sequence(kernel._handle, xp, op, 1, case.batch, case.im_size, 20, C.c_void_p(stream), None))
+        capi.check(L.pl_sparse_conv_run_sequence(kernel._handle, xp, op, 1, case.batch, case.im_size, 100, C.c_void_p(stream), C.byref(ms)))
+        per_layer.append(ms.value * 10.0)  # us per launch
+    for _ in range(max(1, args.warmup // 13)):
+        sequence()
+    torch.cuda.synchronize()
+    steps = max(1, args.steps // 13)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        sequence()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    seq_us = e0.elapsed_time(e1) * 1e3 / steps
+    line = {
+        "metric": "MobileNetV1 pointwise stack, int8, 90% sparse: nnz-GOP/s of the 13-launch sequence",
+        "value": total_ops * steps / wall / 1e9,
+        "unit": "nnz-GOP/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "ms_per_step": wall * 1e3 / steps,
+        "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": "c5_mobilenet_v1_pointwise_stack", "batch": 64, "layers": 13},
+        "roofline": {"bound": "hbm", "achieved": total_bytes / (seq_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": total_bytes / (seq_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None, "algorithmic_bytes_per_sequence": total_bytes, "sequence_us": seq_us, "sum_of_layer_kernel_us": sum(per_layer)},
+        "per_layer_kernel_us": [round(v, 2) for v in per_layer],
+        "per_layer_frac": [round(c.algorithmic_bytes(helpers.pla.detect_and_pack(c.dense, c.im_size)) / (t * 1e-6) / 1e9 / HBM_PEAK_GBS, 3) for (c, _, _, _), t in zip(layers, per_layer)],
+    }
+    print(json.dumps(line))
+    return 0
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -121,6 +201,8 @@ def main():
         sys.stderr.write("bench.py needs a GPU\n")
         return 2
     torch.cuda.set_device(0)
+    if args.config == "c5":
+        return run_c5(args)
     case = wl.CONFIGS[args.config]()
     algo = {"auto": capi.ALGO_AUTO, "walk": capi.ALGO_ROW_WALK, "mfma": capi.ALGO_BLOCK_MFMA}[args.algo]
     kernel, weights = helpers.make_kernel(case, algo=algo)

@@ -25,7 +25,16 @@ HIPCC_FLAGS = [
     "-Wno-unused-function",
 ]
 
-SOURCES = ["sparse_layout.cc", "sparse_conv_kernels.hip", "sparse_conv_capi.cc"]
+# (source, object name, extra flags); the kernel file is built as four
+# translation units so that they compile in parallel
+SOURCES = [
+    ("sparse_layout.cc", "sparse_layout.o", []),
+    ("sparse_conv_capi.cc", "sparse_conv_capi.o", []),
+    ("sparse_conv_kernels.hip", "sparse_conv_kernels_walk.o", ["-DPL_KERNEL_PART=0"]),
+    ("sparse_conv_kernels.hip", "sparse_conv_kernels_mfma_f32.o", ["-DPL_KERNEL_PART=1"]),
+    ("sparse_conv_kernels.hip", "sparse_conv_kernels_mfma_i8.o", ["-DPL_KERNEL_PART=2"]),
+    ("sparse_conv_kernels.hip", "sparse_conv_kernels_mfma_acc32.o", ["-DPL_KERNEL_PART=3"]),
+]
 
 
 def hipcc():
@@ -35,21 +44,33 @@ def hipcc():
     return exe
 
 
+def _compile_one(job):
+    src, obj_name, extra = job
+    obj = os.path.join(LIB_DIR, obj_name)
+    cmd = [hipcc()] + HIPCC_FLAGS + extra + ["-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
+    return obj, res.returncode, out, " ".join(cmd)
+
+
 def build_library(verbose=False):
     """Compile every source and link the shared library. Always recompiles."""
+    from concurrent.futures import ThreadPoolExecutor
+
     os.makedirs(LIB_DIR, exist_ok=True)
+    for stale in os.listdir(LIB_DIR):
+        if stale.endswith(".o"):
+            os.remove(os.path.join(LIB_DIR, stale))
+    with ThreadPoolExecutor(max_workers=min(6, os.cpu_count() or 1)) as pool:
+        results = list(pool.map(_compile_one, SOURCES))
     objs = []
-    for src in SOURCES:
-        obj = os.path.join(LIB_DIR, os.path.splitext(src)[0] + ".o")
-        cmd = [hipcc()] + HIPCC_FLAGS + ["-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
+    for obj, rc, out, cmd in results:
         if verbose:
-            print(" ".join(cmd), flush=True)
-        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-        out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
-        if res.returncode != 0:
-            raise RuntimeError("hipcc failed for %s:\n%s" % (src, out))
-        if verbose and out.strip():
-            print(out, flush=True)
+            print(cmd, flush=True)
+            if out.strip():
+                print(out, flush=True)
+        if rc != 0:
+            raise RuntimeError("hipcc failed: %s\n%s" % (cmd, out))
         objs.append(obj)
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)

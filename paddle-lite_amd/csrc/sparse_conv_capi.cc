@@ -98,6 +98,9 @@ struct pl_sparse_conv_handle {
   int row_blocks = 0, ksteps = 0;
   int64_t blocks_present = 0;
   DevBuf wblocks, kmask;
+  int wg_slots = 512;       // workgroups resident at once (2 per CU)
+  int mfma_i8_wide = 1;
+  int mfma_tile_quads = 0;  // 0 = chosen per problem
   // epilogue
   DevBuf scale, bias;
   int padded_rows = 0;
@@ -301,6 +304,11 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   pl_sparse_conv_handle* h = new (std::nothrow) pl_sparse_conv_handle();
   if (!h) return Fail(PL_ERR_BAD_ARG, "out of host memory");
   h->device = dev;
+  h->wg_slots = 2 * std::max(1, prop.multiProcessorCount);
+  if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_I8_WIDE")) h->mfma_i8_wide = std::atoi(e) != 0;
+  if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_TILE_QUADS")) h->mfma_tile_quads = std::max(0, std::min(32, std::atoi(e)));
+  // tuning switches for experiments; the defaults are what measured best
+  if (const char* e = std::getenv("PL_SPARSE_CONV_WG_SLOTS")) h->wg_slots = std::max(1, std::atoi(e));
   h->kind = desc->kind;
   h->oc = desc->oc;
   h->ic = desc->ic;
@@ -379,14 +387,25 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.K = h->ic;
     p.hw = im_size;
     p.P = P;
-    p.vec = vec;
     p.small = (P64 * h->ic < (1ll << 31)) && (P64 * h->oc * 4 < (1ll << 31));
     p.act = h->act;
     pl::MfmaConfig c{};
     c.out_kind = OutKind(h->kind);
     c.ks_max = 2;
     while (c.ks_max < h->ksteps) c.ks_max <<= 1;
-    c.waves = 4;  // the kernel's thread mapping is written for 256 threads
+    // Tile width: full 128-position tiles unless that leaves CUs without a
+    // workgroup (narrower tiles measured slower on the 392-workgroup metric
+    // shape: every workgroup pays for its own copy of the weight blocks).
+    const int row_groups = CeilDiv(h->row_blocks, 4);
+    const int64_t quads = static_cast<int64_t>(batch) * ((im_size + 3) / 4);
+    const int64_t full_tiles = (quads + 31) / 32;
+    c.tile_quads = 32;
+    if (full_tiles * row_groups < h->wg_slots / 2) {
+      const int64_t target_tiles = std::max<int64_t>(1, (h->wg_slots / 2) / row_groups);
+      c.tile_quads = static_cast<int>(std::min<int64_t>(32, std::max<int64_t>(8, (quads + target_tiles - 1) / target_tiles)));
+    }
+    c.i8_wide_stores = h->mfma_i8_wide;
+    if (h->mfma_tile_quads > 0) c.tile_quads = h->mfma_tile_quads;
     e = pl::LaunchBlockMfma(c, p, s);
   } else {
     pl::WalkParams p{};

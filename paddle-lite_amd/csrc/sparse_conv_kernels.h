@@ -70,18 +70,25 @@ struct MfmaParams {
   int ksteps;              // ceil(K / 32)
   int M, K;
   int hw;
-  uint32_t P;
-  int vec;
+  uint32_t P;              // batch * hw
   int small;               // 1: input and output tensors are each below 2 GB
-  int tiles;               // filled in by the launcher: position tiles
-  int row_groups;          // and groups of four row blocks
   DevAct act;
+  // filled in by the launcher
+  int vec;                 // hw >= 4: positions are handled four at a time by dword access
+  int quad_aligned;        // hw % 4 == 0: every quad is complete
+  int qpi;                 // quads per image = ceil(hw / 4)
+  uint32_t total_quads;    // batch * qpi
+  int tiles;               // tiles of tile_quads quads
+  int tile_quads;
+  int row_groups;          // groups of four row blocks
+  int i8_stage;            // int8 output is regrouped through LDS for 16-byte stores
 };
 
 struct MfmaConfig {
   int out_kind;
-  int ks_max;   // 2, 4, 8, 16 or 32 (>= ksteps)
-  int waves;    // row blocks per workgroup: 4, 8 or 16
+  int ks_max;          // 2, 4, 8, 16 or 32 (>= ksteps)
+  int tile_quads;      // 1..32 position quads per workgroup tile
+  int i8_wide_stores;  // int8 output: regroup through LDS into 16-byte stores
 };
 
 hipError_t LaunchBlockMfma(const MfmaConfig& cfg, const MfmaParams& p, hipStream_t stream);

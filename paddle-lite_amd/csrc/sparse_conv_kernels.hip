@@ -26,6 +26,23 @@
 #include <atomic>
 #include <type_traits>
 
+// This file is compiled as four translation units (in parallel) selected by
+// PL_KERNEL_PART: 0 = row walk + launch selection, 1 / 2 / 3 = block MFMA
+// kernels with fp32 / int8 / int32 output.  Without the macro everything is
+// built in one unit.
+#ifndef PL_KERNEL_PART
+#define PL_PART_WALK 1
+#define PL_PART_MFMA_F32 1
+#define PL_PART_MFMA_I8 1
+#define PL_PART_MFMA_ACC32 1
+#else
+#define PL_PART_WALK (PL_KERNEL_PART == 0)
+#define PL_PART_MFMA_F32 (PL_KERNEL_PART == 1)
+#define PL_PART_MFMA_I8 (PL_KERNEL_PART == 2)
+#define PL_PART_MFMA_ACC32 (PL_KERNEL_PART == 3)
+#endif
+#define PL_PART_MFMA_ANY (PL_PART_MFMA_F32 || PL_PART_MFMA_I8 || PL_PART_MFMA_ACC32)
+
 // Phase marks for tuning builds; compiled out of the library.
 #ifndef PL_PHASE_MARK
 #define PL_PHASE_MARK(i)
@@ -42,12 +59,25 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 // non-temporally so that they stream to memory instead of sitting dirty in
 // L2 until the end-of-kernel write-back.
 __device__ __forceinline__ void StreamStore(float4 v, void* dst) {
+#ifdef PL_PLAIN_STORES
+  *static_cast<float4*>(dst) = v;
+#else
   __builtin_nontemporal_store(v4f{v.x, v.y, v.z, v.w}, static_cast<v4f*>(dst));
+#endif
 }
 __device__ __forceinline__ void StreamStore(int4 v, void* dst) {
   __builtin_nontemporal_store(v4i{v.x, v.y, v.z, v.w}, static_cast<v4i*>(dst));
 }
 __device__ __forceinline__ void StreamStore(uint32_t v, void* dst) { __builtin_nontemporal_store(v, static_cast<uint32_t*>(dst)); }
+__device__ __forceinline__ void StreamStore(uint16_t v, void* dst) { __builtin_nontemporal_store(v, static_cast<uint16_t*>(dst)); }
+__device__ __forceinline__ void StreamStore(float2 v, void* dst) {
+  typedef float v2f __attribute__((ext_vector_type(2)));
+  __builtin_nontemporal_store(v2f{v.x, v.y}, static_cast<v2f*>(dst));
+}
+__device__ __forceinline__ void StreamStore(int2 v, void* dst) {
+  typedef int v2i __attribute__((ext_vector_type(2)));
+  __builtin_nontemporal_store(v2i{v.x, v.y}, static_cast<v2i*>(dst));
+}
 
 // ---------------------------------------------------------------- epilogue
 __device__ __forceinline__ float Activate(float v, const DevAct& a) {
@@ -237,6 +267,7 @@ __device__ __forceinline__ void StoreRow(const WalkParams& p, int row, uint32_t 
 }
 
 // ---------------------------------------------------------------- row walk
+#if PL_PART_WALK
 template <bool INT8, int OUT, int NR, int TP>
 __global__ void __launch_bounds__(1024) RowWalkKernel(const WalkParams p) {
   extern __shared__ uint32_t tile[];
@@ -333,28 +364,52 @@ __global__ void __launch_bounds__(1024) RowWalkKernel(const WalkParams p) {
   }
 }
 
-// -------------------------------------------------------------- block MFMA
-// LDS layout: xt[kg][slot] 16-byte cells, kg = group of 16 input channels,
-// slot = c*32 + j holds position 4*j + c of the 128-position tile, so that
-// MFMA column j of the four accumulators c = 0..3 are four consecutive
-// positions of one output row (one 16-byte fp32 store, one dword int8 store).
+#endif  // PL_PART_WALK
 
-// Stage with aligned dword loads (hw % 4 == 0).  Every load is unconditional
-// so that all loads of a batch are in flight together.  FAST: all channel
-// groups of the batch are complete, the tile lies inside the tensor and the
-// tensor is below 2 GB, so an address is a uniform base plus one 32-bit
-// per-lane offset (no per-load address arithmetic on the vector ALU).
-// Otherwise addresses are clamped and the results masked.
+// -------------------------------------------------------------- block MFMA
+#if PL_PART_MFMA_ANY
+// Positions are handled four at a time ("quads").  Every image is cut into
+// qpi = ceil(hw / 4) quads, so a quad never leaves its image; when hw is not
+// a multiple of four the last quad of an image holds hw % 4 valid positions.
+// Quads of all images form one sequence (index n*qpi + q); a workgroup
+// (4 wavefronts = 4 blocks of 32 output rows) handles a tile of J <= 32
+// consecutive quads.  MFMA column j of accumulator c is position c of the
+// tile's quad j, so a lane ends up with the four consecutive positions of
+// each of its rows (one 16-byte fp32 store or one dword int8 store).
+// LDS: xt[kg][c*32 + j], 16-byte cells, kg = group of 16 input channels.
+struct QuadInfo {
+  uint32_t n;    // image
+  uint32_t pp;   // first position of the quad in its image
+  int valid;     // 0: beyond the last image; else positions in the quad (1..4)
+};
+
+__device__ __forceinline__ QuadInfo LocateQuad(const MfmaParams& p, uint32_t quad) {
+  QuadInfo q;
+  const bool live = quad < p.total_quads;
+  const uint32_t qs = live ? quad : 0u;
+  q.n = qs / (uint32_t)p.qpi;
+  q.pp = 4u * (qs - q.n * (uint32_t)p.qpi);
+  const int left = p.hw - (int)q.pp;
+  q.valid = !live ? 0 : (left < 4 ? left : 4);
+  return q;
+}
+
+// Issue the dword loads of UNITS channel groups for one quad.  Global memory
+// needs no alignment for dword access.  A partial quad (valid < 4) reads the
+// last four positions of its row and shifts the unwanted ones out, so no
+// load leaves the tensor.  All loads are unconditional so that they are in
+// flight together.  FAST: the channel groups are complete and the tensor is
+// below 2 GB, so an address is a uniform base plus one 32-bit per-lane offset
+// (no per-load address arithmetic on the vector ALU).  Otherwise channel
+// indices are clamped and the values masked in CommitX.  Lanes beyond the
+// last image read the tensor's first bytes and are ignored.
 template <int UNITS, bool FAST>
-__device__ __forceinline__ void StageMfmaVec(uint4* xt, const MfmaParams& p, uint32_t tile0, int kg_base, int kg_lane, int j) {
-  const int n_kg = 2 * p.ksteps;
-  const uint32_t g = tile0 + 4u * j;
-  const bool live = FAST || g < p.P;
-  const uint32_t gs = live ? g : 0u;
-  const uint32_t n = gs / (uint32_t)p.hw, pp = gs % (uint32_t)p.hw;
-  uint32_t r[UNITS][16];
+__device__ __forceinline__ void LoadX(uint32_t (&r)[UNITS][16], const MfmaParams& p, const QuadInfo& q, int kg_base, int kg_lane) {
+  const bool live = q.valid > 0;
+  const uint32_t first = (q.valid == 4 || !live) ? q.pp : (uint32_t)(p.hw - 4);  // hw >= 4 on this path
+  const int sh = (q.valid == 4 || !live) ? 0 : 8 * (4 - q.valid);
   if (FAST) {
-    const uint32_t voff = (n * (uint32_t)p.K + 16u * (uint32_t)kg_lane) * (uint32_t)p.hw + pp;
+    const uint32_t voff = live ? (q.n * (uint32_t)p.K + 16u * (uint32_t)kg_lane) * (uint32_t)p.hw + first : 0u;
 #pragma unroll
     for (int u = 0; u < UNITS; ++u) {
 #pragma unroll
@@ -364,17 +419,30 @@ __device__ __forceinline__ void StageMfmaVec(uint4* xt, const MfmaParams& p, uin
       }
     }
   } else {
-    const int8_t* col = p.x + (size_t)n * p.K * p.hw + pp;
+    const int8_t* col = p.x + (live ? (size_t)q.n * p.K * p.hw + first : (size_t)0);
+    const size_t row_step = live ? (size_t)p.hw : (size_t)0;
 #pragma unroll
     for (int u = 0; u < UNITS; ++u) {
       const int kg = kg_base + kg_lane + 8 * u;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int ch = min(16 * kg + i, p.K - 1);
-        r[u][i] = *reinterpret_cast<const uint32_t*>(col + (size_t)ch * p.hw);
+        r[u][i] = *reinterpret_cast<const uint32_t*>(col + (size_t)ch * row_step);
       }
     }
   }
+  if (!p.quad_aligned) {
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) r[u][i] >>= sh;
+  }
+}
+
+// Transpose to channel-innermost and write the cells of four positions.
+template <int UNITS, bool FAST>
+__device__ __forceinline__ void CommitX(uint32_t (&r)[UNITS][16], uint4* xt, const MfmaParams& p, bool live, bool store, int kg_base, int kg_lane, int j) {
+  const int n_kg = 2 * p.ksteps;
 #pragma unroll
   for (int u = 0; u < UNITS; ++u) {
     const int kg = kg_base + kg_lane + 8 * u;
@@ -384,25 +452,24 @@ __device__ __forceinline__ void StageMfmaVec(uint4* xt, const MfmaParams& p, uin
     }
 #pragma unroll
     for (int b = 0; b < 4; ++b) Transpose4x4(r[u][4 * b], r[u][4 * b + 1], r[u][4 * b + 2], r[u][4 * b + 3]);
-    // now r[u][4b + c] = channels 16kg+4b..+3 of position 4j+c
-    if (FAST || kg < n_kg) {
+    // now r[u][4b + c] = channels 16kg+4b..+3 of the quad's position c
+    if (store && (FAST || kg < n_kg)) {
 #pragma unroll
       for (int c = 0; c < 4; ++c) xt[(size_t)kg * kMfmaTilePos + c * 32 + j] = make_uint4(r[u][c], r[u][4 + c], r[u][8 + c], r[u][12 + c]);
     }
   }
 }
 
-// Any hw: byte loads.
-__device__ __forceinline__ void StageMfmaBytes(uint4* xt, const MfmaParams& p, uint32_t tile0, int kg0, int kg_step, int j) {
+// hw < 4: byte loads, one position at a time.
+__device__ __forceinline__ void StageMfmaBytes(uint4* xt, const MfmaParams& p, uint32_t quad, bool quad_on, int kg0, int j) {
   const int n_kg = 2 * p.ksteps;
-  const uint32_t g = tile0 + 4u * j;
-  for (int kg = kg0; kg < n_kg; kg += kg_step) {
+  if (!quad_on) return;
+  const QuadInfo q = LocateQuad(p, quad);
+  for (int kg = kg0; kg < n_kg; kg += 8) {
     for (int c = 0; c < 4; ++c) {
-      const uint32_t gc = g + c;
       uint32_t d[4] = {0, 0, 0, 0};
-      if (gc < p.P) {
-        const uint32_t n = gc / (uint32_t)p.hw, pp = gc % (uint32_t)p.hw;
-        const int8_t* col = p.x + (size_t)n * p.K * p.hw + pp;
+      if (c < q.valid) {
+        const int8_t* col = p.x + (size_t)q.n * p.K * p.hw + q.pp + c;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const int ch = 16 * kg + i;
@@ -415,155 +482,178 @@ __device__ __forceinline__ void StageMfmaBytes(uint4* xt, const MfmaParams& p, u
   }
 }
 
-// Accumulator register r of lane l is output row 8*(r/4) + 4*(l/32) + r%4 of
-// the 32-row block, column l%32; the four accumulators are four consecutive
-// positions.
-template <int OUT, int ACT, bool VEC>
-__device__ __forceinline__ void MfmaEpilogue(const MfmaParams& p, const v16i (&acc)[4], int rb, int lane, uint32_t tile0) {
-  const uint32_t g = tile0 + 4u * (lane & 31);
-  if (g >= p.P) return;
-  const uint32_t n = g / (uint32_t)p.hw, pp = g % (uint32_t)p.hw;
+template <int OUT>
+__device__ __forceinline__ void StoreRun4(void* dst, const float* v, const int* q) {
+  if (OUT == kOutF32) {
+    StreamStore(make_float4(v[0], v[1], v[2], v[3]), dst);
+  } else if (OUT == kOutI8) {
+    uint32_t w = 0;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) w |= (uint32_t)(QuantizeI8(v[c]) & 0xff) << (8 * c);
+    StreamStore(w, dst);
+  } else {
+    StreamStore(make_int4(q[0], q[1], q[2], q[3]), dst);
+  }
+}
+
+// ACT < 0: activation type read at run time (slow paths only).
+template <int ACT>
+__device__ __forceinline__ float ActivateAny(float v, const DevAct& a) {
+  if (ACT < 0) return Activate(v, a);
+  return ActivateT<(ACT < 0 ? 0 : ACT)>(v, a);
+}
+
+// int8 output of a full tile inside one image: the wavefront's 32 rows x 128
+// positions are packed, written to its own 4 KB of LDS as [row][128 bytes]
+// and stored as 16 bytes per lane (8 rows x 128 contiguous bytes per
+// instruction) instead of one dword per lane.  `stage` is private to the
+// wavefront.
+template <int ACT>
+__device__ __forceinline__ void MfmaEpilogueI8Wide(const MfmaParams& p, const v16i (&acc)[4], int rb, int lane, uint32_t n, uint32_t pp, uint32_t* stage) {
   const int row_base = rb * 32 + 4 * (lane >> 5);
-  if (VEC && p.small && rb * 32 + 32 <= p.M) {
-    // all 32 rows exist and byte offsets fit 32 bits: uniform row base plus
-    // one per-lane offset
-    constexpr uint32_t kElem = OUT == kOutI8 ? 1u : 4u;
-    const uint32_t voff = ((n * (uint32_t)p.M + (uint32_t)row_base) * (uint32_t)p.hw + pp) * kElem;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int ro = 8 * (r >> 2) + (r & 3);
-      char* dst = static_cast<char*>(p.out) + (size_t)ro * (size_t)p.hw * kElem + voff;
-      int q[4];
-#pragma unroll
-      for (int c = 0; c < 4; ++c) q[c] = acc[c][r];
-      if (OUT == kOutAcc32) {
-        StreamStore(make_int4(q[0], q[1], q[2], q[3]), dst);
-      } else {
-        const float s = p.scale[row_base + ro], b = p.bias[row_base + ro];
-        float v[4];
-#pragma unroll
-        for (int c = 0; c < 4; ++c) v[c] = ActivateT<ACT>(__builtin_fmaf((float)q[c], s, b), p.act);
-        if (OUT == kOutF32) {
-          StreamStore(make_float4(v[0], v[1], v[2], v[3]), dst);
-        } else {
-          uint32_t w = (uint32_t)(QuantizeI8(v[0]) & 0xff) | ((uint32_t)(QuantizeI8(v[1]) & 0xff) << 8) |
-                       ((uint32_t)(QuantizeI8(v[2]) & 0xff) << 16) | ((uint32_t)(QuantizeI8(v[3]) & 0xff) << 24);
-          StreamStore(w, dst);
-        }
-      }
-    }
-    return;
-  }
-  float sc[16], bi[16];
-  if (OUT != kOutAcc32) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = row_base + 8 * (r >> 2) + (r & 3);  // scale / bias are padded to 32 rows per block
-      sc[r] = p.scale[row];
-      bi[r] = p.bias[row];
-    }
-  }
+  const int j = lane & 31;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
-    const int row = row_base + 8 * (r >> 2) + (r & 3);
-    if (row >= p.M) continue;
-    float v[4];
+    const int ro = 8 * (r >> 2) + (r & 3);
+    const float s = p.scale[row_base + ro], b = p.bias[row_base + ro];
+    uint32_t w = 0;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) w |= (uint32_t)(QuantizeI8(ActivateAny<ACT>(__builtin_fmaf((float)acc[c][r], s, b), p.act)) & 0xff) << (8 * c);
+    stage[(4 * (lane >> 5) + ro) * 32 + j] = w;  // row-local index 0..31, 32 dwords per row
+  }
+  // the same wavefront reads back: its LDS operations complete in order
+  char* obase = static_cast<char*>(p.out) + ((size_t)n * p.M + (size_t)rb * 32) * p.hw + pp;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = 8 * i + (lane >> 3), chunk = lane & 7;
+    const uint4 v = *reinterpret_cast<const uint4*>(stage + row * 32 + chunk * 4);
+    StreamStore(make_int4((int)v.x, (int)v.y, (int)v.z, (int)v.w), obase + (size_t)row * p.hw + chunk * 16);
+  }
+}
+
+// Accumulator register r of lane l is output row 8*(r/4) + 4*(l/32) + r%4 of
+// the 32-row block, column l%32; the four accumulators are the positions of
+// the lane's quad.  WHOLE: the quad has all four positions and the row block
+// all 32 rows (the common case, kept free of per-row conditions).
+template <int OUT, int ACT, bool WHOLE>
+__device__ __forceinline__ void MfmaEpilogueRows(const MfmaParams& p, const v16i (&acc)[4], int row_base, char* lane_base, int valid) {
+  constexpr uint32_t kElem = OUT == kOutI8 ? 1u : 4u;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int ro = 8 * (r >> 2) + (r & 3);
+    if (!WHOLE && row_base + ro >= p.M) continue;
+    char* dst = lane_base + (size_t)ro * (size_t)p.hw * kElem;
     int q[4];
+    float v[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) q[c] = acc[c][r];
     if (OUT != kOutAcc32) {
+      const float s = p.scale[row_base + ro], b = p.bias[row_base + ro];
 #pragma unroll
-      for (int c = 0; c < 4; ++c) v[c] = ActivateT<ACT>(__builtin_fmaf((float)q[c], sc[r], bi[r]), p.act);
+      for (int c = 0; c < 4; ++c) v[c] = ActivateAny<ACT>(__builtin_fmaf((float)q[c], s, b), p.act);
     }
-    if (VEC) {
-      const size_t idx = ((size_t)n * p.M + row) * p.hw + pp;
-      if (OUT == kOutF32) {
-        *reinterpret_cast<float4*>(static_cast<float*>(p.out) + idx) = make_float4(v[0], v[1], v[2], v[3]);
-      } else if (OUT == kOutI8) {
-        uint32_t w = (uint32_t)(QuantizeI8(v[0]) & 0xff) | ((uint32_t)(QuantizeI8(v[1]) & 0xff) << 8) |
-                     ((uint32_t)(QuantizeI8(v[2]) & 0xff) << 16) | ((uint32_t)(QuantizeI8(v[3]) & 0xff) << 24);
-        *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(p.out) + idx) = w;
-      } else {
-        *reinterpret_cast<int4*>(static_cast<int*>(p.out) + idx) = make_int4(q[0], q[1], q[2], q[3]);
-      }
+    if (WHOLE) {
+      StoreRun4<OUT>(dst, v, q);
     } else {
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        const uint32_t gc = g + c;
-        if (gc < p.P) {
-          const uint32_t nc = gc / (uint32_t)p.hw, pc = gc % (uint32_t)p.hw;
-          StoreOne<OUT>(p.out, ((size_t)nc * p.M + row) * p.hw + pc, v[c], q[c]);
+        if (c < valid) {
+          if (OUT == kOutF32) {
+            reinterpret_cast<float*>(dst)[c] = v[c];
+          } else if (OUT == kOutI8) {
+            reinterpret_cast<int8_t*>(dst)[c] = static_cast<int8_t>(QuantizeI8(v[c]));
+          } else {
+            reinterpret_cast<int*>(dst)[c] = q[c];
+          }
         }
       }
     }
   }
 }
 
-template <int KSMAX, int OUT>
-__global__ void __launch_bounds__(256) BlockMfmaKernel(const MfmaParams p) {
-  extern __shared__ uint4 xt[];
+template <int OUT, int ACT>
+__device__ __forceinline__ void MfmaEpilogue(const MfmaParams& p, const v16i (&acc)[4], int rb, int lane, const QuadInfo& qi) {
+  if (qi.valid == 0) return;
+  const int row_base = rb * 32 + 4 * (lane >> 5);
+  constexpr uint32_t kElem = OUT == kOutI8 ? 1u : 4u;
+  // per-lane part of the address; with a tensor below 2 GB it fits 32 bits
+  // and rows are reached through a uniform base
+  const size_t lane_off = (((size_t)qi.n * p.M + row_base) * p.hw + qi.pp) * kElem;
+  char* lane_base = p.small ? static_cast<char*>(p.out) + (uint32_t)lane_off : static_cast<char*>(p.out) + lane_off;
+  if (rb * 32 + 32 <= p.M && (p.quad_aligned || qi.valid == 4)) {
+    MfmaEpilogueRows<OUT, ACT, true>(p, acc, row_base, lane_base, 4);
+  } else {
+    MfmaEpilogueRows<OUT, ACT, false>(p, acc, row_base, lane_base, qi.valid);
+  }
+}
+
+// One tile: stage, multiply, finish.  The activation loads go out first (they
+// feed the longest chain: transpose, LDS, barrier), the wavefront's weight
+// blocks right behind them.
+template <int KSMAX, int OUT, int ACT, bool VEC>
+__device__ __forceinline__ void MfmaTile(const MfmaParams& p, uint4* xt, uint32_t kmask, int rb, int rbc, bool wave_on, int tile) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  // Workgroups are handed to the 8 XCDs round robin.  Map the linear id so
-  // that the workgroups sharing one activation tile (all row-block groups)
-  // run on the same XCD one after the other: the tile is then fetched into
-  // that XCD's L2 once.
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int tile = (slot / p.row_groups) * 8 + xcd;
-  if (tile >= p.tiles) return;
-  const uint32_t tile0 = (uint32_t)tile * (uint32_t)kMfmaTilePos;
-  const int rb = (slot % p.row_groups) * 4 + wave;
-  const bool wave_on = rb < p.row_blocks;
-  const int rbc = wave_on ? rb : p.row_blocks - 1;
-  PL_PHASE_MARK(0);
-
-  // weight blocks of this wavefront's 32 rows -> registers (blocks of absent
-  // k-steps are never multiplied; their loads are clamped to a valid block)
-  const uint32_t kmask = wave_on ? p.kmask[rbc] : 0u;
+  const int J = p.tile_quads;
+  const int j = tid & 31;    // quad of the tile
+  const int kg0 = tid >> 5;  // 8 channel groups per pass of the workgroup
+  const uint32_t quad0 = (uint32_t)tile * (uint32_t)J;
   v4i a[KSMAX];
+  auto load_weights = [&]() {
+    // blocks of absent k-steps are never multiplied; their loads are clamped
 #pragma unroll
-  for (int ks = 0; ks < KSMAX; ++ks) {
-    const int ksc = min(ks, p.ksteps - 1);
-    a[ks] = static_cast<const v4i*>(p.wblocks)[((size_t)rbc * p.ksteps + ksc) * 64 + lane];
-  }
-
-  PL_PHASE_MARK(1);
-  // ---- stage 128 positions x (32*ksteps) channels, channel-innermost
-  {
-    const int j = tid & 31;    // position quad of the tile
-    const int kg0 = tid >> 5;  // 8 channel groups per pass of the workgroup
-    if (p.vec) {
-      constexpr int kPasses = (2 * KSMAX + 7) / 8;  // passes that cover 2*KSMAX groups
-      constexpr int kBatch = kPasses < 4 ? kPasses : 4;
-      const bool inside = p.small && tile0 + (uint32_t)kMfmaTilePos <= p.P;
+    for (int ks = 0; ks < KSMAX; ++ks) {
+      const int ksc = min(ks, p.ksteps - 1);
+      a[ks] = static_cast<const v4i*>(p.wblocks)[((size_t)rbc * p.ksteps + ksc) * 64 + lane];
+    }
+  };
+  const bool quad_on = j < J;
+  const int jc = quad_on ? j : J - 1;  // idle lanes repeat the last quad's loads
+  if (VEC) {
+    constexpr int kPasses = (2 * KSMAX + 7) / 8;  // passes that cover 2*KSMAX groups
+    constexpr int kBatch = kPasses < 4 ? kPasses : 4;
+    const QuadInfo qs = LocateQuad(p, quad0 + (uint32_t)jc);
+    const bool live = qs.valid > 0;
+    uint32_t r[kBatch][16];
+    const bool fast0 = p.small && 16 * 8 * kBatch <= p.K;
+    if (fast0) {
+      LoadX<kBatch, true>(r, p, qs, 0, kg0);
+    } else {
+      LoadX<kBatch, false>(r, p, qs, 0, kg0);
+    }
+    load_weights();
+    if (fast0) {
+      CommitX<kBatch, true>(r, xt, p, true, quad_on && live, 0, kg0, jc);
+    } else {
+      CommitX<kBatch, false>(r, xt, p, live, quad_on, 0, kg0, jc);
+    }
 #pragma unroll
-      for (int pass = 0; pass < kPasses; pass += kBatch) {
-        if (8 * pass < 2 * p.ksteps) {
-          if (inside && 16 * 8 * (pass + kBatch) <= p.K) {
-            StageMfmaVec<kBatch, true>(xt, p, tile0, 8 * pass, kg0, j);
-          } else {
-            StageMfmaVec<kBatch, false>(xt, p, tile0, 8 * pass, kg0, j);
-          }
+    for (int pass = kBatch; pass < kPasses; pass += kBatch) {
+      if (8 * pass < 2 * p.ksteps) {
+        if (p.small && 16 * 8 * (pass + kBatch) <= p.K) {
+          LoadX<kBatch, true>(r, p, qs, 8 * pass, kg0);
+          CommitX<kBatch, true>(r, xt, p, true, quad_on && live, 8 * pass, kg0, jc);
+        } else {
+          LoadX<kBatch, false>(r, p, qs, 8 * pass, kg0);
+          CommitX<kBatch, false>(r, xt, p, live, quad_on, 8 * pass, kg0, jc);
         }
       }
-    } else {
-      StageMfmaBytes(xt, p, tile0, kg0, 8, j);
     }
+  } else {
+    load_weights();
+    StageMfmaBytes(xt, p, quad0 + (uint32_t)jc, quad_on, kg0, jc);
   }
   PL_PHASE_MARK(2);
   __syncthreads();
   PL_PHASE_MARK(3);
   if (!wave_on) return;
 
-  // ---- multiply: D[32 rows][32 cols] += A[32 x 32k] * B[32k x 32], four
-  //      column blocks
+  // ---- multiply: D[32 rows][32 cols] += A[32 x 32k] * B[32k x 32]
   v16i acc[4];
 #pragma unroll
   for (int c = 0; c < 4; ++c)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[c][i] = 0;
-
   const uint4* bbase = xt + (size_t)(lane >> 5) * kMfmaTilePos + (lane & 31);
 #pragma unroll
   for (int ks = 0; ks < KSMAX; ++ks) {
@@ -576,18 +666,58 @@ __global__ void __launch_bounds__(256) BlockMfmaKernel(const MfmaParams p) {
       }
     }
   }
-
   PL_PHASE_MARK(4);
+  if ((lane & 31) >= J) return;
+  const QuadInfo qo = LocateQuad(p, quad0 + (uint32_t)(lane & 31));
+  if (OUT == kOutI8 && VEC) {
+    // wide stores need a full tile inside one image whose rows all exist and
+    // 16-byte aligned row pieces
+    const QuadInfo q0 = LocateQuad(p, quad0);
+    const bool wide = p.i8_stage && J == 32 && p.small && rb * 32 + 32 <= p.M && (p.hw & 15) == 0 && quad0 + 32u <= p.total_quads && q0.pp + 128u <= (uint32_t)p.hw;
+    if (wide) {
+      uint32_t* stage = reinterpret_cast<uint32_t*>(xt + (size_t)2 * p.ksteps * kMfmaTilePos) + (threadIdx.x >> 6) * 1024;
+      MfmaEpilogueI8Wide<ACT>(p, acc, rb, lane, q0.n, q0.pp, stage);
+      return;
+    }
+  }
+  MfmaEpilogue<OUT, ACT>(p, acc, rb, lane, qo);
+}
+
+template <int KSMAX, int OUT, int ACT, bool VEC>
+__device__ __forceinline__ void MfmaBody(const MfmaParams& p, uint4* xt) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  // Workgroups are handed to the 8 XCDs round robin.  Map the linear id so
+  // that the workgroups sharing one activation tile (all row-block groups)
+  // run on the same XCD one after the other: the tile is then fetched into
+  // that XCD's L2 once.
+  const int xcd = blockIdx.x & 7, wg_slot = blockIdx.x >> 3;
+  const int tile = (wg_slot / p.row_groups) * 8 + xcd;
+  if (tile >= p.tiles) return;
+  const int rb = (wg_slot % p.row_groups) * 4 + wave;
+  const bool wave_on = rb < p.row_blocks;
+  const int rbc = wave_on ? rb : p.row_blocks - 1;
+  const uint32_t kmask = wave_on ? p.kmask[rbc] : 0u;
+  PL_PHASE_MARK(0);
+  MfmaTile<KSMAX, OUT, ACT, VEC>(p, xt, kmask, rb, rbc, wave_on, tile);
+  PL_PHASE_MARK(6);
+}
+
+// At least two workgroups per CU (two wavefronts per SIMD): caps the kernel
+// at 256 VGPRs.
+template <int KSMAX, int OUT>
+__global__ void __launch_bounds__(256, 2) BlockMfmaKernel(const MfmaParams p) {
+  extern __shared__ uint4 xt[];
+  if (!p.vec) {
+    MfmaBody<KSMAX, OUT, -1, false>(p, xt);
+    return;
+  }
   DispatchAct(OUT == kOutAcc32 ? 0 : p.act.type, [&](auto act_c) {
     constexpr int ACT = decltype(act_c)::value;
-    if (p.vec) {
-      MfmaEpilogue<OUT, ACT, true>(p, acc, rb, lane, tile0);
-    } else {
-      MfmaEpilogue<OUT, ACT, false>(p, acc, rb, lane, tile0);
-    }
+    MfmaBody<KSMAX, OUT, ACT, true>(p, xt);
   });
-  PL_PHASE_MARK(5);
 }
+
+#endif  // PL_PART_MFMA_ANY
 
 // ------------------------------------------------------------- launch glue
 // Dynamic LDS above the default limit has to be enabled per kernel and
@@ -610,6 +740,7 @@ hipError_t LaunchWithLds(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipSt
   return hipGetLastError();
 }
 
+#if PL_PART_WALK
 template <bool INT8, int OUT, int NR>
 hipError_t WalkByTile(const WalkConfig& cfg, const WalkParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
   switch (cfg.tile_pos) {
@@ -633,10 +764,12 @@ hipError_t WalkByRows(const WalkConfig& cfg, const WalkParams& p, dim3 grid, dim
   return cfg.nrows == 2 ? WalkByTile<INT8, OUT, 2>(cfg, p, grid, block, lds, s)
                         : WalkByTile<INT8, OUT, 1>(cfg, p, grid, block, lds, s);
 }
+#endif  // PL_PART_WALK
 
+#if PL_PART_MFMA_ANY
 template <int OUT>
-hipError_t MfmaByKs(const MfmaConfig& cfg, const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
-  switch (cfg.ks_max) {
+hipError_t MfmaByKs(int ks_max, const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
+  switch (ks_max) {
     case 2:
       return LaunchWithLds(BlockMfmaKernel<2, OUT>, grid, block, lds, s, p);
     case 4:
@@ -651,9 +784,27 @@ hipError_t MfmaByKs(const MfmaConfig& cfg, const MfmaParams& p, dim3 grid, dim3 
       return hipErrorInvalidValue;
   }
 }
+#endif  // PL_PART_MFMA_ANY
 
 }  // namespace
 
+// The block MFMA kernels of each output kind are compiled in their own
+// translation unit (see the part macros at the top of this file).
+hipError_t LaunchMfmaF32(int ks_max, const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s);
+hipError_t LaunchMfmaI8(int ks_max, const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s);
+hipError_t LaunchMfmaAcc32(int ks_max, const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s);
+
+#if PL_PART_MFMA_F32
+hipError_t LaunchMfmaF32(int ks_max, const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s) { return MfmaByKs<kOutF32>(ks_max, p, grid, block, lds, s); }
+#endif
+#if PL_PART_MFMA_I8
+hipError_t LaunchMfmaI8(int ks_max, const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s) { return MfmaByKs<kOutI8>(ks_max, p, grid, block, lds, s); }
+#endif
+#if PL_PART_MFMA_ACC32
+hipError_t LaunchMfmaAcc32(int ks_max, const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s) { return MfmaByKs<kOutAcc32>(ks_max, p, grid, block, lds, s); }
+#endif
+
+#if PL_PART_WALK
 hipError_t LaunchRowWalk(const WalkConfig& cfg, const WalkParams& p, hipStream_t stream) {
   if (p.P == 0 || p.n_groups == 0) return hipSuccess;
   const size_t lds = (size_t)p.kd * cfg.tile_pos * 4;
@@ -681,24 +832,33 @@ hipError_t LaunchRowWalk(const WalkConfig& cfg, const WalkParams& p, hipStream_t
 hipError_t LaunchBlockMfma(const MfmaConfig& cfg, const MfmaParams& p, hipStream_t stream) {
   if (p.P == 0 || p.row_blocks == 0) return hipSuccess;
   if (p.ksteps > cfg.ks_max || p.ksteps > 32) return hipErrorInvalidValue;
-  const size_t lds = (size_t)2 * p.ksteps * kMfmaTilePos * 16;
+  if (cfg.tile_quads < 1 || cfg.tile_quads > 32 || p.hw < 1) return hipErrorInvalidValue;
+  size_t lds = (size_t)2 * p.ksteps * kMfmaTilePos * 16;
   if (lds > (size_t)kMaxLdsBytes) return hipErrorInvalidValue;
-  const uint32_t tiles = (p.P + kMfmaTilePos - 1) / kMfmaTilePos;
-  if (cfg.waves != 4) return hipErrorInvalidValue;
   MfmaParams q = p;
+  q.qpi = (p.hw + 3) / 4;
+  q.total_quads = (p.P / (uint32_t)p.hw) * (uint32_t)q.qpi;
+  q.vec = p.hw >= 4;
+  q.quad_aligned = p.hw % 4 == 0;
+  q.tile_quads = cfg.tile_quads;
+  const uint32_t tiles = (q.total_quads + cfg.tile_quads - 1) / cfg.tile_quads;
   q.tiles = (int)tiles;
   q.row_groups = (p.row_blocks + 3) / 4;
-  dim3 grid(8u * q.row_groups * ((tiles + 7) / 8)), block(256);
+  // int8 output: 4 KB per wavefront behind the activation tile to widen stores
+  q.i8_stage = cfg.out_kind == kOutI8 && cfg.i8_wide_stores && lds + 16384 <= (size_t)kMaxLdsBytes;
+  if (q.i8_stage) lds += 16384;
+  dim3 grid(8u * q.row_groups * ((tiles + 7) / 8)), block(256);  // one workgroup per (tile, row group)
   switch (cfg.out_kind) {
     case kOutF32:
-      return MfmaByKs<kOutF32>(cfg, q, grid, block, lds, stream);
+      return LaunchMfmaF32(cfg.ks_max, q, grid, block, lds, stream);
     case kOutI8:
-      return MfmaByKs<kOutI8>(cfg, q, grid, block, lds, stream);
+      return LaunchMfmaI8(cfg.ks_max, q, grid, block, lds, stream);
     case kOutAcc32:
-      return MfmaByKs<kOutAcc32>(cfg, q, grid, block, lds, stream);
+      return LaunchMfmaAcc32(cfg.ks_max, q, grid, block, lds, stream);
     default:
       return hipErrorInvalidValue;
   }
 }
+#endif  // PL_PART_WALK
 
 }  // namespace pl
