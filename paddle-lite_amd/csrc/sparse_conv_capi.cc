@@ -158,6 +158,14 @@ int BuildRowWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
         if (nr == 2) wts.push_back(p1);
       }
     }
+    // The kernel takes entries kWalkBatch at a time.  Padding entries have
+    // zero weights; fp32 ones read the all-zero row that the kernel appends
+    // to its tile (index ic), so that a non-finite input cannot leak in.
+    while ((kidx.size() - d.first) % pl::kWalkBatch != 0) {
+      kidx.push_back(h->int8 ? 0u : static_cast<uint32_t>(L.ic));
+      wts.push_back(0u);
+      if (nr == 2) wts.push_back(0u);
+    }
     d.count = static_cast<uint32_t>(kidx.size()) - d.first;
     groups.push_back(d);
   }
@@ -227,7 +235,7 @@ pl::WalkConfig ChooseWalk(const pl_sparse_conv_handle* h, uint32_t P) {
   c.int8 = h->int8;
   c.out_kind = OutKind(h->kind);
   c.nrows = h->semi ? 2 : 1;
-  const size_t row_bytes = static_cast<size_t>(h->kd) * 4;
+  const size_t row_bytes = static_cast<size_t>(h->kd + (h->int8 ? 0 : 1)) * 4;  // fp32 tiles carry a zero row
   // prefer tiles of at most 64 KB (two workgroups per CU), never below one
   // wavefront of positions unless the channel count forces it
   int tp = 256;
@@ -243,6 +251,12 @@ pl::WalkConfig ChooseWalk(const pl_sparse_conv_handle* h, uint32_t P) {
   int slices = static_cast<int>((1024 + tiles - 1) / tiles);
   slices = std::min(slices, std::max(1, h->n_groups / nwaves));
   slices = std::max(1, std::min(slices, 65535));
+  // tuning overrides (power-of-two thread counts only)
+  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_THREADS")) {
+    const int t = std::atoi(e);
+    if (t >= tp && t <= 1024 && (t & (t - 1)) == 0) c.threads = t;
+  }
+  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_SLICES")) slices = std::max(1, std::min(std::atoi(e), std::max(1, h->n_groups)));
   c.slices = slices;
   return c;
 }

@@ -27,6 +27,10 @@ struct DevGroup {
   uint32_t count;
 };
 
+// Entries of an index list are taken this many at a time; every list is
+// padded to a multiple of it with zero-weight entries.
+constexpr int kWalkBatch = 8;
+
 // Row-walk SpMM: arguments common to all instantiations.
 struct WalkParams {
   const void* x;
@@ -39,11 +43,12 @@ struct WalkParams {
   int n_groups;
   int groups_per_slice;
   int M, K;
-  int kd;                // LDS tile rows: K (fp32) or ceil(K/4) (int8)
+  int kd;                // LDS tile rows: K (fp32, plus one all-zero row) or ceil(K/4) (int8)
   int hw;
   uint32_t P;            // batch * hw
   int vec;               // 1: hw % 4 == 0 and pointers 16-byte aligned
   DevAct act;
+  int tiles, slices;     // filled in by the launcher
 };
 
 struct WalkConfig {

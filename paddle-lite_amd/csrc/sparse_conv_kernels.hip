@@ -154,12 +154,16 @@ __device__ __forceinline__ void Transpose4x4(uint32_t& r0, uint32_t& r1, uint32_
 }
 
 // ------------------------------------------------------------ tile staging
-// fp32: tile[k][TP] floats.  int8: tile[q][TP] dwords, dword = channels
-// 4q..4q+3 of one position (channels past K read as zero).
+// fp32: tile[k][TP] floats plus one row of zeros.  int8: tile[q][TP] dwords, dword = channels
+// 4q..4q+3 of one position (channels past K read as zero).  The aligned path
+// issues a batch of row loads before it touches LDS so that they are in
+// flight together.
 template <bool INT8, int TP>
 __device__ __forceinline__ void StageTile(uint32_t* tile, const WalkParams& p, uint32_t tile0) {
   const int tid = threadIdx.x;
   const int nthreads = blockDim.x;
+  // fp32 tiles end in an all-zero row, the target of list padding entries
+  if (!INT8 && tid < TP) tile[(size_t)p.kd * TP + tid] = 0u;
   if (p.vec) {
     constexpr int TPV = TP / 4;  // groups of four positions per row
     const int j4 = tid % TPV;
@@ -167,23 +171,46 @@ __device__ __forceinline__ void StageTile(uint32_t* tile, const WalkParams& p, u
     const bool live = g < p.P;
     const uint32_t n = live ? g / (uint32_t)p.hw : 0u;
     const uint32_t pp = live ? g % (uint32_t)p.hw : 0u;
-    for (int k = tid / TPV; k < p.kd; k += nthreads / TPV) {
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (live) {
-        if (!INT8) {
-          const float* src = static_cast<const float*>(p.x) + ((size_t)n * p.K + k) * p.hw + pp;
-          v = *reinterpret_cast<const uint4*>(src);
-        } else {
-          const int8_t* src = static_cast<const int8_t*>(p.x) + ((size_t)n * p.K + 4 * k) * p.hw + pp;
-          uint32_t r0 = *reinterpret_cast<const uint32_t*>(src);
-          uint32_t r1 = (4 * k + 1 < p.K) ? *reinterpret_cast<const uint32_t*>(src + p.hw) : 0u;
-          uint32_t r2 = (4 * k + 2 < p.K) ? *reinterpret_cast<const uint32_t*>(src + 2 * (size_t)p.hw) : 0u;
-          uint32_t r3 = (4 * k + 3 < p.K) ? *reinterpret_cast<const uint32_t*>(src + 3 * (size_t)p.hw) : 0u;
-          Transpose4x4(r0, r1, r2, r3);
-          v = make_uint4(r0, r1, r2, r3);
+    const int k_step = nthreads / TPV;
+    if (!INT8) {
+      constexpr int kBatch = 8;
+      const float* base = static_cast<const float*>(p.x) + (size_t)n * p.K * p.hw + pp;
+      for (int k0 = tid / TPV; k0 < p.kd; k0 += kBatch * k_step) {
+        uint4 v[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+          const int k = min(k0 + u * k_step, p.kd - 1);
+          v[u] = *reinterpret_cast<const uint4*>(base + (size_t)k * p.hw);
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+          const int k = k0 + u * k_step;
+          if (k < p.kd) *reinterpret_cast<uint4*>(tile + (size_t)k * TP + 4 * j4) = live ? v[u] : make_uint4(0, 0, 0, 0);
         }
       }
-      *reinterpret_cast<uint4*>(tile + (size_t)k * TP + 4 * j4) = v;
+    } else {
+      constexpr int kBatch = 4;
+      const int8_t* base = static_cast<const int8_t*>(p.x) + (size_t)n * p.K * p.hw + pp;
+      for (int k0 = tid / TPV; k0 < p.kd; k0 += kBatch * k_step) {
+        uint32_t r[kBatch][4];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+          const int k = min(k0 + u * k_step, p.kd - 1);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int ch = min(4 * k + i, p.K - 1);
+            r[u][i] = *reinterpret_cast<const uint32_t*>(base + (size_t)ch * p.hw);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+          const int k = k0 + u * k_step;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) r[u][i] = (live && 4 * k + i < p.K) ? r[u][i] : 0u;
+          Transpose4x4(r[u][0], r[u][1], r[u][2], r[u][3]);
+          if (k < p.kd) *reinterpret_cast<uint4*>(tile + (size_t)k * TP + 4 * j4) = make_uint4(r[u][0], r[u][1], r[u][2], r[u][3]);
+        }
+      }
     }
   } else {
     const int j = tid % TP;
@@ -233,18 +260,18 @@ __device__ __forceinline__ void StoreRow(const WalkParams& p, int row, uint32_t 
     if (OUT == kOutF32) {
       float* dst = static_cast<float*>(p.out) + idx;
       if (PPL == 4) {
-        *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+        StreamStore(make_float4(v[0], v[1], v[2], v[3]), dst);
       } else if (PPL == 2) {
-        *reinterpret_cast<float2*>(dst) = make_float2(v[0], v[1]);
+        StreamStore(make_float2(v[0], v[1]), dst);
       } else {
-        dst[0] = v[0];
+        __builtin_nontemporal_store(v[0], dst);
       }
     } else if (OUT == kOutI8) {
       int8_t* dst = static_cast<int8_t*>(p.out) + idx;
       if (PPL == 4) {
         uint32_t w = (uint32_t)(QuantizeI8(v[0]) & 0xff) | ((uint32_t)(QuantizeI8(v[1]) & 0xff) << 8) |
                      ((uint32_t)(QuantizeI8(v[2]) & 0xff) << 16) | ((uint32_t)(QuantizeI8(v[3]) & 0xff) << 24);
-        *reinterpret_cast<uint32_t*>(dst) = w;
+        StreamStore(w, dst);
       } else {
 #pragma unroll
         for (int j = 0; j < PPL; ++j) dst[j] = static_cast<int8_t>(QuantizeI8(v[j]));
@@ -268,27 +295,78 @@ __device__ __forceinline__ void StoreRow(const WalkParams& p, int row, uint32_t 
 
 // ---------------------------------------------------------------- row walk
 #if PL_PART_WALK
-template <bool INT8, int OUT, int NR, int TP>
-__global__ void __launch_bounds__(1024) RowWalkKernel(const WalkParams p) {
-  extern __shared__ uint32_t tile[];
-  constexpr int PPL = TP >= 64 ? TP / 64 : 1;  // positions per lane
-  const uint32_t tile0 = blockIdx.x * (uint32_t)TP;
+// Multiply-accumulate of one index entry into the lane's PPL positions.
+template <bool INT8, int NR, int PPL, int TP>
+__device__ __forceinline__ void WalkEntry(const uint32_t* xbase, uint32_t k, uint32_t w0, uint32_t w1, float (&f0)[PPL], float (&f1)[PPL], int (&a0)[PPL], int (&a1)[PPL]) {
+  const uint32_t* xp = xbase + (size_t)k * TP;
+  uint32_t xv[PPL];
+  if (PPL == 4) {
+    uint4 t = *reinterpret_cast<const uint4*>(xp);
+    xv[0] = t.x;
+    xv[1 % PPL] = t.y;
+    xv[2 % PPL] = t.z;
+    xv[3 % PPL] = t.w;
+  } else if (PPL == 2) {
+    uint2 t = *reinterpret_cast<const uint2*>(xp);
+    xv[0] = t.x;
+    xv[1 % PPL] = t.y;
+  } else {
+    xv[0] = xp[0];
+  }
+#pragma unroll
+  for (int j = 0; j < PPL; ++j) {
+    if (INT8) {
+      a0[j] = __builtin_amdgcn_sdot4((int)xv[j], (int)w0, a0[j], false);
+      if (NR == 2) a1[j] = __builtin_amdgcn_sdot4((int)xv[j], (int)w1, a1[j], false);
+    } else {
+      f0[j] = __builtin_fmaf(__uint_as_float(xv[j]), __uint_as_float(w0), f0[j]);
+      if (NR == 2) f1[j] = __builtin_fmaf(__uint_as_float(xv[j]), __uint_as_float(w1), f1[j]);
+    }
+  }
+}
 
+template <bool INT8, int OUT, int NR, int TP, int ACT>
+__device__ __forceinline__ void RowWalkBody(const WalkParams& p, uint32_t* tile) {
+  constexpr int PPL = TP >= 64 ? TP / 64 : 1;  // positions per lane
+  // Index lists, weights, scales and biases are wave-uniform and written by
+  // the host before the launch: read them through the constant address
+  // space, i.e. with scalar loads.  Left to itself the compiler turns some
+  // of them into vector loads of one address per wavefront, which cost a
+  // full address-coalescing pass each and, for the bias, make the walk wait
+  // for the previous row's output stores.
+  typedef const __attribute__((address_space(4))) float* ConstFloats;
+  typedef const __attribute__((address_space(4))) uint32_t* ConstWords;
+  const ConstFloats biasp = (ConstFloats)p.bias;
+  const ConstFloats scalep = (ConstFloats)p.scale;
+  static_assert(sizeof(DevGroup) == 16, "DevGroup is read as four words");
+  const ConstWords group_words = (ConstWords)p.groups;
+  // 1-D grid; the slices (row ranges) of one tile are neighbours in the
+  // per-XCD order so that the tile is fetched into one L2
+  const int xcd = blockIdx.x & 7, wg_slot = blockIdx.x >> 3;
+  const int tile_id = (wg_slot / p.slices) * 8 + xcd;
+  const int slice = wg_slot % p.slices;
+  if (tile_id >= p.tiles) return;
+  const uint32_t tile0 = (uint32_t)tile_id * (uint32_t)TP;
+
+  PL_PHASE_MARK(0);
   StageTile<INT8, TP>(tile, p, tile0);
+  PL_PHASE_MARK(1);
   __syncthreads();
+  PL_PHASE_MARK(2);
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int nwaves = blockDim.x >> 6;
-  const int g_begin = blockIdx.y * p.groups_per_slice;
+  const int g_begin = slice * p.groups_per_slice;
   const int g_end = min(p.n_groups, g_begin + p.groups_per_slice);
   const bool lane_on = (TP >= 64) || (lane < TP);
   const uint32_t* xbase = tile + (lane_on ? lane * PPL : 0);
 
   for (int g = g_begin + wave; g < g_end; g += nwaves) {
-    const DevGroup grp = p.groups[g];
-    const uint32_t* __restrict__ kp = p.kidx + grp.first;
-    const uint32_t* __restrict__ wp = p.wts + (size_t)grp.first * NR;
+    const ConstWords gw = group_words + (size_t)g * 4;
+    const DevGroup grp = {(int)gw[0], (int)gw[1], gw[2], gw[3]};
+    const ConstWords kp = (ConstWords)p.kidx + grp.first;
+    const ConstWords wp = (ConstWords)p.wts + (size_t)grp.first * NR;
 
     float f0[PPL], f1[PPL];
     int a0[PPL], a1[PPL];
@@ -298,8 +376,9 @@ __global__ void __launch_bounds__(1024) RowWalkKernel(const WalkParams p) {
       f0[j] = f1[j] = 0.0f;
     }
     if (!INT8) {
-      const float b0 = p.bias ? p.bias[grp.row0] : 0.0f;
-      const float b1 = (p.bias && NR == 2 && grp.nrows == 2) ? p.bias[grp.row0 + 1] : 0.0f;
+      // the accumulator starts at the bias, entries follow in index order
+      const float b0 = biasp ? biasp[grp.row0] : 0.0f;
+      const float b1 = (biasp && NR == 2 && grp.nrows == 2) ? biasp[grp.row0 + 1] : 0.0f;
 #pragma unroll
       for (int j = 0; j < PPL; ++j) {
         f0[j] = b0;
@@ -307,36 +386,12 @@ __global__ void __launch_bounds__(1024) RowWalkKernel(const WalkParams p) {
       }
     }
 
-#pragma unroll 4
-    for (uint32_t e = 0; e < grp.count; ++e) {
-      const uint32_t k = kp[e];
-      const uint32_t w0 = wp[(size_t)e * NR];
-      const uint32_t w1 = (NR == 2) ? wp[(size_t)e * NR + 1] : 0u;
-      const uint32_t* xp = xbase + (size_t)k * TP;
-      uint32_t xv[PPL];
-      if (PPL == 4) {
-        uint4 t = *reinterpret_cast<const uint4*>(xp);
-        xv[0] = t.x;
-        xv[1 % PPL] = t.y;
-        xv[2 % PPL] = t.z;
-        xv[3 % PPL] = t.w;
-      } else if (PPL == 2) {
-        uint2 t = *reinterpret_cast<const uint2*>(xp);
-        xv[0] = t.x;
-        xv[1 % PPL] = t.y;
-      } else {
-        xv[0] = xp[0];
-      }
+    // the list length is a multiple of kWalkBatch: no remainder loop, whose
+    // entries would each wait for their own scalar loads
+    for (uint32_t e = 0; e < grp.count; e += kWalkBatch) {
 #pragma unroll
-      for (int j = 0; j < PPL; ++j) {
-        if (INT8) {
-          a0[j] = __builtin_amdgcn_sdot4((int)xv[j], (int)w0, a0[j], false);
-          if (NR == 2) a1[j] = __builtin_amdgcn_sdot4((int)xv[j], (int)w1, a1[j], false);
-        } else {
-          f0[j] = __builtin_fmaf(__uint_as_float(xv[j]), __uint_as_float(w0), f0[j]);
-          if (NR == 2) f1[j] = __builtin_fmaf(__uint_as_float(xv[j]), __uint_as_float(w1), f1[j]);
-        }
-      }
+      for (int j = 0; j < kWalkBatch; ++j)
+        WalkEntry<INT8, NR, PPL, TP>(xbase, kp[e + j], wp[(size_t)(e + j) * NR], NR == 2 ? wp[(size_t)(e + j) * NR + NR - 1] : 0u, f0, f1, a0, a1);
     }
 
     if (!lane_on) continue;
@@ -349,21 +404,30 @@ __global__ void __launch_bounds__(1024) RowWalkKernel(const WalkParams p) {
       const int* acc = r == 0 ? a0 : a1;
       if (INT8) {
         if (OUT != kOutAcc32) {
-          const float s = p.scale[row];
-          const float b = p.bias ? p.bias[row] : 0.0f;
+          const float s = scalep[row];
+          const float b = biasp ? biasp[row] : 0.0f;
 #pragma unroll
-          for (int j = 0; j < PPL; ++j) v[j] = Activate(__builtin_fmaf((float)acc[j], s, b), p.act);
+          for (int j = 0; j < PPL; ++j) v[j] = ActivateT<ACT>(__builtin_fmaf((float)acc[j], s, b), p.act);
         }
       } else {
         const float* f = r == 0 ? f0 : f1;
 #pragma unroll
-        for (int j = 0; j < PPL; ++j) v[j] = Activate(f[j], p.act);
+        for (int j = 0; j < PPL; ++j) v[j] = ActivateT<ACT>(f[j], p.act);
       }
       StoreRow<OUT, PPL>(p, row, gpos, v, acc);
     }
   }
+  PL_PHASE_MARK(3);
 }
 
+template <bool INT8, int OUT, int NR, int TP>
+__global__ void __launch_bounds__(1024) RowWalkKernel(const WalkParams p) {
+  extern __shared__ uint32_t tile[];
+  DispatchAct(OUT == kOutAcc32 ? 0 : p.act.type, [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
+    RowWalkBody<INT8, OUT, NR, TP, ACT>(p, tile);
+  });
+}
 #endif  // PL_PART_WALK
 
 // -------------------------------------------------------------- block MFMA
@@ -807,23 +871,26 @@ hipError_t LaunchMfmaAcc32(int ks_max, const MfmaParams& p, dim3 grid, dim3 bloc
 #if PL_PART_WALK
 hipError_t LaunchRowWalk(const WalkConfig& cfg, const WalkParams& p, hipStream_t stream) {
   if (p.P == 0 || p.n_groups == 0) return hipSuccess;
-  const size_t lds = (size_t)p.kd * cfg.tile_pos * 4;
+  const size_t lds = (size_t)(p.kd + (cfg.int8 ? 0 : 1)) * cfg.tile_pos * 4;
   if (lds > (size_t)kMaxLdsBytes) return hipErrorInvalidValue;
   if (cfg.threads % cfg.tile_pos != 0 && cfg.tile_pos % cfg.threads != 0) return hipErrorInvalidValue;
   if (cfg.threads < cfg.tile_pos) return hipErrorInvalidValue;
   const uint32_t tiles = (p.P + cfg.tile_pos - 1) / cfg.tile_pos;
-  dim3 grid(tiles, cfg.slices), block(cfg.threads);
+  WalkParams q = p;
+  q.tiles = (int)tiles;
+  q.slices = cfg.slices;
+  dim3 grid(8u * (uint32_t)cfg.slices * ((tiles + 7) / 8)), block(cfg.threads);
   if (!cfg.int8) {
     if (cfg.out_kind != kOutF32) return hipErrorInvalidValue;
-    return WalkByRows<false, kOutF32>(cfg, p, grid, block, lds, stream);
+    return WalkByRows<false, kOutF32>(cfg, q, grid, block, lds, stream);
   }
   switch (cfg.out_kind) {
     case kOutF32:
-      return WalkByRows<true, kOutF32>(cfg, p, grid, block, lds, stream);
+      return WalkByRows<true, kOutF32>(cfg, q, grid, block, lds, stream);
     case kOutI8:
-      return WalkByRows<true, kOutI8>(cfg, p, grid, block, lds, stream);
+      return WalkByRows<true, kOutI8>(cfg, q, grid, block, lds, stream);
     case kOutAcc32:
-      return WalkByRows<true, kOutAcc32>(cfg, p, grid, block, lds, stream);
+      return WalkByRows<true, kOutAcc32>(cfg, q, grid, block, lds, stream);
     default:
       return hipErrorInvalidValue;
   }
