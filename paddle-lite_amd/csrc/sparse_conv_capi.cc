@@ -236,15 +236,21 @@ pl::WalkConfig ChooseWalk(const pl_sparse_conv_handle* h, uint32_t P) {
   c.out_kind = OutKind(h->kind);
   c.nrows = h->semi ? 2 : 1;
   const size_t row_bytes = static_cast<size_t>(h->kd + (h->int8 ? 0 : 1)) * 4;  // fp32 tiles carry a zero row
-  // prefer tiles of at most 64 KB (two workgroups per CU), never below one
-  // wavefront of positions unless the channel count forces it
+  // Every workgroup reads its rows' index lists through the scalar cache,
+  // whose fill rate is what bounds the walk: wide tiles amortise a list over
+  // more positions.  256 positions when two tiles still fit a CU, else 128
+  // when one does, else what the channel count leaves room for.
   int tp = 256;
-  while (tp > 64 && row_bytes * tp > 64 * 1024) tp >>= 1;
+  if (row_bytes * tp > 64 * 1024) tp = 128;
   while (tp > 16 && row_bytes * tp > static_cast<size_t>(pl::kMaxLdsBytes)) tp >>= 1;
-  while (tp > 64 && P <= static_cast<uint32_t>(tp) * 64) tp >>= 1;  // small problems: more tiles
+  while (tp > 64 && P <= static_cast<uint32_t>(tp) * 8) tp >>= 1;  // small problems: more tiles
+  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_TILE")) {
+    const int t = std::atoi(e);
+    if (t >= 16 && t <= 256 && (t & (t - 1)) == 0 && row_bytes * t <= static_cast<size_t>(pl::kMaxLdsBytes)) tp = t;
+  }
   c.tile_pos = tp;
   const size_t lds = row_bytes * tp;
-  c.threads = lds > 80 * 1024 ? 1024 : (lds > 40 * 1024 ? 512 : 256);
+  c.threads = lds > 80 * 1024 ? 1024 : (lds >= 32 * 1024 ? 512 : 256);
   if (c.threads < tp) c.threads = tp;
   const int nwaves = c.threads / 64;
   const uint32_t tiles = (P + tp - 1) / tp;

@@ -29,7 +29,10 @@ struct DevGroup {
 
 // Entries of an index list are taken this many at a time; every list is
 // padded to a multiple of it with zero-weight entries.
-constexpr int kWalkBatch = 8;
+#ifndef PL_WALK_BATCH
+#define PL_WALK_BATCH 8
+#endif
+constexpr int kWalkBatch = PL_WALK_BATCH;
 
 // Row-walk SpMM: arguments common to all instantiations.
 struct WalkParams {
