@@ -80,18 +80,20 @@ __device__ __forceinline__ void StreamStore(int2 v, void* dst) {
 }
 
 // ---------------------------------------------------------------- epilogue
+// min(max(v, 0), hi) for any hi as one median instruction: the lower bound
+// min(0, hi) is wave-uniform and makes the median equal hi when hi < 0.
+__device__ __forceinline__ float Clamp0(float v, float hi) { return __builtin_amdgcn_fmed3f(v, fminf(0.0f, hi), hi); }
+
 __device__ __forceinline__ float Activate(float v, const DevAct& a) {
   switch (a.type) {
     case 1:
       return fmaxf(v, 0.0f);
     case 2:
-      return fminf(fmaxf(v, 0.0f), a.relu6_coef);
+      return Clamp0(v, a.relu6_coef);
     case 4:
       return (v >= 0.0f) ? v : v * a.leaky_alpha;
-    case 10: {
-      float gate = fminf(fmaxf(v + a.hs_offset, 0.0f), a.hs_threshold);
-      return (v * a.hs_inv_scale) * gate;
-    }
+    case 10:
+      return (v * a.hs_inv_scale) * Clamp0(v + a.hs_offset, a.hs_threshold);
     default:
       return v;
   }
@@ -102,12 +104,9 @@ __device__ __forceinline__ float Activate(float v, const DevAct& a) {
 template <int ACT>
 __device__ __forceinline__ float ActivateT(float v, const DevAct& a) {
   if (ACT == 1) return fmaxf(v, 0.0f);
-  if (ACT == 2) return fminf(fmaxf(v, 0.0f), a.relu6_coef);
+  if (ACT == 2) return Clamp0(v, a.relu6_coef);
   if (ACT == 4) return (v >= 0.0f) ? v : v * a.leaky_alpha;
-  if (ACT == 10) {
-    float gate = fminf(fmaxf(v + a.hs_offset, 0.0f), a.hs_threshold);
-    return (v * a.hs_inv_scale) * gate;
-  }
+  if (ACT == 10) return (v * a.hs_inv_scale) * Clamp0(v + a.hs_offset, a.hs_threshold);
   return v;
 }
 
@@ -132,11 +131,21 @@ __device__ __forceinline__ void DispatchAct(int type, F&& f) {
   }
 }
 
+// max(v, -127), round half away from zero, min(., 127).  The bounds are
+// integers, so clamping first gives the same result; rounding half away from
+// zero is the truncated sum with the largest float below one half (adding one
+// half itself would carry 0.49999997 up to 1).
 __device__ __forceinline__ int QuantizeI8(float v) {
-  v = fmaxf(v, -127.0f);
-  float r = roundf(v);  // half away from zero
-  r = fminf(r, 127.0f);
-  return static_cast<int>(r);
+  v = __builtin_amdgcn_fmed3f(v, -127.0f, 127.0f);
+  return static_cast<int>(v + __builtin_copysignf(0x1.fffffep-2f, v));
+}
+
+// Low bytes of four quantized values as one dword (a in byte 0).
+__device__ __forceinline__ uint32_t PackI8x4(int a, int b, int c, int d) {
+  // perm(hi, lo, sel): selector 0-3 = byte of lo, 4-7 = byte of hi, 0x0c = zero
+  const uint32_t ab = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);
+  const uint32_t cd = __builtin_amdgcn_perm((uint32_t)d, (uint32_t)c, 0x0c0c0400u);
+  return __builtin_amdgcn_perm(cd, ab, 0x05040100u);
 }
 
 // 4x4 byte transpose: r[i] holds bytes (i, 0..3); on return r[j] holds bytes
@@ -269,9 +278,7 @@ __device__ __forceinline__ void StoreRow(const WalkParams& p, int row, uint32_t 
     } else if (OUT == kOutI8) {
       int8_t* dst = static_cast<int8_t*>(p.out) + idx;
       if (PPL == 4) {
-        uint32_t w = (uint32_t)(QuantizeI8(v[0]) & 0xff) | ((uint32_t)(QuantizeI8(v[1]) & 0xff) << 8) |
-                     ((uint32_t)(QuantizeI8(v[2]) & 0xff) << 16) | ((uint32_t)(QuantizeI8(v[3]) & 0xff) << 24);
-        StreamStore(w, dst);
+        StreamStore(PackI8x4(QuantizeI8(v[0]), QuantizeI8(v[1]), QuantizeI8(v[2]), QuantizeI8(v[3])), dst);
       } else {
 #pragma unroll
         for (int j = 0; j < PPL; ++j) dst[j] = static_cast<int8_t>(QuantizeI8(v[j]));
@@ -551,10 +558,7 @@ __device__ __forceinline__ void StoreRun4(void* dst, const float* v, const int* 
   if (OUT == kOutF32) {
     StreamStore(make_float4(v[0], v[1], v[2], v[3]), dst);
   } else if (OUT == kOutI8) {
-    uint32_t w = 0;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) w |= (uint32_t)(QuantizeI8(v[c]) & 0xff) << (8 * c);
-    StreamStore(w, dst);
+    StreamStore(PackI8x4(QuantizeI8(v[0]), QuantizeI8(v[1]), QuantizeI8(v[2]), QuantizeI8(v[3])), dst);
   } else {
     StreamStore(make_int4(q[0], q[1], q[2], q[3]), dst);
   }
@@ -580,9 +584,10 @@ __device__ __forceinline__ void MfmaEpilogueI8Wide(const MfmaParams& p, const v1
   for (int r = 0; r < 16; ++r) {
     const int ro = 8 * (r >> 2) + (r & 3);
     const float s = p.scale[row_base + ro], b = p.bias[row_base + ro];
-    uint32_t w = 0;
+    int q[4];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) w |= (uint32_t)(QuantizeI8(ActivateAny<ACT>(__builtin_fmaf((float)acc[c][r], s, b), p.act)) & 0xff) << (8 * c);
+    for (int c = 0; c < 4; ++c) q[c] = QuantizeI8(ActivateAny<ACT>(__builtin_fmaf((float)acc[c][r], s, b), p.act));
+    const uint32_t w = PackI8x4(q[0], q[1], q[2], q[3]);
     stage[(4 * (lane >> 5) + ro) * 32 + j] = w;  // row-local index 0..31, 32 dwords per row
   }
   // the same wavefront reads back: its LDS operations complete in order
