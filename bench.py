@@ -21,6 +21,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 LLC_BYTES = 256 << 20  # last-level (Infinity) cache the rotation must exceed
+COPY_CALIBRATION_BYTES = 64 << 20
 
 
 def parse():
@@ -32,6 +33,7 @@ def parse():
     ap.add_argument("--algo", default="auto", choices=["auto", "walk", "mfma"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cache-resident", action="store_true", help="reuse one buffer set (reported, never the headline)")
+    ap.add_argument("--copy-calibration", action="store_true", help="also launch a plain 64 MiB device copy 20 times, the known-size kernel that counter runs scale FETCH_SIZE / WRITE_SIZE by")
     return ap.parse_args()
 
 
@@ -286,6 +288,13 @@ def main():
             "nnz_TOPs_kernel": ops / (kernel_ms * 1e-3) / 1e12,
         },
     }
+    if args.copy_calibration:
+        src = torch.randint(0, 255, (COPY_CALIBRATION_BYTES,), dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(20):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        line["config"]["copy_calibration_bytes"] = COPY_CALIBRATION_BYTES
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(case, weights)
     print(json.dumps(line))

@@ -79,6 +79,18 @@ __device__ __forceinline__ void StreamStore(int2 v, void* dst) {
   __builtin_nontemporal_store(v2i{v.x, v.y}, static_cast<v2i*>(dst));
 }
 
+// Workgroups are handed to the 8 XCDs round robin (linear id mod 8).  For a
+// 1-D grid of 8 * per_tile * ceil(tiles / 8) workgroups, the tile of this
+// workgroup: XCD x owns the contiguous tiles [x*tiles/8, (x+1)*tiles/8), and
+// the per_tile workgroups of one tile follow each other on that XCD.
+// Returns -1 for the surplus workgroups of an XCD with the smaller share.
+__device__ __forceinline__ int XcdTile(int tiles, int per_tile) {
+  const int xcd = blockIdx.x & 7, wg_slot = blockIdx.x >> 3;
+  const int first = (xcd * tiles) >> 3, last = ((xcd + 1) * tiles) >> 3;
+  const int t = first + wg_slot / per_tile;
+  return t < last ? t : -1;
+}
+
 // ---------------------------------------------------------------- epilogue
 // min(max(v, 0), hi) for any hi as one median instruction: the lower bound
 // min(0, hi) is wave-uniform and makes the median equal hi when hi < 0.
@@ -349,10 +361,9 @@ __device__ __forceinline__ void RowWalkBody(const WalkParams& p, uint32_t* tile)
   const ConstWords group_words = (ConstWords)p.groups;
   // 1-D grid; the slices (row ranges) of one tile are neighbours in the
   // per-XCD order so that the tile is fetched into one L2
-  const int xcd = blockIdx.x & 7, wg_slot = blockIdx.x >> 3;
-  const int tile_id = (wg_slot / p.slices) * 8 + xcd;
-  const int slice = wg_slot % p.slices;
-  if (tile_id >= p.tiles) return;
+  const int tile_id = XcdTile(p.tiles, p.slices);
+  const int slice = (blockIdx.x >> 3) % p.slices;
+  if (tile_id < 0) return;
   const uint32_t tile0 = (uint32_t)tile_id * (uint32_t)TP;
 
   PL_PHASE_MARK(0);
@@ -759,10 +770,11 @@ __device__ __forceinline__ void MfmaBody(const MfmaParams& p, uint4* xt) {
   // that the workgroups sharing one activation tile (all row-block groups)
   // run on the same XCD one after the other: the tile is then fetched into
   // that XCD's L2 once.
-  const int xcd = blockIdx.x & 7, wg_slot = blockIdx.x >> 3;
-  const int tile = (wg_slot / p.row_groups) * 8 + xcd;
-  if (tile >= p.tiles) return;
-  const int rb = (wg_slot % p.row_groups) * 4 + wave;
+  // Each XCD takes a contiguous range of tiles: cache lines that straddle
+  // two neighbouring tiles are then fetched by one L2 instead of two.
+  const int tile = XcdTile(p.tiles, p.row_groups);
+  if (tile < 0) return;
+  const int rb = ((blockIdx.x >> 3) % p.row_groups) * 4 + wave;
   const bool wave_on = rb < p.row_blocks;
   const int rbc = wave_on ? rb : p.row_blocks - 1;
   const uint32_t kmask = wave_on ? p.kmask[rbc] : 0u;
