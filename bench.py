@@ -37,6 +37,20 @@ def parse():
     return ap.parse_args()
 
 
+def measured_traffic(workload, algo):
+    """HBM bytes per launch from the committed counter runs (rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE, scaled by a plain copy of known size); None for
+    a workload that has no such run."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            t = json.load(f).get("%s/%s" % (workload, algo))
+    except (OSError, ValueError):
+        return None, None
+    if not t:
+        return None, None
+    return t["read_bytes"] + t["written_bytes"], t
+
+
 def cpu_baseline(case, packed, budget_s=12.0):
     """The reference's CPU path on this host: its naive test reference (the
     real header when oracle/_ref was built, else the restatement), and the
@@ -251,6 +265,8 @@ def main():
     ms_per_step = wall * 1e3 / args.steps
     kernel_ms = ev_ms / args.steps
     achieved = nbytes / (kernel_ms * 1e-3) / 1e9
+    algo_name = {capi.ALGO_ROW_WALK: "row_walk", capi.ALGO_BLOCK_MFMA: "block_mfma"}[info["algo"]]
+    traffic, traffic_detail = measured_traffic(case.name, algo_name)
     line = {
         "metric": "sparse 1x1 conv nnz-GOP/s + % HBM roofline (int8, N=64, 512->512@14x14, 85%)",
         "value": ops * args.steps / wall / 1e9,
@@ -270,7 +286,7 @@ def main():
             "nnz": case.nnz,
             "sparsity": 1.0 - case.nnz / float(case.dense.size),
             "flag_semi": weights.flag_semi,
-            "algo": {capi.ALGO_ROW_WALK: "row_walk", capi.ALGO_BLOCK_MFMA: "block_mfma"}[info["algo"]],
+            "algo": algo_name,
             "weight_blocks_present": [info["mfma_blocks"], info["mfma_blocks_total"]],
             "buffer_sets": n_sets,
             "rotation_MB": n_sets * set_bytes / 1e6,
@@ -282,7 +298,9 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None,
+            "traffic": traffic,
+            "traffic_source": "profiles/hbm_traffic.json (separate rocprofv3 --pmc runs)" if traffic else None,
+            "traffic_detail": traffic_detail,
             "algorithmic_bytes_per_launch": nbytes,
             "kernel_us": kernel_ms * 1e3,
             "nnz_TOPs_kernel": ops / (kernel_ms * 1e-3) / 1e12,
