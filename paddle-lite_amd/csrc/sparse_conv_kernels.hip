@@ -476,69 +476,59 @@ __device__ __forceinline__ QuadInfo LocateQuad(const MfmaParams& p, uint32_t qua
   return q;
 }
 
-// Issue the dword loads of UNITS channel groups for one quad.  Global memory
+// Issue the dword loads of one channel group for one quad.  Global memory
 // needs no alignment for dword access.  A partial quad (valid < 4) reads the
-// last four positions of its row and shifts the unwanted ones out, so no
-// load leaves the tensor.  All loads are unconditional so that they are in
+// last four positions of its row (CommitX shifts the unwanted ones out), so
+// no load leaves the tensor.  All loads are unconditional so that they are in
 // flight together.  FAST: the channel groups are complete and the tensor is
 // below 2 GB, so an address is a uniform base plus one 32-bit per-lane offset
 // (no per-load address arithmetic on the vector ALU).  Otherwise channel
 // indices are clamped and the values masked in CommitX.  Lanes beyond the
 // last image read the tensor's first bytes and are ignored.
-template <int UNITS, bool FAST>
-__device__ __forceinline__ void LoadX(uint32_t (&r)[UNITS][16], const MfmaParams& p, const QuadInfo& q, int kg_base, int kg_lane) {
+template <bool FAST>
+__device__ __forceinline__ void LoadX(uint32_t (&r)[16], const MfmaParams& p, const QuadInfo& q, int kg_base, int kg_lane) {
   const bool live = q.valid > 0;
   const uint32_t first = (q.valid == 4 || !live) ? q.pp : (uint32_t)(p.hw - 4);  // hw >= 4 on this path
-  const int sh = (q.valid == 4 || !live) ? 0 : 8 * (4 - q.valid);
   if (FAST) {
     const uint32_t voff = live ? (q.n * (uint32_t)p.K + 16u * (uint32_t)kg_lane) * (uint32_t)p.hw + first : 0u;
 #pragma unroll
-    for (int u = 0; u < UNITS; ++u) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int8_t* sbase = p.x + (size_t)(16 * (kg_base + 8 * u) + i) * (size_t)p.hw;  // uniform
-        r[u][i] = *reinterpret_cast<const uint32_t*>(sbase + voff);
-      }
+    for (int i = 0; i < 16; ++i) {
+      const int8_t* sbase = p.x + (size_t)(16 * kg_base + i) * (size_t)p.hw;  // uniform
+      r[i] = *reinterpret_cast<const uint32_t*>(sbase + voff);
     }
   } else {
     const int8_t* col = p.x + (live ? (size_t)q.n * p.K * p.hw + first : (size_t)0);
     const size_t row_step = live ? (size_t)p.hw : (size_t)0;
+    const int kg = kg_base + kg_lane;
 #pragma unroll
-    for (int u = 0; u < UNITS; ++u) {
-      const int kg = kg_base + kg_lane + 8 * u;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int ch = min(16 * kg + i, p.K - 1);
-        r[u][i] = *reinterpret_cast<const uint32_t*>(col + (size_t)ch * row_step);
-      }
+    for (int i = 0; i < 16; ++i) {
+      const int ch = min(16 * kg + i, p.K - 1);
+      r[i] = *reinterpret_cast<const uint32_t*>(col + (size_t)ch * row_step);
     }
-  }
-  if (!p.quad_aligned) {
-#pragma unroll
-    for (int u = 0; u < UNITS; ++u)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) r[u][i] >>= sh;
   }
 }
 
 // Transpose to channel-innermost and write the cells of four positions.
-template <int UNITS, bool FAST>
-__device__ __forceinline__ void CommitX(uint32_t (&r)[UNITS][16], uint4* xt, const MfmaParams& p, bool live, bool store, int kg_base, int kg_lane, int j) {
+template <bool FAST>
+__device__ __forceinline__ void CommitX(uint32_t (&r)[16], uint4* xt, const MfmaParams& p, const QuadInfo& q, bool live, bool store, int kg_base, int kg_lane, int j) {
   const int n_kg = 2 * p.ksteps;
+  const int kg = kg_base + kg_lane;
+  if (!p.quad_aligned) {
+    // a partial quad was read from the last four positions of its row
+    const int sh = (q.valid == 4 || q.valid == 0) ? 0 : 8 * (4 - q.valid);
 #pragma unroll
-  for (int u = 0; u < UNITS; ++u) {
-    const int kg = kg_base + kg_lane + 8 * u;
-    if (!FAST) {
+    for (int i = 0; i < 16; ++i) r[i] >>= sh;
+  }
+  if (!FAST) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) r[u][i] = (live && 16 * kg + i < p.K) ? r[u][i] : 0u;
-    }
+    for (int i = 0; i < 16; ++i) r[i] = (live && 16 * kg + i < p.K) ? r[i] : 0u;
+  }
 #pragma unroll
-    for (int b = 0; b < 4; ++b) Transpose4x4(r[u][4 * b], r[u][4 * b + 1], r[u][4 * b + 2], r[u][4 * b + 3]);
-    // now r[u][4b + c] = channels 16kg+4b..+3 of the quad's position c
-    if (store && (FAST || kg < n_kg)) {
+  for (int b = 0; b < 4; ++b) Transpose4x4(r[4 * b], r[4 * b + 1], r[4 * b + 2], r[4 * b + 3]);
+  // now r[4b + c] = channels 16kg+4b..+3 of the quad's position c
+  if (store && (FAST || kg < n_kg)) {
 #pragma unroll
-      for (int c = 0; c < 4; ++c) xt[(size_t)kg * kMfmaTilePos + c * 32 + j] = make_uint4(r[u][c], r[u][4 + c], r[u][8 + c], r[u][12 + c]);
-    }
+    for (int c = 0; c < 4; ++c) xt[(size_t)kg * kMfmaTilePos + c * 32 + j] = make_uint4(r[c], r[4 + c], r[8 + c], r[12 + c]);
   }
 }
 
@@ -667,9 +657,9 @@ __device__ __forceinline__ void MfmaEpilogue(const MfmaParams& p, const v16i (&a
   }
 }
 
-// One tile: stage, multiply, finish.  The activation loads go out first (they
-// feed the longest chain: transpose, LDS, barrier), the wavefront's weight
-// blocks right behind them.
+// One tile: stage, multiply, finish, pipelined over groups of four k-steps
+// (activation loads feed the longest chain: transpose, LDS, barrier; the
+// wavefront's weight blocks of the same k-steps follow right behind them).
 template <int KSMAX, int OUT, int ACT, bool VEC>
 __device__ __forceinline__ void MfmaTile(const MfmaParams& p, uint4* xt, uint32_t kmask, int rb, int rbc, bool wave_on, int tile) {
   const int tid = threadIdx.x;
@@ -679,73 +669,81 @@ __device__ __forceinline__ void MfmaTile(const MfmaParams& p, uint4* xt, uint32_
   const int kg0 = tid >> 5;  // 8 channel groups per pass of the workgroup
   const uint32_t quad0 = (uint32_t)tile * (uint32_t)J;
   v4i a[KSMAX];
-  auto load_weights = [&]() {
+  auto load_weights = [&](int ks0, int ks1) {
     // blocks of absent k-steps are never multiplied; their loads are clamped
 #pragma unroll
-    for (int ks = 0; ks < KSMAX; ++ks) {
-      const int ksc = min(ks, p.ksteps - 1);
-      a[ks] = static_cast<const v4i*>(p.wblocks)[((size_t)rbc * p.ksteps + ksc) * 64 + lane];
+    for (int ks = ks0; ks < ks1; ++ks) {
+      if (ks < KSMAX) {
+        const int ksc = min(ks, p.ksteps - 1);
+        a[ks] = static_cast<const v4i*>(p.wblocks)[((size_t)rbc * p.ksteps + ksc) * 64 + lane];
+      }
     }
   };
   const bool quad_on = j < J;
   const int jc = quad_on ? j : J - 1;  // idle lanes repeat the last quad's loads
-  if (VEC) {
-    constexpr int kPasses = (2 * KSMAX + 7) / 8;  // passes that cover 2*KSMAX groups
-    constexpr int kBatch = kPasses < 4 ? kPasses : 4;
-    const QuadInfo qs = LocateQuad(p, quad0 + (uint32_t)jc);
-    const bool live = qs.valid > 0;
-    uint32_t r[kBatch][16];
-    const bool fast0 = p.small && 16 * 8 * kBatch <= p.K;
-    if (fast0) {
-      LoadX<kBatch, true>(r, p, qs, 0, kg0);
-    } else {
-      LoadX<kBatch, false>(r, p, qs, 0, kg0);
-    }
-    load_weights();
-    if (fast0) {
-      CommitX<kBatch, true>(r, xt, p, true, quad_on && live, 0, kg0, jc);
-    } else {
-      CommitX<kBatch, false>(r, xt, p, live, quad_on, 0, kg0, jc);
-    }
-#pragma unroll
-    for (int pass = kBatch; pass < kPasses; pass += kBatch) {
-      if (8 * pass < 2 * p.ksteps) {
-        if (p.small && 16 * 8 * (pass + kBatch) <= p.K) {
-          LoadX<kBatch, true>(r, p, qs, 8 * pass, kg0);
-          CommitX<kBatch, true>(r, xt, p, true, quad_on && live, 8 * pass, kg0, jc);
-        } else {
-          LoadX<kBatch, false>(r, p, qs, 8 * pass, kg0);
-          CommitX<kBatch, false>(r, xt, p, live, quad_on, 8 * pass, kg0, jc);
-        }
-      }
-    }
-  } else {
-    load_weights();
-    StageMfmaBytes(xt, p, quad0 + (uint32_t)jc, quad_on, kg0, jc);
-  }
-  PL_PHASE_MARK(2);
-  __syncthreads();
-  PL_PHASE_MARK(3);
-  if (!wave_on) return;
-
-  // ---- multiply: D[32 rows][32 cols] += A[32 x 32k] * B[32k x 32]
   v16i acc[4];
 #pragma unroll
   for (int c = 0; c < 4; ++c)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[c][i] = 0;
   const uint4* bbase = xt + (size_t)(lane >> 5) * kMfmaTilePos + (lane & 31);
+  // D[32 rows][32 cols] += A[32 x 32k] * B[32k x 32] for k-steps [ks0, ks1)
+  auto multiply = [&](int ks0, int ks1) {
 #pragma unroll
-  for (int ks = 0; ks < KSMAX; ++ks) {
-    if (kmask & (1u << ks)) {
+    for (int ks = ks0; ks < ks1; ++ks) {
+      if (ks < KSMAX && (kmask & (1u << ks))) {
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const uint4 bq = bbase[(size_t)(2 * ks) * kMfmaTilePos + c * 32];
-        const v4i b = v4i{(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w};
-        acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ks], b, acc[c], 0, 0, 0);
+        for (int c = 0; c < 4; ++c) {
+          const uint4 bq = bbase[(size_t)(2 * ks) * kMfmaTilePos + c * 32];
+          const v4i b = v4i{(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w};
+          acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ks < KSMAX ? ks : 0], b, acc[c], 0, 0, 0);
+        }
       }
     }
+  };
+  if (VEC) {
+    // A pass of the workgroup stages 8 channel groups = 4 k-steps.  The loads
+    // of up to four passes (activations, then that pass's weight blocks) go
+    // out together; each pass is then committed to LDS and multiplied as soon
+    // as its own loads have landed, while the later ones are still in flight.
+    constexpr int kPasses = (2 * KSMAX + 7) / 8;
+    constexpr int kBatch = kPasses < 4 ? kPasses : 4;
+    const QuadInfo qs = LocateQuad(p, quad0 + (uint32_t)jc);
+    const bool live = qs.valid > 0;
+    uint32_t r[kBatch][16];
+    // One straight-line instance per batch and addressing mode: loads under
+    // per-pass conditions would be drained at every join.
+    auto run_batch = [&](auto fast_c, int pass0) {
+      constexpr bool kFast = decltype(fast_c)::value;
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        LoadX<kFast>(r[u], p, qs, 8 * (pass0 + u), kg0);
+        load_weights(4 * (pass0 + u), 4 * (pass0 + u) + 4);
+      }
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        CommitX<kFast>(r[u], xt, p, qs, kFast ? true : live, kFast ? (quad_on && live) : quad_on, 8 * (pass0 + u), kg0, jc);
+        PL_PHASE_MARK(2);
+        __syncthreads();
+        if (wave_on) multiply(4 * (pass0 + u), 4 * (pass0 + u) + 4);
+      }
+    };
+#pragma unroll
+    for (int pass0 = 0; pass0 < kPasses; pass0 += kBatch) {
+      if (pass0 > 0 && 8 * pass0 >= 2 * p.ksteps) break;
+      if (p.small && 16 * 8 * (pass0 + kBatch) <= p.K) {
+        run_batch(std::true_type(), pass0);
+      } else {
+        run_batch(std::false_type(), pass0);
+      }
+    }
+  } else {
+    load_weights(0, KSMAX);
+    StageMfmaBytes(xt, p, quad0 + (uint32_t)jc, quad_on, kg0, jc);
+    __syncthreads();
+    if (wave_on) multiply(0, KSMAX);
   }
+  if (!wave_on) return;
   PL_PHASE_MARK(4);
   if ((lane & 31) >= J) return;
   const QuadInfo qo = LocateQuad(p, quad0 + (uint32_t)(lane & 31));
