@@ -152,6 +152,15 @@ __device__ __forceinline__ int QuantizeI8(float v) {
   return static_cast<int>(v + __builtin_copysignf(0x1.fffffep-2f, v));
 }
 
+// Activation and quantisation of one value.  relu followed by the clamp is
+// one median, and its result has no sign to copy.
+template <int ACT>
+__device__ __forceinline__ int ActQuantI8(float v, const DevAct& a) {
+  if (ACT == 1) return static_cast<int>(__builtin_amdgcn_fmed3f(v, 0.0f, 127.0f) + 0x1.fffffep-2f);
+  if (ACT < 0) return QuantizeI8(Activate(v, a));
+  return QuantizeI8(ActivateT<(ACT < 0 ? 0 : ACT)>(v, a));
+}
+
 // Low bytes of four quantized values as one dword (a in byte 0).
 __device__ __forceinline__ uint32_t PackI8x4(int a, int b, int c, int d) {
   // perm(hi, lo, sel): selector 0-3 = byte of lo, 4-7 = byte of hi, 0x0c = zero
@@ -559,7 +568,7 @@ __device__ __forceinline__ void StoreRun4(void* dst, const float* v, const int* 
   if (OUT == kOutF32) {
     StreamStore(make_float4(v[0], v[1], v[2], v[3]), dst);
   } else if (OUT == kOutI8) {
-    StreamStore(PackI8x4(QuantizeI8(v[0]), QuantizeI8(v[1]), QuantizeI8(v[2]), QuantizeI8(v[3])), dst);
+    StreamStore(PackI8x4(q[0], q[1], q[2], q[3]), dst);  // already quantised
   } else {
     StreamStore(make_int4(q[0], q[1], q[2], q[3]), dst);
   }
@@ -587,7 +596,7 @@ __device__ __forceinline__ void MfmaEpilogueI8Wide(const MfmaParams& p, const v1
     const float s = p.scale[row_base + ro], b = p.bias[row_base + ro];
     int q[4];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) q[c] = QuantizeI8(ActivateAny<ACT>(__builtin_fmaf((float)acc[c][r], s, b), p.act));
+    for (int c = 0; c < 4; ++c) q[c] = ActQuantI8<ACT>(__builtin_fmaf((float)acc[c][r], s, b), p.act);
     const uint32_t w = PackI8x4(q[0], q[1], q[2], q[3]);
     stage[(4 * (lane >> 5) + ro) * 32 + j] = w;  // row-local index 0..31, 32 dwords per row
   }
@@ -620,7 +629,14 @@ __device__ __forceinline__ void MfmaEpilogueRows(const MfmaParams& p, const v16i
     if (OUT != kOutAcc32) {
       const float s = p.scale[row_base + ro], b = p.bias[row_base + ro];
 #pragma unroll
-      for (int c = 0; c < 4; ++c) v[c] = ActivateAny<ACT>(__builtin_fmaf((float)q[c], s, b), p.act);
+      for (int c = 0; c < 4; ++c) {
+        const float t = __builtin_fmaf((float)q[c], s, b);
+        if (OUT == kOutI8) {
+          q[c] = ActQuantI8<ACT>(t, p.act);  // from here on q holds the output bytes
+        } else {
+          v[c] = ActivateAny<ACT>(t, p.act);
+        }
+      }
     }
     if (WHOLE) {
       StoreRun4<OUT>(dst, v, q);
@@ -631,7 +647,7 @@ __device__ __forceinline__ void MfmaEpilogueRows(const MfmaParams& p, const v16i
           if (OUT == kOutF32) {
             reinterpret_cast<float*>(dst)[c] = v[c];
           } else if (OUT == kOutI8) {
-            reinterpret_cast<int8_t*>(dst)[c] = static_cast<int8_t>(QuantizeI8(v[c]));
+            reinterpret_cast<int8_t*>(dst)[c] = static_cast<int8_t>(q[c]);
           } else {
             reinterpret_cast<int*>(dst)[c] = q[c];
           }
