@@ -101,6 +101,7 @@ struct pl_sparse_conv_handle {
   int wg_slots = 512;       // workgroups resident at once (2 per CU)
   int mfma_i8_wide = 1;
   int mfma_tile_quads = 0;  // 0 = chosen per problem
+  int mfma_sub_tiles = 1;   // several tiles per workgroup for <= 64 input channels: 0 never, 1 when enough workgroups remain, 2 always
   // epilogue
   DevBuf scale, bias;
   int padded_rows = 0;
@@ -326,6 +327,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   h->device = dev;
   h->wg_slots = 2 * std::max(1, prop.multiProcessorCount);
   if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_I8_WIDE")) h->mfma_i8_wide = std::atoi(e) != 0;
+  if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_SUB_TILES")) h->mfma_sub_tiles = std::max(0, std::min(2, std::atoi(e)));
   if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_TILE_QUADS")) h->mfma_tile_quads = std::max(0, std::min(32, std::atoi(e)));
   // tuning switches for experiments; the defaults are what measured best
   if (const char* e = std::getenv("PL_SPARSE_CONV_WG_SLOTS")) h->wg_slots = std::max(1, std::atoi(e));
@@ -425,6 +427,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
       c.tile_quads = static_cast<int>(std::min<int64_t>(32, std::max<int64_t>(8, (quads + target_tiles - 1) / target_tiles)));
     }
     c.i8_wide_stores = h->mfma_i8_wide;
+    c.sub_tiles = h->mfma_sub_tiles;
     if (h->mfma_tile_quads > 0) c.tile_quads = h->mfma_tile_quads;
     e = pl::LaunchBlockMfma(c, p, s);
   } else {

@@ -88,6 +88,7 @@ struct MfmaParams {
   uint32_t total_quads;    // batch * qpi
   int tiles;               // tiles of tile_quads quads
   int tile_quads;
+  int sub_tiles;           // tiles per workgroup (1, 2 or 4)
   int row_groups;          // groups of four row blocks
   int i8_stage;            // int8 output is regrouped through LDS for 16-byte stores
 };
@@ -96,6 +97,7 @@ struct MfmaConfig {
   int out_kind;
   int ks_max;          // 2, 4, 8, 16 or 32 (>= ksteps)
   int tile_quads;      // 1..32 position quads per workgroup tile
+  int sub_tiles;       // several tiles per workgroup for at most 64 input channels: 0 never, 1 when enough workgroups remain, 2 always
   int i8_wide_stores;  // int8 output: regroup through LDS into 16-byte stores
 };
 

@@ -673,6 +673,25 @@ __device__ __forceinline__ void MfmaEpilogue(const MfmaParams& p, const v16i (&a
   }
 }
 
+// Epilogue of one (tile, row block) pair.  `stage` is the workgroup's LDS
+// behind the activation tiles (4 KB per wavefront when p.i8_stage is set).
+template <int OUT, int ACT, bool VEC>
+__device__ __forceinline__ void MfmaFinish(const MfmaParams& p, uint32_t* stage, const v16i (&acc)[4], int rb, int lane, uint32_t quad0, int J) {
+  if ((lane & 31) >= J) return;
+  const QuadInfo qo = LocateQuad(p, quad0 + (uint32_t)(lane & 31));
+  if (OUT == kOutI8 && VEC) {
+    // wide stores need a full tile inside one image whose rows all exist and
+    // 16-byte aligned row pieces
+    const QuadInfo q0 = LocateQuad(p, quad0);
+    const bool wide = p.i8_stage && J == 32 && p.small && rb * 32 + 32 <= p.M && (p.hw & 15) == 0 && quad0 + 32u <= p.total_quads && q0.pp + 128u <= (uint32_t)p.hw;
+    if (wide) {
+      MfmaEpilogueI8Wide<ACT>(p, acc, rb, lane, q0.n, q0.pp, stage + (threadIdx.x >> 6) * 1024);
+      return;
+    }
+  }
+  MfmaEpilogue<OUT, ACT>(p, acc, rb, lane, qo);
+}
+
 // One tile: stage, multiply, finish, pipelined over groups of four k-steps
 // (activation loads feed the longest chain: transpose, LDS, barrier; the
 // wavefront's weight blocks of the same k-steps follow right behind them).
@@ -761,20 +780,69 @@ __device__ __forceinline__ void MfmaTile(const MfmaParams& p, uint4* xt, uint32_
   }
   if (!wave_on) return;
   PL_PHASE_MARK(4);
-  if ((lane & 31) >= J) return;
-  const QuadInfo qo = LocateQuad(p, quad0 + (uint32_t)(lane & 31));
-  if (OUT == kOutI8 && VEC) {
-    // wide stores need a full tile inside one image whose rows all exist and
-    // 16-byte aligned row pieces
-    const QuadInfo q0 = LocateQuad(p, quad0);
-    const bool wide = p.i8_stage && J == 32 && p.small && rb * 32 + 32 <= p.M && (p.hw & 15) == 0 && quad0 + 32u <= p.total_quads && q0.pp + 128u <= (uint32_t)p.hw;
-    if (wide) {
-      uint32_t* stage = reinterpret_cast<uint32_t*>(xt + (size_t)2 * p.ksteps * kMfmaTilePos) + (threadIdx.x >> 6) * 1024;
-      MfmaEpilogueI8Wide<ACT>(p, acc, rb, lane, q0.n, q0.pp, stage);
-      return;
+  MfmaFinish<OUT, ACT, VEC>(p, reinterpret_cast<uint32_t*>(xt + (size_t)2 * p.ksteps * kMfmaTilePos), acc, rb, lane, quad0, J);
+}
+
+// Few input channels (at most 64, KSMAX <= 2): the channel groups of one
+// tile fill only 2 * ksteps of the 8 group slots of a staging pass, so the
+// workgroup takes T = 4 / ksteps neighbouring tiles at once (LDS: tile after
+// tile) and each wavefront finishes T * RB / 4 (tile, row block) pairs with
+// one set of weight blocks, RB = row blocks of the group (1, 2 or 4).
+template <int KSMAX, int OUT, int ACT>
+__device__ __forceinline__ void MfmaTilesFewChannels(const MfmaParams& p, uint4* xt, int wg_tile, int group, int wave) {
+  const int tid = threadIdx.x, lane = tid & 63, j = tid & 31, kg0 = tid >> 5;
+  const int T = p.sub_tiles;
+  const int n_kg = 2 * p.ksteps;  // == 8 / T
+  const int sub_l = kg0 / n_kg, kgl = kg0 - sub_l * n_kg;
+  const int RB = min(4, p.row_blocks - 4 * group);
+  const int rb = 4 * group + (wave & (RB - 1));
+  const uint32_t kmask = p.kmask[rb];
+  v4i a[KSMAX];
+  const size_t tile_cells = (size_t)n_kg * kMfmaTilePos;
+  {
+    const QuadInfo qs = LocateQuad(p, ((uint32_t)wg_tile * T + sub_l) * 32u + j);
+    const bool live = qs.valid > 0;
+    uint32_t r[16];
+    uint4* xs = xt + (size_t)sub_l * tile_cells;
+    const bool fast = p.small && p.K == 32 * p.ksteps;
+    if (fast) {
+      LoadX<true>(r, p, qs, 0, kgl);
+    } else {
+      LoadX<false>(r, p, qs, 0, kgl);
+    }
+#pragma unroll
+    for (int ks = 0; ks < KSMAX; ++ks) a[ks] = static_cast<const v4i*>(p.wblocks)[((size_t)rb * p.ksteps + min(ks, p.ksteps - 1)) * 64 + lane];
+    if (fast) {
+      CommitX<true>(r, xs, p, qs, true, live, 0, kgl, j);
+    } else {
+      CommitX<false>(r, xs, p, qs, live, true, 0, kgl, j);
     }
   }
-  MfmaEpilogue<OUT, ACT>(p, acc, rb, lane, qo);
+  __syncthreads();
+  uint32_t* stage = reinterpret_cast<uint32_t*>(xt + (size_t)T * tile_cells);
+  for (int it = wave; it < T * RB; it += 4) {
+    const int sub = it / RB;
+    const uint32_t quad0 = ((uint32_t)wg_tile * T + sub) * 32u;
+    if (quad0 >= p.total_quads) break;
+    v16i acc[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[c][i] = 0;
+    const uint4* bbase = xt + (size_t)sub * tile_cells + (size_t)(lane >> 5) * kMfmaTilePos + (lane & 31);
+#pragma unroll
+    for (int ks = 0; ks < KSMAX; ++ks) {
+      if (kmask & (1u << ks)) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const uint4 bq = bbase[(size_t)(2 * ks) * kMfmaTilePos + c * 32];
+          const v4i b = v4i{(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w};
+          acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ks], b, acc[c], 0, 0, 0);
+        }
+      }
+    }
+    MfmaFinish<OUT, ACT, true>(p, stage, acc, rb, lane, quad0, 32);
+  }
 }
 
 template <int KSMAX, int OUT, int ACT, bool VEC>
@@ -788,6 +856,10 @@ __device__ __forceinline__ void MfmaBody(const MfmaParams& p, uint4* xt) {
   // two neighbouring tiles are then fetched by one L2 instead of two.
   const int tile = XcdTile(p.tiles, p.row_groups);
   if (tile < 0) return;
+  if (KSMAX <= 2 && VEC && p.sub_tiles > 1) {
+    MfmaTilesFewChannels<(KSMAX <= 2 ? KSMAX : 1), OUT, (ACT < 0 ? 0 : ACT)>(p, xt, tile, (blockIdx.x >> 3) % p.row_groups, wave);
+    return;
+  }
   const int rb = ((blockIdx.x >> 3) % p.row_groups) * 4 + wave;
   const bool wave_on = rb < p.row_blocks;
   const int rbc = wave_on ? rb : p.row_blocks - 1;
@@ -931,17 +1003,26 @@ hipError_t LaunchBlockMfma(const MfmaConfig& cfg, const MfmaParams& p, hipStream
   if (p.P == 0 || p.row_blocks == 0) return hipSuccess;
   if (p.ksteps > cfg.ks_max || p.ksteps > 32) return hipErrorInvalidValue;
   if (cfg.tile_quads < 1 || cfg.tile_quads > 32 || p.hw < 1) return hipErrorInvalidValue;
-  size_t lds = (size_t)2 * p.ksteps * kMfmaTilePos * 16;
-  if (lds > (size_t)kMaxLdsBytes) return hipErrorInvalidValue;
   MfmaParams q = p;
   q.qpi = (p.hw + 3) / 4;
   q.total_quads = (p.P / (uint32_t)p.hw) * (uint32_t)q.qpi;
   q.vec = p.hw >= 4;
   q.quad_aligned = p.hw % 4 == 0;
   q.tile_quads = cfg.tile_quads;
-  const uint32_t tiles = (q.total_quads + cfg.tile_quads - 1) / cfg.tile_quads;
-  q.tiles = (int)tiles;
+  uint32_t tiles = (q.total_quads + cfg.tile_quads - 1) / cfg.tile_quads;
   q.row_groups = (p.row_blocks + 3) / 4;
+  // at most 64 input channels: a workgroup takes 4 / ksteps tiles at once
+  // (every row group must have 1, 2 or 4 row blocks, and enough workgroups
+  // must remain to fill the chip)
+  q.sub_tiles = 1;
+  if (cfg.ks_max == 2 && cfg.sub_tiles && q.vec && cfg.tile_quads == 32 && (p.row_blocks % 4 == 0 || p.row_blocks <= 2)) {
+    const uint32_t t = 4u / (uint32_t)p.ksteps;
+    if (cfg.sub_tiles == 2 || (tiles / t) * q.row_groups >= 1024u) q.sub_tiles = (int)t;
+  }
+  tiles = (tiles + q.sub_tiles - 1) / q.sub_tiles;
+  q.tiles = (int)tiles;  // workgroup-level tiles
+  size_t lds = (size_t)q.sub_tiles * 2 * p.ksteps * kMfmaTilePos * 16;
+  if (lds > (size_t)kMaxLdsBytes) return hipErrorInvalidValue;
   // int8 output: 4 KB per wavefront behind the activation tile to widen stores
   q.i8_stage = cfg.out_kind == kOutI8 && cfg.i8_wide_stores && lds + 16384 <= (size_t)kMaxLdsBytes;
   if (q.i8_stage) lds += 16384;

@@ -74,6 +74,28 @@ def test_int8_outputs_bit_exact(paired, out_int8, act, algo):
             assert np.abs(got.astype(int)).max() <= 127
 
 
+# at most 64 input channels: a workgroup of the block MFMA kernel takes two
+# or four tiles at once; forced here, the library only does so by itself on
+# problems that keep more than 1024 workgroups.  (batch, ic, oc, h, w): full and
+# ragged channel groups, 1 / 2 / 4 / 8 row blocks, aligned and odd images,
+# a tile count that is not a multiple of the tiles per workgroup.
+FEW_CHANNEL_SHAPES = [(3, 32, 64, 16, 16), (2, 64, 128, 12, 12), (2, 20, 32, 16, 8), (3, 50, 256, 10, 10), (2, 32, 48, 7, 7), (5, 64, 64, 8, 8), (1, 32, 96, 16, 16)]
+
+
+@pytest.mark.parametrize("kind", ["acc32", "fp32out", "int8out"])
+@pytest.mark.parametrize("shape", FEW_CHANNEL_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_few_channel_tiles_bit_exact(shape, kind, monkeypatch):
+    announce("few-channel", shape, kind)
+    monkeypatch.setenv("PL_SPARSE_CONV_MFMA_SUB_TILES", "2")
+    k = {"acc32": capi.KIND_INT8_ACC32, "fp32out": capi.KIND_INT8_FP32, "int8out": capi.KIND_INT8_INT8}[kind]
+    batch, ic, oc, h, w = shape
+    for act in ("relu", "hswish"):
+        case = small_case(k, batch, ic, oc, h, w, 0.6, False, AP() if kind == "acc32" else ACTS[act], seed=3 * ic + oc, output_scale=0.05 if kind == "int8out" else 1.0)
+        got = run_hip(case, capi.ALGO_BLOCK_MFMA)
+        want = run_oracle(case, oracle_pack(case))
+        assert_same(case, got, want, "few-channel %s %s %s" % (kind, act, shape))
+
+
 @pytest.mark.parametrize("act", sorted(ACTS))
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
