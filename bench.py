@@ -29,7 +29,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib"])
     ap.add_argument("--algo", default="auto", choices=["auto", "walk", "mfma"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cache-resident", action="store_true", help="reuse one buffer set (reported, never the headline)")
@@ -120,6 +120,51 @@ def cpu_baseline(case, packed, budget_s=12.0):
     }
     del packed
     return naive
+
+
+def run_calib(args):
+    """The precision changes either side of an int8 layer (the reference's
+    calib op): fp32 -> int8 and int8 -> fp32 over a 64x128x56x56 tensor, each
+    timed with HIP events over rotating buffers.  Not the headline metric:
+    printed as its own JSON line."""
+    import numpy as np
+    import torch
+
+    import helpers
+    from oracle import oracle as O
+
+    capi = helpers.capi
+    L = capi.lib()
+    n = 64 * 128 * 56 * 56
+    scale = 0.0371
+    n_sets = 4  # 4 x 128 MB
+    rng = np.random.RandomState(0)
+    xf_host = (rng.standard_normal(n) * 2.5).astype(np.float32)
+    xf = [torch.from_numpy(xf_host).cuda() for _ in range(n_sets)]
+    q = [torch.empty(n, dtype=torch.int8, device="cuda") for _ in range(n_sets)]
+    stream = torch.cuda.current_stream().cuda_stream
+    out = {}
+    for name, fn, src, dst, nbytes in (("fp32_to_int8", L.pl_calib_fp32_to_int8, xf, q, 5 * n), ("int8_to_fp32", L.pl_calib_int8_to_fp32, q, xf, 5 * n)):
+        def step(i):
+            capi.check(fn(C.c_void_p(src[i % n_sets].data_ptr()), C.c_void_p(dst[i % n_sets].data_ptr()), n, C.c_float(scale), C.c_void_p(stream)))
+        step(0)
+        torch.cuda.synchronize()
+        if name == "fp32_to_int8":
+            assert np.array_equal(q[0][:1 << 20].cpu().numpy(), O.fp32_to_int8(xf_host[:1 << 20], scale)), "fp32_to_int8 differs from the oracle"
+        else:
+            assert np.array_equal(xf[0][:1 << 20].cpu().numpy(), O.int8_to_fp32(q[0][:1 << 20].cpu().numpy(), scale)), "int8_to_fp32 differs from the oracle"
+        for i in range(args.warmup):
+            step(i)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(args.steps):
+            step(i)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / args.steps
+        out[name] = {"kernel_us": us, "algorithmic_bytes_per_launch": nbytes, "achieved_GBs": nbytes / (us * 1e-6) / 1e9, "frac": nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
+    print(json.dumps({"metric": "calib fp32<->int8, 64x128x56x56", "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "data": "synthetic", "config": {"workload": "calib", "elements": n, "rotation_MB": n_sets * 5 * n / 1e6, "parity_checked": True}, "roofline": {"bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s", "kernels": out}}))
+    return 0
 
 
 def run_c5(args):
@@ -219,6 +264,8 @@ def main():
     torch.cuda.set_device(0)
     if args.config == "c5":
         return run_c5(args)
+    if args.config == "calib":
+        return run_calib(args)
     case = wl.CONFIGS[args.config]()
     algo = {"auto": capi.ALGO_AUTO, "walk": capi.ALGO_ROW_WALK, "mfma": capi.ALGO_BLOCK_MFMA}[args.algo]
     kernel, weights = helpers.make_kernel(case, algo=algo)

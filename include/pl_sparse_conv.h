@@ -197,6 +197,20 @@ int pl_sparse_pack(int32_t dtype, int32_t flag_semi, const void* dense,
                    void* nonzero_weights, int64_t n_weights,
                    uint32_t* oc_nonzeros, int32_t* diffs, int64_t n_diffs);
 
+/* Precision changes either side of an int8 sparse convolution (device
+ * pointers, n elements, per-tensor scale; enqueued on `stream`) -----------
+ * Replaces lite::arm::math::fp32_to_int8 as CalibComputeFp32ToInt8::Run calls
+ * it (lite/kernels/arm/calib_compute.cc:31-38, lite/backends/arm/math/
+ * type_trans.cc:35-160): out = saturate(round-half-away(x * (1 / scale))),
+ * never below -127. */
+int pl_calib_fp32_to_int8(const float* x_dev, int8_t* out_dev, int64_t n,
+                          float scale, void* stream);
+
+/* Replaces lite::arm::math::int8_to_fp32 as CalibComputeInt8ToFp32::Run calls
+ * it (calib_compute.cc:60-68, type_trans.cc:int8_to_fp32): out = x * scale. */
+int pl_calib_int8_to_fp32(const int8_t* x_dev, float* out_dev, int64_t n,
+                          float scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -16,4 +16,6 @@ from .sparse_conv import (  # noqa: F401
     detect_and_pack,
 )
 
-__all__ = ["capi", "ActivationParam", "SparseConvParam", "SparseConvKernel", "SparseWeights", "detect_and_pack"]
+from .calib import CalibParam, CalibComputeFp32ToInt8, CalibComputeInt8ToFp32  # noqa: F401
+
+__all__ = ["capi", "ActivationParam", "SparseConvParam", "SparseConvKernel", "SparseWeights", "detect_and_pack", "CalibParam", "CalibComputeFp32ToInt8", "CalibComputeInt8ToFp32"]

@@ -30,6 +30,7 @@ HIPCC_FLAGS = [
 SOURCES = [
     ("sparse_layout.cc", "sparse_layout.o", []),
     ("sparse_conv_capi.cc", "sparse_conv_capi.o", []),
+    ("calib_kernels.hip", "calib_kernels.o", []),
     ("sparse_conv_kernels.hip", "sparse_conv_kernels_walk.o", ["-DPL_KERNEL_PART=0"]),
     ("sparse_conv_kernels.hip", "sparse_conv_kernels_mfma_f32.o", ["-DPL_KERNEL_PART=1"]),
     ("sparse_conv_kernels.hip", "sparse_conv_kernels_mfma_i8.o", ["-DPL_KERNEL_PART=2"]),
@@ -91,8 +92,10 @@ LITE_SOURCES = [
     "core/optimizer/mir/sparse_conv_detect_pass.cc",
     "operators/sparse_conv_op.cc",
     "operators/io_copy_op.cc",
+    "operators/calib_op.cc",
     "kernels/hip/sparse_conv_compute.cc",
     "kernels/hip/io_copy_compute.cc",
+    "kernels/hip/calib_compute.cc",
 ]
 
 

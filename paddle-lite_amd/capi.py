@@ -25,6 +25,8 @@ EXPORTS = [
     "pl_sparse_count_semi",
     "pl_sparse_count_zeros",
     "pl_sparse_pack",
+    "pl_calib_fp32_to_int8",
+    "pl_calib_int8_to_fp32",
 ]
 
 
@@ -118,6 +120,10 @@ def lib():
     L.pl_sparse_count_zeros.restype = C.c_int
     L.pl_sparse_pack.argtypes = [C.c_int32, C.c_int32, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int64]
     L.pl_sparse_pack.restype = C.c_int
+    L.pl_calib_fp32_to_int8.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_float, C.c_void_p]
+    L.pl_calib_fp32_to_int8.restype = C.c_int
+    L.pl_calib_int8_to_fp32.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_float, C.c_void_p]
+    L.pl_calib_int8_to_fp32.restype = C.c_int
     if L.pl_sparse_conv_abi_version() != ABI_VERSION:
         raise LibraryMissing("libpl_sparse_conv.so has ABI %d, binding expects %d" % (L.pl_sparse_conv_abi_version(), ABI_VERSION))
     _lib = L

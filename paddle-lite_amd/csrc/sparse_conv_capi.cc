@@ -8,6 +8,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
+#include <cmath>
 #include <cstring>
 #include <new>
 #include <string>
@@ -508,6 +509,31 @@ int pl_sparse_conv_set_epilogue(pl_sparse_conv_handle* h, const float* scale, co
 }
 
 void pl_sparse_conv_destroy(pl_sparse_conv_handle* h) { delete h; }
+
+namespace {
+int CheckCalibArgs(const void* x, const void* out, int64_t n, float scale) {
+  if (n < 0) return Fail(PL_ERR_BAD_ARG, "negative element count");
+  if (n > 0 && (!x || !out)) return Fail(PL_ERR_BAD_ARG, "null device pointer");
+  if (!(scale > 0.0f) || !std::isfinite(scale)) return Fail(PL_ERR_BAD_ARG, "scale must be positive and finite");
+  static const int devices = pl_device_count();  // looked up once per process
+  if (n > 0 && devices == 0) return Fail(PL_ERR_NO_DEVICE, "no gfx950 device");
+  return PL_OK;
+}
+}  // namespace
+
+int pl_calib_fp32_to_int8(const float* x_dev, int8_t* out_dev, int64_t n, float scale, void* stream) {
+  const int rc = CheckCalibArgs(x_dev, out_dev, n, scale);
+  if (rc != PL_OK || n == 0) return rc;
+  const hipError_t e = pl::LaunchFp32ToInt8(x_dev, out_dev, n, scale, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? PL_OK : FailHip(e, "fp32 -> int8 launch");
+}
+
+int pl_calib_int8_to_fp32(const int8_t* x_dev, float* out_dev, int64_t n, float scale, void* stream) {
+  const int rc = CheckCalibArgs(x_dev, out_dev, n, scale);
+  if (rc != PL_OK || n == 0) return rc;
+  const hipError_t e = pl::LaunchInt8ToFp32(x_dev, out_dev, n, scale, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? PL_OK : FailHip(e, "int8 -> fp32 launch");
+}
 
 // ------------------------------------------------------------ host packers
 int pl_sparse_count_semi(int32_t dtype, const void* dense, int32_t oc, int32_t ic, int32_t* count_nonzeroes, int32_t* count_channels, int32_t* count_blocks, int32_t* flag_semi) {

@@ -107,4 +107,8 @@ hipError_t LaunchBlockMfma(const MfmaConfig& cfg, const MfmaParams& p, hipStream
 constexpr int kMaxLdsBytes = 160 * 1024;
 constexpr int kMfmaTilePos = 128;
 
+// Precision changes around an int8 convolution (calib_kernels.hip).
+hipError_t LaunchFp32ToInt8(const float* x, int8_t* out, int64_t n, float scale, hipStream_t stream);
+hipError_t LaunchInt8ToFp32(const int8_t* x, float* out, int64_t n, float scale, hipStream_t stream);
+
 }  // namespace pl

@@ -72,6 +72,13 @@ struct IoCopyParam : ParamBase {
   int process_type{0};
 };
 
+// reference: lite/operators/op_params.h:74-78
+struct CalibParam : ParamBase {
+  const lite::Tensor* input{};
+  lite::Tensor* output{};
+  float scale{1.0f};
+};
+
 }  // namespace operators
 }  // namespace lite
 }  // namespace paddle

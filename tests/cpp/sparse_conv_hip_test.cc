@@ -331,6 +331,93 @@ static void RegistryAndErrorPaths() {
   }
 }
 
+// The precision changes either side of an int8 convolution: op attach /
+// shape inference / registrations on the host, and on the device the chain
+// fp32 -> io_copy -> calib(fp32_to_int8) -> calib(int8_to_fp32) -> io_copy
+// against the oracle's fp32_to_int8 / int8_to_fp32.
+static void CalibChain(bool run_on_device) {
+  std::printf("calib chain\n");
+  std::fflush(stdout);
+  auto all = KernelRegistry::Global().Create("calib", TARGET(kHIP), PRECISION(kInt8), DATALAYOUT(kNCHW));
+  EXPECT(all.size() == 2);
+  bool a = false, b = false;
+  for (auto& k : all) {
+    a |= k->alias() == "fp32_to_int8";
+    b |= k->alias() == "int8_to_fp32";
+  }
+  EXPECT(a && b);
+
+  Scope scope;
+  const int64_t n = 3 * 5 * 7 * 11 + 0;  // not a multiple of 16
+  const float scale = 0.0371f;
+  Tensor* x = scope.Var("cx")->GetMutable<Tensor>();
+  x->Resize({3, 5, 7, 11});
+  float* xd = x->mutable_data<float>(TargetType::kHost);
+  std::mt19937 rng(5);
+  std::normal_distribution<float> dist(0.f, 2.5f);
+  for (int64_t i = 0; i < n; ++i) xd[i] = dist(rng);
+  xd[0] = 0.5f * scale;
+  xd[1] = -0.5f * scale;
+  xd[2] = 500.f;
+  xd[3] = -500.f;
+  scope.Var("cx_dev");
+  scope.Var("cq");
+  scope.Var("cf");
+
+  OpInfo q("calib");
+  q.SetInput("Input", {"cx_dev"});
+  q.SetOutput("Out", {"cq"});
+  q.SetAttr<float>("scale", scale);
+  OpInfo dq("calib");
+  dq.SetInput("Input", {"cq"});
+  dq.SetOutput("Out", {"cf"});
+  dq.SetAttr<float>("scale", scale);
+  OpInfo missing("calib");
+  missing.SetInput("Input", {"nowhere"});
+  missing.SetOutput("Out", {"cq"});
+  EXPECT(Throws([&] { LiteOpRegistry::Global().Create("calib")->Attach(missing, &scope); }));
+  if (!run_on_device) {
+    // shape inference needs no device: attach on the host tensor
+    q.SetInput("Input", {"cx"});
+    auto op = LiteOpRegistry::Global().Create("calib");
+    EXPECT(op != nullptr && op->Attach(q, &scope) && op->CheckShape() && op->InferShape());
+    EXPECT(scope.FindMutableTensor("cq")->dims() == DDim({3, 5, 7, 11}));
+    return;
+  }
+  OpInfo h2d("io_copy");
+  h2d.SetInput("Input", {"cx"});
+  h2d.SetOutput("Out", {"cx_dev"});
+  auto copy_op = LiteOpRegistry::Global().Create("io_copy");
+  EXPECT(copy_op->Attach(h2d, &scope) && copy_op->InferShape());
+  auto copy_kernels = copy_op->CreateKernels({paddle::lite_api::Place(TARGET(kHIP), PRECISION(kAny), DATALAYOUT(kAny))}, "io_copy/host_to_device");
+  EXPECT(copy_kernels.size() == 1);
+  copy_kernels[0]->Launch();
+
+  auto q_op = LiteOpRegistry::Global().Create("calib");
+  EXPECT(q_op->Attach(q, &scope) && q_op->CheckShape() && q_op->InferShape());
+  auto qk = q_op->CreateKernels({paddle::lite_api::Place(TARGET(kHIP), PRECISION(kInt8), DATALAYOUT(kNCHW))}, "calib/fp32_to_int8");
+  EXPECT(qk.size() == 1);
+  qk[0]->Launch();
+  auto dq_op = LiteOpRegistry::Global().Create("calib");
+  EXPECT(dq_op->Attach(dq, &scope) && dq_op->InferShape());
+  auto dqk = dq_op->CreateKernels({paddle::lite_api::Place(TARGET(kHIP), PRECISION(kInt8), DATALAYOUT(kNCHW))}, "calib/int8_to_fp32");
+  EXPECT(dqk.size() == 1);
+  dqk[0]->Launch();
+  dqk[0]->mutable_context_as<HIPContext>()->Sync();
+  qk[0]->mutable_context_as<HIPContext>()->Sync();
+
+  Tensor q_host, f_host;
+  q_host.CopyDataFrom(*scope.FindMutableTensor("cq"), TargetType::kHost);
+  f_host.CopyDataFrom(*scope.FindMutableTensor("cf"), TargetType::kHost);
+  std::vector<int8_t> want_q(n);
+  std::vector<float> want_f(n);
+  plo_fp32_to_int8(xd, want_q.data(), scale, n);
+  plo_int8_to_fp32(want_q.data(), want_f.data(), scale, n);
+  EXPECT(std::memcmp(want_q.data(), q_host.raw_data(), n) == 0);
+  EXPECT(std::memcmp(want_f.data(), f_host.raw_data(), n * 4) == 0);
+  EXPECT(want_q[2] == 127 && want_q[3] == -127);
+}
+
 int main(int argc, char** argv) {
   const bool gpu = argc > 1 && std::string(argv[1]) == "--gpu";
   RegistryAndErrorPaths();
@@ -350,6 +437,7 @@ int main(int argc, char** argv) {
     return 2;
   }
   for (const Problem& p : problems) RunProblem(p, gpu);
+  CalibChain(gpu);
   std::printf("%s: %d failure(s)\n", gpu ? "gpu" : "cpu", g_failures);
   return g_failures ? 1 : 0;
 }
