@@ -202,9 +202,10 @@ def run_c5(args):
         total_ops += case.algorithmic_ops()
         total_bytes += case.algorithmic_bytes(weights)
 
-    def sequence():
+    def sequence(on_stream=None):
+        st = stream if on_stream is None else on_stream
         for case, kernel, x, out in layers:
-            capi.check(L.pl_sparse_conv_run(kernel._handle, x.data_ptr(), out.data_ptr(), case.batch, case.im_size, C.c_void_p(stream)))
+            capi.check(L.pl_sparse_conv_run(kernel._handle, x.data_ptr(), out.data_ptr(), case.batch, case.im_size, C.c_void_p(st)))
 
     # per-layer kernel time (events around repeated launches of one layer)
     per_layer = []
@@ -228,6 +229,26 @@ def run_c5(args):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     seq_us = e0.elapsed_time(e1) * 1e3 / steps
+    # the same 13 launches captured once as a HIP graph (kernel nodes only)
+    # and replayed; every replay is compared with the eager results
+    eager_last = [layers[i][3].clone() for i in (0, 6, 12)]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        sequence(torch.cuda.current_stream().cuda_stream)
+    graph_ok = True
+    for _ in range(3):
+        for i in (0, 6, 12):
+            layers[i][3].zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        graph_ok = graph_ok and all(torch.equal(layers[i][3], ref) for i, ref in zip((0, 6, 12), eager_last))
+    g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    g0.record()
+    for _ in range(steps):
+        graph.replay()
+    g1.record()
+    torch.cuda.synchronize()
+    graph_us = g0.elapsed_time(g1) * 1e3 / steps
     line = {
         "metric": "MobileNetV1 pointwise stack, int8, 90% sparse: nnz-GOP/s of the 13-launch sequence",
         "value": total_ops * steps / wall / 1e9,
@@ -239,7 +260,8 @@ def run_c5(args):
         "data": "synthetic",
         "config": {"workload": "c5_mobilenet_v1_pointwise_stack", "batch": 64, "layers": 13},
         "roofline": {"bound": "hbm", "achieved": total_bytes / (seq_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": total_bytes / (seq_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
-                     "traffic": None, "algorithmic_bytes_per_sequence": total_bytes, "sequence_us": seq_us, "sum_of_layer_kernel_us": sum(per_layer)},
+                     "traffic": None, "algorithmic_bytes_per_sequence": total_bytes, "sequence_us": seq_us, "sum_of_layer_kernel_us": sum(per_layer),
+                     "graph_replay_us": graph_us, "graph_replay_matches_eager": graph_ok},
         "per_layer_kernel_us": [round(v, 2) for v in per_layer],
         "per_layer_frac": [round(c.algorithmic_bytes(helpers.pla.detect_and_pack(c.dense, c.im_size)) / (t * 1e-6) / 1e9 / HBM_PEAK_GBS, 3) for (c, _, _, _), t in zip(layers, per_layer)],
     }
