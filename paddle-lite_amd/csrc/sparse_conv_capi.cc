@@ -96,7 +96,7 @@ struct pl_sparse_conv_handle {
   int64_t walk_entries = 0;
   DevBuf groups, kidx, wts;
   // block MFMA
-  int row_blocks = 0, ksteps = 0;
+  int row_blocks = 0, ksteps = 0, kmask_words = 1;
   int64_t blocks_present = 0;
   DevBuf wblocks, kmask;
   int wg_slots = 512;       // workgroups resident at once (2 per CU)
@@ -187,7 +187,8 @@ int BuildRowWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
 int BuildBlockMfma(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
   const int rbs = CeilDiv(L.oc, 32), kss = CeilDiv(L.ic, 32);
   std::vector<int8_t> blocks(static_cast<size_t>(rbs) * kss * 64 * 16, 0);
-  std::vector<uint32_t> mask(rbs, 0u);
+  const int words = CeilDiv(kss, 32);  // mask words per row block
+  std::vector<uint32_t> mask(static_cast<size_t>(rbs) * words, 0u);
   auto put = [&](int row, uint32_t c, uint32_t wbits) {
     const int8_t w = static_cast<int8_t>(wbits & 0xffu);
     if (w == 0) return;
@@ -195,7 +196,7 @@ int BuildBlockMfma(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
     const int ks = c >> 5, kk = c & 31;
     const int lane = i + 32 * (kk >> 4), t = kk & 15;
     blocks[((static_cast<size_t>(rb) * kss + ks) * 64 + lane) * 16 + t] = w;
-    mask[rb] |= 1u << ks;
+    mask[static_cast<size_t>(rb) * words + (ks >> 5)] |= 1u << (ks & 31);
   };
   for (const pl::RowGroup& g : L.groups) {
     for (uint32_t j = 0; j < g.count; ++j) {
@@ -205,6 +206,7 @@ int BuildBlockMfma(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
   }
   h->row_blocks = rbs;
   h->ksteps = kss;
+  h->kmask_words = words;
   h->blocks_present = 0;
   for (uint32_t m : mask) h->blocks_present += __builtin_popcount(m);
   hipError_t e = h->wblocks.Upload(blocks.data(), blocks.size());
@@ -344,12 +346,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   h->padded_rows = CeilDiv(desc->oc, 32) * 32;
 
   int algo = desc->algo;
-  const bool mfma_ok = int8 && CeilDiv(desc->ic, 32) <= 32;
-  if (algo == PL_ALGO_BLOCK_MFMA && !mfma_ok) {
-    delete h;
-    return Fail(PL_ERR_UNSUPPORTED, "block MFMA needs ic <= 1024 (got %d)", desc->ic);
-  }
-  if (algo == PL_ALGO_AUTO) algo = mfma_ok ? PL_ALGO_BLOCK_MFMA : PL_ALGO_ROW_WALK;
+  if (algo == PL_ALGO_AUTO) algo = int8 ? PL_ALGO_BLOCK_MFMA : PL_ALGO_ROW_WALK;
   if (algo == PL_ALGO_ROW_WALK) {
     const size_t row_bytes = static_cast<size_t>(int8 ? CeilDiv(desc->ic, 4) : desc->ic) * 4;
     if (row_bytes * 16 > static_cast<size_t>(pl::kMaxLdsBytes)) {
@@ -402,6 +399,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.out = out_dev;
     p.wblocks = h->wblocks.ptr;
     p.kmask = static_cast<const uint32_t*>(h->kmask.ptr);
+    p.kmask_words = h->kmask_words;
     p.scale = static_cast<const float*>(h->scale.ptr);
     p.bias = static_cast<const float*>(h->bias.ptr);
     p.row_blocks = h->row_blocks;
@@ -415,7 +413,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     pl::MfmaConfig c{};
     c.out_kind = OutKind(h->kind);
     c.ks_max = 2;
-    while (c.ks_max < h->ksteps) c.ks_max <<= 1;
+    while (c.ks_max < h->ksteps && c.ks_max < 64) c.ks_max <<= 1;  // 64: any count, a chunk at a time
     // Tile width: full 128-position tiles unless that leaves CUs without a
     // workgroup (narrower tiles measured slower on the 392-workgroup metric
     // shape: every workgroup pays for its own copy of the weight blocks).

@@ -71,7 +71,8 @@ struct MfmaParams {
   const int8_t* x;
   void* out;
   const void* wblocks;     // [row_blocks][ksteps][64 lanes][16 bytes]
-  const uint32_t* kmask;   // [row_blocks] bit ks set = block (rb, ks) has a nonzero
+  const uint32_t* kmask;   // [row_blocks][kmask_words] bit ks set = block (rb, ks) has a nonzero
+  int kmask_words;         // ceil(ksteps / 32)
   const float* scale;      // padded to 32 * row_blocks
   const float* bias;       // padded likewise (zeros when the op has no bias)
   int row_blocks;
@@ -106,6 +107,9 @@ hipError_t LaunchBlockMfma(const MfmaConfig& cfg, const MfmaParams& p, hipStream
 // Largest dynamic LDS size a kernel of this library may be given.
 constexpr int kMaxLdsBytes = 160 * 1024;
 constexpr int kMfmaTilePos = 128;
+// More than 32 k-steps (1024 input channels): the block MFMA kernel takes
+// them this many at a time through one LDS tile.
+constexpr int kLoopChunk = 8;
 
 // Precision changes around an int8 convolution (calib_kernels.hip).
 hipError_t LaunchFp32ToInt8(const float* x, int8_t* out, int64_t n, float scale, hipStream_t stream);

@@ -519,9 +519,9 @@ __device__ __forceinline__ void LoadX(uint32_t (&r)[16], const MfmaParams& p, co
 
 // Transpose to channel-innermost and write the cells of four positions.
 template <bool FAST>
-__device__ __forceinline__ void CommitX(uint32_t (&r)[16], uint4* xt, const MfmaParams& p, const QuadInfo& q, bool live, bool store, int kg_base, int kg_lane, int j) {
+__device__ __forceinline__ void CommitX(uint32_t (&r)[16], uint4* xt, const MfmaParams& p, const QuadInfo& q, bool live, bool store, int kg_base, int kg_lane, int j, int kg_lds0 = 0) {
   const int n_kg = 2 * p.ksteps;
-  const int kg = kg_base + kg_lane;
+  const int kg = kg_base + kg_lane;  // kg_lds0: the channel group held by LDS row 0
   if (!p.quad_aligned) {
     // a partial quad was read from the last four positions of its row
     const int sh = (q.valid == 4 || q.valid == 0) ? 0 : 8 * (4 - q.valid);
@@ -537,16 +537,16 @@ __device__ __forceinline__ void CommitX(uint32_t (&r)[16], uint4* xt, const Mfma
   // now r[4b + c] = channels 16kg+4b..+3 of the quad's position c
   if (store && (FAST || kg < n_kg)) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) xt[(size_t)kg * kMfmaTilePos + c * 32 + j] = make_uint4(r[c], r[4 + c], r[8 + c], r[12 + c]);
+    for (int c = 0; c < 4; ++c) xt[(size_t)(kg - kg_lds0) * kMfmaTilePos + c * 32 + j] = make_uint4(r[c], r[4 + c], r[8 + c], r[12 + c]);
   }
 }
 
-// hw < 4: byte loads, one position at a time.
-__device__ __forceinline__ void StageMfmaBytes(uint4* xt, const MfmaParams& p, uint32_t quad, bool quad_on, int kg0, int j) {
-  const int n_kg = 2 * p.ksteps;
+// hw < 4: byte loads, one position at a time.  Stages the channel groups
+// [kg_first, kg_end) into LDS rows 0 .. kg_end - kg_first.
+__device__ __forceinline__ void StageMfmaBytes(uint4* xt, const MfmaParams& p, uint32_t quad, bool quad_on, int kg0, int j, int kg_first, int kg_end) {
   if (!quad_on) return;
   const QuadInfo q = LocateQuad(p, quad);
-  for (int kg = kg0; kg < n_kg; kg += 8) {
+  for (int kg = kg_first + kg0; kg < kg_end; kg += 8) {
     for (int c = 0; c < 4; ++c) {
       uint32_t d[4] = {0, 0, 0, 0};
       if (c < q.valid) {
@@ -558,7 +558,7 @@ __device__ __forceinline__ void StageMfmaBytes(uint4* xt, const MfmaParams& p, u
           d[i >> 2] |= b << (8 * (i & 3));
         }
       }
-      xt[(size_t)kg * kMfmaTilePos + c * 32 + j] = make_uint4(d[0], d[1], d[2], d[3]);
+      xt[(size_t)(kg - kg_first) * kMfmaTilePos + c * 32 + j] = make_uint4(d[0], d[1], d[2], d[3]);
     }
   }
 }
@@ -703,17 +703,11 @@ __device__ __forceinline__ void MfmaTile(const MfmaParams& p, uint4* xt, uint32_
   const int j = tid & 31;    // quad of the tile
   const int kg0 = tid >> 5;  // 8 channel groups per pass of the workgroup
   const uint32_t quad0 = (uint32_t)tile * (uint32_t)J;
-  v4i a[KSMAX];
-  auto load_weights = [&](int ks0, int ks1) {
-    // blocks of absent k-steps are never multiplied; their loads are clamped
-#pragma unroll
-    for (int ks = ks0; ks < ks1; ++ks) {
-      if (ks < KSMAX) {
-        const int ksc = min(ks, p.ksteps - 1);
-        a[ks] = static_cast<const v4i*>(p.wblocks)[((size_t)rbc * p.ksteps + ksc) * 64 + lane];
-      }
-    }
-  };
+  // KSMAX > 32 stands for any number of k-steps, taken kLoopChunk at a time
+  // through one LDS tile; the accumulators stay in registers across chunks.
+  constexpr bool kLoopK = KSMAX > 32;
+  constexpr int KC = kLoopK ? kLoopChunk : KSMAX;  // k-steps held at once
+  v4i a[KC];
   const bool quad_on = j < J;
   const int jc = quad_on ? j : J - 1;  // idle lanes repeat the last quad's loads
   v16i acc[4];
@@ -722,65 +716,89 @@ __device__ __forceinline__ void MfmaTile(const MfmaParams& p, uint4* xt, uint32_
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[c][i] = 0;
   const uint4* bbase = xt + (size_t)(lane >> 5) * kMfmaTilePos + (lane & 31);
-  // D[32 rows][32 cols] += A[32 x 32k] * B[32k x 32] for k-steps [ks0, ks1)
-  auto multiply = [&](int ks0, int ks1) {
+  const QuadInfo qs = LocateQuad(p, quad0 + (uint32_t)jc);
+  const bool live = qs.valid > 0;
+  auto do_chunk = [&](int chunk) {
+    const int ks_first = kLoopK ? chunk * KC : 0;  // first k-step of the chunk; LDS row 0 is channel group 2 * ks_first
+    // bit i of cmask: k-step ks_first + i holds a nonzero of this row block
+    const uint32_t cmask = kLoopK ? (p.kmask[(size_t)rbc * p.kmask_words + (ks_first >> 5)] >> (ks_first & 31)) & ((1u << kLoopChunk) - 1u) : kmask;
+    auto load_weights = [&](int i0, int i1) {
+      // blocks of absent k-steps are never multiplied; their loads are clamped
 #pragma unroll
-    for (int ks = ks0; ks < ks1; ++ks) {
-      if (ks < KSMAX && (kmask & (1u << ks))) {
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const uint4 bq = bbase[(size_t)(2 * ks) * kMfmaTilePos + c * 32];
-          const v4i b = v4i{(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w};
-          acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ks < KSMAX ? ks : 0], b, acc[c], 0, 0, 0);
+      for (int i = i0; i < i1; ++i) {
+        if (i < KC) {
+          const int ksc = min(ks_first + i, p.ksteps - 1);
+          a[i] = static_cast<const v4i*>(p.wblocks)[((size_t)rbc * p.ksteps + ksc) * 64 + lane];
         }
       }
-    }
-  };
-  if (VEC) {
-    // A pass of the workgroup stages 8 channel groups = 4 k-steps.  The loads
-    // of up to four passes (activations, then that pass's weight blocks) go
-    // out together; each pass is then committed to LDS and multiplied as soon
-    // as its own loads have landed, while the later ones are still in flight.
-    constexpr int kPasses = (2 * KSMAX + 7) / 8;
-    constexpr int kBatch = kPasses < 4 ? kPasses : 4;
-    const QuadInfo qs = LocateQuad(p, quad0 + (uint32_t)jc);
-    const bool live = qs.valid > 0;
-    uint32_t r[kBatch][16];
-    // One straight-line instance per batch and addressing mode: loads under
-    // per-pass conditions would be drained at every join.
-    auto run_batch = [&](auto fast_c, int pass0) {
-      constexpr bool kFast = decltype(fast_c)::value;
+    };
+    // D[32 rows][32 cols] += A[32 x 32k] * B[32k x 32] for the chunk's k-steps [i0, i1)
+    auto multiply = [&](int i0, int i1) {
 #pragma unroll
-      for (int u = 0; u < kBatch; ++u) {
-        LoadX<kFast>(r[u], p, qs, 8 * (pass0 + u), kg0);
-        load_weights(4 * (pass0 + u), 4 * (pass0 + u) + 4);
-      }
+      for (int i = i0; i < i1; ++i) {
+        if (i < KC && (cmask & (1u << i))) {
 #pragma unroll
-      for (int u = 0; u < kBatch; ++u) {
-        CommitX<kFast>(r[u], xt, p, qs, kFast ? true : live, kFast ? (quad_on && live) : quad_on, 8 * (pass0 + u), kg0, jc);
-        PL_PHASE_MARK(2);
-        __syncthreads();
-        if (wave_on) multiply(4 * (pass0 + u), 4 * (pass0 + u) + 4);
+          for (int c = 0; c < 4; ++c) {
+            const uint4 bq = bbase[(size_t)(2 * i) * kMfmaTilePos + c * 32];
+            const v4i b = v4i{(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w};
+            acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i < KC ? i : 0], b, acc[c], 0, 0, 0);
+          }
+        }
       }
     };
+    // the previous chunk's tile is read until every wavefront has multiplied
+    if (kLoopK && chunk > 0) __syncthreads();
+    if (VEC) {
+      // A pass of the workgroup stages 8 channel groups = 4 k-steps.  The
+      // loads of up to four passes (activations, then that pass's weight
+      // blocks) go out together; each pass is then committed to LDS and
+      // multiplied as soon as its own loads have landed, while the later
+      // ones are still in flight.
+      constexpr int kPasses = (2 * KC + 7) / 8;
+      constexpr int kBatch = kPasses < 4 ? kPasses : 4;
+      uint32_t r[kBatch][16];
+      // One straight-line instance per batch and addressing mode: loads
+      // under per-pass conditions would be drained at every join.
+      auto run_batch = [&](auto fast_c, int pass0) {
+        constexpr bool kFast = decltype(fast_c)::value;
 #pragma unroll
-    for (int pass0 = 0; pass0 < kPasses; pass0 += kBatch) {
-      if (pass0 > 0 && 8 * pass0 >= 2 * p.ksteps) break;
-      if (p.small && 16 * 8 * (pass0 + kBatch) <= p.K) {
-        run_batch(std::true_type(), pass0);
-      } else {
-        run_batch(std::false_type(), pass0);
+        for (int u = 0; u < kBatch; ++u) {
+          LoadX<kFast>(r[u], p, qs, 2 * ks_first + 8 * (pass0 + u), kg0);
+          load_weights(4 * (pass0 + u), 4 * (pass0 + u) + 4);
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+          CommitX<kFast>(r[u], xt, p, qs, kFast ? true : live, kFast ? (quad_on && live) : quad_on, 2 * ks_first + 8 * (pass0 + u), kg0, jc, 2 * ks_first);
+          PL_PHASE_MARK(2);
+          __syncthreads();
+          if (wave_on) multiply(4 * (pass0 + u), 4 * (pass0 + u) + 4);
+        }
+      };
+#pragma unroll
+      for (int pass0 = 0; pass0 < kPasses; pass0 += kBatch) {
+        if (pass0 > 0 && 2 * ks_first + 8 * pass0 >= 2 * p.ksteps) continue;
+        if (p.small && 16 * (2 * ks_first + 8 * (pass0 + kBatch)) <= p.K) {
+          run_batch(std::true_type(), pass0);
+        } else {
+          run_batch(std::false_type(), pass0);
+        }
       }
+    } else {
+      load_weights(0, KC);
+      StageMfmaBytes(xt, p, quad0 + (uint32_t)jc, quad_on, kg0, jc, 2 * ks_first, min(2 * (ks_first + KC), 2 * p.ksteps));
+      __syncthreads();
+      if (wave_on) multiply(0, KC);
     }
+  };
+  if (kLoopK) {
+    const int n_chunks = (p.ksteps + KC - 1) / KC;
+    for (int chunk = 0; chunk < n_chunks; ++chunk) do_chunk(chunk);
   } else {
-    load_weights(0, KSMAX);
-    StageMfmaBytes(xt, p, quad0 + (uint32_t)jc, quad_on, kg0, jc);
-    __syncthreads();
-    if (wave_on) multiply(0, KSMAX);
+    do_chunk(0);
   }
   if (!wave_on) return;
   PL_PHASE_MARK(4);
-  MfmaFinish<OUT, ACT, VEC>(p, reinterpret_cast<uint32_t*>(xt + (size_t)2 * p.ksteps * kMfmaTilePos), acc, rb, lane, quad0, J);
+  MfmaFinish<OUT, ACT, VEC>(p, reinterpret_cast<uint32_t*>(xt + (size_t)2 * (kLoopK ? KC : p.ksteps) * kMfmaTilePos), acc, rb, lane, quad0, J);
 }
 
 // Few input channels (at most 64, KSMAX <= 2): the channel groups of one
@@ -796,7 +814,7 @@ __device__ __forceinline__ void MfmaTilesFewChannels(const MfmaParams& p, uint4*
   const int sub_l = kg0 / n_kg, kgl = kg0 - sub_l * n_kg;
   const int RB = min(4, p.row_blocks - 4 * group);
   const int rb = 4 * group + (wave & (RB - 1));
-  const uint32_t kmask = p.kmask[rb];
+  const uint32_t kmask = p.kmask[(size_t)rb * p.kmask_words];
   v4i a[KSMAX];
   const size_t tile_cells = (size_t)n_kg * kMfmaTilePos;
   {
@@ -863,7 +881,7 @@ __device__ __forceinline__ void MfmaBody(const MfmaParams& p, uint4* xt) {
   const int rb = ((blockIdx.x >> 3) % p.row_groups) * 4 + wave;
   const bool wave_on = rb < p.row_blocks;
   const int rbc = wave_on ? rb : p.row_blocks - 1;
-  const uint32_t kmask = wave_on ? p.kmask[rbc] : 0u;
+  const uint32_t kmask = wave_on ? p.kmask[(size_t)rbc * p.kmask_words] : 0u;  // first 32 k-steps; chunked kernels read their own words
   PL_PHASE_MARK(0);
   MfmaTile<KSMAX, OUT, ACT, VEC>(p, xt, kmask, rb, rbc, wave_on, tile);
   PL_PHASE_MARK(6);
@@ -947,6 +965,8 @@ hipError_t MfmaByKs(int ks_max, const MfmaParams& p, dim3 grid, dim3 block, size
       return LaunchWithLds(BlockMfmaKernel<16, OUT>, grid, block, lds, s, p);
     case 32:
       return LaunchWithLds(BlockMfmaKernel<32, OUT>, grid, block, lds, s, p);
+    case 64:
+      return LaunchWithLds(BlockMfmaKernel<64, OUT>, grid, block, lds, s, p);
     default:
       return hipErrorInvalidValue;
   }
@@ -1001,7 +1021,7 @@ hipError_t LaunchRowWalk(const WalkConfig& cfg, const WalkParams& p, hipStream_t
 
 hipError_t LaunchBlockMfma(const MfmaConfig& cfg, const MfmaParams& p, hipStream_t stream) {
   if (p.P == 0 || p.row_blocks == 0) return hipSuccess;
-  if (p.ksteps > cfg.ks_max || p.ksteps > 32) return hipErrorInvalidValue;
+  if (p.ksteps > cfg.ks_max && cfg.ks_max <= 32) return hipErrorInvalidValue;  // ks_max 64 = any count, kLoopChunk at a time
   if (cfg.tile_quads < 1 || cfg.tile_quads > 32 || p.hw < 1) return hipErrorInvalidValue;
   MfmaParams q = p;
   q.qpi = (p.hw + 3) / 4;
@@ -1021,7 +1041,7 @@ hipError_t LaunchBlockMfma(const MfmaConfig& cfg, const MfmaParams& p, hipStream
   }
   tiles = (tiles + q.sub_tiles - 1) / q.sub_tiles;
   q.tiles = (int)tiles;  // workgroup-level tiles
-  size_t lds = (size_t)q.sub_tiles * 2 * p.ksteps * kMfmaTilePos * 16;
+  size_t lds = (size_t)q.sub_tiles * 2 * (cfg.ks_max > 32 ? kLoopChunk : p.ksteps) * kMfmaTilePos * 16;
   if (lds > (size_t)kMaxLdsBytes) return hipErrorInvalidValue;
   // int8 output: 4 KB per wavefront behind the activation tile to widen stores
   q.i8_stage = cfg.out_kind == kOutI8 && cfg.i8_wide_stores && lds + 16384 <= (size_t)kMaxLdsBytes;

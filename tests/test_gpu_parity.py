@@ -96,6 +96,28 @@ def test_few_channel_tiles_bit_exact(shape, kind, monkeypatch):
         assert_same(case, got, want, "few-channel %s %s %s" % (kind, act, shape))
 
 
+# more than 1024 input channels: the block MFMA kernel takes the k-steps a
+# chunk at a time through one LDS tile.  Aligned and odd images, a channel
+# count off the 32 grid, images smaller than a quad, a chunk count of one
+# plus a remainder.
+MANY_CHANNEL_SHAPES = [(2, 2048, 64, 4, 4), (1, 1100, 40, 6, 6), (1, 1030, 33, 7, 7), (3, 1500, 20, 1, 2), (1, 1056, 128, 8, 8)]
+
+
+@pytest.mark.parametrize("kind", ["acc32", "fp32out", "int8out"])
+@pytest.mark.parametrize("shape", MANY_CHANNEL_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_many_channels_bit_exact(shape, kind):
+    announce("many-channel", shape, kind)
+    k = {"acc32": capi.KIND_INT8_ACC32, "fp32out": capi.KIND_INT8_FP32, "int8out": capi.KIND_INT8_INT8}[kind]
+    batch, ic, oc, h, w = shape
+    case = small_case(k, batch, ic, oc, h, w, 0.9, False, AP() if kind == "acc32" else ACTS["leaky"], seed=ic + oc, output_scale=0.2 if kind == "int8out" else 1.0)
+    got = run_hip(case, capi.ALGO_BLOCK_MFMA)
+    want = run_oracle(case, oracle_pack(case))
+    assert_same(case, got, want, "many-channel %s %s" % (kind, shape))
+    # the default choice for int8 is the same kernel now
+    got_auto = run_hip(case, capi.ALGO_AUTO)
+    assert np.array_equal(got_auto, got)
+
+
 @pytest.mark.parametrize("act", sorted(ACTS))
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
