@@ -95,6 +95,10 @@ struct pl_sparse_conv_handle {
   int kd = 0;
   int64_t walk_entries = 0;
   DevBuf groups, kidx, wts;
+  // fp32 row walk over channel chunks (built beside the plain form)
+  DevBuf cw_desc, cw_idx, cw_wts;
+  int cw_chunks = 0, cw_slices = 0;
+  int walk_chunked = 1;  // 0 never, 1 when the problem is large enough, 2 whenever the shape allows
   // block MFMA
   int row_blocks = 0, ksteps = 0, kmask_words = 1;
   int64_t blocks_present = 0;
@@ -108,7 +112,7 @@ struct pl_sparse_conv_handle {
   int padded_rows = 0;
 
   int64_t DeviceBytes() const {
-    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + wblocks.bytes + kmask.bytes + scale.bytes + bias.bytes);
+    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + cw_desc.bytes + cw_idx.bytes + cw_wts.bytes + wblocks.bytes + kmask.bytes + scale.bytes + bias.bytes);
   }
 };
 
@@ -178,6 +182,59 @@ int BuildRowWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
   if (e == hipSuccess) e = h->kidx.Upload(kidx.data(), kidx.size() * sizeof(uint32_t));
   if (e == hipSuccess) e = h->wts.Upload(wts.data(), wts.size() * sizeof(uint32_t));
   if (e != hipSuccess) return FailHip(e, "uploading the row-walk index");
+  return PL_OK;
+}
+
+// Device-side form for the fp32 walk over channel chunks: per (slice, chunk,
+// wavefront, group of the wavefront) the batches of four entries whose channel
+// lies in the chunk, in index order, padded with zero-weight entries that
+// point at the tile's zero row.
+int BuildChunkWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
+  const int nr = L.semi ? 2 : 1;
+  const int per_slice = pl::kChunkWalkWaves * pl::kChunkWalkGroups;
+  const int n_groups = static_cast<int>(L.groups.size());
+  const int slices = CeilDiv(n_groups, per_slice);
+  const int chunks = CeilDiv(L.ic, pl::kChunkWalkChunk);
+  std::vector<uint32_t> desc(static_cast<size_t>(slices) * chunks * per_slice * 2, 0u);
+  std::vector<uint32_t> idx, wts;
+  for (int sl = 0; sl < slices; ++sl) {
+    for (int c = 0; c < chunks; ++c) {
+      for (int gl = 0; gl < per_slice; ++gl) {  // gl = wave * groups-per-wave + group of the wave
+        const int g = sl * per_slice + gl;
+        uint32_t* d = &desc[((static_cast<size_t>(sl) * chunks + c) * per_slice + gl) * 2];
+        d[0] = static_cast<uint32_t>(idx.size());
+        if (g >= n_groups) continue;
+        const pl::RowGroup& rg = L.groups[g];
+        uint32_t packed = 0;
+        int fill = 0;
+        auto flush = [&]() {
+          for (; fill < 4; ++fill) {  // padding entries: zero row, zero weights
+            packed |= static_cast<uint32_t>(pl::kChunkWalkChunk) << (8 * fill);
+            for (int r = 0; r < nr; ++r) wts.push_back(0u);
+          }
+          idx.push_back(packed);
+          packed = 0;
+          fill = 0;
+        };
+        for (uint32_t j = 0; j < rg.count; ++j) {
+          const uint32_t k = L.ic_index[rg.first + j];
+          if (static_cast<int>(k / pl::kChunkWalkChunk) != c) continue;
+          packed |= (k % pl::kChunkWalkChunk) << (8 * fill);
+          wts.push_back(L.w0[rg.first + j]);
+          if (nr == 2) wts.push_back(L.w1[rg.first + j]);
+          if (++fill == 4) flush();
+        }
+        if (fill > 0) flush();
+        d[1] = static_cast<uint32_t>(idx.size()) - d[0];
+      }
+    }
+  }
+  h->cw_chunks = chunks;
+  h->cw_slices = slices;
+  hipError_t e = h->cw_desc.Upload(desc.data(), desc.size() * sizeof(uint32_t));
+  if (e == hipSuccess) e = h->cw_idx.Upload(idx.empty() ? nullptr : idx.data(), idx.size() * sizeof(uint32_t));
+  if (e == hipSuccess) e = h->cw_wts.Upload(wts.empty() ? nullptr : wts.data(), wts.size() * sizeof(uint32_t));
+  if (e != hipSuccess) return FailHip(e, "uploading the chunked row-walk index");
   return PL_OK;
 }
 
@@ -330,6 +387,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   h->device = dev;
   h->wg_slots = 2 * std::max(1, prop.multiProcessorCount);
   if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_I8_WIDE")) h->mfma_i8_wide = std::atoi(e) != 0;
+  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_CHUNKED")) h->walk_chunked = std::max(0, std::min(2, std::atoi(e)));
   if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_SUB_TILES")) h->mfma_sub_tiles = std::max(0, std::min(2, std::atoi(e)));
   if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_TILE_QUADS")) h->mfma_tile_quads = std::max(0, std::min(32, std::atoi(e)));
   // tuning switches for experiments; the defaults are what measured best
@@ -357,6 +415,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   h->algo = algo;
 
   int rc = algo == PL_ALGO_BLOCK_MFMA ? BuildBlockMfma(L, h) : BuildRowWalk(L, h);
+  if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8) rc = BuildChunkWalk(L, h);
   if (rc == PL_OK) {
     // the MFMA epilogue always reads a bias; give it zeros when the op has none
     std::vector<float> zeros;
@@ -429,6 +488,27 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     c.sub_tiles = h->mfma_sub_tiles;
     if (h->mfma_tile_quads > 0) c.tile_quads = h->mfma_tile_quads;
     e = pl::LaunchBlockMfma(c, p, s);
+  } else if (!h->int8 && vec && h->walk_chunked > 0 && h->cw_chunks > 0 &&
+             (h->walk_chunked == 2 || (h->ic > 128 && static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kChunkWalkTile)) * h->cw_slices >= 256))) {
+    // fp32 with many channels and enough work for every CU: walk over
+    // channel chunks (256 positions per list fetch)
+    pl::ChunkWalkParams p{};
+    p.x = x_dev;
+    p.out = out_dev;
+    p.groups = static_cast<const pl::DevGroup*>(h->groups.ptr);
+    p.desc = static_cast<const uint32_t*>(h->cw_desc.ptr);
+    p.idx = static_cast<const uint32_t*>(h->cw_idx.ptr);
+    p.wts = static_cast<const uint32_t*>(h->cw_wts.ptr);
+    p.bias = h->has_bias ? static_cast<const float*>(h->bias.ptr) : nullptr;
+    p.n_groups = h->n_groups;
+    p.n_chunks = h->cw_chunks;
+    p.slices = h->cw_slices;
+    p.M = h->oc;
+    p.K = h->ic;
+    p.hw = im_size;
+    p.P = P;
+    p.act = h->act;
+    e = pl::LaunchChunkWalk(h->semi ? 2 : 1, p, s);
   } else {
     pl::WalkParams p{};
     p.x = x_dev;

@@ -65,6 +65,36 @@ struct WalkConfig {
 
 hipError_t LaunchRowWalk(const WalkConfig& cfg, const WalkParams& p, hipStream_t stream);
 
+// fp32 row walk over channel chunks (chunk_walk_kernels.hip): a workgroup of
+// kChunkWalkWaves wavefronts takes kChunkWalkTile positions and a slice of
+// kChunkWalkWaves * kChunkWalkGroups row groups, and stages kChunkWalkChunk
+// channels at a time.
+constexpr int kChunkWalkTile = 256;
+constexpr int kChunkWalkChunk = 64;
+constexpr int kChunkWalkWaves = 8;
+constexpr int kChunkWalkGroups = 8;
+
+struct ChunkWalkParams {
+  const void* x;
+  void* out;
+  const DevGroup* groups;  // row0 / nrows of every row group
+  // [slice][chunk][wave][group of the wave]: first batch, number of batches
+  const uint32_t* desc;
+  const uint32_t* idx;     // per batch of four entries: four chunk-local channels, 8 bits each (kChunkWalkChunk = zero row)
+  const uint32_t* wts;     // per batch: 4 entries x nrows float bit patterns
+  const float* bias;       // may be null
+  int n_groups;
+  int n_chunks, slices;
+  int M, K;
+  int hw;
+  uint32_t P;
+  DevAct act;
+  int tiles;               // filled in by the launcher
+};
+
+// Needs hw % 4 == 0 and 16-byte aligned x / out.
+hipError_t LaunchChunkWalk(int nrows, const ChunkWalkParams& p, hipStream_t stream);
+
 // Block MFMA SpMM (int8): dense 32x32 weight blocks pre-arranged in operand
 // order, empty blocks skipped through a per-row-block bit mask.
 struct MfmaParams {

@@ -134,6 +134,31 @@ def test_fp32_within_tolerance(shape, paired, act):
         np.testing.assert_allclose(got.reshape(batch, oc, -1), ref, rtol=1e-4, atol=1e-5)
 
 
+# fp32 walk over channel chunks (256 positions per workgroup, 64 channels
+# staged at a time); forced here, the library picks it by itself only for
+# large problems.  Needs H*W % 4 == 0.  (batch, ic, oc, h, w): one chunk and
+# several, a channel count off the chunk grid, more row groups than one slice
+# holds (64), an odd row count, a tile that spans images.
+CHUNKED_SHAPES = [(2, 64, 64, 4, 4), (1, 96, 48, 8, 6), (3, 130, 67, 4, 5), (1, 300, 150, 16, 16), (5, 70, 33, 2, 2), (2, 257, 20, 12, 12)]
+
+
+@pytest.mark.parametrize("act", ["none", "relu6", "hswish"])
+@pytest.mark.parametrize("shape", CHUNKED_SHAPES, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
+def test_fp32_chunked_walk(shape, paired, act, monkeypatch):
+    announce("fp32 chunked", shape, paired, act)
+    batch, ic, oc, h, w = shape
+    case = small_case(capi.KIND_FP32, batch, ic, oc, h, w, 0.75, paired, ACTS[act], seed=ic + 3 * oc)
+    want = run_oracle(case, oracle_pack(case, force_semi=paired))
+    monkeypatch.setenv("PL_SPARSE_CONV_WALK_CHUNKED", "2")
+    got = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired)
+    assert_same(case, got, want, "fp32 chunked %s %s" % (act, shape))
+    # and the plain walk gives the same bits (same order of fused multiply-adds)
+    monkeypatch.setenv("PL_SPARSE_CONV_WALK_CHUNKED", "0")
+    plain = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired)
+    assert np.array_equal(got, plain)
+
+
 def test_no_bias_and_single_scale():
     announce("nobias")
     for kind in (capi.KIND_FP32, capi.KIND_INT8_FP32, capi.KIND_INT8_INT8):
