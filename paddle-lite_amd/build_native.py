@@ -91,6 +91,7 @@ LITE_SOURCES = [
     "core/tensor.cc",
     "core/op_lite.cc",
     "core/optimizer/mir/sparse_conv_detect_pass.cc",
+    "core/optimizer/mir/int8_chain_pass.cc",
     "operators/sparse_conv_op.cc",
     "operators/io_copy_op.cc",
     "operators/calib_op.cc",

@@ -1,0 +1,62 @@
+// What the reference's optimiser does around quantised ops, restated for a
+// linear list of sparse_conv2d ops that all run on TARGET(kHIP):
+//  * the output-type rule of static_kernel_pick_pass
+//    (lite/core/optimizer/mir/static_kernel_pick_pass.cc:97-135): an op with
+//    enable_int8 produces int8 only if every consumer of its output has
+//    enable_int8 too; its output scale is then the consumer's input scale;
+//  * the calib op type_precision_cast_pass puts where a producer's precision
+//    differs from what the picked kernel declares
+//    (lite/core/optimizer/mir/type_precision_cast_pass.cc);
+//  * the io_copy op type_target_cast_pass puts where a tensor lives on
+//    another target than the kernel declares
+//    (lite/core/optimizer/mir/type_target_cast_pass.cc).
+// The result is a list of steps (op description + kernel alias + place) that
+// HipProgram runs in order, the counterpart of RuntimeProgram::Run
+// (lite/core/program.cc:789-816) for this slice.
+#pragma once
+
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "lite/api/paddle_place.h"
+#include "lite/core/kernel.h"
+#include "lite/core/op_desc.h"
+#include "lite/core/op_lite.h"
+#include "lite/core/scope.h"
+
+namespace paddle {
+namespace lite {
+namespace mir {
+
+struct ProgramStep {
+  OpInfo op;
+  std::string kernel;      // "op_type/alias"
+  lite_api::Place place;   // place the kernel is created for
+};
+
+class Int8ChainPass {
+ public:
+  // `ops`: sparse_conv2d ops in execution order (after SparseConvDetectPass).
+  // `feeds`: fp32 host tensors in `scope`.  `fetches`: variables wanted back
+  // on the host as fp32; the host copy of "v" is named "v/host".
+  std::vector<ProgramStep> Apply(const std::vector<OpInfo>& ops, const std::vector<std::string>& feeds, const std::vector<std::string>& fetches, Scope* scope) const;
+};
+
+// Creates the op and the kernel of every step once, then launches them in
+// order on one stream.
+class HipProgram {
+ public:
+  HipProgram(const std::vector<ProgramStep>& steps, Scope* scope);
+  void Run();   // enqueue every step and wait for the stream
+  size_t size() const { return kernels_.size(); }
+  const KernelBase& kernel(size_t i) const { return *kernels_[i]; }
+
+ private:
+  std::vector<std::shared_ptr<OpLite>> ops_;
+  std::vector<std::unique_ptr<KernelBase>> kernels_;
+};
+
+}  // namespace mir
+}  // namespace lite
+}  // namespace paddle

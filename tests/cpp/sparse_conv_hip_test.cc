@@ -15,6 +15,7 @@
 #include <vector>
 
 #include "lite/core/op_registry.h"
+#include "lite/core/optimizer/mir/int8_chain_pass.h"
 #include "lite/core/optimizer/mir/sparse_conv_detect_pass.h"
 #include "lite/kernels/hip/sparse_conv_compute.h"
 #include "lite/operators/sparse_conv_op.h"
@@ -418,6 +419,124 @@ static void CalibChain(bool run_on_device) {
   EXPECT(want_q[2] == 127 && want_q[3] == -127);
 }
 
+// Three quantised 1x1 convolutions in a row, fed and fetched as fp32 on the
+// host: detect pass -> output-type rule / calib / io_copy insertion ->
+// program run on the device, against the oracle's chain
+// fp32_to_int8 -> int8 conv (int8 out) x2 -> int8 conv (fp32 out).
+static void Int8Chain(bool run_on_device) {
+  std::printf("int8 chain\n");
+  std::fflush(stdout);
+  const int batch = 2, hw_h = 8, hw_w = 6, hw = hw_h * hw_w;
+  const int ch[4] = {40, 64, 33, 48};
+  const float act_scale[3] = {0.02f, 0.05f, 0.04f};  // input scale of layer 1..3
+  Scope scope;
+  std::mt19937 gen(77);
+  std::uniform_real_distribution<float> uni(0.f, 1.f);
+  std::normal_distribution<float> nrm(0.f, 1.f);
+  Tensor* a0 = scope.NewTensor("a0");
+  a0->Resize({batch, ch[0], hw_h, hw_w});
+  float* a0d = a0->mutable_data<float>(TargetType::kHost);
+  for (int64_t i = 0; i < a0->numel(); ++i) a0d[i] = uni(gen) * 2.f - 1.f;
+  std::vector<OpInfo> ops;
+  std::vector<std::vector<int8_t>> w8(3);
+  std::vector<std::vector<float>> ws(3), bias(3);
+  for (int l = 0; l < 3; ++l) {
+    const int ic = ch[l], oc = ch[l + 1];
+    const std::string n = std::to_string(l + 1);
+    Tensor* w = scope.NewTensor("w" + n);
+    w->Resize({oc, ic, 1, 1});
+    int8_t* wd = w->mutable_data<int8_t>(TargetType::kHost);
+    for (int64_t i = 0; i < w->numel(); ++i) {
+      int v = static_cast<int>(uni(gen) * 127.f) + 1;
+      if (uni(gen) < 0.5f) v = -v;
+      wd[i] = uni(gen) >= 0.7f ? static_cast<int8_t>(v) : 0;
+    }
+    w8[l].assign(wd, wd + w->numel());
+    Tensor* b = scope.NewTensor("b" + n);
+    b->Resize({oc});
+    float* bd = b->mutable_data<float>(TargetType::kHost);
+    bias[l].resize(oc);
+    for (int i = 0; i < oc; ++i) bias[l][i] = bd[i] = nrm(gen) * 0.1f;
+    ws[l].resize(oc);
+    for (float& v : ws[l]) v = 0.001f + 0.004f * uni(gen);
+    OpInfo conv("conv2d");
+    conv.SetInput("Input", {"a" + std::to_string(l)});
+    conv.SetInput("Filter", {"w" + n});
+    conv.SetInput("Bias", {"b" + n});
+    conv.SetOutput("Output", {"a" + n});
+    scope.NewTensor("a" + n);
+    conv.SetAttr<std::vector<int>>("strides", {1, 1});
+    conv.SetAttr<std::vector<int>>("paddings", {0, 0});
+    conv.SetAttr<std::vector<int>>("dilations", {1, 1});
+    conv.SetAttr<int>("groups", 1);
+    conv.SetAttr<bool>("with_act", true);
+    conv.SetAttr<std::string>("act_type", "relu");
+    conv.SetAttr<bool>("enable_int8", true);
+    conv.SetInputScale("Input0_scale", {act_scale[l]}, true);
+    conv.SetInputScale("Filter0_scale", ws[l], true);
+    conv.SetOutputScale("Output0_scale", {1.f}, true);  // the pick rule overwrites it where the output stays int8
+    ops.push_back(conv);
+  }
+  // the first layer's input tensor must have a shape for the detect pass
+  mir::SparseConvDetectPass detect;
+  detect.SetSparseThreshold(0.5f);
+  // the pass needs the spatial size of every conv input: give the later
+  // inputs their shapes (shape inference would have done so in a graph)
+  for (int l = 1; l < 3; ++l) scope.FindMutableTensor("a" + std::to_string(l))->Resize({batch, ch[l], hw_h, hw_w});
+  EXPECT(detect.Apply(&ops, &scope) == 3);
+
+  mir::Int8ChainPass chain;
+  std::vector<mir::ProgramStep> steps = chain.Apply(ops, {"a0"}, {"a3"}, &scope);
+  EXPECT(steps.size() == 6);
+  if (steps.size() == 6) {
+    EXPECT(steps[0].kernel == "io_copy/host_to_device");
+    EXPECT(steps[1].kernel == "calib/fp32_to_int8" && steps[1].op.GetAttr<float>("scale") == act_scale[0]);
+    EXPECT(steps[2].kernel == "sparse_conv2d/int8_int8_out" && steps[2].op.GetOutputScale("Output0_scale", true)[0] == act_scale[1]);
+    EXPECT(steps[3].kernel == "sparse_conv2d/int8_int8_out" && steps[3].op.GetOutputScale("Output0_scale", true)[0] == act_scale[2]);
+    EXPECT(steps[4].kernel == "sparse_conv2d/int8_fp32_out");
+    EXPECT(steps[5].kernel == "io_copy/device_to_host" && steps[5].op.Output("Out").front() == "a3/host");
+    EXPECT(steps[2].op.Input("Input").front() == "a0/hip/int8");
+  }
+  // an fp32 consumer in the middle keeps its producer's output fp32
+  {
+    std::vector<OpInfo> mixed = ops;
+    mixed[1].SetAttr<bool>("enable_int8", false);
+    Scope dummy;
+    dummy.NewTensor("a0");
+    auto st = chain.Apply({mixed[0]}, {"a0"}, {"a1"}, &dummy);
+    EXPECT(st.size() == 4 && st[2].kernel == "sparse_conv2d/int8_fp32_out");
+  }
+  EXPECT(Throws([&] { chain.Apply(ops, {"a0"}, {"nothing"}, &scope); }));
+  if (!run_on_device) return;
+
+  mir::HipProgram program(steps, &scope);
+  program.Run();
+  program.Run();  // second epoch
+  const Tensor* got = scope.FindMutableTensor("a3/host");
+  EXPECT(got != nullptr && got->dims() == DDim({batch, ch[3], hw_h, hw_w}));
+
+  // oracle chain
+  std::vector<int8_t> q(a0->numel());
+  plo_fp32_to_int8(a0d, q.data(), act_scale[0], a0->numel());
+  std::vector<float> want;
+  for (int l = 0; l < 3; ++l) {
+    const int ic = ch[l], oc = ch[l + 1];
+    plo_act act{1, 6.f, 0.1f, 6.f, 3.f, 6.f};
+    std::vector<float> ms(oc), mb(oc);
+    const int kind = l < 2 ? 2 : 1;
+    EXPECT(plo_merge_params(kind, oc, ws[l].data(), oc, act_scale[l], l < 2 ? act_scale[l + 1] : 1.f, bias[l].data(), ms.data(), mb.data(), &act) == 0);
+    if (kind == 2) {
+      std::vector<int8_t> next(static_cast<size_t>(batch) * oc * hw);
+      plo_dense_conv1x1(2, w8[l].data(), q.data(), mb.data(), ms.data(), next.data(), batch, oc, ic, hw, &act, 1);
+      q.swap(next);
+    } else {
+      want.resize(static_cast<size_t>(batch) * oc * hw);
+      plo_dense_conv1x1(1, w8[l].data(), q.data(), bias[l].data(), ms.data(), want.data(), batch, oc, ic, hw, &act, 1);
+    }
+  }
+  if (got) EXPECT(std::memcmp(want.data(), got->raw_data(), want.size() * 4) == 0);
+}
+
 int main(int argc, char** argv) {
   const bool gpu = argc > 1 && std::string(argv[1]) == "--gpu";
   RegistryAndErrorPaths();
@@ -438,6 +557,7 @@ int main(int argc, char** argv) {
   }
   for (const Problem& p : problems) RunProblem(p, gpu);
   CalibChain(gpu);
+  Int8Chain(gpu);
   std::printf("%s: %d failure(s)\n", gpu ? "gpu" : "cpu", g_failures);
   return g_failures ? 1 : 0;
 }
