@@ -446,6 +446,8 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
   if (batch < 0 || im_size <= 0) return Fail(PL_ERR_BAD_ARG, "batch must be >= 0 and im_size > 0");
   if (batch == 0) return PL_OK;
   if (!x_dev || !out_dev) return Fail(PL_ERR_BAD_ARG, "null device pointer");
+  int cur_dev = -1;
+  if (hipGetDevice(&cur_dev) != hipSuccess || cur_dev != h->device) return Fail(PL_ERR_BAD_ARG, "the handle belongs to device %d, the current device is %d", h->device, cur_dev);
   const int64_t P64 = static_cast<int64_t>(batch) * im_size;
   if (P64 >= (1ll << 31) - 512) return Fail(PL_ERR_UNSUPPORTED, "batch * im_size = %lld exceeds 2^31", static_cast<long long>(P64));
   const uint32_t P = static_cast<uint32_t>(P64);

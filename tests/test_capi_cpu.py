@@ -132,3 +132,17 @@ def test_workloads_are_seeded_and_shaped():
     c2 = workloads.config2(batch=1)
     assert O.count_semi(c2.dense)["flag_semi"] == 1 and c2.dense.dtype == np.float32
     assert len(workloads.MOBILENET_V1_POINTWISE) == 13
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """Every box has one GPU: bench.py --gpus N > 1 exits with a message
+    instead of measuring anything."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+    assert res.returncode != 0
+    assert "one GPU" in res.stderr
+    assert res.stdout.strip() == ""
