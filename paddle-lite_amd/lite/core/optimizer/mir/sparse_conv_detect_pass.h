@@ -20,11 +20,14 @@ class SparseConvDetectPass {
  public:
   // reference default 0.6 (lite/api/paddle_api.h:473-474); the predictor
   // passes 1.5 to disable the pass (lite/api/cxx_api_impl.cc:112-123)
-  // The optimiser tool refuses a threshold outside [0, 1]
+  // Any value is accepted here: the predictor passes 1.5 to switch the pass
+  // off (reference: lite/api/cxx_api_impl.cc:117-123).
+  void SetSparseThreshold(float t) { sparse_threshold_ = t; }
+  // The range check of the optimiser tool, which only takes [0, 1]
   // (reference: lite/api/tools/opt_base.cc:78-81).
-  void SetSparseThreshold(float t) {
+  static float CheckedToolThreshold(float t) {
     CHECK(t >= 0.f && t <= 1.f) << "Please set sparse_threshold between 0.0 and 1.0.";
-    sparse_threshold_ = t;
+    return t;
   }
   float sparse_threshold() const { return sparse_threshold_; }
 

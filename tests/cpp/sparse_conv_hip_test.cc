@@ -254,11 +254,9 @@ static void RegistryAndErrorPaths() {
   }
   EXPECT(static_cast<int>(TARGET(kHIP)) == 19 && static_cast<int>(TARGET(kNNAdapter)) == 18);
   {
-    mir::SparseConvDetectPass range;
-    EXPECT(Throws([&] { range.SetSparseThreshold(1.5f); }));
-    EXPECT(Throws([&] { range.SetSparseThreshold(-0.1f); }));
-    range.SetSparseThreshold(1.0f);
-    EXPECT(range.sparse_threshold() == 1.0f);
+    EXPECT(Throws([&] { mir::SparseConvDetectPass::CheckedToolThreshold(1.5f); }));
+    EXPECT(Throws([&] { mir::SparseConvDetectPass::CheckedToolThreshold(-0.1f); }));
+    EXPECT(mir::SparseConvDetectPass::CheckedToolThreshold(1.0f) == 1.0f);
   }
 
   // unknown fused activation and bad paddings are fatal in the op
