@@ -31,6 +31,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib"])
     ap.add_argument("--algo", default="auto", choices=["auto", "walk", "mfma"])
+    ap.add_argument("--fp16", action="store_true", help="run an fp32 configuration (c1, c2) through the half-precision kernel")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cache-resident", action="store_true", help="reuse one buffer set (reported, never the headline)")
     ap.add_argument("--copy-calibration", action="store_true", help="also launch a plain 64 MiB device copy 20 times, the known-size kernel that counter runs scale FETCH_SIZE / WRITE_SIZE by")
@@ -289,6 +290,14 @@ def main():
     if args.config == "calib":
         return run_calib(args)
     case = wl.CONFIGS[args.config]()
+    if args.fp16:
+        if case.kind != capi.KIND_FP32:
+            sys.stderr.write("--fp16 applies to the fp32 configurations\n")
+            return 2
+        case.kind = capi.KIND_FP16
+        case.x = case.x.astype(np.float16)
+        case.name += "_fp16"
+        args.no_cpu_baseline = True  # the CPU baselines are fp32 / int8 paths
     algo = {"auto": capi.ALGO_AUTO, "walk": capi.ALGO_ROW_WALK, "mfma": capi.ALGO_BLOCK_MFMA}[args.algo]
     kernel, weights = helpers.make_kernel(case, algo=algo)
     info = kernel.info()
@@ -296,9 +305,9 @@ def main():
     nbytes = case.algorithmic_bytes(weights)
 
     # rotating buffer sets: footprint above the last-level cache
-    out_dtype = {capi.KIND_FP32: torch.float32, capi.KIND_INT8_FP32: torch.float32, capi.KIND_INT8_INT8: torch.int8}[case.kind]
+    out_dtype = {capi.KIND_FP32: torch.float32, capi.KIND_INT8_FP32: torch.float32, capi.KIND_INT8_INT8: torch.int8, capi.KIND_FP16: torch.float16}[case.kind]
     oc = case.dense.shape[0]
-    set_bytes = case.x.nbytes + case.batch * oc * case.im_size * (1 if out_dtype == torch.int8 else 4)
+    set_bytes = case.x.nbytes + case.batch * oc * case.im_size * {torch.int8: 1, torch.float16: 2}.get(out_dtype, 4)
     n_sets = 1 if args.cache_resident else int(LLC_BYTES * 1.25 // set_bytes) + 1
     x0 = torch.from_numpy(case.x).cuda()
     xs = [x0] + [x0.clone() for _ in range(n_sets - 1)]
@@ -319,7 +328,9 @@ def main():
     nchk = min(case.batch, 2)
     want = helpers.run_oracle(case, x=case.x[:nchk])
     got = outs[0][:nchk].cpu().numpy()
-    if case.kind == capi.KIND_FP32:
+    if case.kind == capi.KIND_FP16:
+        assert np.array_equal(got, want), "timed kernel output differs from the oracle"
+    elif case.kind == capi.KIND_FP32:
         np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
     else:
         assert np.array_equal(got, want), "timed kernel output differs from the oracle"
@@ -371,7 +382,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32" if case.kind == capi.KIND_FP32 else "int8",
+        "dtype": {capi.KIND_FP32: "f32", capi.KIND_FP16: "f16"}.get(case.kind, "int8"),
         "data": "synthetic",
         "config": {
             "workload": case.name,

@@ -38,12 +38,19 @@ enum {
 /* Kernel variants = the registrations of the reference
  * (lite/kernels/arm/sparse_conv_compute.cc:369-430): fp32 "def",
  * "int8_fp32_out" and "int8_int8_out".  PL_KIND_INT8_ACC32 additionally
- * exposes the raw int32 accumulators of the int8 path for verification. */
+ * exposes the raw int32 accumulators of the int8 path for verification.
+ * PL_KIND_FP16 is the half-precision kernel (sparse_conv_compute.cc:270-356,
+ * lite/backends/arm/math/fp16/sparse_conv_fp16.cc, sparse_semi_conv_fp16.cc):
+ * the descriptor carries the fp32 sparse tensors and the fp32 bias of the
+ * pass, which prepare converts to binary16 like that kernel's PrepareForRun;
+ * x_dev / out_dev are binary16, and accumulation and activation run in
+ * half precision. */
 enum {
   PL_KIND_FP32 = 0,
   PL_KIND_INT8_FP32 = 1,
   PL_KIND_INT8_INT8 = 2,
-  PL_KIND_INT8_ACC32 = 3
+  PL_KIND_INT8_ACC32 = 3,
+  PL_KIND_FP16 = 4
 };
 
 /* lite_api::ActivationType values the sparse kernels implement
@@ -196,6 +203,12 @@ int pl_sparse_pack(int32_t dtype, int32_t flag_semi, const void* dense,
                    int32_t oc, int32_t ic, int32_t im_size,
                    void* nonzero_weights, int64_t n_weights,
                    uint32_t* oc_nonzeros, int32_t* diffs, int64_t n_diffs);
+
+/* Host: float -> IEEE binary16 bit patterns, round to nearest even.  Replaces
+ * lite::arm::math::fp16::fp32_to_fp16 as the half-precision kernel class
+ * uses it on weights and bias (lite/kernels/arm/sparse_conv_compute.cc:
+ * 275-297); prepare applies the same conversion for PL_KIND_FP16. */
+int pl_fp32_to_fp16(const float* in, uint16_t* out, int64_t n);
 
 /* Precision changes either side of an int8 sparse convolution (device
  * pointers, n elements, per-tensor scale; enqueued on `stream`) -----------

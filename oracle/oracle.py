@@ -192,6 +192,27 @@ def sparse_conv_fp32(pk, x, bias=None, act=None):
     return out
 
 
+def fp32_to_fp16(x):
+    """Element-wise conversion (round to nearest even); returns float16."""
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, dtype=np.uint16)
+    lib().plo_fp32_to_fp16(_p(x), _p(out), C.c_int64(x.size))
+    return out.view(np.float16)
+
+
+def sparse_conv_fp16(pk, x, bias=None, act=None):
+    """pk: the fp32 packing of the pass; x: float16 activations; bias: fp32
+    (converted like the kernel class does).  Returns float16."""
+    x = _c(x, np.float16)
+    batch, K, N = x.shape[0], x.shape[1], int(np.prod(x.shape[2:]))
+    out = np.empty((batch, pk.M) + x.shape[2:], dtype=np.uint16)
+    w16 = _c(fp32_to_fp16(pk.nonzero_weights).view(np.uint16))
+    b16 = _c(fp32_to_fp16(bias).view(np.uint16)) if bias is not None else None
+    lib().plo_sparse_conv_fp16(_p(w16), _p(_c(x.view(np.uint16))), _p(_c(pk.diffs)), _p(_c(pk.oc_nonzeros)), _p(b16), _p(out), batch, pk.M, K, N,
+                               pk.first_ic, pk.flag_semi, C.byref(act) if act else None)
+    return out.view(np.float16)
+
+
 def sparse_conv_int8(pk, x, scale, bias=None, act=None, out_int8=False):
     x = _c(x, np.int8)
     batch, K, N = x.shape[0], x.shape[1], int(np.prod(x.shape[2:]))

@@ -357,6 +357,169 @@ void plo_sparse_conv_fp32(const float* A, const float* x,
   }
 }
 
+/* ------------------------------------------------------------------------ */
+/* fp16 path (IEEE binary16 on bit patterns; every operation rounds once,   */
+/* to nearest even, like the NEON half-precision instructions)              */
+/* ------------------------------------------------------------------------ */
+static double h2d(uint16_t h) {
+  const int sign = h >> 15, e = (h >> 10) & 31, m = h & 1023;
+  double v;
+  if (e == 31)
+    v = m ? NAN : INFINITY;
+  else if (e == 0)
+    v = ldexp((double)m, -24);
+  else
+    v = ldexp((double)(m + 1024), e - 25);
+  return sign ? -v : v;
+}
+
+/* exact double -> binary16, round to nearest even */
+static uint16_t d2h(double d) {
+  uint16_t sign = signbit(d) ? 0x8000u : 0;
+  if (isnan(d)) return (uint16_t)(sign | 0x7e00u);
+  double a = fabs(d);
+  if (a >= 65520.0) return (uint16_t)(sign | 0x7c00u); /* rounds to infinity */
+  if (a < ldexp(1.0, -14)) {
+    /* subnormal range: multiples of 2^-24; 1024 carries into the smallest
+     * normal number by itself */
+    return (uint16_t)(sign | (uint16_t)nearbyint(ldexp(a, 24)));
+  }
+  int e;
+  double m = frexp(a, &e);               /* a = m * 2^e, m in [0.5, 1) */
+  double q = nearbyint(ldexp(m, 11));    /* 1024 .. 2048 */
+  if (q == 2048.0) {
+    q = 1024.0;
+    ++e;
+  }
+  /* value = q * 2^(e-11), biased exponent = e - 1 + 15 */
+  return (uint16_t)(sign | (uint16_t)((e + 14) << 10) | ((uint16_t)q & 1023u));
+}
+
+uint16_t plo_f32_to_f16(float f) { return d2h((double)f); }
+float plo_f16_to_f32(uint16_t h) { return (float)h2d(h); }
+
+/* fused multiply-add: the product of two halves is exact in double; the sum
+ * may not be, so it is rounded to odd first (error term from TwoSum), which
+ * makes the final rounding to 11 bits the correctly rounded result */
+static uint16_t h_fma(uint16_t a, uint16_t b, uint16_t c) {
+  const double p = h2d(a) * h2d(b), cc = h2d(c);
+  double s = p + cc;
+  if (isfinite(s) && s != 0.0) {
+    const double bb = s - p;
+    const double err = (p - (s - bb)) + (cc - bb);
+    if (err != 0.0) {
+      uint64_t bits;
+      memcpy(&bits, &s, 8);
+      if ((bits & 1u) == 0) {
+        /* one ulp towards the exact sum */
+        if ((err > 0.0) == (s > 0.0))
+          bits += 1;
+        else
+          bits -= 1;
+        memcpy(&s, &bits, 8);
+      }
+    }
+  }
+  return d2h(s);
+}
+static uint16_t h_mul(uint16_t a, uint16_t b) { return d2h(h2d(a) * h2d(b)); }
+static uint16_t h_add(uint16_t a, uint16_t b) { return d2h(h2d(a) + h2d(b)); }
+static uint16_t h_max(uint16_t a, uint16_t b) { return h2d(a) >= h2d(b) ? a : b; }
+static uint16_t h_min(uint16_t a, uint16_t b) { return h2d(a) <= h2d(b) ? a : b; }
+
+void plo_fp32_to_fp16(const float* in, uint16_t* out, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) out[i] = plo_f32_to_f16(in[i]);
+}
+void plo_fp16_to_fp32(const uint16_t* in, float* out, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) out[i] = plo_f16_to_f32(in[i]);
+}
+
+typedef struct h_act {
+  int type;
+  uint16_t alpha; /* relu6 bound or leaky slope */
+  uint16_t hs_offset, hs_inv_scale, hs_threshold;
+} h_act;
+
+/* reference: lite/backends/arm/math/fp16/sparse_conv_fp16.cc:1301-1325
+ * (constants), :668-1173 (instruction order of the activations) */
+static h_act make_h_act(const plo_act* act) {
+  h_act a = {0, 0, 0, 0, 0};
+  if (!act) return a;
+  a.type = act->type;
+  if (act->type == PLO_ACT_RELU6) a.alpha = plo_f32_to_f16(act->relu6_coef);
+  if (act->type == PLO_ACT_LEAKY_RELU) a.alpha = plo_f32_to_f16(act->leaky_alpha);
+  if (act->type == PLO_ACT_HARD_SWISH) {
+    a.hs_offset = plo_f32_to_f16(act->hs_offset);
+    a.hs_inv_scale = d2h(1.0 / (double)act->hs_scale);
+    a.hs_threshold = plo_f32_to_f16(act->hs_threshold);
+  }
+  return a;
+}
+
+static uint16_t apply_h_act(uint16_t v, const h_act* a) {
+  switch (a->type) {
+    case PLO_ACT_RELU:
+      return h_max(v, 0);
+    case PLO_ACT_RELU6:
+      return h_min(h_max(v, 0), a->alpha);
+    case PLO_ACT_LEAKY_RELU:
+      return h2d(v) >= 0.0 ? v : h_mul(v, a->alpha);
+    case PLO_ACT_HARD_SWISH: {
+      uint16_t t = h_add(v, a->hs_offset);
+      uint16_t u = h_mul(v, a->hs_inv_scale);
+      t = h_min(h_max(t, 0), a->hs_threshold);
+      return h_mul(u, t);
+    }
+    default:
+      return v;
+  }
+}
+
+/* The three sparse tensors are those the pass makes for fp32 weights (rows
+ * padded to four, or the semi layout); the kernel class converts weights and
+ * bias to fp16 and halves the byte offsets
+ * (lite/kernels/arm/sparse_conv_compute.cc:270-304); here the weights and the
+ * bias arrive converted, the offsets as the pass wrote them. */
+void plo_sparse_conv_fp16(const uint16_t* A, const uint16_t* x,
+                          const int32_t* diffs, const uint32_t* ends,
+                          const uint16_t* bias, uint16_t* out, int batch,
+                          int M, int K, int N, int first_ic, int flag_semi,
+                          const plo_act* act) {
+  const h_act ha = make_h_act(act);
+  const int layout = flag_semi ? 2 : 1;
+  const int pairs = flag_semi ? M / 2 : 0;
+  const int groups = flag_semi ? pairs + (M & 1) : M;
+  for (int b = 0; b < batch; ++b) {
+    const char* start = (const char*)(x + ((size_t)b * K + first_ic) * N);
+    uint16_t* o = out + (size_t)b * M * N;
+    for (int g = 0; g < groups; ++g) {
+      row_span s = span_of(layout, ends, diffs, g);
+      const int is_pair = flag_semi && g < pairs;
+      const int row0 = flag_semi ? (is_pair ? 2 * g : 2 * pairs) : g;
+      const uint16_t* w =
+          flag_semi ? A + 2 * (size_t)s.first : A + (size_t)s.first;
+      for (int p = 0; p < N; ++p) {
+        uint16_t a0 = bias ? bias[row0] : 0;
+        uint16_t a1 = (is_pair && bias) ? bias[row0 + 1] : 0;
+        const char* ptr = start + s.start / 2 + (size_t)p * sizeof(uint16_t);
+        for (uint32_t j = 0; j < s.count; ++j) {
+          uint16_t xv;
+          memcpy(&xv, ptr, 2);
+          if (is_pair) {
+            a0 = h_fma(xv, w[2 * j], a0);
+            a1 = h_fma(xv, w[2 * j + 1], a1);
+          } else {
+            a0 = h_fma(xv, w[j], a0);
+          }
+          ptr += diffs[s.first + j] / 2;
+        }
+        o[(size_t)row0 * N + p] = apply_h_act(a0, &ha);
+        if (is_pair) o[(size_t)(row0 + 1) * N + p] = apply_h_act(a1, &ha);
+      }
+    }
+  }
+}
+
 /* int8 accumulation core: calls sink(row, p, acc) for every output */
 typedef struct i8_sink {
   int kind; /* 0 raw acc, 1 fp32 out, 2 int8 out */

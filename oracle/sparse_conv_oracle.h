@@ -124,6 +124,26 @@ void plo_sparse_conv_int8_int8(const int8_t* nonzero_weights, const int8_t* x,
                                int M, int K, int N, int first_ic,
                                int flag_semi, const plo_act* act);
 
+/* fp16 path: values are IEEE binary16 bit patterns.  Weights and bias are the
+ * fp32 layout of the pass converted element by element (round to nearest
+ * even), `diffs` are the byte offsets as the pass wrote them for fp32 (the
+ * function halves them like the kernel class does); accumulation, bias and
+ * activation all happen in half precision, one rounding per instruction.
+ * reference: lite/kernels/arm/sparse_conv_compute.cc:270-356,
+ * lite/backends/arm/math/fp16/sparse_conv_fp16.cc (fmla chains, activation
+ * macros :668-1173, constants :1301-1325), sparse_semi_conv_fp16.cc.
+ * Parity unpinned: the reference has no vectors for it and its test only
+ * compares with an fp32 computation under a tolerance. */
+uint16_t plo_f32_to_f16(float f);
+float plo_f16_to_f32(uint16_t h);
+void plo_fp32_to_fp16(const float* in, uint16_t* out, int64_t n);
+void plo_fp16_to_fp32(const uint16_t* in, float* out, int64_t n);
+void plo_sparse_conv_fp16(const uint16_t* nonzero_weights, const uint16_t* x,
+                          const int32_t* diffs, const uint32_t* oc_nonzeros,
+                          const uint16_t* bias, uint16_t* out, int batch,
+                          int M, int K, int N, int first_ic, int flag_semi,
+                          const plo_act* act);
+
 /* Raw int32 accumulators of the int8 path (no epilogue), for the bit-exact
  * accumulator check. */
 void plo_sparse_conv_int8_acc(const int8_t* nonzero_weights, const int8_t* x,

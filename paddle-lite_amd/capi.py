@@ -8,7 +8,7 @@ LIB_PATH = os.path.join(PKG, "lib", "libpl_sparse_conv.so")
 ABI_VERSION = 1
 
 PL_OK, PL_ERR_BAD_ARG, PL_ERR_BAD_LAYOUT, PL_ERR_UNSUPPORTED, PL_ERR_HIP, PL_ERR_NO_DEVICE = 0, -1, -2, -3, -4, -5
-KIND_FP32, KIND_INT8_FP32, KIND_INT8_INT8, KIND_INT8_ACC32 = 0, 1, 2, 3
+KIND_FP32, KIND_INT8_FP32, KIND_INT8_INT8, KIND_INT8_ACC32, KIND_FP16 = 0, 1, 2, 3, 4
 ACT_NONE, ACT_RELU, ACT_RELU6, ACT_LEAKY_RELU, ACT_HARD_SWISH = 0, 1, 2, 4, 10
 ALGO_AUTO, ALGO_ROW_WALK, ALGO_BLOCK_MFMA = 0, 1, 2
 
@@ -25,6 +25,7 @@ EXPORTS = [
     "pl_sparse_count_semi",
     "pl_sparse_count_zeros",
     "pl_sparse_pack",
+    "pl_fp32_to_fp16",
     "pl_calib_fp32_to_int8",
     "pl_calib_int8_to_fp32",
 ]
@@ -120,6 +121,8 @@ def lib():
     L.pl_sparse_count_zeros.restype = C.c_int
     L.pl_sparse_pack.argtypes = [C.c_int32, C.c_int32, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int64]
     L.pl_sparse_pack.restype = C.c_int
+    L.pl_fp32_to_fp16.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+    L.pl_fp32_to_fp16.restype = C.c_int
     L.pl_calib_fp32_to_int8.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_float, C.c_void_p]
     L.pl_calib_fp32_to_int8.restype = C.c_int
     L.pl_calib_int8_to_fp32.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_float, C.c_void_p]

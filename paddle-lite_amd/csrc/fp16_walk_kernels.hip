@@ -1,0 +1,215 @@
+// Row walk in half precision: activations, weights, bias, accumulators and
+// the activation function are all IEEE binary16, one rounding per
+// instruction (v_pk_fma_f16 for the multiply-accumulate), in index order.
+//
+// A workgroup stages a tile of TP positions x all channels in LDS
+// ([channel][position] halves plus one all-zero row for the padding entries
+// of the index lists); a wavefront owns one output row (or row pair) at a
+// time, a lane two neighbouring positions.  Index lists and weights are read
+// through the constant address space (scalar loads).
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "sparse_conv_kernels.h"
+
+namespace pl {
+namespace {
+
+typedef _Float16 h1;
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef const __attribute__((address_space(4))) uint32_t* ConstWords;
+typedef const __attribute__((address_space(4))) uint16_t* ConstHalves;
+
+__device__ __forceinline__ h1 HalfBits(uint16_t b) { return __builtin_bit_cast(h1, b); }
+__device__ __forceinline__ uint16_t BitsOf(h1 v) { return __builtin_bit_cast(uint16_t, v); }
+__device__ __forceinline__ h2 Both(h1 v) { return h2{v, v}; }
+
+__device__ __forceinline__ int XcdTile(int tiles, int per_tile) {
+  const int xcd = blockIdx.x & 7, wg_slot = blockIdx.x >> 3;
+  const int first = (xcd * tiles) >> 3, last = ((xcd + 1) * tiles) >> 3;
+  const int t = first + wg_slot / per_tile;
+  return t < last ? t : -1;
+}
+
+// Activation on two values, every step its own half-precision instruction:
+// relu max(v,0); relu6 min(max(v,0),six); leaky v >= 0 ? v : v*alpha;
+// hard_swish (v * (1/scale)) * min(max(v + offset, 0), threshold).
+template <int ACT>
+__device__ __forceinline__ h2 ActivateH(h2 v, const DevActH& a) {
+  const h2 zero = {(h1)0, (h1)0};
+  if (ACT == 1) return __builtin_elementwise_max(v, zero);
+  if (ACT == 2) return __builtin_elementwise_min(__builtin_elementwise_max(v, zero), Both(HalfBits(a.alpha)));
+  if (ACT == 4) {
+    const h2 m = v * Both(HalfBits(a.alpha));
+    return h2{v.x >= (h1)0 ? v.x : m.x, v.y >= (h1)0 ? v.y : m.y};
+  }
+  if (ACT == 10) {
+    h2 t = v + Both(HalfBits(a.hs_offset));
+    const h2 u = v * Both(HalfBits(a.hs_inv_scale));
+    t = __builtin_elementwise_min(__builtin_elementwise_max(t, zero), Both(HalfBits(a.hs_threshold)));
+    return u * t;
+  }
+  return v;
+}
+
+template <int NR, int TP, int ACT>
+__device__ __forceinline__ void HalfWalkBody(const HalfWalkParams& p, uint32_t* tile32) {
+  uint16_t* tile = reinterpret_cast<uint16_t*>(tile32);
+  const int tile_id = XcdTile(p.tiles, p.slices);
+  if (tile_id < 0) return;
+  const int slice = (blockIdx.x >> 3) % p.slices;
+  const uint32_t tile0 = (uint32_t)tile_id * (uint32_t)TP;
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+
+  // ---- staging: [channel][TP] halves; row K is zero
+  if (p.pair) {
+    // positions two at a time (hw even, x 4-byte aligned: a pair never
+    // leaves its image)
+    constexpr int TP2 = TP / 2;
+    const int j2 = tid % TP2;
+    const uint32_t g = tile0 + 2u * j2;
+    const bool live = g < p.P;
+    const uint32_t n = live ? g / (uint32_t)p.hw : 0u, pp = live ? g % (uint32_t)p.hw : 0u;
+    const uint16_t* col = p.x + (size_t)n * p.K * p.hw + pp;
+    for (int k = tid / TP2; k <= p.K; k += nthreads / TP2) {
+      uint32_t v = 0;
+      if (live && k < p.K) v = *reinterpret_cast<const uint32_t*>(col + (size_t)k * p.hw);
+      tile32[(size_t)k * TP2 + j2] = v;
+    }
+  } else {
+    const int j = tid % TP;
+    const uint32_t g = tile0 + j;
+    const bool live = g < p.P;
+    const uint32_t n = live ? g / (uint32_t)p.hw : 0u, pp = live ? g % (uint32_t)p.hw : 0u;
+    const uint16_t* col = p.x + (size_t)n * p.K * p.hw + pp;
+    for (int k = tid / TP; k <= p.K; k += nthreads / TP) tile[(size_t)k * TP + j] = (live && k < p.K) ? col[(size_t)k * p.hw] : (uint16_t)0;
+  }
+  __syncthreads();
+
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nwaves = nthreads >> 6;
+  const bool lane_on = 2 * lane < TP;
+  const uint32_t* xlane = tile32 + (lane_on ? lane : 0);  // the lane's two positions of channel 0
+  const ConstWords group_words = (ConstWords)p.groups;
+  const ConstWords kidx = (ConstWords)p.kidx;
+  const ConstWords wts = (ConstWords)p.wts;
+  const ConstHalves bias = (ConstHalves)p.bias;
+  const int g_begin = slice * p.groups_per_slice;
+  const int g_end = min(p.n_groups, g_begin + p.groups_per_slice);
+
+  for (int g = g_begin + wave; g < g_end; g += nwaves) {
+    const ConstWords gw = group_words + (size_t)g * 4;
+    const int row0 = (int)gw[0], nrows = (int)gw[1];
+    const uint32_t first = gw[2], count = gw[3];
+    h2 a0 = {(h1)0, (h1)0}, a1 = {(h1)0, (h1)0};
+    if (bias) {
+      a0 = Both(HalfBits(bias[row0]));
+      if (NR == 2 && nrows == 2) a1 = Both(HalfBits(bias[row0 + 1]));
+    }
+    const ConstWords kp = kidx + first;
+    const ConstWords wp = wts + first;
+    // list lengths are multiples of kWalkBatch
+    for (uint32_t e = 0; e < count; e += kWalkBatch) {
+#pragma unroll
+      for (int i = 0; i < kWalkBatch; ++i) {
+        const uint32_t k = kp[e + i], w = wp[e + i];
+        const h2 xv = __builtin_bit_cast(h2, xlane[(size_t)k * (TP / 2)]);
+        a0 = __builtin_elementwise_fma(xv, Both(HalfBits((uint16_t)(w & 0xffffu))), a0);
+        if (NR == 2) a1 = __builtin_elementwise_fma(xv, Both(HalfBits((uint16_t)(w >> 16))), a1);
+      }
+    }
+    if (!lane_on) continue;
+    const uint32_t gpos = tile0 + 2u * (uint32_t)lane;
+    if (gpos >= p.P) continue;
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+      if (r < nrows) {
+        const h2 v = ActivateH<ACT>(r == 0 ? a0 : a1, p.act);
+        const int row = row0 + r;
+        if (p.pair) {
+          const uint32_t n = gpos / (uint32_t)p.hw, pp = gpos % (uint32_t)p.hw;
+          __builtin_nontemporal_store(__builtin_bit_cast(uint32_t, v), reinterpret_cast<uint32_t*>(p.out + ((size_t)n * p.M + row) * p.hw + pp));
+        } else {
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const uint32_t gj = gpos + j;
+            if (gj < p.P) {
+              const uint32_t n = gj / (uint32_t)p.hw, pp = gj % (uint32_t)p.hw;
+              p.out[((size_t)n * p.M + row) * p.hw + pp] = BitsOf(j == 0 ? v.x : v.y);
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int NR, int TP>
+__global__ void __launch_bounds__(1024) HalfWalkKernel(const HalfWalkParams p) {
+  extern __shared__ uint32_t tile32[];
+  switch (p.act.type) {
+    case 1:
+      HalfWalkBody<NR, TP, 1>(p, tile32);
+      break;
+    case 2:
+      HalfWalkBody<NR, TP, 2>(p, tile32);
+      break;
+    case 4:
+      HalfWalkBody<NR, TP, 4>(p, tile32);
+      break;
+    case 10:
+      HalfWalkBody<NR, TP, 10>(p, tile32);
+      break;
+    default:
+      HalfWalkBody<NR, TP, 0>(p, tile32);
+      break;
+  }
+}
+
+template <typename K>
+hipError_t LaunchBig(K kernel, dim3 grid, dim3 block, size_t lds, hipStream_t s, const HalfWalkParams& p) {
+  // once per kernel and device: allow more than 64 KB of dynamic LDS
+  static bool done[64] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (lds > 48 * 1024 && dev >= 0 && dev < 64 && !done[dev]) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
+    if (e != hipSuccess) return e;
+    done[dev] = true;
+  }
+  hipLaunchKernelGGL(kernel, grid, block, lds, s, p);
+  return hipGetLastError();
+}
+
+template <int NR>
+hipError_t ByTile(int tp, dim3 grid, dim3 block, size_t lds, hipStream_t s, const HalfWalkParams& p) {
+  switch (tp) {
+    case 128:
+      return LaunchBig(HalfWalkKernel<NR, 128>, grid, block, lds, s, p);
+    case 64:
+      return LaunchBig(HalfWalkKernel<NR, 64>, grid, block, lds, s, p);
+    case 32:
+      return LaunchBig(HalfWalkKernel<NR, 32>, grid, block, lds, s, p);
+    case 16:
+      return LaunchBig(HalfWalkKernel<NR, 16>, grid, block, lds, s, p);
+    default:
+      return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace
+
+hipError_t LaunchHalfWalk(int nrows, int tile_pos, int threads, const HalfWalkParams& p, hipStream_t stream) {
+  if (p.P == 0 || p.n_groups == 0) return hipSuccess;
+  const size_t lds = (size_t)(p.K + 1) * tile_pos * 2;
+  if (lds > (size_t)kMaxLdsBytes || threads < tile_pos || threads % 64 != 0 || p.slices < 1) return hipErrorInvalidValue;
+  HalfWalkParams q = p;
+  q.tiles = (int)((p.P + tile_pos - 1) / tile_pos);
+  dim3 grid(8u * (uint32_t)q.slices * (((uint32_t)q.tiles + 7) / 8)), block(threads);
+  return nrows == 2 ? ByTile<2>(tile_pos, grid, block, lds, stream, q) : ByTile<1>(tile_pos, grid, block, lds, stream, q);
+}
+
+}  // namespace pl

@@ -78,6 +78,47 @@ pl::DevAct ToDevAct(const pl_activation& a) {
 
 int CeilDiv(int a, int b) { return (a + b - 1) / b; }
 
+// double (or float, which widens exactly) -> IEEE binary16 bit pattern with
+// one rounding to nearest even (what the reference's fp32_to_fp16 and
+// static_cast<float16_t> do).
+uint16_t HalfBits(double f) {
+  uint64_t u;
+  std::memcpy(&u, &f, 8);
+  const uint16_t sign = static_cast<uint16_t>((u >> 48) & 0x8000u);
+  const uint64_t a = u & 0x7fffffffffffffffull;
+  if (a > 0x7ff0000000000000ull) return static_cast<uint16_t>(sign | 0x7e00u);  // NaN
+  const double mag = std::fabs(f);
+  if (mag >= 65520.0) return static_cast<uint16_t>(sign | 0x7c00u);  // rounds to infinity
+  if (mag < 2.9802322387695312e-08) return sign;                     // < 2^-25 rounds to zero
+  const int e = static_cast<int>(a >> 52) - 1023;                    // unbiased (mag is a normal double here)
+  const uint64_t m = (a & 0xfffffffffffffull) | 0x10000000000000ull;  // 53-bit significand
+  // keep 10 fraction bits (fewer for subnormal results)
+  const int shift = e >= -14 ? 42 : 42 + (-14 - e);
+  const uint64_t kept = m >> shift, rest = m & ((1ull << shift) - 1ull), half = 1ull << (shift - 1);
+  const uint32_t r = static_cast<uint32_t>(kept + ((rest > half || (rest == half && (kept & 1ull))) ? 1ull : 0ull));
+  if (e >= -14) {
+    // r carries the implicit bit at position 10: adding it to the exponent
+    // field below also handles the carry out of the fraction
+    return static_cast<uint16_t>(sign | ((static_cast<uint32_t>(e + 14) << 10) + r));
+  }
+  return static_cast<uint16_t>(sign | r);  // subnormal; r == 1024 is the smallest normal number
+}
+
+pl::DevActH ToDevActH(const pl_activation& a) {
+  pl::DevActH d{};
+  d.type = a.type;
+  if (a.type == PL_ACT_RELU6) d.alpha = HalfBits(a.relu6_coef);
+  if (a.type == PL_ACT_LEAKY_RELU) d.alpha = HalfBits(a.leaky_alpha);
+  if (a.type == PL_ACT_HARD_SWISH) {
+    // (float16_t)(1.0 / scale): formed in double and narrowed once
+    // (lite/backends/arm/math/fp16/sparse_conv_fp16.cc:1318-1322)
+    d.hs_offset = HalfBits(a.hs_offset);
+    d.hs_inv_scale = HalfBits(1.0 / static_cast<double>(a.hs_scale));
+    d.hs_threshold = HalfBits(a.hs_threshold);
+  }
+  return d;
+}
+
 }  // namespace
 
 struct pl_sparse_conv_handle {
@@ -99,6 +140,10 @@ struct pl_sparse_conv_handle {
   DevBuf cw_desc, cw_idx, cw_wts;
   int cw_chunks = 0, cw_slices = 0;
   int walk_chunked = 1;  // 0 never, 1 when the problem is large enough, 2 whenever the shape allows
+  // half-precision row walk
+  bool half = false;
+  pl::DevActH act_h{};
+  DevBuf hw_kidx, hw_wts, hw_bias;
   // block MFMA
   int row_blocks = 0, ksteps = 0, kmask_words = 1;
   int64_t blocks_present = 0;
@@ -112,7 +157,7 @@ struct pl_sparse_conv_handle {
   int padded_rows = 0;
 
   int64_t DeviceBytes() const {
-    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + cw_desc.bytes + cw_idx.bytes + cw_wts.bytes + wblocks.bytes + kmask.bytes + scale.bytes + bias.bytes);
+    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + cw_desc.bytes + cw_idx.bytes + cw_wts.bytes + hw_kidx.bytes + hw_wts.bytes + hw_bias.bytes + wblocks.bytes + kmask.bytes + scale.bytes + bias.bytes);
   }
 };
 
@@ -182,6 +227,50 @@ int BuildRowWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
   if (e == hipSuccess) e = h->kidx.Upload(kidx.data(), kidx.size() * sizeof(uint32_t));
   if (e == hipSuccess) e = h->wts.Upload(wts.data(), wts.size() * sizeof(uint32_t));
   if (e != hipSuccess) return FailHip(e, "uploading the row-walk index");
+  return PL_OK;
+}
+
+// Device-side form for the half-precision walk: groups as for the plain walk,
+// per entry the channel and the weights of both rows as binary16 in one
+// dword; lists padded to kWalkBatch with zero-weight entries that read the
+// tile's zero row (index ic).
+int BuildHalfWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
+  std::vector<pl::DevGroup> groups;
+  std::vector<uint32_t> kidx, wts;
+  for (const pl::RowGroup& g : L.groups) {
+    pl::DevGroup d;
+    d.row0 = g.row0;
+    d.nrows = g.nrows;
+    d.first = static_cast<uint32_t>(kidx.size());
+    for (uint32_t j = 0; j < g.count; ++j) {
+      float w0, w1 = 0.f;
+      std::memcpy(&w0, &L.w0[g.first + j], 4);
+      if (g.nrows == 2) std::memcpy(&w1, &L.w1[g.first + j], 4);
+      kidx.push_back(L.ic_index[g.first + j]);
+      wts.push_back(static_cast<uint32_t>(HalfBits(w0)) | (static_cast<uint32_t>(HalfBits(w1)) << 16));
+    }
+    while ((kidx.size() - d.first) % pl::kWalkBatch != 0) {
+      kidx.push_back(static_cast<uint32_t>(L.ic));
+      wts.push_back(0u);
+    }
+    d.count = static_cast<uint32_t>(kidx.size()) - d.first;
+    groups.push_back(d);
+  }
+  h->n_groups = static_cast<int>(groups.size());
+  hipError_t e = h->groups.Upload(groups.data(), groups.size() * sizeof(pl::DevGroup));
+  if (e == hipSuccess) e = h->hw_kidx.Upload(kidx.empty() ? nullptr : kidx.data(), kidx.size() * sizeof(uint32_t));
+  if (e == hipSuccess) e = h->hw_wts.Upload(wts.empty() ? nullptr : wts.data(), wts.size() * sizeof(uint32_t));
+  if (e != hipSuccess) return FailHip(e, "uploading the half-precision index");
+  return PL_OK;
+}
+
+int UploadHalfBias(pl_sparse_conv_handle* h, const float* bias) {
+  if (!bias) return PL_OK;
+  std::vector<uint16_t> b(static_cast<size_t>(h->oc));
+  for (int i = 0; i < h->oc; ++i) b[i] = HalfBits(bias[i]);
+  const hipError_t e = h->hw_bias.Upload(b.data(), b.size() * sizeof(uint16_t));
+  if (e != hipSuccess) return FailHip(e, "uploading biases");
+  h->has_bias = true;
   return PL_OK;
 }
 
@@ -354,11 +443,12 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   if (!desc || !out_handle) return Fail(PL_ERR_BAD_ARG, "null argument");
   *out_handle = nullptr;
   if (desc->struct_size != sizeof(pl_sparse_conv_desc)) return Fail(PL_ERR_BAD_ARG, "pl_sparse_conv_desc size mismatch (%u vs %zu)", desc->struct_size, sizeof(pl_sparse_conv_desc));
-  if (desc->kind < PL_KIND_FP32 || desc->kind > PL_KIND_INT8_ACC32) return Fail(PL_ERR_BAD_ARG, "unknown kind %d", desc->kind);
+  if (desc->kind < PL_KIND_FP32 || desc->kind > PL_KIND_FP16) return Fail(PL_ERR_BAD_ARG, "unknown kind %d", desc->kind);
   if (desc->algo < PL_ALGO_AUTO || desc->algo > PL_ALGO_BLOCK_MFMA) return Fail(PL_ERR_BAD_ARG, "unknown algo %d", desc->algo);
   if (desc->oc <= 0 || desc->ic <= 0 || desc->im_size <= 0) return Fail(PL_ERR_BAD_ARG, "oc, ic and im_size must be positive");
   if (!desc->oc_nonzeros || (desc->n_weights > 0 && (!desc->nonzero_weights || !desc->diffs))) return Fail(PL_ERR_BAD_ARG, "null weight tensors");
-  const bool int8 = desc->kind != PL_KIND_FP32;
+  const bool half = desc->kind == PL_KIND_FP16;
+  const bool int8 = desc->kind != PL_KIND_FP32 && !half;
   if (int8 && desc->kind != PL_KIND_INT8_ACC32 && !desc->scale) return Fail(PL_ERR_BAD_ARG, "int8 kinds need per-channel scales");
   if (desc->algo == PL_ALGO_BLOCK_MFMA && !int8) return Fail(PL_ERR_UNSUPPORTED, "the block MFMA algorithm exists for int8 only");
 
@@ -396,8 +486,10 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   h->oc = desc->oc;
   h->ic = desc->ic;
   h->int8 = int8;
+  h->half = half;
   h->semi = desc->flag_semi != 0;
   h->act = ToDevAct(desc->act);
+  h->act_h = ToDevActH(desc->act);
   h->nnz = L.nnz;
   h->stored = L.stored_weights;
   h->entries = static_cast<int64_t>(L.ic_index.size());
@@ -405,6 +497,22 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
 
   int algo = desc->algo;
   if (algo == PL_ALGO_AUTO) algo = int8 ? PL_ALGO_BLOCK_MFMA : PL_ALGO_ROW_WALK;
+  if (half) {
+    // half precision: its own walk; a tile of 16 positions must fit LDS
+    if (static_cast<size_t>(desc->ic + 1) * 16 * 2 > static_cast<size_t>(pl::kMaxLdsBytes)) {
+      delete h;
+      return Fail(PL_ERR_UNSUPPORTED, "ic = %d does not fit an LDS tile", desc->ic);
+    }
+    h->algo = PL_ALGO_ROW_WALK;
+    int hrc = BuildHalfWalk(L, h);
+    if (hrc == PL_OK) hrc = UploadHalfBias(h, desc->bias);
+    if (hrc != PL_OK) {
+      delete h;
+      return hrc;
+    }
+    *out_handle = h;
+    return PL_OK;
+  }
   if (algo == PL_ALGO_ROW_WALK) {
     const size_t row_bytes = static_cast<size_t>(int8 ? CeilDiv(desc->ic, 4) : desc->ic) * 4;
     if (row_bytes * 16 > static_cast<size_t>(pl::kMaxLdsBytes)) {
@@ -454,7 +562,37 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
   const int vec = (im_size % 4 == 0) && (reinterpret_cast<uintptr_t>(x_dev) % 16 == 0) && (reinterpret_cast<uintptr_t>(out_dev) % 16 == 0);
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipError_t e;
-  if (h->algo == PL_ALGO_BLOCK_MFMA) {
+  if (h->half) {
+    pl::HalfWalkParams p{};
+    p.x = static_cast<const uint16_t*>(x_dev);
+    p.out = static_cast<uint16_t*>(out_dev);
+    p.groups = static_cast<const pl::DevGroup*>(h->groups.ptr);
+    p.kidx = static_cast<const uint32_t*>(h->hw_kidx.ptr);
+    p.wts = static_cast<const uint32_t*>(h->hw_wts.ptr);
+    p.bias = h->has_bias ? static_cast<const uint16_t*>(h->hw_bias.ptr) : nullptr;
+    p.n_groups = h->n_groups;
+    p.M = h->oc;
+    p.K = h->ic;
+    p.hw = im_size;
+    p.P = P;
+    p.pair = (im_size % 2 == 0) && (reinterpret_cast<uintptr_t>(x_dev) % 4 == 0) && (reinterpret_cast<uintptr_t>(out_dev) % 4 == 0);
+    p.act = h->act_h;
+    // widest tile of which two fit a CU, else the widest that fits at all
+    const size_t row_bytes = static_cast<size_t>(h->ic + 1) * 2;
+    int tp = 128;
+    while (tp > 16 && row_bytes * tp > 64 * 1024) tp >>= 1;
+    if (row_bytes * tp > 64 * 1024) {
+      tp = 128;
+      while (tp > 16 && row_bytes * tp > static_cast<size_t>(pl::kMaxLdsBytes)) tp >>= 1;
+    }
+    const int threads = row_bytes * tp > 32 * 1024 ? 512 : 256;
+    const uint32_t tiles = (P + tp - 1) / tp;
+    int slices = static_cast<int>((1024 + tiles - 1) / tiles);
+    slices = std::max(1, std::min(slices, std::max(1, h->n_groups / (threads / 64))));
+    p.groups_per_slice = CeilDiv(h->n_groups, slices);
+    p.slices = CeilDiv(h->n_groups, p.groups_per_slice);
+    e = pl::LaunchHalfWalk(h->semi ? 2 : 1, tp, threads, p, s);
+  } else if (h->algo == PL_ALGO_BLOCK_MFMA) {
     pl::MfmaParams p{};
     p.x = static_cast<const int8_t*>(x_dev);
     p.out = out_dev;
@@ -581,14 +719,23 @@ int pl_sparse_conv_get_info(const pl_sparse_conv_handle* h, pl_sparse_conv_info*
 
 int pl_sparse_conv_set_epilogue(pl_sparse_conv_handle* h, const float* scale, const float* bias, const pl_activation* act) {
   if (!h) return Fail(PL_ERR_BAD_ARG, "null handle");
-  if (scale && !h->int8) return Fail(PL_ERR_BAD_ARG, "fp32 kernels take no scales");
-  int rc = UploadEpilogue(h, scale, bias);
+  if (scale && !h->int8) return Fail(PL_ERR_BAD_ARG, "floating-point kernels take no scales");
+  int rc = h->half ? UploadHalfBias(h, bias) : UploadEpilogue(h, scale, bias);
   if (rc != PL_OK) return rc;
-  if (act) h->act = ToDevAct(*act);
+  if (act) {
+    h->act = ToDevAct(*act);
+    h->act_h = ToDevActH(*act);
+  }
   return PL_OK;
 }
 
 void pl_sparse_conv_destroy(pl_sparse_conv_handle* h) { delete h; }
+
+int pl_fp32_to_fp16(const float* in, uint16_t* out, int64_t n) {
+  if (n < 0 || (n > 0 && (!in || !out))) return Fail(PL_ERR_BAD_ARG, "bad conversion arguments");
+  for (int64_t i = 0; i < n; ++i) out[i] = HalfBits(in[i]);
+  return PL_OK;
+}
 
 namespace {
 int CheckCalibArgs(const void* x, const void* out, int64_t n, float scale) {

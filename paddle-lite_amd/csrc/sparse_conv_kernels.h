@@ -95,6 +95,36 @@ struct ChunkWalkParams {
 // Needs hw % 4 == 0 and 16-byte aligned x / out.
 hipError_t LaunchChunkWalk(int nrows, const ChunkWalkParams& p, hipStream_t stream);
 
+// Half-precision row walk (fp16_walk_kernels.hip).  Activation constants as
+// binary16 bit patterns.
+struct DevActH {
+  int type;
+  uint16_t alpha;         // relu6 bound or leaky slope
+  uint16_t hs_offset;
+  uint16_t hs_inv_scale;  // (half)(1.0 / scale)
+  uint16_t hs_threshold;
+};
+
+struct HalfWalkParams {
+  const uint16_t* x;
+  uint16_t* out;
+  const DevGroup* groups;
+  const uint32_t* kidx;   // per entry: input channel (K = the tile's zero row)
+  const uint32_t* wts;    // per entry: weight of row 0 in the low half, of row 1 in the high half
+  const uint16_t* bias;   // may be null
+  int n_groups;
+  int groups_per_slice;
+  int M, K;
+  int hw;
+  uint32_t P;
+  int pair;               // 1: hw even and x / out 4-byte aligned
+  DevActH act;
+  int tiles, slices;      // tiles filled in by the launcher
+};
+
+// tile_pos: 128, 64, 32 or 16 positions with (K + 1) * tile_pos * 2 bytes of LDS.
+hipError_t LaunchHalfWalk(int nrows, int tile_pos, int threads, const HalfWalkParams& p, hipStream_t stream);
+
 // Block MFMA SpMM (int8): dense 32x32 weight blocks pre-arranged in operand
 // order, empty blocks skipped through a per-row-block bit mask.
 struct MfmaParams {

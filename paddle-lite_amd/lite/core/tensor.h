@@ -86,6 +86,8 @@ template <> struct PrecisionOf<int32_t> { static constexpr PrecisionType value =
 template <> struct PrecisionOf<uint32_t> { static constexpr PrecisionType value = PrecisionType::kInt32; };
 template <> struct PrecisionOf<int64_t> { static constexpr PrecisionType value = PrecisionType::kInt64; };
 template <> struct PrecisionOf<uint8_t> { static constexpr PrecisionType value = PrecisionType::kUInt8; };
+// binary16 values travel as their bit patterns on the host side
+template <> struct PrecisionOf<uint16_t> { static constexpr PrecisionType value = PrecisionType::kFP16; };
 
 using LoD = std::vector<std::vector<uint64_t>>;
 

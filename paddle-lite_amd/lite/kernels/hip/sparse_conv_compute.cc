@@ -119,6 +119,16 @@ void SparseConvCompute<PRECISION(kInt8), PRECISION(kInt8)>::PrepareForRun() {
   Upload(PL_KIND_INT8_INT8);
 }
 
+// Half precision: the reference converts the fp32 weights and bias in place
+// and halves the byte offsets
+// (lite/kernels/arm/sparse_conv_compute.cc:270-304); here the library does
+// the conversion when it builds its device-side form, the host tensors stay
+// as the pass wrote them.
+template <>
+void SparseConvCompute<PRECISION(kFP16), PRECISION(kFP16)>::PrepareForRun() {
+  Upload(PL_KIND_FP16);
+}
+
 template <PrecisionType P, PrecisionType O>
 void SparseConvCompute<P, O>::Run() {
   auto& param = this->template Param<param_t>();
@@ -130,7 +140,8 @@ void SparseConvCompute<P, O>::Run() {
   const int batch = static_cast<int>(xd[0]);
   const int im_size = static_cast<int>(od[2] * od[3]);
   void* out = (O == PRECISION(kFloat)) ? static_cast<void*>(param.output->template mutable_data<float>(TargetType::kHIP))
-                                       : static_cast<void*>(param.output->template mutable_data<int8_t>(TargetType::kHIP));
+              : (O == PRECISION(kFP16)) ? static_cast<void*>(param.output->template mutable_data<uint16_t>(TargetType::kHIP))
+                                        : static_cast<void*>(param.output->template mutable_data<int8_t>(TargetType::kHIP));
   const int rc = pl_sparse_conv_run(handle_, param.x->raw_data(), out, batch, im_size, ctx.stream());
   if (rc != PL_OK) LOG(FATAL) << "pl_sparse_conv_run failed (" << rc << "): " << pl_last_error();
 }
@@ -138,6 +149,7 @@ void SparseConvCompute<P, O>::Run() {
 template class SparseConvCompute<PRECISION(kFloat), PRECISION(kFloat)>;
 template class SparseConvCompute<PRECISION(kInt8), PRECISION(kFloat)>;
 template class SparseConvCompute<PRECISION(kInt8), PRECISION(kInt8)>;
+template class SparseConvCompute<PRECISION(kFP16), PRECISION(kFP16)>;
 
 }  // namespace hip
 }  // namespace kernels
@@ -177,4 +189,16 @@ REGISTER_LITE_KERNEL(sparse_conv2d, kHIP, kInt8, kNCHW, SparseConvHipInt8Int8, i
     .BindInput("Diffs", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost), PRECISION(kInt32))})
     .BindInput("Bias", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost), PRECISION(kFloat))})
     .BindOutput("Output", {paddle::lite::LiteType::GetTensorTy(TARGET(kHIP), PRECISION(kInt8))})
+    .Finalize();
+
+// lite/kernels/arm/sparse_conv_compute.cc:365-381 (under ENABLE_ARM_FP16).  The
+// weight tensors and the bias are the fp32 ones of the pass on the host.
+typedef paddle::lite::kernels::hip::SparseConvCompute<PRECISION(kFP16), PRECISION(kFP16)> SparseConvHipFp16;
+REGISTER_LITE_KERNEL(sparse_conv2d, kHIP, kFP16, kNCHW, SparseConvHipFp16, def)
+    .BindInput("Input", {paddle::lite::LiteType::GetTensorTy(TARGET(kHIP), PRECISION(kFP16))})
+    .BindInput("NonZeroWeights", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost), PRECISION(kFloat))})
+    .BindInput("OcNonZeros", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost), PRECISION(kInt32))})
+    .BindInput("Diffs", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost), PRECISION(kInt32))})
+    .BindInput("Bias", {paddle::lite::LiteType::GetTensorTy(TARGET(kHost), PRECISION(kFloat))})
+    .BindOutput("Output", {paddle::lite::LiteType::GetTensorTy(TARGET(kHIP), PRECISION(kFP16))})
     .Finalize();

@@ -128,7 +128,8 @@ class SparseConvParam(object):
         self.bit_length = 8
 
 
-_KINDS = {("float32", "float32"): capi.KIND_FP32, ("int8", "float32"): capi.KIND_INT8_FP32, ("int8", "int8"): capi.KIND_INT8_INT8, ("int8", "int32"): capi.KIND_INT8_ACC32}
+_KINDS = {("float32", "float32"): capi.KIND_FP32, ("int8", "float32"): capi.KIND_INT8_FP32, ("int8", "int8"): capi.KIND_INT8_INT8, ("int8", "int32"): capi.KIND_INT8_ACC32,
+          ("float16", "float16"): capi.KIND_FP16}
 
 
 class SparseConvKernel(object):
@@ -137,7 +138,10 @@ class SparseConvKernel(object):
     precision/out_precision select the registration: ("float32","float32") =
     def, ("int8","float32") = int8_fp32_out, ("int8","int8") = int8_int8_out
     (reference: lite/kernels/arm/sparse_conv_compute.cc:369-430).
-    ("int8","int32") exposes the raw accumulators for verification.
+    ("int8","int32") exposes the raw accumulators for verification;
+    ("float16","float16") is the half-precision kernel
+    (sparse_conv_compute.cc:270-356): fp32 sparse tensors and bias in the
+    parameter, converted to fp16 at PrepareForRun, fp16 activations.
 
     reference_quirks=True reproduces what the reference computes through its
     kernel class for int8 output: the leaky slope is divided by output_scale
@@ -168,7 +172,7 @@ class SparseConvKernel(object):
         act = p.activation_param.copy()
         bias = p.bias
         scale = None
-        if self.kind != capi.KIND_FP32:
+        if self.kind not in (capi.KIND_FP32, capi.KIND_FP16):
             ws = list(p.weight_scale)
             if len(ws) != 1 and len(ws) != oc:
                 raise ValueError("weights scale size must equal to filter size")
@@ -243,11 +247,11 @@ class SparseConvKernel(object):
             raise RuntimeError("PrepareForRun has not been called")
         if not x.is_cuda or not x.is_contiguous():
             raise ValueError("x must be a contiguous device tensor")
-        want_in = torch.float32 if self.kind == capi.KIND_FP32 else torch.int8
+        want_in = {capi.KIND_FP32: torch.float32, capi.KIND_FP16: torch.float16}.get(self.kind, torch.int8)
         if x.dtype != want_in or x.dim() != 4 or x.shape[1] != self.param.weights.ic:
             raise ValueError("x must be %s NCHW with %d channels" % (want_in, self.param.weights.ic))
         n, _, hh, ww = x.shape
-        odt = {capi.KIND_FP32: torch.float32, capi.KIND_INT8_FP32: torch.float32, capi.KIND_INT8_INT8: torch.int8, capi.KIND_INT8_ACC32: torch.int32}[self.kind]
+        odt = {capi.KIND_FP32: torch.float32, capi.KIND_INT8_FP32: torch.float32, capi.KIND_INT8_INT8: torch.int8, capi.KIND_INT8_ACC32: torch.int32, capi.KIND_FP16: torch.float16}[self.kind]
         # output shape as SparseConvOp::InferShapeImpl for 1x1 / stride 1 / pad 0
         # (reference: lite/operators/sparse_conv_op.cc:46-65)
         shape = (n, self.param.weights.oc, hh, ww)

@@ -45,7 +45,7 @@ class Case(object):
     def algorithmic_bytes(self, weights):
         """Input + output + compressed weights, each once."""
         oc, ic = self.dense.shape
-        out_item = {capi.KIND_FP32: 4, capi.KIND_INT8_FP32: 4, capi.KIND_INT8_INT8: 1, capi.KIND_INT8_ACC32: 4}[self.kind]
+        out_item = {capi.KIND_FP32: 4, capi.KIND_INT8_FP32: 4, capi.KIND_INT8_INT8: 1, capi.KIND_INT8_ACC32: 4, capi.KIND_FP16: 2}[self.kind]
         p = self.batch * self.im_size
         wbytes = weights.nonzero_weights.nbytes + weights.diffs.nbytes + 12 * oc
         return float(self.x.nbytes + p * oc * out_item + wbytes)

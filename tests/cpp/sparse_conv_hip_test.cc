@@ -424,6 +424,65 @@ static void CalibChain(bool run_on_device) {
   EXPECT(want_q[2] == 127 && want_q[3] == -127);
 }
 
+// The half-precision registration: fp32 sparse tensors from the pass, fp16
+// activations on the device, checked against the oracle's binary16 walker.
+static void HalfPrecision(bool run_on_device) {
+  std::printf("half precision\n");
+  std::fflush(stdout);
+  auto regs = KernelRegistry::Global().Create("sparse_conv2d", TARGET(kHIP), PRECISION(kFP16), DATALAYOUT(kNCHW));
+  EXPECT(regs.size() == 1 && regs.front()->alias() == "def");
+  if (!run_on_device) return;
+  Problem p{2, 70, 33, 6, 6, 0.7f, true, false, false, true, "hard_swish", 21};
+  Scope scope;
+  std::vector<float> ws;
+  float is = 1.f, os = 1.f;
+  std::vector<OpInfo> ops{MakeConv(p, &scope, &ws, &is, &os)};
+  const int hw = p.h * p.w;
+  const int64_t xn = static_cast<int64_t>(p.batch) * p.ic * hw;
+  // fp16 copy of the input
+  const float* xf = scope.FindMutableTensor("x")->data<float>();
+  Tensor* xh = scope.NewTensor("xh");
+  xh->Resize({p.batch, p.ic, p.h, p.w});
+  uint16_t* xhd = xh->mutable_data<uint16_t>(TargetType::kHost);
+  plo_fp32_to_fp16(xf, xhd, xn);
+  mir::SparseConvDetectPass pass;
+  pass.SetSparseThreshold(0.5f);
+  EXPECT(pass.Apply(&ops, &scope) == 1);
+  // oracle on the tensors the pass made
+  const Tensor* nzw = scope.FindMutableTensor("conv_w_nonzeros_output");
+  const Tensor* ocn = scope.FindMutableTensor("conv_w_oc_nonzeros");
+  const Tensor* dif = scope.FindMutableTensor("conv_w_ic_diffs");
+  EXPECT(nzw && ocn && dif);
+  if (!(nzw && ocn && dif)) return;
+  std::vector<uint16_t> w16(nzw->numel()), b16(p.oc), want(static_cast<size_t>(p.batch) * p.oc * hw);
+  plo_fp32_to_fp16(nzw->data<float>(), w16.data(), nzw->numel());
+  plo_fp32_to_fp16(scope.FindMutableTensor("conv_b")->data<float>(), b16.data(), p.oc);
+  plo_act act{10, 6.f, 0.1f, 6.f, 3.f, 6.f};
+  plo_sparse_conv_fp16(w16.data(), xhd, dif->data<int32_t>(), ocn->data<uint32_t>(), b16.data(), want.data(), p.batch, p.oc, p.ic, hw, ops[0].GetAttr<int>("first_ic"), ops[0].GetAttr<int>("flag_semi"), &act);
+
+  OpInfo h2d("io_copy");
+  h2d.SetInput("Input", {"xh"});
+  h2d.SetOutput("Out", {"xh_dev"});
+  auto copy_op = LiteOpRegistry::Global().Create("io_copy");
+  EXPECT(copy_op->Attach(h2d, &scope) && copy_op->InferShape());
+  auto ck = copy_op->CreateKernels({paddle::lite_api::Place(TARGET(kHIP), PRECISION(kAny), DATALAYOUT(kAny))}, "io_copy/host_to_device");
+  EXPECT(ck.size() == 1);
+  ck[0]->Launch();
+  ops[0].SetInput("Input", {"xh_dev"});
+  auto op = LiteOpRegistry::Global().Create("sparse_conv2d");
+  EXPECT(op->Attach(ops[0], &scope) && op->CheckShape() && op->InferShape());
+  auto ks = op->CreateKernels({paddle::lite_api::Place(TARGET(kHIP), PRECISION(kFP16), DATALAYOUT(kNCHW))}, "sparse_conv2d/def");
+  EXPECT(ks.size() == 1);
+  ks[0]->Launch();
+  ks[0]->mutable_context_as<HIPContext>()->Sync();
+  Tensor y_host;
+  y_host.CopyDataFrom(*scope.FindMutableTensor("y"), TargetType::kHost);
+  const uint16_t* got = static_cast<const uint16_t*>(y_host.raw_data());
+  size_t bad = 0;
+  for (size_t i = 0; i < want.size(); ++i) bad += (got[i] != want[i]) && !(((got[i] | want[i]) & 0x7fffu) == 0);  // zeros of either sign agree
+  EXPECT(bad == 0);
+}
+
 // Three quantised 1x1 convolutions in a row, fed and fetched as fp32 on the
 // host: detect pass -> output-type rule / calib / io_copy insertion ->
 // program run on the device, against the oracle's chain
@@ -563,6 +622,7 @@ int main(int argc, char** argv) {
   for (const Problem& p : problems) RunProblem(p, gpu);
   CalibChain(gpu);
   Int8Chain(gpu);
+  HalfPrecision(gpu);
   std::printf("%s: %d failure(s)\n", gpu ? "gpu" : "cpu", g_failures);
   return g_failures ? 1 : 0;
 }

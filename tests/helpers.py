@@ -23,7 +23,7 @@ def merged_for_oracle(case, quirks=False):
     here with explicit numpy float32 arithmetic (not through the package)."""
     act = case.act.copy()
     bias = case.bias
-    if case.kind == capi.KIND_FP32:
+    if case.kind in (capi.KIND_FP32, capi.KIND_FP16):
         return None, bias, oracle_act(act)
     ws = np.asarray(case.weight_scale, np.float32)
     if ws.size == 1:
@@ -63,17 +63,19 @@ def run_oracle(case, packed=None, quirks=False, x=None):
     scale, bias, act = merged_for_oracle(case, quirks)
     if case.kind == capi.KIND_FP32:
         return O.sparse_conv_fp32(pk, x, bias, act)
+    if case.kind == capi.KIND_FP16:
+        return O.sparse_conv_fp16(pk, x, bias, act)
     if case.kind == capi.KIND_INT8_ACC32:
         return O.sparse_conv_int8_acc(pk, x)
     return O.sparse_conv_int8(pk, x, scale, bias, act, out_int8=(case.kind == capi.KIND_INT8_INT8))
 
 
-_PREC = {capi.KIND_FP32: ("float32", "float32"), capi.KIND_INT8_FP32: ("int8", "float32"), capi.KIND_INT8_INT8: ("int8", "int8"), capi.KIND_INT8_ACC32: ("int8", "int32")}
+_PREC = {capi.KIND_FP32: ("float32", "float32"), capi.KIND_INT8_FP32: ("int8", "float32"), capi.KIND_INT8_INT8: ("int8", "int8"), capi.KIND_INT8_ACC32: ("int8", "int32"), capi.KIND_FP16: ("float16", "float16")}
 
 
 def make_kernel(case, algo=capi.ALGO_AUTO, force_semi=None, quirks=False, im_size=None):
     weights = pla.detect_and_pack(case.dense, im_size or case.im_size, force_semi=force_semi)
-    param = pla.SparseConvParam(weights, bias=case.bias, activation_param=case.act, enable_int8=case.kind != capi.KIND_FP32, input_scale=case.input_scale,
+    param = pla.SparseConvParam(weights, bias=case.bias, activation_param=case.act, enable_int8=case.kind not in (capi.KIND_FP32, capi.KIND_FP16), input_scale=case.input_scale,
                                 weight_scale=case.weight_scale if case.weight_scale is not None else (), output_scale=case.output_scale)
     prec = _PREC[case.kind]
     k = pla.SparseConvKernel(param, prec[0], prec[1], algo=algo, reference_quirks=quirks)
@@ -93,6 +95,12 @@ def run_hip(case, algo=capi.ALGO_AUTO, force_semi=None, quirks=False, x=None, ke
 
 def assert_same(case, got, want, what=""):
     assert got.shape == want.shape and got.dtype == want.dtype, (what, got.shape, want.shape, got.dtype, want.dtype)
+    if case.kind == capi.KIND_FP16:
+        # fp16: the same sequence of half-precision instructions -> the same
+        # values (zeros compare equal whatever their sign)
+        bad = ~((got == want) | (np.isnan(got) & np.isnan(want)))
+        assert not bad.any(), "%s: %d of %d fp16 values differ, first %r vs %r" % (what, int(bad.sum()), got.size, got[bad][0], want[bad][0])
+        return
     if case.kind == capi.KIND_FP32:
         # fp32: 1e-5 relative (the reference's own tests allow 1e-4 / 5e-5)
         np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6, err_msg=what)

@@ -146,3 +146,15 @@ def test_bench_refuses_more_than_one_gpu():
     assert res.returncode != 0
     assert "one GPU" in res.stderr
     assert res.stdout.strip() == ""
+
+
+def test_host_fp16_conversion_matches_the_oracle():
+    import ctypes as C
+    from oracle import oracle as O
+
+    rng = np.random.default_rng(1)
+    f = np.concatenate([rng.standard_normal(100000).astype(np.float32) * np.float32(10.0) ** rng.integers(-8, 5, 100000).astype(np.float32),
+                        np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e-8, 5.96e-8, 2.98e-8, 2.9802322e-8, 2.9802326e-8, np.inf, -np.inf], np.float32)])
+    out = np.empty(f.size, np.uint16)
+    assert capi.lib().pl_fp32_to_fp16(f.ctypes.data, out.ctypes.data, f.size) == capi.PL_OK
+    assert np.array_equal(out, O.fp32_to_fp16(f).view(np.uint16))

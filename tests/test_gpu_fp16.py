@@ -1,0 +1,48 @@
+"""Half-precision sparse_conv2d on the GPU (through the C ABI) against the
+oracle's binary16 restatement: same values for every output (the kernel
+issues the same sequence of half-precision operations)."""
+import numpy as np
+import pytest
+
+from helpers import capi, workloads, pla, run_hip, run_oracle, oracle_pack, assert_same
+
+pytestmark = pytest.mark.gpu
+
+AP = pla.ActivationParam
+ACTS = {
+    "none": AP(),
+    "relu": AP("relu"),
+    "relu6": AP("relu6", Relu_clipped_coef=6.0),
+    "leaky": AP("leaky_relu", Leaky_relu_alpha=0.1),
+    "hswish": AP("hard_swish"),
+}
+# (batch, ic, oc, h, w): even and odd images, a single pixel, channel counts
+# off the batch-of-eight grid, more channels than one 128-position tile
+# holds, odd row counts for the semi layout's tail row
+SHAPES = [(2, 64, 64, 4, 4), (3, 37, 29, 7, 7), (1, 96, 48, 8, 6), (2, 130, 67, 5, 3), (1, 1, 1, 1, 1), (5, 8, 33, 1, 1), (1, 700, 40, 14, 14), (2, 256, 96, 28, 28)]
+
+
+def half_case(batch, ic, oc, h, w, sparsity, paired, act, seed):
+    c = workloads.make_fp32("t", batch, ic, oc, h, w, sparsity, paired, act, seed=seed)
+    c.kind = capi.KIND_FP16
+    c.x = c.x.astype(np.float16)
+    return c
+
+
+@pytest.mark.parametrize("act", sorted(ACTS))
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
+def test_fp16_same_values(shape, paired, act):
+    batch, ic, oc, h, w = shape
+    case = half_case(batch, ic, oc, h, w, 0.7, paired, ACTS[act], seed=ic + 5 * oc)
+    got = run_hip(case, capi.ALGO_AUTO, force_semi=paired)
+    want = run_oracle(case, oracle_pack(case, force_semi=paired))
+    assert got.dtype == np.float16
+    assert_same(case, got, want, "fp16 %s %s" % (act, shape))
+
+
+def test_fp16_no_bias_and_new_epilogue():
+    case = half_case(2, 48, 20, 6, 6, 0.6, False, ACTS["relu"], seed=3)
+    case.bias = None
+    got = run_hip(case)
+    assert_same(case, got, run_oracle(case), "fp16 without bias")
