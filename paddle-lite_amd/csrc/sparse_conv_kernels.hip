@@ -581,19 +581,40 @@ __device__ __forceinline__ float ActivateAny(float v, const DevAct& a) {
   return ActivateT<(ACT < 0 ? 0 : ACT)>(v, a);
 }
 
+// Scales and biases of the 16 output rows a lane finishes (row
+// 8*(r/4) + 4*(lane/32) + r%4 of the wavefront's row block), fetched ahead of
+// the multiply so that the epilogue does not start with a memory wait.
+struct RowConsts {
+  float s[16], b[16];
+};
+
+template <int OUT>
+__device__ __forceinline__ void LoadRowConsts(RowConsts& rc, const MfmaParams& p, int rb, int lane) {
+  if (OUT == kOutAcc32) return;
+  const int row_base = rb * 32 + 4 * (lane >> 5);
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    // four consecutive rows: one 16-byte load each (arrays are padded to 32 * row_blocks)
+    const float4 sv = *reinterpret_cast<const float4*>(p.scale + row_base + 8 * g);
+    const float4 bv = *reinterpret_cast<const float4*>(p.bias + row_base + 8 * g);
+    rc.s[4 * g] = sv.x, rc.s[4 * g + 1] = sv.y, rc.s[4 * g + 2] = sv.z, rc.s[4 * g + 3] = sv.w;
+    rc.b[4 * g] = bv.x, rc.b[4 * g + 1] = bv.y, rc.b[4 * g + 2] = bv.z, rc.b[4 * g + 3] = bv.w;
+  }
+}
+
 // int8 output of a full tile inside one image: the wavefront's 32 rows x 128
 // positions are packed, written to its own 4 KB of LDS as [row][128 bytes]
 // and stored as 16 bytes per lane (8 rows x 128 contiguous bytes per
 // instruction) instead of one dword per lane.  `stage` is private to the
 // wavefront.
 template <int ACT>
-__device__ __forceinline__ void MfmaEpilogueI8Wide(const MfmaParams& p, const v16i (&acc)[4], int rb, int lane, uint32_t n, uint32_t pp, uint32_t* stage) {
+__device__ __forceinline__ void MfmaEpilogueI8Wide(const MfmaParams& p, const v16i (&acc)[4], const RowConsts& rc, int rb, int lane, uint32_t n, uint32_t pp, uint32_t* stage) {
   const int row_base = rb * 32 + 4 * (lane >> 5);
   const int j = lane & 31;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int ro = 8 * (r >> 2) + (r & 3);
-    const float s = p.scale[row_base + ro], b = p.bias[row_base + ro];
+    const float s = rc.s[r], b = rc.b[r];
     int q[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) q[c] = ActQuantI8<ACT>(__builtin_fmaf((float)acc[c][r], s, b), p.act);
@@ -615,7 +636,7 @@ __device__ __forceinline__ void MfmaEpilogueI8Wide(const MfmaParams& p, const v1
 // the lane's quad.  WHOLE: the quad has all four positions and the row block
 // all 32 rows (the common case, kept free of per-row conditions).
 template <int OUT, int ACT, bool WHOLE>
-__device__ __forceinline__ void MfmaEpilogueRows(const MfmaParams& p, const v16i (&acc)[4], int row_base, char* lane_base, int valid) {
+__device__ __forceinline__ void MfmaEpilogueRows(const MfmaParams& p, const v16i (&acc)[4], const RowConsts& rc, int row_base, char* lane_base, int valid) {
   constexpr uint32_t kElem = OUT == kOutI8 ? 1u : 4u;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
@@ -627,7 +648,7 @@ __device__ __forceinline__ void MfmaEpilogueRows(const MfmaParams& p, const v16i
 #pragma unroll
     for (int c = 0; c < 4; ++c) q[c] = acc[c][r];
     if (OUT != kOutAcc32) {
-      const float s = p.scale[row_base + ro], b = p.bias[row_base + ro];
+      const float s = rc.s[r], b = rc.b[r];
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         const float t = __builtin_fmaf((float)q[c], s, b);
@@ -658,7 +679,7 @@ __device__ __forceinline__ void MfmaEpilogueRows(const MfmaParams& p, const v16i
 }
 
 template <int OUT, int ACT>
-__device__ __forceinline__ void MfmaEpilogue(const MfmaParams& p, const v16i (&acc)[4], int rb, int lane, const QuadInfo& qi) {
+__device__ __forceinline__ void MfmaEpilogue(const MfmaParams& p, const v16i (&acc)[4], const RowConsts& rc, int rb, int lane, const QuadInfo& qi) {
   if (qi.valid == 0) return;
   const int row_base = rb * 32 + 4 * (lane >> 5);
   constexpr uint32_t kElem = OUT == kOutI8 ? 1u : 4u;
@@ -667,16 +688,16 @@ __device__ __forceinline__ void MfmaEpilogue(const MfmaParams& p, const v16i (&a
   const size_t lane_off = (((size_t)qi.n * p.M + row_base) * p.hw + qi.pp) * kElem;
   char* lane_base = p.small ? static_cast<char*>(p.out) + (uint32_t)lane_off : static_cast<char*>(p.out) + lane_off;
   if (rb * 32 + 32 <= p.M && (p.quad_aligned || qi.valid == 4)) {
-    MfmaEpilogueRows<OUT, ACT, true>(p, acc, row_base, lane_base, 4);
+    MfmaEpilogueRows<OUT, ACT, true>(p, acc, rc, row_base, lane_base, 4);
   } else {
-    MfmaEpilogueRows<OUT, ACT, false>(p, acc, row_base, lane_base, qi.valid);
+    MfmaEpilogueRows<OUT, ACT, false>(p, acc, rc, row_base, lane_base, qi.valid);
   }
 }
 
 // Epilogue of one (tile, row block) pair.  `stage` is the workgroup's LDS
 // behind the activation tiles (4 KB per wavefront when p.i8_stage is set).
 template <int OUT, int ACT, bool VEC>
-__device__ __forceinline__ void MfmaFinish(const MfmaParams& p, uint32_t* stage, const v16i (&acc)[4], int rb, int lane, uint32_t quad0, int J) {
+__device__ __forceinline__ void MfmaFinish(const MfmaParams& p, uint32_t* stage, const v16i (&acc)[4], const RowConsts& rc, int rb, int lane, uint32_t quad0, int J) {
   if ((lane & 31) >= J) return;
   const QuadInfo qo = LocateQuad(p, quad0 + (uint32_t)(lane & 31));
   if (OUT == kOutI8 && VEC) {
@@ -685,11 +706,11 @@ __device__ __forceinline__ void MfmaFinish(const MfmaParams& p, uint32_t* stage,
     const QuadInfo q0 = LocateQuad(p, quad0);
     const bool wide = p.i8_stage && J == 32 && p.small && rb * 32 + 32 <= p.M && (p.hw & 15) == 0 && quad0 + 32u <= p.total_quads && q0.pp + 128u <= (uint32_t)p.hw;
     if (wide) {
-      MfmaEpilogueI8Wide<ACT>(p, acc, rb, lane, q0.n, q0.pp, stage + (threadIdx.x >> 6) * 1024);
+      MfmaEpilogueI8Wide<ACT>(p, acc, rc, rb, lane, q0.n, q0.pp, stage + (threadIdx.x >> 6) * 1024);
       return;
     }
   }
-  MfmaEpilogue<OUT, ACT>(p, acc, rb, lane, qo);
+  MfmaEpilogue<OUT, ACT>(p, acc, rc, rb, lane, qo);
 }
 
 // One tile: stage, multiply, finish, pipelined over groups of four k-steps
@@ -708,6 +729,12 @@ __device__ __forceinline__ void MfmaTile(const MfmaParams& p, uint4* xt, uint32_
   constexpr bool kLoopK = KSMAX > 32;
   constexpr int KC = kLoopK ? kLoopChunk : KSMAX;  // k-steps held at once
   v4i a[KC];
+  // Held across the multiply only by the 16-k-step kernel: the smaller ones
+  // would lose a resident wavefront per SIMD to the 32 extra registers, the
+  // 32-k-step one has no room left.
+  constexpr bool kEarlyConsts = KSMAX == 16;
+  RowConsts rc;
+  if (kEarlyConsts) LoadRowConsts<OUT>(rc, p, rbc, lane);
   const bool quad_on = j < J;
   const int jc = quad_on ? j : J - 1;  // idle lanes repeat the last quad's loads
   v16i acc[4];
@@ -798,7 +825,8 @@ __device__ __forceinline__ void MfmaTile(const MfmaParams& p, uint4* xt, uint32_
   }
   if (!wave_on) return;
   PL_PHASE_MARK(4);
-  MfmaFinish<OUT, ACT, VEC>(p, reinterpret_cast<uint32_t*>(xt + (size_t)2 * (kLoopK ? KC : p.ksteps) * kMfmaTilePos), acc, rb, lane, quad0, J);
+  if (!kEarlyConsts) LoadRowConsts<OUT>(rc, p, rbc, lane);
+  MfmaFinish<OUT, ACT, VEC>(p, reinterpret_cast<uint32_t*>(xt + (size_t)2 * (kLoopK ? KC : p.ksteps) * kMfmaTilePos), acc, rc, rb, lane, quad0, J);
 }
 
 // Few input channels (at most 64, KSMAX <= 2): the channel groups of one
@@ -815,6 +843,8 @@ __device__ __forceinline__ void MfmaTilesFewChannels(const MfmaParams& p, uint4*
   const int RB = min(4, p.row_blocks - 4 * group);
   const int rb = 4 * group + (wave & (RB - 1));
   const uint32_t kmask = p.kmask[(size_t)rb * p.kmask_words];
+  RowConsts rc;
+  LoadRowConsts<OUT>(rc, p, rb, lane);
   v4i a[KSMAX];
   const size_t tile_cells = (size_t)n_kg * kMfmaTilePos;
   {
@@ -859,7 +889,7 @@ __device__ __forceinline__ void MfmaTilesFewChannels(const MfmaParams& p, uint4*
         }
       }
     }
-    MfmaFinish<OUT, ACT, true>(p, stage, acc, rb, lane, quad0, 32);
+    MfmaFinish<OUT, ACT, true>(p, stage, acc, rc, rb, lane, quad0, 32);
   }
 }
 
