@@ -87,12 +87,15 @@ LITE_LIB_PATH = os.path.join(LIB_DIR, "libpl_lite_hip.so")
 ROOT = os.path.dirname(PKG)
 HOST_TEST_SRC = os.path.join(ROOT, "tests", "cpp", "sparse_conv_hip_test.cc")
 HOST_TEST_BIN = os.path.join(ROOT, "tests", "cpp", "sparse_conv_hip_test")
+MODEL_TOOL_SRC = os.path.join(ROOT, "tests", "cpp", "model_file_tool.cc")
+MODEL_TOOL_BIN = os.path.join(ROOT, "tests", "cpp", "model_file_tool")
 
 LITE_SOURCES = [
     "core/tensor.cc",
     "core/op_lite.cc",
     "core/optimizer/mir/sparse_conv_detect_pass.cc",
     "core/optimizer/mir/int8_chain_pass.cc",
+    "model_parser/model_parser.cc",
     "operators/sparse_conv_op.cc",
     "operators/io_copy_op.cc",
     "operators/calib_op.cc",
@@ -123,6 +126,8 @@ def build_host_mirror(verbose=False):
     _run(["make", "-C", oracle_dir, "-s", "libsparse_conv_oracle.so"], verbose)
     _run(["g++"] + flags + inc + ["-I" + oracle_dir, "-o", HOST_TEST_BIN, HOST_TEST_SRC, "-L" + LIB_DIR, "-lpl_lite_hip", "-lpl_sparse_conv", "-L" + oracle_dir, "-lsparse_conv_oracle",
                                   "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN/../../paddle-lite_amd/lib:$ORIGIN/../../oracle:/opt/rocm/lib"], verbose)
+    _run(["g++"] + flags + inc + ["-o", MODEL_TOOL_BIN, MODEL_TOOL_SRC, "-L" + LIB_DIR, "-lpl_lite_hip", "-lpl_sparse_conv", "-L/opt/rocm/lib", "-lamdhip64",
+                                  "-Wl,-rpath,$ORIGIN/../../paddle-lite_amd/lib:/opt/rocm/lib"], verbose)
     return LITE_LIB_PATH, HOST_TEST_BIN
 
 

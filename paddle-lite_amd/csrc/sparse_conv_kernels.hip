@@ -761,6 +761,29 @@ __device__ __forceinline__ void MfmaTile(const MfmaParams& p, uint4* xt, uint32_
     };
     // D[32 rows][32 cols] += A[32 x 32k] * B[32k x 32] for the chunk's k-steps [i0, i1)
     auto multiply = [&](int i0, int i1) {
+      if (KSMAX != 32 && i1 - i0 == 4 && i1 <= KC && ((cmask >> i0) & 15u) == 15u) {
+        // all four k-steps present: no branches, and the cells of the next
+        // k-step are read from LDS while this one is multiplied (the
+        // 32-k-step kernel has no registers left for the second set of cells)
+        uint4 bq[2][4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) bq[0][c] = bbase[(size_t)(2 * i0) * kMfmaTilePos + c * 32];
+#pragma unroll
+        for (int i = i0; i < i1; ++i) {
+          if (i + 1 < i1) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) bq[(i + 1 - i0) & 1][c] = bbase[(size_t)(2 * (i + 1)) * kMfmaTilePos + c * 32];
+          }
+          __builtin_amdgcn_sched_barrier(0);  // keeps the reads ahead of the multiplies
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const uint4 q = bq[(i - i0) & 1][c];
+            acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i < KC ? i : 0], v4i{(int)q.x, (int)q.y, (int)q.z, (int)q.w}, acc[c], 0, 0, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        return;
+      }
 #pragma unroll
       for (int i = i0; i < i1; ++i) {
         if (i < KC && (cmask & (1u << i))) {

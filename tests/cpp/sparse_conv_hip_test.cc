@@ -11,6 +11,7 @@
 #include <cstdio>
 #include <cstring>
 #include <random>
+#include <unistd.h>
 #include <string>
 #include <vector>
 
@@ -18,6 +19,7 @@
 #include "lite/core/optimizer/mir/int8_chain_pass.h"
 #include "lite/core/optimizer/mir/sparse_conv_detect_pass.h"
 #include "lite/kernels/hip/sparse_conv_compute.h"
+#include "lite/model_parser/model_parser.h"
 #include "lite/operators/sparse_conv_op.h"
 #include "pl_sparse_conv.h"
 #include "sparse_conv_oracle.h"
@@ -601,6 +603,99 @@ static void Int8Chain(bool run_on_device) {
   if (got) EXPECT(std::memcmp(want.data(), got->raw_data(), want.size() * 4) == 0);
 }
 
+// Runs a sparse_conv2d description against the tensors of `scope` on the
+// device ("x" is copied over first) and returns the output on the host.
+static Tensor RunSparseOnDevice(OpInfo info, Scope* scope, PrecisionType prec, const std::string& alias) {
+  OpInfo h2d("io_copy");
+  h2d.SetInput("Input", {"x"});
+  h2d.SetOutput("Out", {"x_dev"});
+  auto copy_op = LiteOpRegistry::Global().Create("io_copy");
+  EXPECT(copy_op->Attach(h2d, scope) && copy_op->InferShape());
+  auto copy_kernels = copy_op->CreateKernels({paddle::lite_api::Place(TARGET(kHIP), PRECISION(kAny), DATALAYOUT(kAny))}, "io_copy/host_to_device");
+  copy_kernels[0]->Launch();
+  info.SetInput("Input", {"x_dev"});
+  scope->NewTensor(info.Output("Output").front());
+  auto op = LiteOpRegistry::Global().Create("sparse_conv2d");
+  EXPECT(op->Attach(info, scope) && op->CheckShape() && op->InferShape());
+  auto kernels = op->CreateKernels({paddle::lite_api::Place(TARGET(kHIP), prec, DATALAYOUT(kNCHW))}, "sparse_conv2d/" + alias);
+  EXPECT(kernels.size() == 1);
+  kernels[0]->Launch();
+  kernels[0]->mutable_context_as<HIPContext>()->Sync();
+  Tensor y_host;
+  y_host.CopyDataFrom(*scope->FindMutableTensor(info.Output("Output").front()), TargetType::kHost);
+  return y_host;
+}
+
+// The optimised-model file: what the detect pass produced is written as a
+// "<name>.nb" file, read back into an empty scope, and the loaded
+// sparse_conv2d gives the same output bytes as the one that was saved.
+static void ModelFile(bool run_on_device) {
+  std::printf("case model file round trip\n");
+  std::fflush(stdout);
+  const std::vector<Problem> problems = {
+      {2, 64, 48, 7, 7, 0.8f, true, false, false, true, "relu6", 31},
+      {2, 128, 64, 7, 7, 0.85f, false, true, false, true, "leaky_relu", 32},
+      {2, 96, 32, 8, 8, 0.75f, true, true, true, true, "hard_swish", 33},
+  };
+  for (const Problem& p : problems) {
+    Scope scope;
+    std::vector<float> ws;
+    float in_scale = 1.f, out_scale = 1.f;
+    std::vector<OpInfo> ops{MakeConv(p, &scope, &ws, &in_scale, &out_scale)};
+    mir::SparseConvDetectPass pass;
+    pass.SetSparseThreshold(0.5f);
+    EXPECT(pass.Apply(&ops, &scope) == 1);
+
+    cpp::ProgramDesc prog;
+    cpp::BlockDesc* block = prog.AddBlock();
+    block->SetParentIdx(-1);
+    prog.SetVersion(1);
+    auto add_var = [&](const std::string& name, bool persistable) {
+      cpp::VarDesc* v = block->AddVar();
+      v->SetName(name);
+      v->SetPersistable(persistable);
+      const Tensor* t = scope.FindMutableTensor(name);
+      v->SetShape(t->dims().Vectorize());
+      v->SetDataType(t->precision() == PRECISION(kInt8) ? VarDataType::INT8 : t->precision() == PRECISION(kInt32) ? VarDataType::INT32 : VarDataType::FP32);
+    };
+    add_var("x", false);
+    for (const char* arg : {"NonZeroWeights", "OcNonZeros", "Diffs", "Bias"}) add_var(ops[0].Input(arg).front(), true);
+    *block->AddOp() = ops[0];
+
+    const std::string base = "/tmp/pl_model_file_test_" + std::to_string(static_cast<long>(getpid())) + "_" + std::to_string(p.seed);
+    SaveModelNaive(base, scope, prog);
+    Scope loaded;
+    cpp::ProgramDesc back;
+    LoadModelNaiveFromFile(base + ".nb", &loaded, &back);
+    std::remove((base + ".nb").c_str());
+    EXPECT(back.BlocksSize() == 1 && back.GetBlock(0)->OpsSize() == 1);
+    if (back.BlocksSize() != 1 || back.GetBlock(0)->OpsSize() != 1) continue;
+    const OpInfo& op2 = back.GetBlock(0)->GetOp(0);
+    EXPECT(op2.Type() == "sparse_conv2d");
+    EXPECT(op2.GetAttr<int>("first_ic") == ops[0].GetAttr<int>("first_ic") && op2.GetAttr<int>("flag_semi") == ops[0].GetAttr<int>("flag_semi"));
+    EXPECT(op2.GetAttr<std::string>("act_type") == p.act);
+    if (p.int8) EXPECT(op2.GetInputScale("Filter0_scale", true) == ws);
+    for (const char* arg : {"NonZeroWeights", "OcNonZeros", "Diffs", "Bias"}) {
+      const std::string name = ops[0].Input(arg).front();
+      const Tensor* a = scope.FindMutableTensor(name);
+      const Tensor* b = loaded.FindMutableTensor(name);
+      EXPECT(b != nullptr && b->persistable() && b->dims() == a->dims() && b->precision() == a->precision() && b->memory_size() == a->memory_size());
+      if (b && b->memory_size() == a->memory_size()) EXPECT(std::memcmp(a->raw_data(), b->raw_data(), a->memory_size()) == 0);
+    }
+    EXPECT(loaded.FindVar("x") == nullptr);
+    if (!run_on_device) continue;
+    // the input is not part of the file
+    const Tensor* x = scope.FindMutableTensor("x");
+    loaded.NewTensor("x")->CopyDataFrom(*x, TargetType::kHost);
+    const PrecisionType prec = p.int8 ? PRECISION(kInt8) : PRECISION(kFloat);
+    const std::string alias = !p.int8 ? "def" : (p.out_int8 ? "int8_int8_out" : "int8_fp32_out");
+    const Tensor y_saved = RunSparseOnDevice(ops[0], &scope, prec, alias);
+    const Tensor y_loaded = RunSparseOnDevice(op2, &loaded, prec, alias);
+    EXPECT(y_saved.memory_size() > 0 && y_saved.memory_size() == y_loaded.memory_size());
+    if (y_saved.memory_size() == y_loaded.memory_size()) EXPECT(std::memcmp(y_saved.raw_data(), y_loaded.raw_data(), y_saved.memory_size()) == 0);
+  }
+}
+
 int main(int argc, char** argv) {
   const bool gpu = argc > 1 && std::string(argv[1]) == "--gpu";
   RegistryAndErrorPaths();
@@ -623,6 +718,7 @@ int main(int argc, char** argv) {
   CalibChain(gpu);
   Int8Chain(gpu);
   HalfPrecision(gpu);
+  ModelFile(gpu);
   std::printf("%s: %d failure(s)\n", gpu ? "gpu" : "cpu", g_failures);
   return g_failures ? 1 : 0;
 }
