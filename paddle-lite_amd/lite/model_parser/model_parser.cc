@@ -1,5 +1,7 @@
 #include "lite/model_parser/model_parser.h"
 
+#include <climits>
+#include <cstdint>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -545,6 +547,55 @@ std::string SerializeModelNaive(const Scope& exec_scope, const cpp::ProgramDesc&
     out.append(reinterpret_cast<const char*>(param.data()), param.size());
   }
   return out;
+}
+
+int RebakeSparseConvDiffs(cpp::ProgramDesc* prog, Scope* scope, int64_t new_h, int64_t new_w) {
+  CHECK(prog && scope);
+  CHECK(new_h > 0 && new_w > 0) << "the new input size must be positive";
+  if (prog->BlocksSize() == 0) return 0;
+  cpp::BlockDesc* block = prog->GetBlock(0);
+  auto find_var = [&](const std::string& name) -> cpp::VarDesc* {
+    for (cpp::VarDesc& v : block->vars())
+      if (v.Name() == name) return &v;
+    return nullptr;
+  };
+  // sizes first: several ops may read one variable, whose shape changes below
+  std::vector<std::pair<OpInfo*, int64_t>> todo;
+  for (OpInfo& op : block->ops()) {
+    if (op.Type() != "sparse_conv2d") continue;
+    const cpp::VarDesc* x = find_var(op.Input("Input").front());
+    if (!x || x->GetShape().size() != 4 || x->GetShape()[2] <= 0 || x->GetShape()[3] <= 0) continue;
+    todo.emplace_back(&op, x->GetShape()[2] * x->GetShape()[3]);
+  }
+  const int64_t new_size = new_h * new_w;
+  std::set<std::string> done;  // a Diffs tensor shared by two ops is rewritten once
+  for (auto& item : todo) {
+    const OpInfo& op = *item.first;
+    const int64_t old_size = item.second;
+    const std::string diffs_name = op.Input("Diffs").front();
+    if (!done.insert(diffs_name).second) continue;
+    Tensor* diffs = scope->FindMutableTensor(diffs_name);
+    CHECK(diffs && diffs->precision() == PrecisionType::kInt32) << "sparse_conv2d without an int32 Diffs tensor";
+    int32_t* d = diffs->mutable_data<int32_t>(TargetType::kHost);
+    for (int64_t i = 0; i < diffs->numel(); ++i) {
+      CHECK(d[i] % old_size == 0) << "Diffs entry " << i << " is not a multiple of the recorded input size " << old_size;
+      const int64_t v = static_cast<int64_t>(d[i]) / old_size * new_size;
+      CHECK(v >= INT32_MIN && v <= INT32_MAX) << "Diffs entry " << i << " does not fit 32 bits at the new input size";
+      d[i] = static_cast<int32_t>(v);
+    }
+  }
+  auto reshape = [&](cpp::VarDesc* v) {
+    if (!v || v->GetShape().size() != 4) return;
+    std::vector<int64_t> s = v->GetShape();
+    s[2] = new_h;
+    s[3] = new_w;
+    v->SetShape(s);
+  };
+  for (auto& item : todo) {
+    reshape(find_var(item.first->Input("Input").front()));
+    reshape(find_var(item.first->Output("Output").front()));
+  }
+  return static_cast<int>(todo.size());
 }
 
 void SaveModelNaive(const std::string& model_file, const Scope& exec_scope, const cpp::ProgramDesc& cpp_prog) {

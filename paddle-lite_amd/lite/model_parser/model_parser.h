@@ -38,6 +38,16 @@ bool TryLoadModelNaiveFromMemory(const std::string& model_buffer, Scope* scope, 
 void SaveModelNaive(const std::string& model_file, const Scope& exec_scope, const cpp::ProgramDesc& cpp_prog);
 std::string SerializeModelNaive(const Scope& exec_scope, const cpp::ProgramDesc& cpp_prog, uint16_t meta_version = 2);
 
+// The Diffs tensor of a sparse_conv2d holds byte distances that include the
+// H*W of the op's input at optimisation time (the detect pass multiplies the
+// channel distance by it, lite/core/optimizer/mir/sparse_conv_detect_pass.cc:
+// 35-91), so a saved model runs at that resolution only.  This rewrites the
+// Diffs of every sparse_conv2d of block 0 from the recorded shape of its
+// Input variable to new_h * new_w and records the new shape, which makes the
+// loaded model usable at another resolution.  Returns the number of ops
+// changed; an op whose Input has no static 4-D shape is left alone.
+int RebakeSparseConvDiffs(cpp::ProgramDesc* prog, Scope* scope, int64_t new_h, int64_t new_w);
+
 namespace fbs {
 // The two FlatBuffers payloads on their own.
 std::vector<uint8_t> SerializeProgramDesc(const cpp::ProgramDesc& prog);

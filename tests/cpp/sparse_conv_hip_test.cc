@@ -683,6 +683,31 @@ static void ModelFile(bool run_on_device) {
       if (b && b->memory_size() == a->memory_size()) EXPECT(std::memcmp(a->raw_data(), b->raw_data(), a->memory_size()) == 0);
     }
     EXPECT(loaded.FindVar("x") == nullptr);
+    {
+      // another resolution: the reloaded Diffs, rewritten for 5x3 inputs,
+      // equal what the detect pass makes of the same weights at 5x3
+      Problem q = p;
+      q.h = 5, q.w = 3;
+      Scope scope_q;
+      std::vector<float> ws_q;
+      float is_q, os_q;
+      std::vector<OpInfo> ops_q{MakeConv(q, &scope_q, &ws_q, &is_q, &os_q)};
+      EXPECT(pass.Apply(&ops_q, &scope_q) == 1);
+      Scope again;
+      cpp::ProgramDesc prog_q;
+      SaveModelNaive(base, scope, prog);
+      LoadModelNaiveFromFile(base + ".nb", &again, &prog_q);
+      std::remove((base + ".nb").c_str());
+      EXPECT(RebakeSparseConvDiffs(&prog_q, &again, q.h, q.w) == 1);
+      const std::string dn = ops[0].Input("Diffs").front();
+      const Tensor* want = scope_q.FindMutableTensor(dn);
+      const Tensor* got = again.FindMutableTensor(dn);
+      EXPECT(want->numel() == got->numel() && std::memcmp(want->raw_data(), got->raw_data(), want->memory_size()) == 0);
+      EXPECT(prog_q.GetBlock(0)->GetVar(0).GetShape() == (std::vector<int64_t>{q.batch, q.ic, q.h, q.w}));
+      // the saved model itself is unchanged, and a second rewrite starts from the recorded 5x3
+      EXPECT(RebakeSparseConvDiffs(&prog_q, &again, p.h, p.w) == 1);
+      EXPECT(std::memcmp(scope.FindMutableTensor(dn)->raw_data(), again.FindMutableTensor(dn)->raw_data(), got->memory_size()) == 0);
+    }
     if (!run_on_device) continue;
     // the input is not part of the file
     const Tensor* x = scope.FindMutableTensor("x");
