@@ -224,6 +224,43 @@ int pl_calib_fp32_to_int8(const float* x_dev, int8_t* out_dev, int64_t n,
 int pl_calib_int8_to_fp32(const int8_t* x_dev, float* out_dev, int64_t n,
                           float scale, void* stream);
 
+/* ---- int8 depthwise 3x3 convolution (the layer between the pointwise
+ * convolutions of a MobileNet) -------------------------------------------
+ * Replaces lite::arm::math::conv_depthwise_3x3_int8_fp32 / _int8_int8 as
+ * DepthwiseConv<kInt8, *>::Run calls them (lite/kernels/arm/conv_depthwise.cc:
+ * 359-412, lite/backends/arm/math/conv_impl.cc:1858-2090): one 3x3 filter per
+ * channel, stride 1 or 2, zero padding 0 or 1 on all four sides, dilation 1;
+ * int32 accumulation, then fmaf(float(acc), scale[c], bias[c]), activation,
+ * and for int8 output max(v, -127), round half away from zero, saturate
+ * (conv_block_utils.h:3888-3950, :4328-4420).  hard_swish follows
+ * cvt_kernel there: (v * hs_scale) * min(max(v + hs_offset, 0), hs_threshold),
+ * i.e. hs_scale multiplies.  scale / bias are the merged per-channel values
+ * of PrepareForRun (conv_depthwise.cc:158-322).  All desc pointers are host
+ * pointers read only during prepare. */
+typedef struct pl_dwconv_desc {
+  uint32_t struct_size;     /* sizeof(pl_dwconv_desc)                        */
+  int32_t kind;             /* PL_KIND_INT8_FP32 or PL_KIND_INT8_INT8        */
+  int32_t channels;
+  int32_t stride;           /* 1 or 2 (both directions)                      */
+  int32_t pad;              /* 0 or 1 (all four sides)                       */
+  const int8_t* weights;    /* [channels][3][3]                              */
+  const float* scale;       /* [channels]                                    */
+  const float* bias;        /* [channels] or NULL                            */
+  pl_activation act;
+} pl_dwconv_desc;
+
+typedef struct pl_dwconv_handle pl_dwconv_handle;
+
+int pl_dwconv3x3_prepare(const pl_dwconv_desc* desc, pl_dwconv_handle** out_handle);
+
+/* x_dev: int8 NCHW [batch, channels, h, w]; out_dev: fp32 or int8 NCHW
+ * [batch, channels, oh, ow] with oh = (h + 2 * pad - 3) / stride + 1.
+ * Enqueues on `stream` and returns. */
+int pl_dwconv3x3_run(pl_dwconv_handle* handle, const int8_t* x_dev, void* out_dev,
+                     int32_t batch, int32_t h, int32_t w, void* stream);
+
+void pl_dwconv3x3_destroy(pl_dwconv_handle* handle);
+
 #ifdef __cplusplus
 }
 #endif

@@ -288,6 +288,42 @@ def ref_conv1x1_s8_s32(x, w, omp=False):
     return out
 
 
+def dwconv_out_size(size, stride, pad):
+    return (size + 2 * pad - 3) // stride + 1
+
+
+def dwconv3x3_int8(x, w, scale=None, bias=None, act=None, out="int8", stride=1,
+                   pad=1):
+    """int8 depthwise 3x3; out: "fp32", "int8" or "acc" (raw int32 sums)."""
+    x, w = _c(x, np.int8), _c(w, np.int8)
+    n, ch, h, ww = x.shape
+    assert w.shape == (ch, 3, 3)
+    kind = {"fp32": 1, "int8": 2, "acc": 3}[out]
+    oh, ow = dwconv_out_size(h, stride, pad), dwconv_out_size(ww, stride, pad)
+    res = np.zeros((n, ch, oh, ow),
+                   dtype={1: np.float32, 2: np.int8, 3: np.int32}[kind])
+    scale = None if scale is None else _c(scale, np.float32)
+    bias = None if bias is None else _c(bias, np.float32)
+    act = act or Act()
+    rc = lib().plo_dwconv3x3_int8(_p(x), _p(w), _p(scale), _p(bias),
+                                  C.byref(act), kind, n, ch, h, ww, stride,
+                                  pad, _p(res))
+    if rc != 0:
+        raise ValueError("plo_dwconv3x3_int8: bad argument")
+    return res
+
+
+def ref_dwconv3x3_s8_s32(x, w, stride=1, pad=1):
+    """The reference header's conv_basic<int8, int32> with group == channels."""
+    x, w = _c(x, np.int8), _c(w, np.int8)
+    n, ch, h, ww = x.shape
+    oh, ow = dwconv_out_size(h, stride, pad), dwconv_out_size(ww, stride, pad)
+    out = np.zeros((n, ch, oh, ow), dtype=np.int32)
+    ref().ref_dwconv3x3_s8_s32(_p(x), _p(out), n, ch, oh, ow, h, ww, _p(w),
+                               stride, pad)
+    return out
+
+
 def fp32_to_int8(x, scale):
     x = _c(x, np.float32)
     out = np.empty(x.shape, dtype=np.int8)

@@ -43,4 +43,13 @@ void ref_conv1x1_s8_s32(const int8_t* x, int32_t* out, int num, int chout,
                               nullptr, 1, 1, 1, 1, 1, 1, 1, 0, 0, false, 0);
 }
 
+// Depthwise 3x3 (group == channels), int8 inputs, int32 accumulators.
+void ref_dwconv3x3_s8_s32(const int8_t* x, int32_t* out, int num, int ch,
+                          int hout, int wout, int hin, int win,
+                          const int8_t* weights, int stride, int pad) {
+  conv_basic<int8_t, int32_t>(x, out, num, ch, hout, wout, ch, hin, win,
+                              weights, nullptr, ch, 3, 3, stride, stride, 1, 1,
+                              pad, pad, false, 0);
+}
+
 }  // extern "C"

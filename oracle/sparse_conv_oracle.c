@@ -800,3 +800,61 @@ int plo_dense_conv1x1(int out_kind, const void* w_dense, const void* x,
   }
   return used;
 }
+
+/* ------------------------------------------------------------------------ */
+/* int8 depthwise 3x3 convolution                                            */
+/* ------------------------------------------------------------------------ */
+/* Accumulators as the reference's naive conv_basic<int8_t, int> computes them
+ * for group == channels (lite/tests/utils/naive_math_impl.h:395-519: zero
+ * padding, out = (in + 2 pad - 3) / stride + 1), then the epilogue of the
+ * ARM depthwise kernels (lite/backends/arm/math/conv_block_utils.h:3696-3753
+ * cvt_kernel; the NEON bodies use fmla, :3888-3950): fmaf(acc, scale, bias),
+ * activation - hard_swish there is (v * alpha) * min(max(v + offset, 0),
+ * threshold) with alpha = hard_swish_scale, the scale MULTIPLIES - and for
+ * int8 output max(v, -127), round half away from zero, saturate.
+ * out_kind: 1 fp32, 2 int8, 3 raw int32 accumulators.
+ * Pinned by tests/test_oracle_dwconv.py: accumulators against conv_basic from
+ * the reference header (oracle/_ref) and against a numpy statement; the
+ * epilogue pieces are those of the sparse convolution, pinned there. */
+int plo_dwconv3x3_int8(const int8_t* x, const int8_t* w, const float* scale,
+                       const float* bias, const plo_act* act, int out_kind,
+                       int batch, int channels, int h, int wd, int stride,
+                       int pad, void* out) {
+  if (!x || !w || !out || batch < 0 || channels <= 0 || h <= 0 || wd <= 0)
+    return -1;
+  if ((stride != 1 && stride != 2) || (pad != 0 && pad != 1)) return -1;
+  if (out_kind < 1 || out_kind > 3 || (out_kind != 3 && !scale)) return -1;
+  if (h + 2 * pad < 3 || wd + 2 * pad < 3) return -1;
+  const int oh = (h + 2 * pad - 3) / stride + 1;
+  const int ow = (wd + 2 * pad - 3) / stride + 1;
+  const float hs_mul = act ? act->hs_scale : 0.0f;
+  for (int n = 0; n < batch; ++n)
+    for (int c = 0; c < channels; ++c) {
+      const int8_t* xp = x + ((size_t)n * channels + c) * h * wd;
+      const int8_t* wp = w + (size_t)c * 9;
+      const size_t obase = ((size_t)n * channels + c) * oh * ow;
+      for (int oy = 0; oy < oh; ++oy)
+        for (int ox = 0; ox < ow; ++ox) {
+          int32_t acc = 0;
+          for (int ky = 0; ky < 3; ++ky)
+            for (int kx = 0; kx < 3; ++kx) {
+              const int iy = oy * stride - pad + ky;
+              const int ix = ox * stride - pad + kx;
+              if (iy < 0 || iy >= h || ix < 0 || ix >= wd) continue;
+              acc += (int32_t)xp[(size_t)iy * wd + ix] * (int32_t)wp[ky * 3 + kx];
+            }
+          const size_t o = obase + (size_t)oy * ow + ox;
+          if (out_kind == 3) {
+            ((int32_t*)out)[o] = acc;
+            continue;
+          }
+          float v = fmaf((float)acc, scale[c], bias ? bias[c] : 0.0f);
+          v = apply_act(v, act, hs_mul);
+          if (out_kind == 1)
+            ((float*)out)[o] = v;
+          else
+            ((int8_t*)out)[o] = to_int8_sat(v);
+        }
+    }
+  return 0;
+}

@@ -194,6 +194,19 @@ int plo_dense_conv1x1(int out_kind, const void* w_dense, const void* x,
                       int batch, int M, int K, int N, const plo_act* act,
                       int threads);
 
+/* ---------------------------------------------------------------------------
+ * int8 depthwise 3x3 convolution, stride 1 or 2, zero padding 0 or 1
+ * (reference: lite/tests/utils/naive_math_impl.h:395-519 for the sums,
+ * lite/backends/arm/math/conv_block_utils.h:3696-3753 for the epilogue; note
+ * that hard_swish multiplies by act->hs_scale here).
+ * x [batch, channels, h, w], w [channels, 3, 3]; out_kind 1 fp32, 2 int8,
+ * 3 raw int32 accumulators.  Returns 0, or -1 for a bad argument.
+ * ------------------------------------------------------------------------ */
+int plo_dwconv3x3_int8(const int8_t* x, const int8_t* w, const float* scale,
+                       const float* bias, const plo_act* act, int out_kind,
+                       int batch, int channels, int h, int wd, int stride,
+                       int pad, void* out);
+
 #ifdef __cplusplus
 }
 #endif

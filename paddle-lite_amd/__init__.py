@@ -19,3 +19,4 @@ from .sparse_conv import (  # noqa: F401
 from .calib import CalibParam, CalibComputeFp32ToInt8, CalibComputeInt8ToFp32  # noqa: F401
 
 __all__ = ["capi", "ActivationParam", "SparseConvParam", "SparseConvKernel", "SparseWeights", "detect_and_pack", "CalibParam", "CalibComputeFp32ToInt8", "CalibComputeInt8ToFp32"]
+from .depthwise_conv import ConvParam, DepthwiseConv  # noqa: F401

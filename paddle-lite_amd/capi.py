@@ -28,6 +28,9 @@ EXPORTS = [
     "pl_fp32_to_fp16",
     "pl_calib_fp32_to_int8",
     "pl_calib_int8_to_fp32",
+    "pl_dwconv3x3_prepare",
+    "pl_dwconv3x3_run",
+    "pl_dwconv3x3_destroy",
 ]
 
 
@@ -39,6 +42,20 @@ class Activation(C.Structure):
         ("hs_scale", C.c_float),
         ("hs_offset", C.c_float),
         ("hs_threshold", C.c_float),
+    ]
+
+
+class DwConvDesc(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32),
+        ("kind", C.c_int32),
+        ("channels", C.c_int32),
+        ("stride", C.c_int32),
+        ("pad", C.c_int32),
+        ("weights", C.c_void_p),
+        ("scale", C.c_void_p),
+        ("bias", C.c_void_p),
+        ("act", Activation),
     ]
 
 
@@ -127,6 +144,12 @@ def lib():
     L.pl_calib_fp32_to_int8.restype = C.c_int
     L.pl_calib_int8_to_fp32.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_float, C.c_void_p]
     L.pl_calib_int8_to_fp32.restype = C.c_int
+    L.pl_dwconv3x3_prepare.argtypes = [C.POINTER(DwConvDesc), C.POINTER(C.c_void_p)]
+    L.pl_dwconv3x3_prepare.restype = C.c_int
+    L.pl_dwconv3x3_run.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]
+    L.pl_dwconv3x3_run.restype = C.c_int
+    L.pl_dwconv3x3_destroy.argtypes = [C.c_void_p]
+    L.pl_dwconv3x3_destroy.restype = None
     if L.pl_sparse_conv_abi_version() != ABI_VERSION:
         raise LibraryMissing("libpl_sparse_conv.so has ABI %d, binding expects %d" % (L.pl_sparse_conv_abi_version(), ABI_VERSION))
     _lib = L

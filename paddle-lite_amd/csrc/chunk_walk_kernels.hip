@@ -17,6 +17,7 @@
 #include <cstdint>
 #include <type_traits>
 
+#include "epilogue.h"
 #include "sparse_conv_kernels.h"
 
 namespace pl {
@@ -26,16 +27,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef const __attribute__((address_space(4))) uint32_t* ConstWords;
 typedef const __attribute__((address_space(4))) float* ConstFloats;
 
-__device__ __forceinline__ float Clamp0(float v, float hi) { return __builtin_amdgcn_fmed3f(v, fminf(0.0f, hi), hi); }
-
-template <int ACT>
-__device__ __forceinline__ float ActivateT(float v, const DevAct& a) {
-  if (ACT == 1) return fmaxf(v, 0.0f);
-  if (ACT == 2) return Clamp0(v, a.relu6_coef);
-  if (ACT == 4) return (v >= 0.0f) ? v : v * a.leaky_alpha;
-  if (ACT == 10) return (v * a.hs_inv_scale) * Clamp0(v + a.hs_offset, a.hs_threshold);
-  return v;
-}
+using epilogue::ActivateT;
 
 // Workgroup id -> tile: each XCD (linear id mod 8) owns a contiguous range of
 // tiles, the per_tile workgroups of one tile follow each other on it.

@@ -1,0 +1,35 @@
+// Device-side interface of the int8 depthwise 3x3 convolution.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "sparse_conv_kernels.h"
+
+namespace pl {
+
+struct DwConvParams {
+  const int8_t* x;         // NCHW [batch, channels, h, w]
+  void* out;               // NCHW [batch, channels, oh, ow], fp32 or int8
+  const uint32_t* wpack;   // [channels][4]: weight rows as bytes (w0, w1, w2, 0); the fourth dword is unused
+  const float* scale;      // [channels]
+  const float* bias;       // [channels] (zeros when the op has no bias)
+  int channels;
+  int h, w, oh, ow;
+  int pad;                 // 0 or 1, all four sides
+  uint32_t planes;         // batch * channels
+  int64_t in_bytes;        // planes * h * w
+  DevAct act;
+  // filled in by the launcher
+  int groups_w;            // ceil(ow / 4): a thread makes four neighbouring outputs of a row
+  int items;               // oh * groups_w per plane
+  int planes_per_block;    // several small planes share a workgroup
+  uint32_t magic_items;    // ceil(2^32 / items) for items >= 2: x / items == mulhi(x, magic) for x * items < 2^32
+  uint32_t magic_groups;   // likewise for groups_w
+};
+
+// stride 1 or 2; out_kind kOutF32 or kOutI8.
+hipError_t LaunchDwConv3x3(int stride, int out_kind, const DwConvParams& p, hipStream_t stream);
+
+}  // namespace pl

@@ -10,11 +10,13 @@
 #include <cstdlib>
 #include <cmath>
 #include <cstring>
+#include <memory>
 #include <new>
 #include <string>
 #include <vector>
 
 #include "../../include/pl_sparse_conv.h"
+#include "dwconv_kernels.h"
 #include "sparse_conv_kernels.h"
 #include "sparse_layout.h"
 
@@ -829,5 +831,98 @@ int pl_sparse_pack(int32_t dtype, int32_t flag_semi, const void* dense, int32_t 
   if (dtype == 0) return pl::PackWeights(static_cast<const float*>(dense), oc, ic, im_size, flag_semi != 0, static_cast<float*>(nonzero_weights), oc_nonzeros, diffs);
   return pl::PackWeights(static_cast<const int8_t*>(dense), oc, ic, im_size, flag_semi != 0, static_cast<int8_t*>(nonzero_weights), oc_nonzeros, diffs);
 }
+
+// ------------------------------------------------ depthwise 3x3 convolution
+struct pl_dwconv_handle {
+  int device = 0;
+  int kind = 0, channels = 0, stride = 1, pad = 0;
+  DevBuf wpack, scale, bias;
+  pl::DevAct act{};
+};
+
+int pl_dwconv3x3_prepare(const pl_dwconv_desc* desc, pl_dwconv_handle** out_handle) {
+  if (!desc || !out_handle) return Fail(PL_ERR_BAD_ARG, "null argument");
+  *out_handle = nullptr;
+  if (desc->struct_size != sizeof(pl_dwconv_desc)) return Fail(PL_ERR_BAD_ARG, "pl_dwconv_desc size mismatch (%u vs %zu)", desc->struct_size, sizeof(pl_dwconv_desc));
+  if (desc->kind != PL_KIND_INT8_FP32 && desc->kind != PL_KIND_INT8_INT8) return Fail(PL_ERR_BAD_ARG, "kind must be int8 -> fp32 or int8 -> int8");
+  if (desc->channels <= 0) return Fail(PL_ERR_BAD_ARG, "channels must be positive");
+  if (desc->stride != 1 && desc->stride != 2) return Fail(PL_ERR_UNSUPPORTED, "stride %d: only 1 and 2 exist", desc->stride);
+  if (desc->pad != 0 && desc->pad != 1) return Fail(PL_ERR_UNSUPPORTED, "padding %d: only 0 and 1 exist", desc->pad);
+  if (!desc->weights || !desc->scale) return Fail(PL_ERR_BAD_ARG, "null weights or scales");
+  switch (desc->act.type) {
+    case PL_ACT_NONE:
+    case PL_ACT_RELU:
+    case PL_ACT_RELU6:
+    case PL_ACT_LEAKY_RELU:
+    case PL_ACT_HARD_SWISH:
+      break;
+    default:
+      return Fail(PL_ERR_UNSUPPORTED, "activation %d has no kernel", desc->act.type);
+  }
+  if (pl_device_count() == 0) return Fail(PL_ERR_NO_DEVICE, "no gfx950 device: this library has no CPU path");
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return FailHip(e, "hipGetDevice");
+  hipDeviceProp_t prop;
+  e = hipGetDeviceProperties(&prop, dev);
+  if (e != hipSuccess) return FailHip(e, "hipGetDeviceProperties");
+  if (!std::strstr(prop.gcnArchName, "gfx950")) return Fail(PL_ERR_NO_DEVICE, "device %d is %s; the kernels are built for gfx950 only", dev, prop.gcnArchName);
+
+  std::unique_ptr<pl_dwconv_handle> h(new pl_dwconv_handle);
+  h->device = dev;
+  h->kind = desc->kind;
+  h->channels = desc->channels;
+  h->stride = desc->stride;
+  h->pad = desc->pad;
+  h->act = ToDevAct(desc->act);
+  h->act.hs_inv_scale = desc->act.hs_scale;  // this op multiplies by the scale itself
+  // filter rows as the dot-product operand (w0, w1, w2, 0)
+  std::vector<uint32_t> wpack(static_cast<size_t>(desc->channels) * 4, 0u);
+  for (int c = 0; c < desc->channels; ++c)
+    for (int r = 0; r < 3; ++r) {
+      const int8_t* w = desc->weights + (static_cast<size_t>(c) * 3 + r) * 3;
+      wpack[static_cast<size_t>(c) * 4 + r] = static_cast<uint32_t>(static_cast<uint8_t>(w[0])) | static_cast<uint32_t>(static_cast<uint8_t>(w[1])) << 8 | static_cast<uint32_t>(static_cast<uint8_t>(w[2])) << 16;
+    }
+  std::vector<float> bias(desc->channels, 0.0f);
+  if (desc->bias) std::memcpy(bias.data(), desc->bias, sizeof(float) * desc->channels);
+  if ((e = h->wpack.Upload(wpack.data(), wpack.size() * 4)) != hipSuccess) return FailHip(e, "uploading the filters");
+  if ((e = h->scale.Upload(desc->scale, sizeof(float) * desc->channels)) != hipSuccess) return FailHip(e, "uploading the scales");
+  if ((e = h->bias.Upload(bias.data(), sizeof(float) * desc->channels)) != hipSuccess) return FailHip(e, "uploading the biases");
+  *out_handle = h.release();
+  return PL_OK;
+}
+
+int pl_dwconv3x3_run(pl_dwconv_handle* h, const int8_t* x_dev, void* out_dev, int32_t batch, int32_t height, int32_t width, void* stream) {
+  if (!h) return Fail(PL_ERR_BAD_ARG, "null handle");
+  if (batch < 0 || height <= 0 || width <= 0) return Fail(PL_ERR_BAD_ARG, "bad batch or input size");
+  const int oh = (height + 2 * h->pad - 3) / h->stride + 1, ow = (width + 2 * h->pad - 3) / h->stride + 1;
+  if (height + 2 * h->pad < 3 || width + 2 * h->pad < 3) return Fail(PL_ERR_BAD_ARG, "the input is smaller than the filter");
+  if (batch == 0) return PL_OK;
+  if (!x_dev || !out_dev) return Fail(PL_ERR_BAD_ARG, "null device pointer");
+  int cur_dev = -1;
+  if (hipGetDevice(&cur_dev) != hipSuccess || cur_dev != h->device) return Fail(PL_ERR_BAD_ARG, "the handle belongs to device %d, the current device is %d", h->device, cur_dev);
+  const int64_t planes = static_cast<int64_t>(batch) * h->channels;
+  if (planes > 0x7fffffffll || planes * height * width >= (1ll << 40)) return Fail(PL_ERR_UNSUPPORTED, "tensor too large");
+  if (static_cast<int64_t>(oh) * ((ow + 3) / 4) > 46000) return Fail(PL_ERR_UNSUPPORTED, "output planes above 46000 groups of four outputs are not supported");
+  pl::DwConvParams p{};
+  p.x = x_dev;
+  p.out = out_dev;
+  p.wpack = static_cast<const uint32_t*>(h->wpack.ptr);
+  p.scale = static_cast<const float*>(h->scale.ptr);
+  p.bias = static_cast<const float*>(h->bias.ptr);
+  p.channels = h->channels;
+  p.h = height;
+  p.w = width;
+  p.oh = oh;
+  p.ow = ow;
+  p.pad = h->pad;
+  p.planes = static_cast<uint32_t>(planes);
+  p.in_bytes = planes * height * width;
+  p.act = h->act;
+  const hipError_t e = pl::LaunchDwConv3x3(h->stride, h->kind == PL_KIND_INT8_INT8 ? pl::kOutI8 : pl::kOutF32, p, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? PL_OK : FailHip(e, "depthwise convolution launch");
+}
+
+void pl_dwconv3x3_destroy(pl_dwconv_handle* h) { delete h; }
 
 }  // extern "C"

@@ -21,6 +21,7 @@
 //
 // Positions are the flattened (image, pixel) index g = n*hw + p, so tiles do
 // not care about image boundaries.
+#include "epilogue.h"
 #include "sparse_conv_kernels.h"
 
 #include <atomic>
@@ -92,82 +93,7 @@ __device__ __forceinline__ int XcdTile(int tiles, int per_tile) {
 }
 
 // ---------------------------------------------------------------- epilogue
-// min(max(v, 0), hi) for any hi as one median instruction: the lower bound
-// min(0, hi) is wave-uniform and makes the median equal hi when hi < 0.
-__device__ __forceinline__ float Clamp0(float v, float hi) { return __builtin_amdgcn_fmed3f(v, fminf(0.0f, hi), hi); }
-
-__device__ __forceinline__ float Activate(float v, const DevAct& a) {
-  switch (a.type) {
-    case 1:
-      return fmaxf(v, 0.0f);
-    case 2:
-      return Clamp0(v, a.relu6_coef);
-    case 4:
-      return (v >= 0.0f) ? v : v * a.leaky_alpha;
-    case 10:
-      return (v * a.hs_inv_scale) * Clamp0(v + a.hs_offset, a.hs_threshold);
-    default:
-      return v;
-  }
-}
-
-// Same, with the activation fixed at compile time; DispatchAct turns the
-// run-time type into that constant once per kernel instead of once per value.
-template <int ACT>
-__device__ __forceinline__ float ActivateT(float v, const DevAct& a) {
-  if (ACT == 1) return fmaxf(v, 0.0f);
-  if (ACT == 2) return Clamp0(v, a.relu6_coef);
-  if (ACT == 4) return (v >= 0.0f) ? v : v * a.leaky_alpha;
-  if (ACT == 10) return (v * a.hs_inv_scale) * Clamp0(v + a.hs_offset, a.hs_threshold);
-  return v;
-}
-
-template <typename F>
-__device__ __forceinline__ void DispatchAct(int type, F&& f) {
-  switch (type) {
-    case 1:
-      f(std::integral_constant<int, 1>());
-      break;
-    case 2:
-      f(std::integral_constant<int, 2>());
-      break;
-    case 4:
-      f(std::integral_constant<int, 4>());
-      break;
-    case 10:
-      f(std::integral_constant<int, 10>());
-      break;
-    default:
-      f(std::integral_constant<int, 0>());
-      break;
-  }
-}
-
-// max(v, -127), round half away from zero, min(., 127).  The bounds are
-// integers, so clamping first gives the same result; rounding half away from
-// zero is the truncated sum with the largest float below one half (adding one
-// half itself would carry 0.49999997 up to 1).
-__device__ __forceinline__ int QuantizeI8(float v) {
-  v = __builtin_amdgcn_fmed3f(v, -127.0f, 127.0f);
-  return static_cast<int>(v + __builtin_copysignf(0x1.fffffep-2f, v));
-}
-
-// Activation and quantisation of one value.  relu followed by the clamp is
-// one median, and its result has no sign to copy.
-template <int ACT>
-__device__ __forceinline__ int ActQuantI8(float v, const DevAct& a) {
-  if (ACT == 1) return static_cast<int>(__builtin_amdgcn_fmed3f(v, 0.0f, 127.0f) + 0x1.fffffep-2f);
-  if (ACT < 0) return QuantizeI8(Activate(v, a));
-  return QuantizeI8(ActivateT<(ACT < 0 ? 0 : ACT)>(v, a));
-}
-
-// Low bytes of four quantized values as one dword (a in byte 0).
-__device__ __forceinline__ uint32_t PackI8x4(int a, int b, int c, int d) {
-  // perm(hi, lo, sel): selector 0-3 = byte of lo, 4-7 = byte of hi, 0x0c = zero
-  const uint32_t ab = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);
-  const uint32_t cd = __builtin_amdgcn_perm((uint32_t)d, (uint32_t)c, 0x0c0c0400u);
-  return __builtin_amdgcn_perm(cd, ab, 0x05040100u);
-}
+using namespace epilogue;  // activation, quantisation, packing (epilogue.h)
 
 // 4x4 byte transpose: r[i] holds bytes (i, 0..3); on return r[j] holds bytes
 // (0..3, j).
