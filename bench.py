@@ -29,7 +29,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib"])
+    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib", "mobilenet"])
     ap.add_argument("--algo", default="auto", choices=["auto", "walk", "mfma"])
     ap.add_argument("--fp16", action="store_true", help="run an fp32 configuration (c1, c2) through the half-precision kernel")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -270,6 +270,106 @@ def run_c5(args):
     return 0
 
 
+def run_mobilenet(args):
+    """The convolutional body of MobileNetV1-1.0 at batch 64 in int8: thirteen
+    times (depthwise 3x3, relu) then (pointwise 1x1 through sparse_conv2d, 90 %
+    zeros, relu), every layer consuming the previous layer's int8 output: 26
+    launches per step.  Every layer is compared with the oracle on the first
+    two images of its actual input.  Not the headline metric: printed as its
+    own JSON line."""
+    import numpy as np
+    import torch
+
+    import helpers
+    from oracle import oracle as O
+
+    capi, wl, pla = helpers.capi, helpers.workloads, helpers.pla
+    L = capi.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    batch = 64
+    rng = np.random.RandomState(5)
+    x = torch.from_numpy(rng.randint(-127, 128, size=(batch, 32, 112, 112)).astype(np.int8)).cuda()
+    steps_list = []  # (kind, name, launch, bytes)
+    keep = []
+    total_bytes = 0.0
+    nonzero = []
+    for i in range(13):
+        dwc = wl.config5_depthwise_layer(i)
+        param = pla.ConvParam(dwc.filter, dwc.bias, strides=(dwc.stride, dwc.stride), paddings=(1, 1, 1, 1), activation_param=dwc.act, input_scale=dwc.input_scale,
+                              weight_scale=dwc.weight_scale, output_scale=dwc.output_scale)
+        dw = pla.DepthwiseConv(param, out_precision="int8")
+        dw.PrepareForRun()
+        t = dw.Run(x)
+        torch.cuda.synchronize()
+        a = O.Act()
+        a.type = 1
+        want = O.dwconv3x3_int8(x[:2].cpu().numpy(), dwc.filter[:, 0], dw.w_scale_, dw.bias_, a, out="int8", stride=dwc.stride, pad=1)
+        assert np.array_equal(t[:2].cpu().numpy(), want), "depthwise layer %d differs from the oracle" % (i + 1)
+        dw_bytes = dwc.algorithmic_bytes(batch)
+        steps_list.append(("depthwise", dwc.name, (lambda k=dw, xi=x, ti=t: k.Run(xi, ti)), dw_bytes))
+        case = wl.config5_layer(i)
+        kernel, weights = helpers.make_kernel(case)
+        ic, oc, hw = wl.MOBILENET_V1_POINTWISE[i]
+        out = torch.empty((batch, oc, hw, hw), dtype=torch.int8, device="cuda")
+        capi.check(L.pl_sparse_conv_run(kernel._handle, t.data_ptr(), out.data_ptr(), batch, hw * hw, C.c_void_p(stream)))
+        torch.cuda.synchronize()
+        assert np.array_equal(out[:2].cpu().numpy(), helpers.run_oracle(case, x=t[:2].cpu().numpy())), "pointwise layer %d differs from the oracle" % (i + 1)
+        pw_bytes = case.algorithmic_bytes(weights)
+        steps_list.append(("pointwise", case.name, (lambda h=kernel._handle, ti=t, oi=out, n=hw * hw: capi.check(L.pl_sparse_conv_run(h, ti.data_ptr(), oi.data_ptr(), batch, n, C.c_void_p(stream)))), pw_bytes))
+        keep.append((dw, kernel, t, out))
+        nonzero.append(round(float((out != 0).float().mean().item()), 3))
+        total_bytes += dw_bytes + pw_bytes
+        x = out
+
+    def sequence():
+        for _, _, launch, _ in steps_list:
+            launch()
+
+    per_layer = []
+    for kind, name, launch, nbytes in steps_list:
+        for _ in range(10):
+            launch()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(50):
+            launch()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / 50
+        per_layer.append({"layer": name, "kind": kind, "kernel_us": round(us, 2), "frac": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 3)})
+    for _ in range(max(1, args.warmup // 26)):
+        sequence()
+    torch.cuda.synchronize()
+    steps = max(1, args.steps // 26)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        sequence()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    seq_us = e0.elapsed_time(e1) * 1e3 / steps
+    dw_us = sum(p["kernel_us"] for p in per_layer if p["kind"] == "depthwise")
+    pw_us = sum(p["kernel_us"] for p in per_layer if p["kind"] == "pointwise")
+    print(json.dumps({
+        "metric": "MobileNetV1-1.0 convolutional body, int8, batch 64: images/s of the 26-launch sequence",
+        "value": batch * steps / wall,
+        "unit": "images/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "ms_per_step": wall * 1e3 / steps,
+        "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": "mobilenet_v1_body_int8", "batch": batch, "launches": 26, "pointwise_sparsity": 0.9, "parity_checked": True},
+        "roofline": {"bound": "hbm", "achieved": total_bytes / (seq_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": total_bytes / (seq_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_sequence": total_bytes, "sequence_us": seq_us, "sum_depthwise_kernel_us": round(dw_us, 1), "sum_pointwise_kernel_us": round(pw_us, 1)},
+        "per_layer": per_layer,
+        "nonzero_fraction_of_pointwise_outputs": nonzero,
+    }))
+    return 0
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -289,6 +389,8 @@ def main():
         return run_c5(args)
     if args.config == "calib":
         return run_calib(args)
+    if args.config == "mobilenet":
+        return run_mobilenet(args)
     case = wl.CONFIGS[args.config]()
     if args.fp16:
         if case.kind != capi.KIND_FP32:

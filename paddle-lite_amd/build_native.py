@@ -100,9 +100,11 @@ LITE_SOURCES = [
     "operators/sparse_conv_op.cc",
     "operators/io_copy_op.cc",
     "operators/calib_op.cc",
+    "operators/conv_op.cc",
     "kernels/hip/sparse_conv_compute.cc",
     "kernels/hip/io_copy_compute.cc",
     "kernels/hip/calib_compute.cc",
+    "kernels/hip/conv_depthwise.cc",
 ]
 
 

@@ -65,6 +65,26 @@ struct SparseConvParam : ParamBase {
   int bit_length{8};
 };
 
+// The fields of the reference's ConvParam that the int8 depthwise kernels
+// read (lite/operators/op_params.h ConvParam), same names and defaults.
+struct ConvParam : ParamBase {
+  const lite::Tensor* x{};
+  lite::Tensor* filter{};
+  lite::Tensor* bias{nullptr};
+  lite::Tensor* output{};
+  std::vector<int> strides{1, 1};
+  std::shared_ptr<std::vector<int>> paddings;
+  int groups{1};
+  std::shared_ptr<std::vector<int>> dilations;
+  bool fuse_relu{false};
+  ActivationParam activation_param;
+  bool enable_int8{false};
+  float input_scale{1.0f};
+  std::vector<float> weight_scale{};
+  float output_scale{1.0f};
+  int bit_length{8};
+};
+
 // reference: lite/operators/op_params.h (IoCopyParam)
 struct IoCopyParam : ParamBase {
   const lite::Tensor* x{};

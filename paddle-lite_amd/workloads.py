@@ -126,4 +126,48 @@ def config5_layer(index, batch=64, sparsity=0.90):
     return c
 
 
+# stride of the depthwise 3x3 layer in front of each pointwise layer above
+MOBILENET_V1_DEPTHWISE_STRIDES = [1, 2, 1, 2, 1, 2, 1, 1, 1, 1, 1, 2, 1]
+
+
+class DepthwiseCase(object):
+    """One int8 depthwise 3x3 layer (padding 1, relu): filter [C, 1, 3, 3],
+    per-channel weight scales, bias, input / output scales."""
+
+    def __init__(self, name, channels, in_size, stride, filt, bias, weight_scale, input_scale, output_scale):
+        self.name = name
+        self.channels, self.in_size, self.stride = channels, in_size, stride
+        self.out_size = (in_size + 2 - 3) // stride + 1
+        self.filter = filt
+        self.bias = bias
+        self.weight_scale = weight_scale
+        self.input_scale = input_scale
+        self.output_scale = output_scale
+        self.act = ActivationParam("relu")
+
+    def algorithmic_bytes(self, batch):
+        """Input + output + filters, scales and biases, each once."""
+        c = self.channels
+        return float(batch * c * (self.in_size ** 2 + self.out_size ** 2) + 9 * c + 8 * c)
+
+
+def config5_depthwise_layer(index, sparsity=0.0):
+    """The depthwise layer in front of pointwise layer `index` (0..12) of
+    MobileNetV1-1.0: channels = that layer's input channels, int8 -> int8,
+    relu.  Filters U{-127..127}, weight scales U[0.001, 0.02], input scale
+    0.01; the output scale keeps the requantised output of typical inputs
+    below saturation: 3 * sigma(acc * scale) / 127 with sigma(acc) =
+    sqrt(9) * 73.3 * 40 (mean |w| of the uniform filters times a mean |x| of 40
+    for inputs that went through a relu)."""
+    ic, _, hw = MOBILENET_V1_POINTWISE[index]
+    stride = MOBILENET_V1_DEPTHWISE_STRIDES[index]
+    rng = np.random.RandomState(300 + index)
+    filt = rng.randint(-127, 128, size=(ic, 1, 3, 3)).astype(np.int8)
+    ws = rng.uniform(0.001, 0.02, size=ic).astype(np.float32)
+    bias = (rng.standard_normal(ic) * 0.1).astype(np.float32)
+    input_scale = 0.01
+    output_scale = float(3.0 * 3.0 * 73.3 * 40.0 * float(np.mean(ws)) * input_scale / 127.0)
+    return DepthwiseCase("c5_dw%02d_%d_%d_s%d" % (index + 1, ic, hw * stride, stride), ic, hw * stride, stride, filt, bias, ws, input_scale, output_scale)
+
+
 CONFIGS = {"c1": config1, "c2": config2, "c3": config3, "c4": config4}

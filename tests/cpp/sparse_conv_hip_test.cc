@@ -20,6 +20,7 @@
 #include "lite/core/optimizer/mir/sparse_conv_detect_pass.h"
 #include "lite/kernels/hip/sparse_conv_compute.h"
 #include "lite/model_parser/model_parser.h"
+#include "lite/operators/conv_op.h"
 #include "lite/operators/sparse_conv_op.h"
 #include "pl_sparse_conv.h"
 #include "sparse_conv_oracle.h"
@@ -721,6 +722,105 @@ static void ModelFile(bool run_on_device) {
   }
 }
 
+// depthwise_conv2d (int8, 3x3) through the op and the registered kHIP
+// kernels, against the oracle with the parameters merged as the reference's
+// DepthwiseConv::PrepareForRun merges them.
+static void Depthwise(bool run_on_device) {
+  std::printf("case depthwise 3x3\n");
+  std::fflush(stdout);
+  struct Dw {
+    int n, c, h, w, stride, pad;
+    bool out_int8;
+    std::string act;
+    unsigned seed;
+  };
+  const std::vector<Dw> cases = {{2, 16, 14, 14, 1, 1, true, "relu", 41}, {2, 8, 15, 13, 2, 1, true, "relu6", 42}, {1, 5, 9, 6, 1, 0, false, "leaky_relu", 43}, {2, 32, 7, 7, 2, 1, false, "", 44}};
+  for (const Dw& q : cases) {
+    std::mt19937 gen(q.seed);
+    std::uniform_real_distribution<float> uni(0.f, 1.f);
+    Scope scope;
+    Tensor* x = scope.NewTensor("x");
+    x->Resize({q.n, q.c, q.h, q.w});
+    int8_t* xd = x->mutable_data<int8_t>(TargetType::kHost);
+    for (int64_t i = 0; i < x->numel(); ++i) xd[i] = static_cast<int8_t>(static_cast<int>(uni(gen) * 255.f) - 127);
+    Tensor* f = scope.NewTensor("dw_w");
+    f->Resize({q.c, 1, 3, 3});
+    int8_t* fd = f->mutable_data<int8_t>(TargetType::kHost);
+    for (int64_t i = 0; i < f->numel(); ++i) fd[i] = static_cast<int8_t>(static_cast<int>(uni(gen) * 255.f) - 127);
+    Tensor* b = scope.NewTensor("dw_b");
+    b->Resize({q.c});
+    float* bd = b->mutable_data<float>(TargetType::kHost);
+    for (int i = 0; i < q.c; ++i) bd[i] = uni(gen) - 0.5f;
+    scope.NewTensor("y");
+    std::vector<float> ws(q.c);
+    for (float& v : ws) v = 0.002f + 0.018f * uni(gen);
+    const float in_scale = 0.02f, out_scale = q.out_int8 ? 0.11f : 1.f;
+    OpInfo info("depthwise_conv2d");
+    info.SetInput("Input", {"x"});
+    info.SetInput("Filter", {"dw_w"});
+    info.SetInput("Bias", {"dw_b"});
+    info.SetOutput("Output", {"y"});
+    info.SetAttr<std::vector<int>>("strides", {q.stride, q.stride});
+    info.SetAttr<std::vector<int>>("paddings", {q.pad, q.pad});
+    info.SetAttr<std::vector<int>>("dilations", {1, 1});
+    info.SetAttr<int>("groups", q.c);
+    if (!q.act.empty()) {
+      info.SetAttr<bool>("with_act", true);
+      info.SetAttr<std::string>("act_type", q.act);
+      info.SetAttr<float>("fuse_brelu_threshold", 6.f);
+      info.SetAttr<float>("leaky_relu_alpha", 0.1f);
+    }
+    info.SetAttr<bool>("enable_int8", true);
+    info.SetInputScale("Input0_scale", {in_scale}, true);
+    info.SetInputScale("Filter0_scale", ws, true);
+    info.SetOutputScale("Output0_scale", {out_scale}, true);
+
+    auto op = LiteOpRegistry::Global().Create("depthwise_conv2d");
+    EXPECT(op != nullptr);
+    EXPECT(op->Attach(info, &scope) && op->CheckShape() && op->InferShape());
+    const int oh = (q.h + 2 * q.pad - 3) / q.stride + 1, ow = (q.w + 2 * q.pad - 3) / q.stride + 1;
+    Tensor* y = scope.FindMutableTensor("y");
+    EXPECT(y->dims() == DDim({q.n, q.c, oh, ow}));
+    if (!run_on_device) {
+      EXPECT(KernelRegistry::Global().Create("depthwise_conv2d", TARGET(kHIP), PRECISION(kInt8), DATALAYOUT(kNCHW)).size() == 2u);
+      continue;
+    }
+    OpInfo h2d("io_copy");
+    h2d.SetInput("Input", {"x"});
+    h2d.SetOutput("Out", {"x_dev"});
+    auto copy_op = LiteOpRegistry::Global().Create("io_copy");
+    EXPECT(copy_op->Attach(h2d, &scope) && copy_op->InferShape());
+    auto copy_kernels = copy_op->CreateKernels({paddle::lite_api::Place(TARGET(kHIP), PRECISION(kAny), DATALAYOUT(kAny))}, "io_copy/host_to_device");
+    copy_kernels[0]->Launch();
+    info.SetInput("Input", {"x_dev"});
+    EXPECT(op->Attach(info, &scope) && op->InferShape());
+    auto kernels = op->CreateKernels({paddle::lite_api::Place(TARGET(kHIP), PRECISION(kInt8), DATALAYOUT(kNCHW))}, std::string("depthwise_conv2d/") + (q.out_int8 ? "int8_out" : "fp32_out"));
+    EXPECT(kernels.size() == 1);
+    if (kernels.size() != 1) continue;
+    kernels[0]->Launch();
+    kernels[0]->Launch();
+    kernels[0]->mutable_context_as<HIPContext>()->Sync();
+    Tensor y_host;
+    y_host.CopyDataFrom(*y, TargetType::kHost);
+    // merged parameters (conv_depthwise.cc:158-200, :257-322)
+    std::vector<float> ms(q.c), mb(q.c);
+    for (int i = 0; i < q.c; ++i) {
+      ms[i] = q.out_int8 ? ws[i] * in_scale / out_scale : ws[i] * in_scale;
+      mb[i] = q.out_int8 ? bd[i] / out_scale : bd[i];
+    }
+    plo_act act{ActCode(q.act), q.out_int8 ? 6.f / out_scale : 6.f, 0.1f, 6.f, 3.f, 6.f};
+    if (q.out_int8) {
+      std::vector<int8_t> want(static_cast<size_t>(q.n) * q.c * oh * ow);
+      EXPECT(plo_dwconv3x3_int8(xd, fd, ms.data(), mb.data(), &act, 2, q.n, q.c, q.h, q.w, q.stride, q.pad, want.data()) == 0);
+      EXPECT(y_host.memory_size() == want.size() && std::memcmp(want.data(), y_host.raw_data(), want.size()) == 0);
+    } else {
+      std::vector<float> want(static_cast<size_t>(q.n) * q.c * oh * ow);
+      EXPECT(plo_dwconv3x3_int8(xd, fd, ms.data(), mb.data(), &act, 1, q.n, q.c, q.h, q.w, q.stride, q.pad, want.data()) == 0);
+      EXPECT(y_host.memory_size() == want.size() * 4 && std::memcmp(want.data(), y_host.raw_data(), want.size() * 4) == 0);
+    }
+  }
+}
+
 int main(int argc, char** argv) {
   const bool gpu = argc > 1 && std::string(argv[1]) == "--gpu";
   RegistryAndErrorPaths();
@@ -744,6 +844,7 @@ int main(int argc, char** argv) {
   Int8Chain(gpu);
   HalfPrecision(gpu);
   ModelFile(gpu);
+  Depthwise(gpu);
   std::printf("%s: %d failure(s)\n", gpu ? "gpu" : "cpu", g_failures);
   return g_failures ? 1 : 0;
 }
