@@ -51,8 +51,10 @@ std::vector<ProgramStep> Int8ChainPass::Apply(const std::vector<OpInfo>& ops, co
 
   for (size_t i = 0; i < ops.size(); ++i) {
     OpInfo op = ops[i];
-    CHECK(op.Type() == "sparse_conv2d") << "this pass handles chains of sparse_conv2d, got " << op.Type();
+    const bool depthwise = op.Type() == "depthwise_conv2d";
+    CHECK(op.Type() == "sparse_conv2d" || depthwise) << "this pass handles chains of sparse_conv2d and depthwise_conv2d, got " << op.Type();
     const bool int8 = IsInt8Op(op);
+    CHECK(int8 || !depthwise) << "depthwise_conv2d has int8 kernels only on this target";
     const std::string in = op.Input("Input").front();
     const std::string out = op.Output("Output").front();
     CHECK(vars.count(in) != 0) << "input " << in << " of op " << i << " has no producer and is not fed";
@@ -97,7 +99,9 @@ std::vector<ProgramStep> Int8ChainPass::Apply(const std::vector<OpInfo>& ops, co
 
     ProgramStep s;
     s.op = op;
-    s.kernel = std::string("sparse_conv2d/") + (!int8 ? "def" : (out_int8 ? "int8_int8_out" : "int8_fp32_out"));
+    // aliases as the reference registers them (sparse_conv_compute.cc:393-430, conv_compute.cc:252-300)
+    s.kernel = depthwise ? std::string("depthwise_conv2d/") + (out_int8 ? "int8_out" : "fp32_out")
+                         : std::string("sparse_conv2d/") + (!int8 ? "def" : (out_int8 ? "int8_int8_out" : "int8_fp32_out"));
     s.place = lite_api::Place(TARGET(kHIP), int8 ? PRECISION(kInt8) : PRECISION(kFloat), DATALAYOUT(kNCHW));
     steps.push_back(s);
     vars[out] = VarState{true, out_int8, out};

@@ -1,5 +1,6 @@
 // What the reference's optimiser does around quantised ops, restated for a
-// linear list of sparse_conv2d ops that all run on TARGET(kHIP):
+// linear list of sparse_conv2d and int8 depthwise_conv2d ops that all run on
+// TARGET(kHIP):
 //  * the output-type rule of static_kernel_pick_pass
 //    (lite/core/optimizer/mir/static_kernel_pick_pass.cc:97-135): an op with
 //    enable_int8 produces int8 only if every consumer of its output has
@@ -37,7 +38,7 @@ struct ProgramStep {
 
 class Int8ChainPass {
  public:
-  // `ops`: sparse_conv2d ops in execution order (after SparseConvDetectPass).
+  // `ops`: sparse_conv2d / depthwise_conv2d ops in execution order (after SparseConvDetectPass).
   // `feeds`: fp32 host tensors in `scope`.  `fetches`: variables wanted back
   // on the host as fp32; the host copy of "v" is named "v/host".
   std::vector<ProgramStep> Apply(const std::vector<OpInfo>& ops, const std::vector<std::string>& feeds, const std::vector<std::string>& fetches, Scope* scope) const;

@@ -821,6 +821,195 @@ static void Depthwise(bool run_on_device) {
   }
 }
 
+// Two MobileNet blocks (depthwise 3x3 then pointwise 1x1, twice; the second
+// depthwise layer has stride 2): conv2d -> sparse_conv2d by the detect pass,
+// the whole program saved as a model file and loaded into an empty scope,
+// precision and target casts placed by the chain pass, run on the device from
+// an fp32 feed to an fp32 fetch, and compared with the oracle's chain.
+static void MobileNetBlocks(bool run_on_device) {
+  std::printf("mobilenet blocks from a model file\n");
+  std::fflush(stdout);
+  const int batch = 2, size0 = 12;
+  const int ch[3] = {24, 40, 56};            // channels: input, after block 1, after block 2
+  const int dw_stride[2] = {1, 2};
+  // input scale of: dw1, pw1, dw2, pw2
+  const float in_scale[4] = {0.02f, 0.03f, 0.025f, 0.04f};
+  Scope scope;
+  std::mt19937 gen(99);
+  std::uniform_real_distribution<float> uni(0.f, 1.f);
+  Tensor* a0 = scope.NewTensor("t0");
+  a0->Resize({batch, ch[0], size0, size0});
+  float* a0d = a0->mutable_data<float>(TargetType::kHost);
+  for (int64_t i = 0; i < a0->numel(); ++i) a0d[i] = uni(gen) * 2.f - 1.f;
+  std::vector<float> feed(a0d, a0d + a0->numel());
+  std::vector<OpInfo> ops;
+  std::vector<std::vector<int8_t>> dw_w(2), pw_w(2);
+  std::vector<std::vector<float>> dw_ws(2), pw_ws(2), dw_b(2), pw_b(2);
+  int size = size0;
+  cpp::ProgramDesc prog;
+  cpp::BlockDesc* block = prog.AddBlock();
+  block->SetParentIdx(-1);
+  auto add_var = [&](const std::string& name, bool persistable, VarDataType dt, const std::vector<int64_t>& shape) {
+    cpp::VarDesc* v = block->AddVar();
+    v->SetName(name);
+    v->SetPersistable(persistable);
+    v->SetDataType(dt);
+    v->SetShape(shape);
+  };
+  add_var("t0", false, VarDataType::FP32, {batch, ch[0], size0, size0});
+  for (int l = 0; l < 2; ++l) {
+    const int c = ch[l], oc = ch[l + 1];
+    const std::string n = std::to_string(l + 1);
+    const int out_size = (size + 2 - 3) / dw_stride[l] + 1;
+    // depthwise
+    Tensor* f = scope.NewTensor("dw_w" + n);
+    f->Resize({c, 1, 3, 3});
+    int8_t* fd = f->mutable_data<int8_t>(TargetType::kHost);
+    for (int64_t i = 0; i < f->numel(); ++i) fd[i] = static_cast<int8_t>(static_cast<int>(uni(gen) * 255.f) - 127);
+    dw_w[l].assign(fd, fd + f->numel());
+    Tensor* b = scope.NewTensor("dw_b" + n);
+    b->Resize({c});
+    float* bd = b->mutable_data<float>(TargetType::kHost);
+    dw_b[l].resize(c);
+    for (int i = 0; i < c; ++i) dw_b[l][i] = bd[i] = uni(gen) - 0.5f;
+    dw_ws[l].resize(c);
+    for (float& v : dw_ws[l]) v = 0.0005f + 0.001f * uni(gen);
+    OpInfo dw("depthwise_conv2d");
+    dw.SetInput("Input", {"t" + std::to_string(2 * l)});
+    dw.SetInput("Filter", {"dw_w" + n});
+    dw.SetInput("Bias", {"dw_b" + n});
+    dw.SetOutput("Output", {"t" + std::to_string(2 * l + 1)});
+    dw.SetAttr<std::vector<int>>("strides", {dw_stride[l], dw_stride[l]});
+    dw.SetAttr<std::vector<int>>("paddings", {1, 1});
+    dw.SetAttr<std::vector<int>>("dilations", {1, 1});
+    dw.SetAttr<int>("groups", c);
+    dw.SetAttr<bool>("with_act", true);
+    dw.SetAttr<std::string>("act_type", "relu");
+    dw.SetAttr<bool>("enable_int8", true);
+    dw.SetInputScale("Input0_scale", {in_scale[2 * l]}, true);
+    dw.SetInputScale("Filter0_scale", dw_ws[l], true);
+    dw.SetOutputScale("Output0_scale", {1.f}, true);
+    ops.push_back(dw);
+    add_var("dw_w" + n, true, VarDataType::INT8, {c, 1, 3, 3});
+    add_var("dw_b" + n, true, VarDataType::FP32, {c});
+    add_var("t" + std::to_string(2 * l + 1), false, VarDataType::FP32, {batch, c, out_size, out_size});
+    // pointwise
+    Tensor* w = scope.NewTensor("pw_w" + n);
+    w->Resize({oc, c, 1, 1});
+    int8_t* wd = w->mutable_data<int8_t>(TargetType::kHost);
+    for (int64_t i = 0; i < w->numel(); ++i) {
+      int v = static_cast<int>(uni(gen) * 127.f) + 1;
+      if (uni(gen) < 0.5f) v = -v;
+      wd[i] = uni(gen) >= 0.7f ? static_cast<int8_t>(v) : 0;
+    }
+    pw_w[l].assign(wd, wd + w->numel());
+    Tensor* pb = scope.NewTensor("pw_b" + n);
+    pb->Resize({oc});
+    float* pbd = pb->mutable_data<float>(TargetType::kHost);
+    pw_b[l].resize(oc);
+    for (int i = 0; i < oc; ++i) pw_b[l][i] = pbd[i] = (uni(gen) - 0.5f) * 0.2f;
+    pw_ws[l].resize(oc);
+    for (float& v : pw_ws[l]) v = 0.001f + 0.004f * uni(gen);
+    OpInfo conv("conv2d");
+    conv.SetInput("Input", {"t" + std::to_string(2 * l + 1)});
+    conv.SetInput("Filter", {"pw_w" + n});
+    conv.SetInput("Bias", {"pw_b" + n});
+    conv.SetOutput("Output", {"t" + std::to_string(2 * l + 2)});
+    conv.SetAttr<std::vector<int>>("strides", {1, 1});
+    conv.SetAttr<std::vector<int>>("paddings", {0, 0});
+    conv.SetAttr<std::vector<int>>("dilations", {1, 1});
+    conv.SetAttr<int>("groups", 1);
+    conv.SetAttr<bool>("with_act", true);
+    conv.SetAttr<std::string>("act_type", "relu");
+    conv.SetAttr<bool>("enable_int8", true);
+    conv.SetInputScale("Input0_scale", {in_scale[2 * l + 1]}, true);
+    conv.SetInputScale("Filter0_scale", pw_ws[l], true);
+    conv.SetOutputScale("Output0_scale", {1.f}, true);
+    ops.push_back(conv);
+    // the detect pass reads the spatial size of the conv input from its tensor
+    scope.NewTensor("t" + std::to_string(2 * l + 1))->Resize({batch, c, out_size, out_size});
+    scope.NewTensor("t" + std::to_string(2 * l + 2));
+    add_var("pw_b" + n, true, VarDataType::FP32, {oc});
+    add_var("t" + std::to_string(2 * l + 2), false, VarDataType::FP32, {batch, oc, out_size, out_size});
+    size = out_size;
+  }
+  mir::SparseConvDetectPass detect;
+  detect.SetSparseThreshold(0.5f);
+  EXPECT(detect.Apply(&ops, &scope) == 2);  // the two pointwise layers; the depthwise ops are left alone
+  EXPECT(ops[0].Type() == "depthwise_conv2d" && ops[1].Type() == "sparse_conv2d");
+  for (int l = 0; l < 2; ++l) {
+    const std::string n = std::to_string(l + 1);
+    const OpInfo& sp = ops[2 * l + 1];
+    const Tensor* nz = scope.FindMutableTensor(sp.Input("NonZeroWeights").front());
+    const Tensor* dif = scope.FindMutableTensor(sp.Input("Diffs").front());
+    add_var(sp.Input("NonZeroWeights").front(), true, VarDataType::INT8, nz->dims().Vectorize());
+    add_var(sp.Input("OcNonZeros").front(), true, VarDataType::INT32, {ch[l + 1]});
+    add_var(sp.Input("Diffs").front(), true, VarDataType::INT32, dif->dims().Vectorize());
+  }
+  for (const OpInfo& op : ops) *block->AddOp() = op;
+
+  // through a model file into an empty scope
+  const std::string base = "/tmp/pl_mobilenet_blocks_" + std::to_string(static_cast<long>(getpid()));
+  SaveModelNaive(base, scope, prog);
+  Scope loaded;
+  cpp::ProgramDesc back;
+  LoadModelNaiveFromFile(base + ".nb", &loaded, &back);
+  std::remove((base + ".nb").c_str());
+  EXPECT(back.BlocksSize() == 1 && back.GetBlock(0)->OpsSize() == 4);
+  if (back.BlocksSize() != 1 || back.GetBlock(0)->OpsSize() != 4) return;
+  EXPECT(loaded.FindVar("pw_w1") == nullptr && loaded.FindVar("dw_w1") != nullptr);  // dense pointwise filters are gone
+  loaded.NewTensor("t0")->Assign<float>(feed.data(), DDim({batch, ch[0], size0, size0}));
+  mir::Int8ChainPass chain;
+  std::vector<mir::ProgramStep> steps = chain.Apply(back.GetBlock(0)->ops(), {"t0"}, {"t4"}, &loaded);
+  EXPECT(steps.size() == 7);
+  if (steps.size() == 7) {
+    EXPECT(steps[1].kernel == "calib/fp32_to_int8" && steps[2].kernel == "depthwise_conv2d/int8_out" && steps[3].kernel == "sparse_conv2d/int8_int8_out");
+    EXPECT(steps[4].kernel == "depthwise_conv2d/int8_out" && steps[5].kernel == "sparse_conv2d/int8_fp32_out" && steps[6].kernel == "io_copy/device_to_host");
+    EXPECT(steps[2].op.GetOutputScale("Output0_scale", true)[0] == in_scale[1]);
+  }
+  if (!run_on_device) return;
+  mir::HipProgram program(steps, &loaded);
+  program.Run();
+  program.Run();
+  const Tensor* got = loaded.FindMutableTensor("t4/host");
+  EXPECT(got != nullptr);
+  if (!got) return;
+
+  // oracle chain
+  std::vector<int8_t> q(feed.size());
+  plo_fp32_to_int8(feed.data(), q.data(), in_scale[0], static_cast<int64_t>(feed.size()));
+  std::vector<float> want;
+  size = size0;
+  plo_act relu{1, 6.f, 0.1f, 6.f, 3.f, 6.f};
+  for (int l = 0; l < 2; ++l) {
+    const int c = ch[l], oc = ch[l + 1];
+    const int out_size = (size + 2 - 3) / dw_stride[l] + 1;
+    const float dw_out = in_scale[2 * l + 1];
+    std::vector<float> ms(c), mb(c);
+    for (int i = 0; i < c; ++i) {
+      ms[i] = dw_ws[l][i] * in_scale[2 * l] / dw_out;
+      mb[i] = dw_b[l][i] / dw_out;
+    }
+    std::vector<int8_t> t(static_cast<size_t>(batch) * c * out_size * out_size);
+    EXPECT(plo_dwconv3x3_int8(q.data(), dw_w[l].data(), ms.data(), mb.data(), &relu, 2, batch, c, size, size, dw_stride[l], 1, t.data()) == 0);
+    const int hw = out_size * out_size;
+    std::vector<float> ps(oc), pb(oc);
+    plo_act act = relu;
+    const bool last = l == 1;
+    EXPECT(plo_merge_params(last ? 1 : 2, oc, pw_ws[l].data(), oc, in_scale[2 * l + 1], last ? 1.f : in_scale[2 * l + 2], pw_b[l].data(), ps.data(), pb.data(), &act) == 0);
+    if (!last) {
+      std::vector<int8_t> next(static_cast<size_t>(batch) * oc * hw);
+      plo_dense_conv1x1(2, pw_w[l].data(), t.data(), pb.data(), ps.data(), next.data(), batch, oc, c, hw, &act, 1);
+      q.swap(next);
+    } else {
+      want.resize(static_cast<size_t>(batch) * oc * hw);
+      plo_dense_conv1x1(1, pw_w[l].data(), t.data(), pw_b[l].data(), ps.data(), want.data(), batch, oc, c, hw, &act, 1);
+    }
+    size = out_size;
+  }
+  EXPECT(got->memory_size() == want.size() * 4 && std::memcmp(want.data(), got->raw_data(), want.size() * 4) == 0);
+}
+
 int main(int argc, char** argv) {
   const bool gpu = argc > 1 && std::string(argv[1]) == "--gpu";
   RegistryAndErrorPaths();
@@ -845,6 +1034,7 @@ int main(int argc, char** argv) {
   HalfPrecision(gpu);
   ModelFile(gpu);
   Depthwise(gpu);
+  MobileNetBlocks(gpu);
   std::printf("%s: %d failure(s)\n", gpu ? "gpu" : "cpu", g_failures);
   return g_failures ? 1 : 0;
 }
