@@ -21,9 +21,10 @@ struct DwConvParams {
   uint32_t planes;         // batch * channels
   int64_t in_bytes;        // planes * h * w
   DevAct act;
+  int item_rows;           // output rows per thread: 2 or 4, 0 = chosen by the launcher
   // filled in by the launcher
-  int groups_w;            // ceil(ow / 4): a thread makes four neighbouring outputs of R rows (R = 2 or 4)
-  int items;               // ceil(oh / R) * groups_w per plane
+  int groups_w;            // column groups per output row
+  int items;               // ceil(oh / rows) * groups_w per plane
   int planes_per_block;    // several small planes share a workgroup
   int blocks_per_plane;    // a plane above 256 items is cut into pieces of 256
   uint32_t magic_items;    // ceil(2^32 / items) for items >= 2: x / items == mulhi(x, magic) for x * items < 2^32

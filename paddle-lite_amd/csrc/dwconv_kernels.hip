@@ -35,63 +35,63 @@ __device__ __forceinline__ uint32_t LoadBytes4(const int8_t* ptr, const int8_t* 
   return v;
 }
 
-// One item: the outputs ox0 .. ox0+3 (ox0 = 4g) of the output rows R*oyr ..
-// R*oyr + R-1 of one plane.  Window byte i of an input row is column col0 + i
-// with col0 = STRIDE * ox0 - pad; output k multiplies window bytes STRIDE*k ..
-// STRIDE*k + 2.  The window is cut from the dwords A, B, C that start at
-// columns cb - 4, cb, cb + 4, cb = col0 + 1 (for stride 1 and padding 1 that is
-// column 4g: B holds the inputs right under the thread's outputs).
+// One item: 4 * CG neighbouring outputs (from column ox0 = 4 * CG * g) of the
+// R output rows R*oyr .. R*oyr + R-1 of one plane.  With col0 = STRIDE * ox0 -
+// pad the column of the first input under the first output, the item reads,
+// per input row, the K dwords that start at columns cb - 4, cb, cb + 4, ...
+// (cb = col0 + 1; for stride 1 and padding 1 that is column ox0 itself).
+// Output j multiplies the three bytes from column col0 + STRIDE * j on: they
+// are the low bytes of the dword pair (k, k + 1) shifted right by sh bytes,
+// k = (STRIDE*j + 3) / 4, sh = (STRIDE*j + 3) % 4, both compile-time values.
 // Neighbouring output rows share 2 of their 3 input rows at stride 1 (1 of 3
 // at stride 2).
-template <int STRIDE, int R, int OUT, int ACT, bool SAFE>
+template <int STRIDE, int R, int CG, int OUT, int ACT, bool SAFE>
 __device__ __forceinline__ void DwItem(const DwConvParams& p, uint32_t plane, int c, int oyr, int g) {
-  constexpr int kRows = 3 + STRIDE * (R - 1);  // input rows under R output rows
-  const int ox0 = 4 * g;
+  constexpr int kRows = 3 + STRIDE * (R - 1);                  // input rows under R output rows
+  constexpr int NOUT = 4 * CG;                                 // outputs per row
+  constexpr int K = (STRIDE * (NOUT - 1) + 3 + 2) / 4 + 1;     // dwords per input row (the last window starts in dword K - 2)
+  const int ox0 = NOUT * g;
   const int cb = STRIDE * ox0 - p.pad + 1;  // 0 <= cb < w for every existing output
   const int8_t* plane_ptr = p.x + (int64_t)plane * (uint32_t)(p.h * p.w);
   // Columns outside [0, w) are zero padding (a dword may also run into the
-  // next row or plane).  A reaches below column 0 only for g == 0: with
-  // padding 1 it is then all padding, without padding its last byte is column 0.
-  const uint32_t mA = g == 0 ? (p.pad ? 0u : 0xff000000u) : 0xffffffffu;
-  const int in_b = p.w - cb;  // >= 1 bytes of B inside the row
-  const uint32_t mB = 0xffffffffu >> (8 * max(4 - in_b, 0));
-  const int in_c = in_b - 4;  // bytes of C inside the row (may be <= 0)
-  const uint32_t mC = in_c <= 0 ? 0u : 0xffffffffu >> (8 * max(4 - in_c, 0));
+  // next row or plane).  Only dword 0 can reach below column 0, and only for
+  // g == 0: with padding 1 it is then all padding, without padding its last
+  // byte is column 0.
+  uint32_t mask[K];
+  mask[0] = g == 0 ? (p.pad ? 0u : 0xff000000u) : 0xffffffffu;
+#pragma unroll
+  for (int k = 1; k < K; ++k) {
+    const int inside = p.w - (cb + 4 * (k - 1));  // bytes of dword k inside the row, from its first byte
+    mask[k] = inside <= 0 ? 0u : 0xffffffffu >> (8 * max(4 - inside, 0));
+  }
   const uint32_t wrow[3] = {p.wpack[4 * c], p.wpack[4 * c + 1], p.wpack[4 * c + 2]};
   const int iy0 = STRIDE * R * oyr - p.pad;
-  int acc[R][4];
+  int acc[R][NOUT];
 #pragma unroll
   for (int o = 0; o < R; ++o)
 #pragma unroll
-    for (int k = 0; k < 4; ++k) acc[o][k] = 0;
-  uint32_t A[kRows], B[kRows], C[kRows];
+    for (int j = 0; j < NOUT; ++j) acc[o][j] = 0;
+  uint32_t D[kRows][K];
 #pragma unroll
   for (int r = 0; r < kRows; ++r) {
     // a row outside [0, h) is zero padding: it reads its neighbour and meets a zero filter row below
     const int8_t* row = plane_ptr + (uint32_t)(min(max(iy0 + r, 0), p.h - 1) * p.w) + cb;
-    A[r] = LoadBytes4<SAFE>(row - 4, p.x, p.x + p.in_bytes);
-    B[r] = LoadBytes4<SAFE>(row, p.x, p.x + p.in_bytes);
-    C[r] = LoadBytes4<SAFE>(row + 4, p.x, p.x + p.in_bytes);
+#pragma unroll
+    for (int k = 0; k < K; ++k) D[r][k] = LoadBytes4<SAFE>(row + 4 * (k - 1), p.x, p.x + p.in_bytes);
   }
 #pragma unroll
   for (int r = 0; r < kRows; ++r) {
     const int iy = iy0 + r;
     const uint32_t row_on = (iy >= 0 && iy < p.h) ? 0xffffffffu : 0u;
-    const uint32_t a = A[r] & mA, b = B[r] & mB, cc = C[r] & mC;
-    // window bytes 0..3 = columns cb-1 .. cb+2, bytes 4..7 = cb+3 .. cb+6
-    const uint32_t win_lo = __builtin_amdgcn_alignbyte(b, a, 3);
-    const uint32_t win_hi = __builtin_amdgcn_alignbyte(cc, b, 3);
-    int win[4];
-    if (STRIDE == 1) {
-      win[0] = (int)win_lo;
-      win[1] = (int)__builtin_amdgcn_alignbyte(win_hi, win_lo, 1);
-      win[2] = (int)__builtin_amdgcn_alignbyte(win_hi, win_lo, 2);
-      win[3] = (int)__builtin_amdgcn_alignbyte(win_hi, win_lo, 3);
-    } else {
-      win[0] = (int)win_lo;
-      win[1] = (int)__builtin_amdgcn_alignbyte(win_hi, win_lo, 2);
-      win[2] = (int)win_hi;
-      win[3] = (int)__builtin_amdgcn_alignbyte(cc >> 24, win_hi, 2);  // cc >> 24: window byte 8 = column cb + 7
+    uint32_t d[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) d[k] = D[r][k] & mask[k];
+    int win[NOUT];
+#pragma unroll
+    for (int j = 0; j < NOUT; ++j) {
+      const int first = STRIDE * j + 3;  // byte index of the window's first byte in the dword sequence
+      const int k = first / 4, sh = first % 4;
+      win[j] = sh == 0 ? (int)d[k] : (int)__builtin_amdgcn_alignbyte(k + 1 < K ? d[k + 1] : 0u, d[k], sh);
     }
 #pragma unroll
     for (int o = 0; o < R; ++o) {
@@ -99,39 +99,44 @@ __device__ __forceinline__ void DwItem(const DwConvParams& p, uint32_t plane, in
       if (fr < 0 || fr > 2) continue;
       const int wr = (int)(wrow[fr] & row_on);
 #pragma unroll
-      for (int k = 0; k < 4; ++k) acc[o][k] = __builtin_amdgcn_sdot4(win[k], wr, acc[o][k], false);
+      for (int j = 0; j < NOUT; ++j) acc[o][j] = __builtin_amdgcn_sdot4(win[j], wr, acc[o][j], false);
     }
   }
   const float s = p.scale[c], b = p.bias[c];
-  const int n_out = min(4, p.ow - ox0);
 #pragma unroll
   for (int o = 0; o < R; ++o) {
     const int oy = R * oyr + o;
     if (oy >= p.oh) break;
-    const size_t at = ((size_t)plane * (uint32_t)p.oh + (uint32_t)oy) * (uint32_t)p.ow + (uint32_t)ox0;
-    if (OUT == kOutI8) {
-      int q[4];
 #pragma unroll
-      for (int k = 0; k < 4; ++k) q[k] = ActQuantI8<ACT>(__builtin_fmaf((float)acc[o][k], s, b), p.act);
-      int8_t* dst = static_cast<int8_t*>(p.out) + at;
-      if (n_out == 4 && (at & 3) == 0) {
-        __builtin_nontemporal_store(PackI8x4(q[0], q[1], q[2], q[3]), reinterpret_cast<uint32_t*>(dst));
+    for (int q4 = 0; q4 < CG; ++q4) {
+      const int ox = ox0 + 4 * q4;
+      const int n_out = min(4, p.ow - ox);
+      if (n_out <= 0) break;
+      const size_t at = ((size_t)plane * (uint32_t)p.oh + (uint32_t)oy) * (uint32_t)p.ow + (uint32_t)ox;
+      if (OUT == kOutI8) {
+        int q[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) q[k] = ActQuantI8<ACT>(__builtin_fmaf((float)acc[o][4 * q4 + k], s, b), p.act);
+        int8_t* dst = static_cast<int8_t*>(p.out) + at;
+        if (n_out == 4 && (at & 3) == 0) {
+          __builtin_nontemporal_store(PackI8x4(q[0], q[1], q[2], q[3]), reinterpret_cast<uint32_t*>(dst));
+        } else {
+#pragma unroll
+          for (int k = 0; k < 4; ++k)
+            if (k < n_out) dst[k] = (int8_t)q[k];
+        }
       } else {
+        float v[4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k)
-          if (k < n_out) dst[k] = (int8_t)q[k];
-      }
-    } else {
-      float v[4];
+        for (int k = 0; k < 4; ++k) v[k] = ActivateT<ACT>(__builtin_fmaf((float)acc[o][4 * q4 + k], s, b), p.act);
+        float* dst = static_cast<float*>(p.out) + at;
+        if (n_out == 4 && (at & 3) == 0) {
+          __builtin_nontemporal_store(v4f{v[0], v[1], v[2], v[3]}, reinterpret_cast<v4f*>(dst));
+        } else {
 #pragma unroll
-      for (int k = 0; k < 4; ++k) v[k] = ActivateT<ACT>(__builtin_fmaf((float)acc[o][k], s, b), p.act);
-      float* dst = static_cast<float*>(p.out) + at;
-      if (n_out == 4 && (at & 3) == 0) {
-        __builtin_nontemporal_store(v4f{v[0], v[1], v[2], v[3]}, reinterpret_cast<v4f*>(dst));
-      } else {
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-          if (k < n_out) dst[k] = v[k];
+          for (int k = 0; k < 4; ++k)
+            if (k < n_out) dst[k] = v[k];
+        }
       }
     }
   }
@@ -141,7 +146,7 @@ __device__ __forceinline__ void DwItem(const DwConvParams& p, uint32_t plane, in
 // wait for later loads only by waiting for the stores as well, so a second
 // item in the same thread would start after the first one's stores have
 // reached memory.
-template <int STRIDE, int R, int OUT, int ACT, bool SAFE>
+template <int STRIDE, int R, int CG, int OUT, int ACT, bool SAFE>
 __device__ __forceinline__ void DwItems(const DwConvParams& p, uint32_t plane0, int v) {
   if (v >= p.planes_per_block * p.items) return;
   const int pl = p.items == 1 ? v : (int)__umulhi((uint32_t)v, p.magic_items);  // v / items
@@ -152,10 +157,10 @@ __device__ __forceinline__ void DwItems(const DwConvParams& p, uint32_t plane0, 
   const int g = item - oyr * p.groups_w;
   int c = (int)(plane0 % (uint32_t)p.channels) + pl;  // the first term is uniform
   if (c >= p.channels) c = p.channels > p.planes_per_block ? c - p.channels : c % p.channels;
-  DwItem<STRIDE, R, OUT, ACT, SAFE>(p, plane, c, oyr, g);
+  DwItem<STRIDE, R, CG, OUT, ACT, SAFE>(p, plane, c, oyr, g);
 }
 
-template <int STRIDE, int R, int OUT, int ACT>
+template <int STRIDE, int R, int CG, int OUT, int ACT>
 __device__ __forceinline__ void DwBody(const DwConvParams& p) {
   // a workgroup takes planes_per_block whole planes, or one of the
   // blocks_per_plane pieces of 256 items of one plane
@@ -163,24 +168,34 @@ __device__ __forceinline__ void DwBody(const DwConvParams& p) {
   const int piece = (int)(blockIdx.x - unit * (uint32_t)p.blocks_per_plane);
   const uint32_t plane0 = unit * (uint32_t)p.planes_per_block;
   const int v = piece * 256 + (int)threadIdx.x;
-  // The dwords A and C reach 4 bytes before and 7 bytes after the window:
-  // only the workgroups with the first and the last plane can leave the tensor
-  // (with planes of at least 8 bytes, so that one neighbouring plane covers the reach)
-  if (plane0 > 0 && plane0 + (uint32_t)p.planes_per_block < p.planes && p.h * p.w >= 8) {
-    DwItems<STRIDE, R, OUT, ACT, true>(p, plane0, v);
+  // The dwords of a row reach 4 bytes before its first column and up to 15
+  // bytes past its last one: only the workgroups with the first and the last
+  // plane can leave the tensor (with planes of at least 16 bytes, so that one
+  // neighbouring plane covers the reach)
+  if (plane0 > 0 && plane0 + (uint32_t)p.planes_per_block < p.planes && p.h * p.w >= 16) {
+    DwItems<STRIDE, R, CG, OUT, ACT, true>(p, plane0, v);
   } else {
-    DwItems<STRIDE, R, OUT, ACT, false>(p, plane0, v);
+    DwItems<STRIDE, R, CG, OUT, ACT, false>(p, plane0, v);
   }
 }
 
-// R: output rows per item (the per-item address and mask arithmetic is shared
-// by R rows of four outputs).
-template <int STRIDE, int R, int OUT>
+// R output rows by 4 * CG columns per item (the per-item address and mask
+// arithmetic is shared by all of them).
+template <int STRIDE, int R, int CG, int OUT>
 __global__ void __launch_bounds__(256) DwConv3x3Kernel(const DwConvParams p) {
   DispatchAct(p.act.type, [&](auto act_c) {
     constexpr int ACT = decltype(act_c)::value;
-    DwBody<STRIDE, R, OUT, ACT>(p);
+    DwBody<STRIDE, R, CG, OUT, ACT>(p);
   });
+}
+
+template <int STRIDE, int R, int CG>
+void LaunchShape(int out_kind, dim3 grid, hipStream_t stream, const DwConvParams& q) {
+  if (out_kind == kOutI8) {
+    hipLaunchKernelGGL((DwConv3x3Kernel<STRIDE, R, CG, kOutI8>), grid, dim3(256), 0, stream, q);
+  } else {
+    hipLaunchKernelGGL((DwConv3x3Kernel<STRIDE, R, CG, kOutF32>), grid, dim3(256), 0, stream, q);
+  }
 }
 
 // ceil(2^32 / d) for d >= 2 (a divisor of 1 is handled by the kernel: its magic would need 33 bits)
@@ -192,11 +207,17 @@ hipError_t LaunchDwConv3x3(int stride, int out_kind, const DwConvParams& p, hipS
   if (p.planes == 0 || p.oh <= 0 || p.ow <= 0) return hipSuccess;
   if ((stride != 1 && stride != 2) || (p.pad != 0 && p.pad != 1) || (out_kind != kOutF32 && out_kind != kOutI8)) return hipErrorInvalidValue;
   DwConvParams q = p;
-  q.groups_w = (p.ow + 3) / 4;
-  // two output rows per item; four for the large planes at stride 1 (measured:
-  // fewer, longer wavefronts pay off only when there are many of them)
-  const int rows = (stride == 1 && p.oh >= 48 && p.oh < 96) ? 4 : 2;
-  const int64_t items = (int64_t)((p.oh + rows - 1) / rows) * q.groups_w;  // an item is `rows` output rows by four columns
+  // Item shape.  Measured on the MobileNet shapes: two output rows by four
+  // columns per thread is best almost everywhere (more work per thread lowers
+  // the instruction count per output but leaves too few wavefronts to hide the
+  // load latency; eight columns per thread were slower on every shape); four
+  // rows pay off for planes of 48 to 95 rows at stride 1.
+  constexpr int cg = 1;
+  int rows = p.item_rows;
+  if (rows != 2 && rows != 4) rows = (stride == 1 && p.oh >= 48 && p.oh < 96) ? 4 : 2;
+  if (stride == 2) rows = 2;
+  q.groups_w = (p.ow + 4 * cg - 1) / (4 * cg);
+  const int64_t items = (int64_t)((p.oh + rows - 1) / rows) * q.groups_w;
   // the magic divisions need v * items < 2^32 for every v below the workgroup's span
   if (items > 46000) return hipErrorInvalidValue;
   q.items = (int)items;
@@ -205,25 +226,15 @@ hipError_t LaunchDwConv3x3(int stride, int out_kind, const DwConvParams& p, hipS
   q.magic_groups = Magic(q.groups_w);
   q.blocks_per_plane = q.items > 256 ? (q.items + 255) / 256 : 1;
   const uint32_t blocks = (p.planes + q.planes_per_block - 1) / q.planes_per_block * (uint32_t)q.blocks_per_plane;
-  dim3 grid(blocks), block(256);
-  if (stride == 1 && rows == 4) {
-    if (out_kind == kOutI8) {
-      hipLaunchKernelGGL((DwConv3x3Kernel<1, 4, kOutI8>), grid, block, 0, stream, q);
+  dim3 grid(blocks);
+  if (stride == 1) {
+    if (rows == 4) {
+      LaunchShape<1, 4, cg>(out_kind, grid, stream, q);
     } else {
-      hipLaunchKernelGGL((DwConv3x3Kernel<1, 4, kOutF32>), grid, block, 0, stream, q);
-    }
-  } else if (stride == 1) {
-    if (out_kind == kOutI8) {
-      hipLaunchKernelGGL((DwConv3x3Kernel<1, 2, kOutI8>), grid, block, 0, stream, q);
-    } else {
-      hipLaunchKernelGGL((DwConv3x3Kernel<1, 2, kOutF32>), grid, block, 0, stream, q);
+      LaunchShape<1, 2, cg>(out_kind, grid, stream, q);
     }
   } else {
-    if (out_kind == kOutI8) {
-      hipLaunchKernelGGL((DwConv3x3Kernel<2, 2, kOutI8>), grid, block, 0, stream, q);
-    } else {
-      hipLaunchKernelGGL((DwConv3x3Kernel<2, 2, kOutF32>), grid, block, 0, stream, q);
-    }
+    LaunchShape<2, 2, cg>(out_kind, grid, stream, q);
   }
   return hipGetLastError();
 }
