@@ -280,7 +280,8 @@ int UploadHalfBias(pl_sparse_conv_handle* h, const float* bias) {
 // wavefront, group of the wavefront) the batches of four entries whose channel
 // lies in the chunk, in index order, padded with zero-weight entries that
 // point at the tile's zero row.
-int BuildChunkWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
+// half: one weight dword per entry, the two rows' binary16 patterns in its halves
+int BuildChunkWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h, bool half = false) {
   const int nr = L.semi ? 2 : 1;
   const int per_slice = pl::kChunkWalkWaves * pl::kChunkWalkGroups;
   const int n_groups = static_cast<int>(L.groups.size());
@@ -301,7 +302,7 @@ int BuildChunkWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
         auto flush = [&]() {
           for (; fill < 4; ++fill) {  // padding entries: zero row, zero weights
             packed |= static_cast<uint32_t>(pl::kChunkWalkChunk) << (8 * fill);
-            for (int r = 0; r < nr; ++r) wts.push_back(0u);
+            for (int r = 0; r < (half ? 1 : nr); ++r) wts.push_back(0u);
           }
           idx.push_back(packed);
           packed = 0;
@@ -311,8 +312,15 @@ int BuildChunkWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
           const uint32_t k = L.ic_index[rg.first + j];
           if (static_cast<int>(k / pl::kChunkWalkChunk) != c) continue;
           packed |= (k % pl::kChunkWalkChunk) << (8 * fill);
-          wts.push_back(L.w0[rg.first + j]);
-          if (nr == 2) wts.push_back(L.w1[rg.first + j]);
+          if (half) {
+            float w0, w1 = 0.f;
+            std::memcpy(&w0, &L.w0[rg.first + j], 4);
+            if (nr == 2) std::memcpy(&w1, &L.w1[rg.first + j], 4);
+            wts.push_back(static_cast<uint32_t>(HalfBits(w0)) | (static_cast<uint32_t>(HalfBits(w1)) << 16));
+          } else {
+            wts.push_back(L.w0[rg.first + j]);
+            if (nr == 2) wts.push_back(L.w1[rg.first + j]);
+          }
           if (++fill == 4) flush();
         }
         if (fill > 0) flush();
@@ -507,6 +515,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
     }
     h->algo = PL_ALGO_ROW_WALK;
     int hrc = BuildHalfWalk(L, h);
+    if (hrc == PL_OK) hrc = BuildChunkWalk(L, h, true);
     if (hrc == PL_OK) hrc = UploadHalfBias(h, desc->bias);
     if (hrc != PL_OK) {
       delete h;
@@ -564,7 +573,27 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
   const int vec = (im_size % 4 == 0) && (reinterpret_cast<uintptr_t>(x_dev) % 16 == 0) && (reinterpret_cast<uintptr_t>(out_dev) % 16 == 0);
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipError_t e;
-  if (h->half) {
+  if (h->half && (im_size % 4 == 0) && (reinterpret_cast<uintptr_t>(x_dev) % 8 == 0) && (reinterpret_cast<uintptr_t>(out_dev) % 8 == 0) && h->walk_chunked > 0 && h->cw_chunks > 0 &&
+      (h->walk_chunked == 2 || (h->ic > 128 && static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kChunkWalkTile)) * h->cw_slices >= 256))) {
+    // many channels and enough work for every CU: walk over channel chunks
+    pl::HalfChunkWalkParams p{};
+    p.x = static_cast<const uint16_t*>(x_dev);
+    p.out = static_cast<uint16_t*>(out_dev);
+    p.groups = static_cast<const pl::DevGroup*>(h->groups.ptr);
+    p.desc = static_cast<const uint32_t*>(h->cw_desc.ptr);
+    p.idx = static_cast<const uint32_t*>(h->cw_idx.ptr);
+    p.wts = static_cast<const uint32_t*>(h->cw_wts.ptr);
+    p.bias = h->has_bias ? static_cast<const uint16_t*>(h->hw_bias.ptr) : nullptr;
+    p.n_groups = h->n_groups;
+    p.n_chunks = h->cw_chunks;
+    p.slices = h->cw_slices;
+    p.M = h->oc;
+    p.K = h->ic;
+    p.hw = im_size;
+    p.P = P;
+    p.act = h->act_h;
+    e = pl::LaunchHalfChunkWalk(h->semi ? 2 : 1, p, s);
+  } else if (h->half) {
     pl::HalfWalkParams p{};
     p.x = static_cast<const uint16_t*>(x_dev);
     p.out = static_cast<uint16_t*>(out_dev);

@@ -105,6 +105,28 @@ struct DevActH {
   uint16_t hs_threshold;
 };
 
+// Half-precision walk over channel chunks (the layout of ChunkWalkParams; a
+// weight entry is one dword, row 0 in the low half and row 1 in the high half).
+struct HalfChunkWalkParams {
+  const uint16_t* x;
+  uint16_t* out;
+  const DevGroup* groups;
+  const uint32_t* desc;
+  const uint32_t* idx;
+  const uint32_t* wts;
+  const uint16_t* bias;    // may be null
+  int n_groups;
+  int n_chunks, slices;
+  int M, K;
+  int hw;
+  uint32_t P;
+  DevActH act;
+  int tiles;               // filled in by the launcher
+};
+
+// Needs hw % 4 == 0 and 8-byte aligned x / out.
+hipError_t LaunchHalfChunkWalk(int nrows, const HalfChunkWalkParams& p, hipStream_t stream);
+
 struct HalfWalkParams {
   const uint16_t* x;
   uint16_t* out;

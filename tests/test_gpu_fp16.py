@@ -46,3 +46,27 @@ def test_fp16_no_bias_and_new_epilogue():
     case.bias = None
     got = run_hip(case)
     assert_same(case, got, run_oracle(case), "fp16 without bias")
+
+
+# Half-precision walk over channel chunks (256 positions per workgroup, 64
+# channels staged at a time); forced here, the library picks it by itself only
+# for large problems.  Needs H*W % 4 == 0.  (batch, ic, oc, h, w): one chunk
+# and several, a channel count off the chunk grid, more row groups than one
+# slice holds, an odd row count, a tile that spans images.
+CHUNKED_SHAPES = [(2, 64, 64, 4, 4), (1, 96, 48, 8, 6), (3, 130, 67, 4, 5), (1, 300, 150, 16, 16), (5, 70, 33, 2, 2), (2, 257, 20, 12, 12)]
+
+
+@pytest.mark.parametrize("act", ["none", "relu6", "hswish"])
+@pytest.mark.parametrize("shape", CHUNKED_SHAPES, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
+def test_fp16_chunked_walk(shape, paired, act, monkeypatch):
+    batch, ic, oc, h, w = shape
+    case = half_case(batch, ic, oc, h, w, 0.75, paired, ACTS[act], seed=ic + 3 * oc)
+    want = run_oracle(case, oracle_pack(case, force_semi=paired))
+    monkeypatch.setenv("PL_SPARSE_CONV_WALK_CHUNKED", "2")
+    got = run_hip(case, capi.ALGO_AUTO, force_semi=paired)
+    assert_same(case, got, want, "fp16 chunked %s %s" % (act, shape))
+    # the plain half-precision walk gives the same bits (same order of operations)
+    monkeypatch.setenv("PL_SPARSE_CONV_WALK_CHUNKED", "0")
+    plain = run_hip(case, capi.ALGO_AUTO, force_semi=paired)
+    assert np.array_equal(got.view(np.uint16), plain.view(np.uint16))
