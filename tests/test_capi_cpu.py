@@ -122,6 +122,42 @@ def test_no_device_no_compute():
     assert e.value.code == capi.PL_ERR_NO_DEVICE
 
 
+def test_depthwise_host_checks_and_no_device():
+    """The depthwise kernel class refuses what the reference's class refuses
+    before any device work, and without a device prepare fails loudly."""
+    import torch
+
+    filt = np.ones((4, 1, 3, 3), dtype=np.int8)
+    with pytest.raises(NotImplementedError):
+        pla.DepthwiseConv(pla.ConvParam(np.ones((4, 1, 5, 5), dtype=np.int8))).PrepareForRun()  # "this type dw conv not impl"
+    with pytest.raises(NotImplementedError):
+        pla.DepthwiseConv(pla.ConvParam(filt, strides=(3, 3))).PrepareForRun()
+    with pytest.raises(ValueError):
+        pla.DepthwiseConv(pla.ConvParam(filt, weight_scale=[0.1, 0.2])).PrepareForRun()  # neither 1 nor one per channel
+    with pytest.raises(ValueError):
+        pla.ConvParam(np.ones((4, 2, 3, 3), dtype=np.int8))  # not a depthwise filter
+    assert pla.ConvParam(filt, paddings=(1, 0)).paddings == [1, 1, 0, 0]  # two-element form, as ConvOp pads it
+    k = pla.DepthwiseConv(pla.ConvParam(filt, strides=(2, 2)))
+    assert k.out_shape((3, 4, 15, 13)) == (3, 4, 8, 7)
+    if torch.cuda.is_available():
+        pytest.skip("a device is present")
+    with pytest.raises(capi.SparseConvError) as e:
+        k.PrepareForRun()
+    assert e.value.code == capi.PL_ERR_NO_DEVICE
+
+
+def test_mobilenet_depthwise_workloads_chain_with_the_pointwise_ones():
+    size = 112
+    for i in range(13):
+        dw = workloads.config5_depthwise_layer(i)
+        ic, oc, hw = workloads.MOBILENET_V1_POINTWISE[i]
+        assert dw.channels == ic and dw.in_size == size and dw.out_size == hw
+        assert dw.filter.shape == (ic, 1, 3, 3) and dw.filter.dtype == np.int8
+        size = hw
+    a, b = workloads.config5_depthwise_layer(3), workloads.config5_depthwise_layer(3)
+    assert np.array_equal(a.filter, b.filter) and a.output_scale == b.output_scale
+
+
 def test_workloads_are_seeded_and_shaped():
     a, b = workloads.config3(batch=2), workloads.config3(batch=2)
     assert np.array_equal(a.x, b.x) and np.array_equal(a.dense, b.dense)
