@@ -21,7 +21,8 @@ struct DwConvParams {
   uint32_t planes;         // batch * channels
   int64_t in_bytes;        // planes * h * w
   DevAct act;
-  int item_rows;           // output rows per thread: 2 or 4, 0 = chosen by the launcher
+  int item_rows;           // output rows per thread: 1, 2 or 4, 0 = chosen by the launcher
+  int item_cols;           // groups of 4 output columns per thread: 1, 2 or 4, 0 = chosen by the launcher
   int share_lanes;         // 1: lanes load only their own dwords and exchange the rest; 0: every lane loads all; -1 = chosen by the launcher
   // filled in by the launcher
   int groups_w;            // column groups per output row

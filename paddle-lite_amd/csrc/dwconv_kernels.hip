@@ -24,15 +24,26 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 
 // Dword at `ptr` (any alignment).  SAFE: the caller knows that the four
 // bytes lie inside the tensor.  Otherwise bytes outside [lo, hi) read as zero
-// (only the workgroups at the two ends of the tensor take this path).
+// (only the workgroups at the two ends of the tensor take this path, but the
+// kernel lasts as long as they do): the load is moved inside the tensor and
+// the value shifted, without a branch, so that all loads of an item are in
+// flight together as on the safe path.
 template <bool SAFE>
 __device__ __forceinline__ uint32_t LoadBytes4(const int8_t* ptr, const int8_t* lo, const int8_t* hi) {
   if (SAFE) return *reinterpret_cast<const uint32_t*>(ptr);
-  uint32_t v = 0;
+  if (hi - lo < 4) {
+    uint32_t v = 0;
 #pragma unroll
-  for (int b = 0; b < 4; ++b)
-    if (ptr + b >= lo && ptr + b < hi) v |= (uint32_t)(uint8_t)ptr[b] << (8 * b);
-  return v;
+    for (int b = 0; b < 4; ++b)
+      if (ptr + b >= lo && ptr + b < hi) v |= (uint32_t)(uint8_t)ptr[b] << (8 * b);
+    return v;
+  }
+  const int8_t* at = ptr < lo ? lo : (ptr > hi - 4 ? hi - 4 : ptr);
+  const uint32_t v = *reinterpret_cast<const uint32_t*>(at);
+  const int d = (int)(ptr - at);  // < 0: the dword starts below the tensor, > 0: it ends above
+  const uint32_t up = d > -4 ? v << (8 * (-d & 3)) : 0u;
+  const uint32_t down = d < 4 ? v >> (8 * (d & 3)) : 0u;
+  return d == 0 ? v : (d < 0 ? up : down);
 }
 
 // One item: 4 * CG neighbouring outputs (from column ox0 = 4 * CG * g) of the
@@ -161,20 +172,21 @@ __device__ __forceinline__ void DwItem(const DwConvParams& p, uint32_t plane, in
 #pragma unroll
         for (int k = 0; k < 4; ++k) q[k] = ActQuantI8<ACT>(__builtin_fmaf((float)acc[o][4 * q4 + k], s, b), p.act);
         int8_t* dst = static_cast<int8_t*>(p.out) + at;
-        if (n_out == 4 && (at & 3) == 0) {
-          __builtin_nontemporal_store(PackI8x4(q[0], q[1], q[2], q[3]), reinterpret_cast<uint32_t*>(dst));
+        // global memory takes dword and short stores at any byte address
+        const uint32_t packed = PackI8x4(q[0], q[1], q[2], q[3]);
+        if (n_out == 4) {
+          *reinterpret_cast<uint32_t*>(dst) = packed;
         } else {
-#pragma unroll
-          for (int k = 0; k < 4; ++k)
-            if (k < n_out) dst[k] = (int8_t)q[k];
+          if (n_out >= 2) *reinterpret_cast<uint16_t*>(dst) = (uint16_t)packed;
+          if (n_out & 1) dst[n_out - 1] = (int8_t)q[n_out - 1];
         }
       } else {
         float v[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) v[k] = ActivateT<ACT>(__builtin_fmaf((float)acc[o][4 * q4 + k], s, b), p.act);
         float* dst = static_cast<float*>(p.out) + at;
-        if (n_out == 4 && (at & 3) == 0) {
-          __builtin_nontemporal_store(v4f{v[0], v[1], v[2], v[3]}, reinterpret_cast<v4f*>(dst));
+        if (n_out == 4) {  // a four-dword store needs dword alignment only
+          *reinterpret_cast<v4f*>(dst) = v4f{v[0], v[1], v[2], v[3]};
         } else {
 #pragma unroll
           for (int k = 0; k < 4; ++k)
@@ -250,19 +262,24 @@ hipError_t LaunchDwConv3x3(int stride, int out_kind, const DwConvParams& p, hipS
   if (p.planes == 0 || p.oh <= 0 || p.ow <= 0) return hipSuccess;
   if ((stride != 1 && stride != 2) || (p.pad != 0 && p.pad != 1) || (out_kind != kOutF32 && out_kind != kOutI8)) return hipErrorInvalidValue;
   DwConvParams q = p;
-  // Item shape.  Measured on the MobileNet shapes: two output rows by four
-  // columns per thread is best almost everywhere (more work per thread lowers
-  // the instruction count per output but leaves too few wavefronts to hide the
-  // load latency; eight columns per thread were slower on every shape); four
-  // rows pay off for planes of 48 to 95 rows at stride 1.
-  constexpr int cg = 1;
-  int rows = p.item_rows;
-  if (rows != 2 && rows != 4) rows = (stride == 1 && p.oh >= 48 && p.oh < 96) ? 4 : 2;
-  if (stride == 2) rows = 2;
+  // Item shape: output rows by groups of four output columns per thread.
+  // More outputs per thread lower the instruction count per output, fewer
+  // leave more wavefronts to hide the load latency.  Measured on the MobileNet
+  // shapes at batch 64 (kernel us for rows x groups 2x1 / 4x1 / 1x2 / 2x2):
+  // stride 1: 112x112 29.6 / 30.8 / - / 26.7, 56x56 33.0 / 28.5 / - / 24.8,
+  // 28x28 17.4 / 14.4 / 17.0 / 14.7, 14x14 10.0 / 10.1 / 11.5 / 10.8;
+  // stride 2 (output size): 56x56 23.5 / - / 20.2 / 22.3, 28x28 12.7 / - /
+  // 11.8 / 13.5, 14x14 8.7 / - / 8.3 / 10.0.
+  int rows = p.item_rows, cg = p.item_cols;
+  const bool rows_given = rows == 1 || rows == 2 || rows == 4, cols_given = cg == 1 || cg == 2 || cg == 4;
+  if (!cols_given) cg = stride == 1 ? ((p.oh >= 48 && p.ow >= 48) ? 2 : 1) : (p.ow >= 14 ? 2 : 1);
+  if (!rows_given) rows = stride == 1 ? ((p.oh >= 24 && p.oh < 48 && cg == 1) ? 4 : 2) : (cg == 2 ? 1 : 2);
+  if (stride == 2 && rows == 4) rows = 2;
+  if (rows * cg > 8 || (rows == 1 && cg == 1)) return hipErrorInvalidValue;  // 8 to 32 outputs per thread
   // Rows that are not 4-byte aligned make the overlapping per-lane loads
   // slow; there the lanes share their dwords instead (measured: 14x14 planes
   // 12.7 -> 10.4 us, 112x112 planes 28.3 -> 31.5 us with sharing).
-  q.share_lanes = p.share_lanes >= 0 ? p.share_lanes : (p.w % 4 != 0 ? 1 : 0);
+  q.share_lanes = cg != 1 ? 0 : (p.share_lanes >= 0 ? p.share_lanes : (p.w % 4 != 0 ? 1 : 0));
   q.groups_w = (p.ow + 4 * cg - 1) / (4 * cg);
   const int64_t items = (int64_t)((p.oh + rows - 1) / rows) * q.groups_w;
   // the magic divisions need v * items < 2^32 for every v below the workgroup's span
@@ -274,14 +291,43 @@ hipError_t LaunchDwConv3x3(int stride, int out_kind, const DwConvParams& p, hipS
   q.blocks_per_plane = q.items > 256 ? (q.items + 255) / 256 : 1;
   const uint32_t blocks = (p.planes + q.planes_per_block - 1) / q.planes_per_block * (uint32_t)q.blocks_per_plane;
   dim3 grid(blocks);
-  if (stride == 1) {
-    if (rows == 4) {
-      LaunchShape<1, 4, cg>(out_kind, grid, stream, q);
-    } else {
-      LaunchShape<1, 2, cg>(out_kind, grid, stream, q);
-    }
-  } else {
-    LaunchShape<2, 2, cg>(out_kind, grid, stream, q);
+  const int shape = 100 * stride + 10 * rows + cg;
+  switch (shape) {
+    case 121:
+      LaunchShape<1, 2, 1>(out_kind, grid, stream, q);
+      break;
+    case 141:
+      LaunchShape<1, 4, 1>(out_kind, grid, stream, q);
+      break;
+    case 112:
+      LaunchShape<1, 1, 2>(out_kind, grid, stream, q);
+      break;
+    case 122:
+      LaunchShape<1, 2, 2>(out_kind, grid, stream, q);
+      break;
+    case 142:
+      LaunchShape<1, 4, 2>(out_kind, grid, stream, q);
+      break;
+    case 114:
+      LaunchShape<1, 1, 4>(out_kind, grid, stream, q);
+      break;
+    case 124:
+      LaunchShape<1, 2, 4>(out_kind, grid, stream, q);
+      break;
+    case 221:
+      LaunchShape<2, 2, 1>(out_kind, grid, stream, q);
+      break;
+    case 212:
+      LaunchShape<2, 1, 2>(out_kind, grid, stream, q);
+      break;
+    case 222:
+      LaunchShape<2, 2, 2>(out_kind, grid, stream, q);
+      break;
+    case 214:
+      LaunchShape<2, 1, 4>(out_kind, grid, stream, q);
+      break;
+    default:
+      return hipErrorInvalidValue;
   }
   return hipGetLastError();
 }

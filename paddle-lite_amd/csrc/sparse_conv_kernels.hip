@@ -869,7 +869,7 @@ __device__ __forceinline__ void MfmaBody(const MfmaParams& p, uint4* xt) {
 // At least two workgroups per CU (two wavefronts per SIMD): caps the kernel
 // at 256 VGPRs.
 template <int KSMAX, int OUT>
-__global__ void __launch_bounds__(256, 2) BlockMfmaKernel(const MfmaParams p) {
+__global__ void __launch_bounds__(256, (KSMAX == 4 ? 4 : 2)) BlockMfmaKernel(const MfmaParams p) {
   extern __shared__ uint4 xt[];
   if (!p.vec) {
     MfmaBody<KSMAX, OUT, -1, false>(p, xt);

@@ -99,6 +99,22 @@ def test_mobilenet_shapes(layer):
     run_case(2, c, size, size, stride, 1, "int8", ACTS["relu"](), True, seed=c + size + stride)
 
 
+# every item shape the launcher can pick (output rows x groups of four output
+# columns per thread), forced through the tuning knobs the library reads when
+# a layer is prepared, on planes that are ragged against each of them
+ITEM_SHAPES = {1: [(2, 1), (4, 1), (1, 2), (2, 2), (4, 2), (1, 4), (2, 4)], 2: [(2, 1), (1, 2), (2, 2), (1, 4)]}
+
+
+@pytest.mark.parametrize("stride,rows,cols", [(s, r, c) for s in (1, 2) for (r, c) in ITEM_SHAPES[s]])
+@pytest.mark.parametrize("out", ["int8", "fp32"])
+def test_item_shapes(monkeypatch, stride, rows, cols, out):
+    monkeypatch.setenv("PL_DWCONV_ROWS", str(rows))
+    monkeypatch.setenv("PL_DWCONV_COLS", str(cols))
+    for i, (n, c, h, w) in enumerate([(2, 3, 7, 7), (1, 5, 14, 14), (2, 2, 33, 17), (1, 4, 30, 61), (2, 40, 28, 28), (1, 2, 3, 70)]):
+        for pad in (0, 1):
+            run_case(n, c, h, w, stride, pad, out, ACTS["relu6"](), True, seed=1000 * rows + 100 * cols + 10 * i + pad + stride)
+
+
 def test_bad_arguments_are_refused():
     import torch
 
