@@ -161,30 +161,50 @@ __device__ __forceinline__ void DwItem(const DwConvParams& p, uint32_t plane, in
   for (int o = 0; o < R; ++o) {
     const int oy = R * oyr + o;
     if (oy >= p.oh) break;
+    const size_t row_at = ((size_t)plane * (uint32_t)p.oh + (uint32_t)oy) * (uint32_t)p.ow + (uint32_t)ox0;
+    if (OUT == kOutI8) {
+      uint32_t packed[CG];
+      int last[CG];  // third value of each group: a tail of three outputs stores it as a byte
 #pragma unroll
-    for (int q4 = 0; q4 < CG; ++q4) {
-      const int ox = ox0 + 4 * q4;
-      const int n_out = min(4, p.ow - ox);
-      if (n_out <= 0) break;
-      const size_t at = ((size_t)plane * (uint32_t)p.oh + (uint32_t)oy) * (uint32_t)p.ow + (uint32_t)ox;
-      if (OUT == kOutI8) {
+      for (int q4 = 0; q4 < CG; ++q4) {
         int q[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) q[k] = ActQuantI8<ACT>(__builtin_fmaf((float)acc[o][4 * q4 + k], s, b), p.act);
-        int8_t* dst = static_cast<int8_t*>(p.out) + at;
-        // global memory takes dword and short stores at any byte address
-        const uint32_t packed = PackI8x4(q[0], q[1], q[2], q[3]);
-        if (n_out == 4) {
-          *reinterpret_cast<uint32_t*>(dst) = packed;
+        packed[q4] = PackI8x4(q[0], q[1], q[2], q[3]);
+        last[q4] = q[2];
+      }
+      int8_t* dst = static_cast<int8_t*>(p.out) + row_at;
+      // global memory takes dword and short stores at any byte address
+      if (CG > 1 && ox0 + 4 * CG <= p.ow) {
+        // the whole item in one store: the wavefront's stores are then contiguous
+        if (CG == 2) {
+          *reinterpret_cast<uint2*>(dst) = make_uint2(packed[0], packed[CG - 1]);
         } else {
-          if (n_out >= 2) *reinterpret_cast<uint16_t*>(dst) = (uint16_t)packed;
-          if (n_out & 1) dst[n_out - 1] = (int8_t)q[n_out - 1];
+          *reinterpret_cast<uint4*>(dst) = make_uint4(packed[0], packed[1 % CG], packed[2 % CG], packed[3 % CG]);
         }
       } else {
+#pragma unroll
+        for (int q4 = 0; q4 < CG; ++q4) {
+          const int n_out = min(4, p.ow - (ox0 + 4 * q4));
+          if (n_out <= 0) break;
+          if (n_out == 4) {
+            *reinterpret_cast<uint32_t*>(dst + 4 * q4) = packed[q4];
+          } else {
+            if (n_out >= 2) *reinterpret_cast<uint16_t*>(dst + 4 * q4) = (uint16_t)packed[q4];
+            if (n_out == 1) dst[4 * q4] = (int8_t)packed[q4];
+            if (n_out == 3) dst[4 * q4 + 2] = (int8_t)last[q4];
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int q4 = 0; q4 < CG; ++q4) {
+        const int n_out = min(4, p.ow - (ox0 + 4 * q4));
+        if (n_out <= 0) break;
         float v[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) v[k] = ActivateT<ACT>(__builtin_fmaf((float)acc[o][4 * q4 + k], s, b), p.act);
-        float* dst = static_cast<float*>(p.out) + at;
+        float* dst = static_cast<float*>(p.out) + row_at + 4 * q4;
         if (n_out == 4) {  // a four-dword store needs dword alignment only
           *reinterpret_cast<v4f*>(dst) = v4f{v[0], v[1], v[2], v[3]};
         } else {
