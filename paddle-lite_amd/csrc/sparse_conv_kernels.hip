@@ -60,11 +60,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 // non-temporally so that they stream to memory instead of sitting dirty in
 // L2 until the end-of-kernel write-back.
 __device__ __forceinline__ void StreamStore(float4 v, void* dst) {
-#ifdef PL_PLAIN_STORES
-  *static_cast<float4*>(dst) = v;
-#else
   __builtin_nontemporal_store(v4f{v.x, v.y, v.z, v.w}, static_cast<v4f*>(dst));
-#endif
 }
 __device__ __forceinline__ void StreamStore(int4 v, void* dst) {
   __builtin_nontemporal_store(v4i{v.x, v.y, v.z, v.w}, static_cast<v4i*>(dst));

@@ -96,23 +96,21 @@ def test_few_channel_tiles_bit_exact(shape, kind, monkeypatch):
         assert_same(case, got, want, "few-channel %s %s %s" % (kind, act, shape))
 
 
-# 512 input channels: a workgroup may take several tiles one after the other
-# (weights loaded once, the next tile's loads issued under the current tile's
-# stores).  Forced here with different tile widths and counts, on shapes whose
-# tile count is not a multiple of the tiles per workgroup.
+# 512 input channels with the tile width forced (the library picks narrower
+# tiles when full ones would leave CUs idle): widths that do and do not divide
+# the quads of an image, on shapes whose last tile is partial.
 @pytest.mark.parametrize("kind", ["acc32", "fp32out", "int8out"])
-@pytest.mark.parametrize("tq,per_wg", [(32, 2), (25, 2), (32, 3), (13, 5)])
+@pytest.mark.parametrize("tq", [32, 25, 13, 8])
 @pytest.mark.parametrize("shape", [(3, 512, 96, 14, 14), (2, 512, 160, 16, 16), (5, 512, 33, 7, 7)], ids=lambda s: "x".join(map(str, s)))
-def test_tile_loop_bit_exact(shape, tq, per_wg, kind, monkeypatch):
-    announce("tile-loop", shape, tq, per_wg, kind)
+def test_tile_widths_bit_exact(shape, tq, kind, monkeypatch):
+    announce("tile-width", shape, tq, kind)
     monkeypatch.setenv("PL_SPARSE_CONV_MFMA_TILE_QUADS", str(tq))
-    monkeypatch.setenv("PL_SPARSE_CONV_MFMA_TILES_PER_WG", str(per_wg))
     k = {"acc32": capi.KIND_INT8_ACC32, "fp32out": capi.KIND_INT8_FP32, "int8out": capi.KIND_INT8_INT8}[kind]
     batch, ic, oc, h, w = shape
     case = small_case(k, batch, ic, oc, h, w, 0.85, False, AP() if kind == "acc32" else ACTS["relu"], seed=oc + tq, output_scale=0.1 if kind == "int8out" else 1.0)
     got = run_hip(case, capi.ALGO_BLOCK_MFMA)
     want = run_oracle(case, oracle_pack(case))
-    assert_same(case, got, want, "tile-loop %s %s tq=%d x%d" % (kind, shape, tq, per_wg))
+    assert_same(case, got, want, "tile-width %s %s tq=%d" % (kind, shape, tq))
 
 
 # more than 1024 input channels: the block MFMA kernel takes the k-steps a
