@@ -77,6 +77,16 @@ __device__ __forceinline__ int QuantizeI8(float v) {
 template <int ACT>
 __device__ __forceinline__ int ActQuantI8(float v, const DevAct& a) {
   if (ACT == 1) return static_cast<int>(__builtin_amdgcn_fmed3f(v, 0.0f, 127.0f) + 0x1.fffffep-2f);
+  if (ACT == 2) {
+    // relu6 followed by the clamp is one median over the intersected bounds
+    // (wave-uniform, computed once), and the sign of its result is the sign
+    // of the coefficient: [0, coef] for coef >= 0, the constant coef below.
+    const float hi = a.relu6_coef;
+    const float lo127 = fmaxf(fminf(0.0f, hi), -127.0f);
+    const float hi127 = fmaxf(fminf(hi, 127.0f), lo127);
+    const float half = hi >= 0.0f ? 0x1.fffffep-2f : -0x1.fffffep-2f;
+    return static_cast<int>(__builtin_amdgcn_fmed3f(v, lo127, hi127) + half);
+  }
   if (ACT < 0) return QuantizeI8(Activate(v, a));
   return QuantizeI8(ActivateT<(ACT < 0 ? 0 : ACT)>(v, a));
 }
