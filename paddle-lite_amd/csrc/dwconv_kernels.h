@@ -27,10 +27,12 @@ struct DwConvParams {
   // filled in by the launcher
   int groups_w;            // column groups per output row
   int items;               // ceil(oh / rows) * groups_w per plane
-  int planes_per_block;    // several small planes share a workgroup
-  int blocks_per_plane;    // a plane above 256 items is cut into pieces of 256
-  uint32_t magic_items;    // ceil(2^32 / items) for items >= 2: x / items == mulhi(x, magic) for x * items < 2^32
+  int planes_per_group;    // the items of this many planes, laid end to end, fill whole workgroups of 256
+  int blocks_per_group;    // planes_per_group * items / 256
+  int planes_per_block;    // bound on the planes one workgroup touches
+  uint32_t magic_items;    // ceil(2^32 / items) for items >= 2: x / items is mulhi(x, magic) or one less, exactly mulhi for x * items < 2^32
   uint32_t magic_groups;   // likewise for groups_w
+  uint32_t magic_blocks;   // likewise for blocks_per_group
 };
 
 // stride 1 or 2; out_kind kOutF32 or kOutI8.

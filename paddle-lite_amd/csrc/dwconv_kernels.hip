@@ -223,7 +223,7 @@ __device__ __forceinline__ void DwItem(const DwConvParams& p, uint32_t plane, in
 // reached memory.
 template <int STRIDE, int R, int CG, int OUT, int ACT, bool SAFE>
 __device__ __forceinline__ void DwItems(const DwConvParams& p, uint32_t plane0, int v) {
-  if (v >= p.planes_per_block * p.items) return;
+  // v = item of plane0 + thread index: below items + 256, so v * items < 2^32
   const int pl = p.items == 1 ? v : (int)__umulhi((uint32_t)v, p.magic_items);  // v / items
   const int item = v - pl * p.items;
   const uint32_t plane = plane0 + (uint32_t)pl;
@@ -235,14 +235,25 @@ __device__ __forceinline__ void DwItems(const DwConvParams& p, uint32_t plane0, 
   DwItem<STRIDE, R, CG, OUT, ACT, SAFE>(p, plane, c, oyr, g);
 }
 
+// x / d for any 32-bit x with magic = ceil(2^32 / d), d >= 2: the multiply-high
+// is the quotient or one more.
+__device__ __forceinline__ uint32_t DivMagic(uint32_t x, uint32_t d, uint32_t magic) {
+  if (d == 1) return x;
+  const uint32_t q = __umulhi(x, magic);
+  return q * d > x ? q - 1 : q;
+}
+
 template <int STRIDE, int R, int CG, int OUT, int ACT>
 __device__ __forceinline__ void DwBody(const DwConvParams& p) {
-  // a workgroup takes planes_per_block whole planes, or one of the
-  // blocks_per_plane pieces of 256 items of one plane
-  const uint32_t unit = blockIdx.x / (uint32_t)p.blocks_per_plane;
-  const int piece = (int)(blockIdx.x - unit * (uint32_t)p.blocks_per_plane);
-  const uint32_t plane0 = unit * (uint32_t)p.planes_per_block;
-  const int v = piece * 256 + (int)threadIdx.x;
+  // The items of planes_per_group planes are laid end to end and cut into
+  // pieces of 256, one per workgroup; planes_per_group * items is a multiple
+  // of 256, so every lane of every workgroup has an item (but for the planes
+  // past the end of the tensor in the last group).
+  const uint32_t group = DivMagic(blockIdx.x, (uint32_t)p.blocks_per_group, p.magic_blocks);
+  const uint32_t first = 256u * (blockIdx.x - group * (uint32_t)p.blocks_per_group);  // first item of the workgroup within its group
+  const uint32_t pl0 = DivMagic(first, (uint32_t)p.items, p.magic_items);
+  const uint32_t plane0 = group * (uint32_t)p.planes_per_group + pl0;
+  const int v = (int)(first - pl0 * (uint32_t)p.items) + (int)threadIdx.x;
   // The dwords of a row reach 4 bytes before its first column and up to 15
   // bytes past its last one: only the workgroups with the first and the last
   // plane can leave the tensor (with planes of at least 16 bytes, so that one
@@ -305,11 +316,22 @@ hipError_t LaunchDwConv3x3(int stride, int out_kind, const DwConvParams& p, hipS
   // the magic divisions need v * items < 2^32 for every v below the workgroup's span
   if (items > 46000) return hipErrorInvalidValue;
   q.items = (int)items;
-  q.planes_per_block = q.items >= 256 ? 1 : 256 / q.items;  // planes_per_block * items <= 256 or one plane
+  // planes per group: the smallest count whose items fill whole workgroups
+  int gcd = 256;
+  for (int a = q.items % 256; a != 0;) {
+    const int t = gcd % a;
+    gcd = a;
+    a = t;
+  }
+  q.planes_per_group = 256 / gcd;
+  q.blocks_per_group = (int)((int64_t)q.planes_per_group * q.items / 256);
+  q.planes_per_block = 256 / q.items + 2;  // bound on the planes one workgroup touches
   q.magic_items = Magic(q.items);
   q.magic_groups = Magic(q.groups_w);
-  q.blocks_per_plane = q.items > 256 ? (q.items + 255) / 256 : 1;
-  const uint32_t blocks = (p.planes + q.planes_per_block - 1) / q.planes_per_block * (uint32_t)q.blocks_per_plane;
+  q.magic_blocks = Magic(q.blocks_per_group);
+  const uint64_t blocks64 = (uint64_t)((p.planes + q.planes_per_group - 1) / q.planes_per_group) * (uint64_t)q.blocks_per_group;
+  if (blocks64 >= (1ull << 31)) return hipErrorInvalidValue;
+  const uint32_t blocks = (uint32_t)blocks64;
   dim3 grid(blocks);
   const int shape = 100 * stride + 10 * rows + cg;
   switch (shape) {
