@@ -296,15 +296,15 @@ hipError_t LaunchDwConv3x3(int stride, int out_kind, const DwConvParams& p, hipS
   // Item shape: output rows by groups of four output columns per thread.
   // More outputs per thread lower the instruction count per output, fewer
   // leave more wavefronts to hide the load latency.  Measured on the MobileNet
-  // shapes at batch 64 (kernel us for rows x groups 2x1 / 4x1 / 1x2 / 2x2):
-  // stride 1: 112x112 29.6 / 30.8 / - / 26.7, 56x56 33.0 / 28.5 / - / 24.8,
-  // 28x28 17.4 / 14.4 / 17.0 / 14.7, 14x14 10.0 / 10.1 / 11.5 / 10.8;
-  // stride 2 (output size): 56x56 23.5 / - / 20.2 / 22.3, 28x28 12.7 / - /
-  // 11.8 / 13.5, 14x14 8.7 / - / 8.3 / 10.0.
+  // shapes at batch 64 (kernel us for rows x groups 2x1 / 4x1 / 1x2 / 2x2 /
+  // 1x4): stride 1: 112x112 28.0 / - / - / 19.7 / 20.1, 56x56 26.5 / 24.4 /
+  // - / 19.4 / 22.6, 28x28 14.2 / 14.1 / - / 12.9 / 13.3, 14x14 9.7 / 9.8 /
+  // - / 9.8 / -; stride 2 (output size): 56x56 20.5 / - / 16.4 / 19.9 / 21.3,
+  // 28x28 11.2 / - / 10.2 / 11.8 / 12.0.
   int rows = p.item_rows, cg = p.item_cols;
   const bool rows_given = rows == 1 || rows == 2 || rows == 4, cols_given = cg == 1 || cg == 2 || cg == 4;
-  if (!cols_given) cg = stride == 1 ? ((p.oh >= 48 && p.ow >= 48) ? 2 : 1) : (p.ow >= 14 ? 2 : 1);
-  if (!rows_given) rows = stride == 1 ? ((p.oh >= 24 && p.oh < 48 && cg == 1) ? 4 : 2) : (cg == 2 ? 1 : 2);
+  if (!cols_given) cg = stride == 1 ? ((p.oh >= 24 && p.ow >= 24) ? 2 : 1) : (p.ow >= 14 ? 2 : 1);
+  if (!rows_given) rows = stride == 1 ? 2 : (cg == 2 ? 1 : 2);
   if (stride == 2 && rows == 4) rows = 2;
   if (rows * cg > 8 || (rows == 1 && cg == 1)) return hipErrorInvalidValue;  // 8 to 32 outputs per thread
   // Rows that are not 4-byte aligned make the overlapping per-lane loads
