@@ -33,6 +33,7 @@ struct DwConvParams {
   uint32_t magic_items;    // ceil(2^32 / items) for items >= 2: x / items is mulhi(x, magic) or one less, exactly mulhi for x * items < 2^32
   uint32_t magic_groups;   // likewise for groups_w
   uint32_t magic_blocks;   // likewise for blocks_per_group
+  uint32_t magic_channels; // likewise for channels
 };
 
 // stride 1 or 2; out_kind kOutF32 or kOutI8.

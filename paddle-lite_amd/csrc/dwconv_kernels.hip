@@ -217,6 +217,14 @@ __device__ __forceinline__ void DwItem(const DwConvParams& p, uint32_t plane, in
   }
 }
 
+// x / d for any 32-bit x with magic = ceil(2^32 / d), d >= 2: the multiply-high
+// is the quotient or one more.
+__device__ __forceinline__ uint32_t DivMagic(uint32_t x, uint32_t d, uint32_t magic) {
+  if (d == 1) return x;
+  const uint32_t q = __umulhi(x, magic);
+  return q * d > x ? q - 1 : q;
+}
+
 // One item per thread and no loop: a wavefront that has stores in flight can
 // wait for later loads only by waiting for the stores as well, so a second
 // item in the same thread would start after the first one's stores have
@@ -230,17 +238,9 @@ __device__ __forceinline__ void DwItems(const DwConvParams& p, uint32_t plane0, 
   if (plane >= p.planes) return;
   const int oyr = p.groups_w == 1 ? item : (int)__umulhi((uint32_t)item, p.magic_groups);  // item / groups_w
   const int g = item - oyr * p.groups_w;
-  int c = (int)(plane0 % (uint32_t)p.channels) + pl;  // the first term is uniform
+  int c = (int)(plane0 - DivMagic(plane0, (uint32_t)p.channels, p.magic_channels) * (uint32_t)p.channels) + pl;  // plane0 % channels (uniform) + pl
   if (c >= p.channels) c = p.channels > p.planes_per_block ? c - p.channels : c % p.channels;
   DwItem<STRIDE, R, CG, OUT, ACT, SAFE>(p, plane, c, oyr, g);
-}
-
-// x / d for any 32-bit x with magic = ceil(2^32 / d), d >= 2: the multiply-high
-// is the quotient or one more.
-__device__ __forceinline__ uint32_t DivMagic(uint32_t x, uint32_t d, uint32_t magic) {
-  if (d == 1) return x;
-  const uint32_t q = __umulhi(x, magic);
-  return q * d > x ? q - 1 : q;
 }
 
 template <int STRIDE, int R, int CG, int OUT, int ACT>
@@ -329,6 +329,7 @@ hipError_t LaunchDwConv3x3(int stride, int out_kind, const DwConvParams& p, hipS
   q.magic_items = Magic(q.items);
   q.magic_groups = Magic(q.groups_w);
   q.magic_blocks = Magic(q.blocks_per_group);
+  q.magic_channels = Magic(p.channels);
   const uint64_t blocks64 = (uint64_t)((p.planes + q.planes_per_group - 1) / q.planes_per_group) * (uint64_t)q.blocks_per_group;
   if (blocks64 >= (1ull << 31)) return hipErrorInvalidValue;
   const uint32_t blocks = (uint32_t)blocks64;
