@@ -373,7 +373,7 @@ def run_mobilenet(args):
 def main():
     args = parse()
     if args.gpus != 1:
-        sys.stderr.write("bench.py measures one GPU; --gpus %d is not supported (this path shards over images with no exchange, see DESIGN.md)\n" % args.gpus)
+        sys.stderr.write("bench.py measures one GPU; --gpus %d is not supported: this path shards over images with no exchange between GPUs, so N GPUs would each run this same kernel on their share of the batch\n" % args.gpus)
         return 2
     import numpy as np
     import torch
