@@ -231,12 +231,14 @@ __device__ __forceinline__ uint32_t DivMagic(uint32_t x, uint32_t d, uint32_t ma
 // reached memory.
 template <int STRIDE, int R, int CG, int OUT, int ACT, bool SAFE>
 __device__ __forceinline__ void DwItems(const DwConvParams& p, uint32_t plane0, int v) {
-  // v = item of plane0 + thread index: below items + 256, so v * items < 2^32
-  const int pl = p.items == 1 ? v : (int)__umulhi((uint32_t)v, p.magic_items);  // v / items
+  // v = item of plane0 + thread index, below items + 256: v / items is 0 or 1
+  // for planes of 256 items and more, else v * items < 2^32 and the
+  // multiply-high is exact
+  const int pl = p.items >= 256 ? (v >= p.items ? 1 : 0) : (p.items == 1 ? v : (int)__umulhi((uint32_t)v, p.magic_items));
   const int item = v - pl * p.items;
   const uint32_t plane = plane0 + (uint32_t)pl;
   if (plane >= p.planes) return;
-  const int oyr = p.groups_w == 1 ? item : (int)__umulhi((uint32_t)item, p.magic_groups);  // item / groups_w
+  const int oyr = (int)DivMagic((uint32_t)item, (uint32_t)p.groups_w, p.magic_groups);  // item / groups_w
   const int g = item - oyr * p.groups_w;
   int c = (int)(plane0 - DivMagic(plane0, (uint32_t)p.channels, p.magic_channels) * (uint32_t)p.channels) + pl;  // plane0 % channels (uniform) + pl
   if (c >= p.channels) c = p.channels > p.planes_per_block ? c - p.channels : c % p.channels;
@@ -313,8 +315,8 @@ hipError_t LaunchDwConv3x3(int stride, int out_kind, const DwConvParams& p, hipS
   q.share_lanes = cg != 1 ? 0 : (p.share_lanes >= 0 ? p.share_lanes : (p.w % 4 != 0 ? 1 : 0));
   q.groups_w = (p.ow + 4 * cg - 1) / (4 * cg);
   const int64_t items = (int64_t)((p.oh + rows - 1) / rows) * q.groups_w;
-  // the magic divisions need v * items < 2^32 for every v below the workgroup's span
-  if (items > 46000) return hipErrorInvalidValue;
+  // 256 * items (the span of a group of planes) must fit 32 bits
+  if (items >= (1 << 24)) return hipErrorInvalidValue;
   q.items = (int)items;
   // planes per group: the smallest count whose items fill whole workgroups
   int gcd = 256;

@@ -938,7 +938,7 @@ int pl_dwconv3x3_run(pl_dwconv_handle* h, const int8_t* x_dev, void* out_dev, in
   if (hipGetDevice(&cur_dev) != hipSuccess || cur_dev != h->device) return Fail(PL_ERR_BAD_ARG, "the handle belongs to device %d, the current device is %d", h->device, cur_dev);
   const int64_t planes = static_cast<int64_t>(batch) * h->channels;
   if (planes > 0x7fffffffll || planes * height * width >= (1ll << 40)) return Fail(PL_ERR_UNSUPPORTED, "tensor too large");
-  if (static_cast<int64_t>((oh + 1) / 2) * ((ow + 3) / 4) > 46000) return Fail(PL_ERR_UNSUPPORTED, "output planes above 46000 items of two rows by four columns are not supported");
+  if (static_cast<int64_t>((oh + 1) / 2) * ((ow + 3) / 4) >= (1ll << 24)) return Fail(PL_ERR_UNSUPPORTED, "output planes of 2^24 and more items of two rows by four columns are not supported");
   pl::DwConvParams p{};
   p.x = x_dev;
   p.out = out_dev;

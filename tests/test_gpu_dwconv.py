@@ -115,6 +115,13 @@ def test_item_shapes(monkeypatch, stride, rows, cols, out):
             run_case(n, c, h, w, stride, pad, out, ACTS["relu6"](), True, seed=1000 * rows + 100 * cols + 10 * i + pad + stride)
 
 
+@pytest.mark.parametrize("stride", [1, 2])
+def test_large_planes(stride):
+    # more than 2^16 items per plane, and a plane whose item count is odd
+    run_case(1, 2, 1100, 900, stride, 1, "int8", ACTS["relu"](), True, seed=77 + stride)
+    run_case(1, 1, 515, 1030, stride, 0, "fp32", ACTS["leaky"](), True, seed=78 + stride)
+
+
 def test_bad_arguments_are_refused():
     import torch
 
