@@ -347,6 +347,7 @@ def run_mobilenet(args):
     for _ in range(steps):
         sequence()
     e1.record()
+    host_us = (time.perf_counter() - t0) * 1e6 / steps  # time the host needs to enqueue one sequence
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     seq_us = e0.elapsed_time(e1) * 1e3 / steps
@@ -363,7 +364,7 @@ def run_mobilenet(args):
         "data": "synthetic",
         "config": {"workload": "mobilenet_v1_body_int8", "batch": batch, "launches": 26, "pointwise_sparsity": 0.9, "parity_checked": True},
         "roofline": {"bound": "hbm", "achieved": total_bytes / (seq_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": total_bytes / (seq_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                     "algorithmic_bytes_per_sequence": total_bytes, "sequence_us": seq_us, "sum_depthwise_kernel_us": round(dw_us, 1), "sum_pointwise_kernel_us": round(pw_us, 1)},
+                     "algorithmic_bytes_per_sequence": total_bytes, "sequence_us": seq_us, "host_enqueue_us_per_sequence": round(host_us, 1), "sum_depthwise_kernel_us": round(dw_us, 1), "sum_pointwise_kernel_us": round(pw_us, 1)},
         "per_layer": per_layer,
         "nonzero_fraction_of_pointwise_outputs": nonzero,
     }))
