@@ -73,3 +73,68 @@ def test_mobilenet_pointwise_layers_at_batch_8(layer):
         assert_same(case, got, want, "layer %d algo %d" % (layer, algo))
     sat = np.mean(got == 127)
     assert sat < 0.2
+
+
+def test_mobilenet_pointwise_stack_chained_at_batch_64():
+    """All thirteen config-5 layers at batch 64, run as the chained sequence
+    the benchmark times: layer i+1 consumes layer i's int8 output on the
+    device where the shapes chain, a fresh uniform int8 tensor is fed at the
+    four spatial breaks.  Every layer is compared with the oracle on the
+    first two and the last image of its actual input."""
+    import torch
+
+    prev = None
+    chained_count = 0
+    for i in range(13):
+        announce("c5 chained layer", i)
+        case = workloads.config5_layer(i)
+        assert case.batch == 64
+        ic, oc, hw = workloads.MOBILENET_V1_POINTWISE[i]
+        kernel, _ = make_kernel(case, capi.ALGO_AUTO)
+        chained = prev is not None and tuple(prev.shape[1:]) == (ic, hw, hw)
+        chained_count += chained
+        x = prev if chained else torch.from_numpy(case.x).cuda()
+        out = kernel.Run(x)
+        torch.cuda.synchronize()
+        assert tuple(out.shape) == (64, oc, hw, hw) and out.dtype == torch.int8
+        pick = [0, 1, 63]
+        want = run_oracle(case, x=np.ascontiguousarray(x[pick].cpu().numpy()))
+        got = out[pick].cpu().numpy()
+        assert_same(case, got, want, "c5 chained layer %d" % i)
+        assert np.mean(got == 127) < 0.2 and np.mean(got != 0) > 0.1, "layer %d output is degenerate" % i
+        prev = out
+    assert chained_count == 8  # 2->3, 4->5, 6->7 .. 10->11, 12->13
+
+
+def test_mobilenet_body_26_launches_at_batch_64():
+    """Depthwise 3x3 + pointwise, thirteen times, every layer consuming the
+    previous layer's int8 output on the device (the `--config mobilenet`
+    sequence of the benchmark), each layer compared with the oracle on the
+    first two images of its actual input."""
+    import torch
+
+    from oracle import oracle as O
+
+    rng = np.random.RandomState(5)
+    x = torch.from_numpy(rng.randint(-127, 128, size=(64, 32, 112, 112)).astype(np.int8)).cuda()
+    for i in range(13):
+        announce("mobilenet block", i)
+        dwc = workloads.config5_depthwise_layer(i)
+        param = pla.ConvParam(dwc.filter, dwc.bias, strides=(dwc.stride, dwc.stride), paddings=(1, 1, 1, 1), activation_param=dwc.act, input_scale=dwc.input_scale,
+                              weight_scale=dwc.weight_scale, output_scale=dwc.output_scale)
+        dw = pla.DepthwiseConv(param, out_precision="int8")
+        dw.PrepareForRun()
+        t = dw.Run(x)
+        torch.cuda.synchronize()
+        a = O.Act()
+        a.type = 1
+        want = O.dwconv3x3_int8(x[:2].cpu().numpy(), dwc.filter[:, 0], dw.w_scale_, dw.bias_, a, out="int8", stride=dwc.stride, pad=1)
+        assert np.array_equal(t[:2].cpu().numpy(), want), "depthwise layer %d differs from the oracle" % i
+        case = workloads.config5_layer(i)
+        kernel, _ = make_kernel(case)
+        out = kernel.Run(t)
+        torch.cuda.synchronize()
+        want = run_oracle(case, x=np.ascontiguousarray(t[:2].cpu().numpy()))
+        assert_same(case, out[:2].cpu().numpy(), want, "pointwise layer %d" % i)
+        x = out
+    assert tuple(x.shape) == (64, 1024, 7, 7)
