@@ -71,8 +71,14 @@ enum {
  *                     nonzero list over an activation tile held in LDS
  *   PL_ALGO_BLOCK_MFMA int8 only: 32x32 blocks of the weight matrix that
  *                     hold at least one nonzero are multiplied on the matrix
- *                     cores, empty blocks are skipped */
-enum { PL_ALGO_AUTO = 0, PL_ALGO_ROW_WALK = 1, PL_ALGO_BLOCK_MFMA = 2 };
+ *                     cores, empty blocks are skipped
+ *   PL_ALGO_IMAGE_MFMA int8 only, oc a multiple of 128, ic = 128 / 256 / 512,
+ *                     H*W a multiple of 4 in [16, 256]: one workgroup per
+ *                     (image, 128 output rows) keeps the whole image in LDS
+ *                     and multiplies it with dense 16x64 weight tiles
+ * With PL_ALGO_AUTO an int8 handle may hold more than one form and choose per
+ * call by batch and H*W: see pl_sparse_conv_algo_for(). */
+enum { PL_ALGO_AUTO = 0, PL_ALGO_ROW_WALK = 1, PL_ALGO_BLOCK_MFMA = 2, PL_ALGO_IMAGE_MFMA = 3 };
 
 /* Activation constants, used as given (replaces the fields of
  * ActivationParam the math functions read,
@@ -166,6 +172,13 @@ int pl_sparse_conv_run_sequence(pl_sparse_conv_handle* handle,
 
 int pl_sparse_conv_get_info(const pl_sparse_conv_handle* handle,
                             pl_sparse_conv_info* info);
+
+/* The algorithm (PL_ALGO_*, never PL_ALGO_AUTO) a pl_sparse_conv_run() call
+ * with this batch and H*W would use on 16-byte aligned tensors, or a negative
+ * status.  No counterpart in the reference, whose kernel choice is fixed by
+ * the registration (lite/kernels/arm/sparse_conv_compute.cc:369-430). */
+int pl_sparse_conv_algo_for(const pl_sparse_conv_handle* handle, int32_t batch,
+                            int32_t im_size);
 
 /* Replace scale / bias / activation without re-uploading weights (what a
  * second PrepareForRun with new quantisation parameters would do). Either

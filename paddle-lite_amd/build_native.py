@@ -34,6 +34,7 @@ SOURCES = [
     ("chunk_walk_kernels.hip", "chunk_walk_kernels.o", []),
     ("fp16_walk_kernels.hip", "fp16_walk_kernels.o", []),
     ("dwconv_kernels.hip", "dwconv_kernels.o", []),
+    ("image_mfma_kernels.hip", "image_mfma_kernels.o", []),
     ("sparse_conv_kernels.hip", "sparse_conv_kernels_walk.o", ["-DPL_KERNEL_PART=0"]),
     ("sparse_conv_kernels.hip", "sparse_conv_kernels_mfma_f32.o", ["-DPL_KERNEL_PART=1"]),
     ("sparse_conv_kernels.hip", "sparse_conv_kernels_mfma_i8.o", ["-DPL_KERNEL_PART=2"]),

@@ -10,7 +10,7 @@ ABI_VERSION = 1
 PL_OK, PL_ERR_BAD_ARG, PL_ERR_BAD_LAYOUT, PL_ERR_UNSUPPORTED, PL_ERR_HIP, PL_ERR_NO_DEVICE = 0, -1, -2, -3, -4, -5
 KIND_FP32, KIND_INT8_FP32, KIND_INT8_INT8, KIND_INT8_ACC32, KIND_FP16 = 0, 1, 2, 3, 4
 ACT_NONE, ACT_RELU, ACT_RELU6, ACT_LEAKY_RELU, ACT_HARD_SWISH = 0, 1, 2, 4, 10
-ALGO_AUTO, ALGO_ROW_WALK, ALGO_BLOCK_MFMA = 0, 1, 2
+ALGO_AUTO, ALGO_ROW_WALK, ALGO_BLOCK_MFMA, ALGO_IMAGE_MFMA = 0, 1, 2, 3
 
 EXPORTS = [
     "pl_sparse_conv_abi_version",
@@ -20,6 +20,7 @@ EXPORTS = [
     "pl_sparse_conv_run",
     "pl_sparse_conv_run_sequence",
     "pl_sparse_conv_get_info",
+    "pl_sparse_conv_algo_for",
     "pl_sparse_conv_set_epilogue",
     "pl_sparse_conv_destroy",
     "pl_sparse_count_semi",
@@ -128,6 +129,8 @@ def lib():
     L.pl_sparse_conv_run_sequence.restype = C.c_int
     L.pl_sparse_conv_get_info.argtypes = [C.c_void_p, C.POINTER(Info)]
     L.pl_sparse_conv_get_info.restype = C.c_int
+    L.pl_sparse_conv_algo_for.argtypes = [C.c_void_p, C.c_int32, C.c_int32]
+    L.pl_sparse_conv_algo_for.restype = C.c_int
     L.pl_sparse_conv_set_epilogue.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Activation)]
     L.pl_sparse_conv_set_epilogue.restype = C.c_int
     L.pl_sparse_conv_destroy.argtypes = [C.c_void_p]

@@ -18,6 +18,7 @@
 #include <type_traits>
 
 #include "epilogue.h"
+#include "launch_lds.h"
 #include "sparse_conv_kernels.h"
 
 namespace pl {
@@ -178,18 +179,7 @@ __global__ void __launch_bounds__(64 * kChunkWalkWaves, 2) ChunkWalkKernel(const
 
 template <typename K>
 hipError_t LaunchBig(K kernel, dim3 grid, dim3 block, size_t lds, hipStream_t s, const ChunkWalkParams& p) {
-  // once per kernel and device: allow more than 64 KB of dynamic LDS
-  static bool done[64] = {};
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return e;
-  if (dev >= 0 && dev < 64 && !done[dev]) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
-    if (e != hipSuccess) return e;
-    done[dev] = true;
-  }
-  hipLaunchKernelGGL(kernel, grid, block, lds, s, p);
-  return hipGetLastError();
+  return LaunchWithLds(kernel, grid, block, lds, s, p);
 }
 
 }  // namespace

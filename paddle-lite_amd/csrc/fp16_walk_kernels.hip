@@ -11,6 +11,7 @@
 
 #include <cstdint>
 
+#include "launch_lds.h"
 #include "sparse_conv_kernels.h"
 
 namespace pl {
@@ -336,18 +337,7 @@ __global__ void __launch_bounds__(64 * kChunkWalkWaves, 2) HalfChunkWalkKernel(c
 
 template <typename K>
 hipError_t LaunchBig(K kernel, dim3 grid, dim3 block, size_t lds, hipStream_t s, const HalfWalkParams& p) {
-  // once per kernel and device: allow more than 64 KB of dynamic LDS
-  static bool done[64] = {};
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return e;
-  if (lds > 48 * 1024 && dev >= 0 && dev < 64 && !done[dev]) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
-    if (e != hipSuccess) return e;
-    done[dev] = true;
-  }
-  hipLaunchKernelGGL(kernel, grid, block, lds, s, p);
-  return hipGetLastError();
+  return LaunchWithLds(kernel, grid, block, lds, s, p);
 }
 
 template <int NR>
@@ -386,17 +376,7 @@ hipError_t HalfChunkLaunch(const HalfChunkWalkParams& p, hipStream_t stream) {
   const size_t lds = (size_t)(kCChunk + 1) * kTile * 2;
   dim3 grid(8u * (uint32_t)q.slices * (((uint32_t)q.tiles + 7) / 8)), block(64 * kCWaves);
   auto kernel = HalfChunkWalkKernel<NR, kChunkWalkGroups, PPL>;
-  static bool done[64] = {};  // once per kernel and device: allow more than 64 KB of dynamic LDS
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return e;
-  if (lds > 48 * 1024 && dev >= 0 && dev < 64 && !done[dev]) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
-    if (e != hipSuccess) return e;
-    done[dev] = true;
-  }
-  hipLaunchKernelGGL(kernel, grid, block, lds, stream, q);
-  return hipGetLastError();
+  return LaunchWithLds(kernel, grid, block, lds, stream, q);
 }
 
 // Needs hw % 4 == 0 and 8-byte aligned x / out.  Four positions per lane (256

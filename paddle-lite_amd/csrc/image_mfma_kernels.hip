@@ -1,0 +1,330 @@
+// Image MFMA: int8 sparse 1x1 convolution for feature maps small enough that
+// one image's activations ([K x H*W] int8, at most 128 KB) fit the LDS of a CU.
+//
+// One workgroup of eight wavefronts computes 128 output rows of one image.
+//   * The image is brought in once as whole cache lines: every wavefront
+//     moves its channel groups (16 channels x H*W bytes, contiguous in NCHW)
+//     from global memory straight into LDS (global_load_lds, no registers),
+//     then turns each group in place into matrix-core operand cells
+//     (16 channels of one position = 16 bytes) with 4x4 byte transposes.
+//   * Weights are dense 16x64 int8 tiles in v_mfma_i32_16x16x64_i8 operand
+//     order, held in registers (a wavefront pair shares 32 rows).  The rows of
+//     a tile are rho, rho + 4, rho + 8, ...: all rows of a tile then start at
+//     the same offset inside a 64-byte sector of the fp32 output, and the
+//     tile's window of 16 position quads is shifted left by that offset so
+//     that every 256-byte row piece it stores covers whole sectors.  Those
+//     are written through to memory (sc1 nt); the few pieces that share a
+//     sector with a neighbouring row are stored plainly and merge in L2.
+//   * The channel loop is innermost: a window is finished and stored while
+//     the other wavefront of the SIMD multiplies, so stores start right after
+//     the first window instead of after the whole tile.
+//   * The quads that the shifted windows leave over at the end of a row are
+//     computed with the operands swapped (positions as matrix rows).
+//
+// Reference semantics: out = act(fmaf(float(acc), scale, bias)) per output,
+// int32 accumulation over all channels (sparse_conv_impl.cc:1661-1685 computes
+// the same sum over the nonzeros only; zeros add nothing to an integer sum).
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <type_traits>
+
+#include "epilogue.h"
+#include "launch_lds.h"
+#include "sparse_conv_kernels.h"
+
+namespace pl {
+namespace {
+
+using epilogue::ActivateT;
+using epilogue::ActQuantI8;
+using epilogue::DispatchAct;
+using epilogue::PackI8x4;
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+
+// 4 dwords holding 4 channels x 4 positions -> 4 positions x 4 channels.
+__device__ __forceinline__ void Transpose4x4(uint32_t& r0, uint32_t& r1, uint32_t& r2, uint32_t& r3) {
+  const uint32_t a = __builtin_amdgcn_perm(r1, r0, 0x05010400u);
+  const uint32_t b = __builtin_amdgcn_perm(r1, r0, 0x07030602u);
+  const uint32_t c = __builtin_amdgcn_perm(r3, r2, 0x05010400u);
+  const uint32_t d = __builtin_amdgcn_perm(r3, r2, 0x07030602u);
+  r0 = __builtin_amdgcn_perm(c, a, 0x05040100u);
+  r1 = __builtin_amdgcn_perm(c, a, 0x07060302u);
+  r2 = __builtin_amdgcn_perm(d, b, 0x05040100u);
+  r3 = __builtin_amdgcn_perm(d, b, 0x07060302u);
+}
+
+// 16 bytes written through to memory as streaming data (sc1 nt).  Measured on
+// 64 x 512 -> 512 @14x14, fp32 output, whole sectors: plain 13.8 us, sc1 12.3,
+// nt 11.1, sc1 nt 10.8.  The wait state after the store keeps the data
+// registers intact until the store has read them (the compiler does not see a
+// store inside the assembly statement).
+__device__ __forceinline__ void StoreThrough(u4 v, void* p) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n s_nop 1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void StorePlain(u4 v, void* p) { *reinterpret_cast<u4*>(p) = v; }
+
+struct Lane {
+  int n;   // column of a 16x16 tile
+  int kq;  // quarter of the wavefront: channel group of an operand, rows 4 kq .. 4 kq + 3 of a result
+};
+
+// Per-wavefront constants of the epilogue.
+struct Rows {
+  float sc[2][4], bi[2][4];  // rows 4 kq + i of the wavefront's two row tiles
+  float sct[2], bit[2];      // row n of each tile (results of the swapped product)
+};
+
+// Epilogue of four accumulators (positions 4 q .. 4 q + 3 of one output row).
+template <int OUT, int ACT>
+__device__ __forceinline__ u4 Finish4(int a0, int a1, int a2, int a3, float s, float b, const DevAct& act) {
+  if (OUT == kOutAcc32) return u4{(uint32_t)a0, (uint32_t)a1, (uint32_t)a2, (uint32_t)a3};
+  const float v0 = __builtin_fmaf((float)a0, s, b), v1 = __builtin_fmaf((float)a1, s, b), v2 = __builtin_fmaf((float)a2, s, b), v3 = __builtin_fmaf((float)a3, s, b);
+  if (OUT == kOutI8) return u4{PackI8x4(ActQuantI8<ACT>(v0, act), ActQuantI8<ACT>(v1, act), ActQuantI8<ACT>(v2, act), ActQuantI8<ACT>(v3, act)), 0u, 0u, 0u};
+  return u4{__float_as_uint(ActivateT<ACT>(v0, act)), __float_as_uint(ActivateT<ACT>(v1, act)), __float_as_uint(ActivateT<ACT>(v2, act)), __float_as_uint(ActivateT<ACT>(v3, act))};
+}
+
+// One window of 16 position quads times NOC row tiles (tiles J0 .. J0 + NOC - 1
+// of the wavefront): 4 * NOC matrix instructions per k-step, then the stores.
+//   q0: first quad of the window (may be negative: the quads in front of the
+//       row belong to the previous row and are not stored)
+//   orow: output row of MFMA row 0 of tile 0, element units of the output type
+template <int KS, int OUT, int NOC, int J0>
+__device__ __forceinline__ void Window(const uint4* __restrict__ xt, int kgs, int qpi, int q0, bool first_sector_shared, const v4i (&a)[2][KS], const Rows& rw, const DevAct& act, char* __restrict__ orow, int hw,
+                                       Lane ln) {
+  const int q = q0 + ln.n;
+  const uint4* bbase = xt + ln.kq * kgs + q;  // + ks * 4 * kgs + c * qpi
+  v4i acc[NOC][4];
+#pragma unroll
+  for (int o = 0; o < NOC; ++o)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[o][c] = v4i{0, 0, 0, 0};
+  uint4 bq[2][4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) bq[0][c] = bbase[c * qpi];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    if (ks + 1 < KS) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) bq[(ks + 1) & 1][c] = bbase[(ks + 1) * 4 * kgs + c * qpi];
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const uint4 u = bq[ks & 1][c];
+      const v4i bv = v4i{(int)u.x, (int)u.y, (int)u.z, (int)u.w};
+#pragma unroll
+      for (int o = 0; o < NOC; ++o) acc[o][c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[J0 + o][ks], bv, acc[o][c], 0, 0, 0);
+    }
+  }
+  constexpr int kElem = OUT == kOutI8 ? 1 : 4;
+  // the first sector of a shifted window is shared with the end of the previous row
+  const bool shared = first_sector_shared && ln.n < 4;
+  DispatchAct(OUT == kOutAcc32 ? 0 : act.type, [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
+#pragma unroll
+    for (int o = 0; o < NOC; ++o) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const u4 v = Finish4<OUT, ACT>(acc[o][0][i], acc[o][1][i], acc[o][2][i], acc[o][3][i], rw.sc[J0 + o][i], rw.bi[J0 + o][i], act);
+        // rows of a tile are 4 apart: MFMA row m of tile j is row 4 (16 j + m) past the wavefront's first row
+        char* ptr = orow + ((size_t)(4 * (16 * (J0 + o) + 4 * ln.kq + i)) * hw + 4 * q) * kElem;
+        if (OUT == kOutI8) {
+          if (q >= 0) *reinterpret_cast<uint32_t*>(ptr) = v.x;
+        } else if (shared) {
+          if (q >= 0) StorePlain(v, ptr);
+        } else {
+          StoreThrough(v, ptr);
+        }
+      }
+    }
+  });
+}
+
+// Four quads starting at quad q0, both row tiles, operands swapped: rows of
+// the product are positions (quad q0 + m / 4, position m % 4), columns are
+// output rows.  A lane ends with the four positions of quad q0 + kq of row n.
+template <int KS, int OUT>
+__device__ __forceinline__ void Tail(const uint4* __restrict__ xt, int kgs, int qpi, int q0, const v4i (&a)[2][KS], const Rows& rw, const DevAct& act, char* __restrict__ orow, int hw, Lane ln) {
+  int tq = q0 + (ln.n >> 2);
+  if (tq > qpi - 1) tq = qpi - 1;  // rows past the end of the image row: any valid cell, results unused
+  const uint4* tb = xt + ln.kq * kgs + (ln.n & 3) * qpi + tq;
+  v4i acc[2] = {v4i{0, 0, 0, 0}, v4i{0, 0, 0, 0}};
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const uint4 u = tb[ks * 4 * kgs];
+    const v4i av = v4i{(int)u.x, (int)u.y, (int)u.z, (int)u.w};
+#pragma unroll
+    for (int o = 0; o < 2; ++o) acc[o] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, a[o][ks], acc[o], 0, 0, 0);
+  }
+  constexpr int kElem = OUT == kOutI8 ? 1 : 4;
+  const int q = q0 + ln.kq;
+  if (q >= qpi) return;
+  DispatchAct(OUT == kOutAcc32 ? 0 : act.type, [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
+#pragma unroll
+    for (int o = 0; o < 2; ++o) {
+      const u4 v = Finish4<OUT, ACT>(acc[o][0], acc[o][1], acc[o][2], acc[o][3], rw.sct[o], rw.bit[o], act);
+      char* ptr = orow + ((size_t)(4 * (16 * o + ln.n)) * hw + 4 * q) * kElem;
+      if (OUT == kOutI8) *reinterpret_cast<uint32_t*>(ptr) = v.x; else StorePlain(v, ptr);
+    }
+  });
+}
+
+template <int KS, int OUT>
+__global__ void __launch_bounds__(512) ImageMfmaKernel(const ImageMfmaParams p) {
+  extern __shared__ uint4 lds_raw[];
+  // shifted windows read up to three cells in front of a row of cells
+  uint4* xt = lds_raw + 16;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // a contiguous range of work items per XCD, the row groups of one image next to each other
+  const int item = (int)(blockIdx.x & 7u) * p.per_xcd + (int)(blockIdx.x >> 3);
+  if (item >= p.items) return;
+  const int n = item / p.row_groups, rg = item - n * p.row_groups;
+  const int rho = wave & 3, half = wave >> 2;
+  const int qpi = p.qpi, kgs = p.kgs, hw = p.hw;
+  constexpr int NKG = 4 * KS, BPW = NKG / 8;
+  static_assert(NKG % 8 == 0, "channel groups are dealt evenly to the eight wavefronts");
+
+  // activations: channel groups straight into LDS, whole lines
+  const int8_t* ximg = p.x + (size_t)n * p.K * hw;
+  char* lbase = reinterpret_cast<char*>(xt);
+  const int blk_bytes = 16 * hw;
+#pragma unroll
+  for (int u = 0; u < BPW; ++u) {
+    const int kg = wave * BPW + u;
+    const int8_t* src = ximg + (size_t)kg * blk_bytes + lane * 16;
+    char* dst = lbase + kg * (kgs * 16);
+    for (int t = 0; t < p.dma_full; ++t)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + t * 1024), (__attribute__((address_space(3))) void*)(dst + t * 1024), 16, 0, 0);
+    if (lane < p.dma_rem_lanes)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + p.dma_full * 1024), (__attribute__((address_space(3))) void*)(dst + p.dma_full * 1024), 16, 0, 0);
+  }
+  // weights of the wavefront's two row tiles, all channels
+  v4i a[2][KS];
+  const v4i* wt = static_cast<const v4i*>(p.wtiles) + ((size_t)(rg * 4 + rho) * 2 * KS) * 64 + lane;
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) a[j][ks] = wt[(j * KS + ks) * 64];
+  Lane ln;
+  ln.n = lane & 15;
+  ln.kq = lane >> 4;
+  const int row0 = rg * 128 + rho;  // the wavefront's rows: row0 + 4 m, m = 0 .. 31
+  Rows rw;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      rw.sc[j][i] = OUT == kOutAcc32 ? 0.f : p.scale[row0 + 4 * (16 * j + 4 * ln.kq + i)];
+      rw.bi[j][i] = OUT == kOutAcc32 ? 0.f : p.bias[row0 + 4 * (16 * j + 4 * ln.kq + i)];
+    }
+    rw.sct[j] = OUT == kOutAcc32 ? 0.f : p.scale[row0 + 4 * (16 * j + ln.n)];
+    rw.bit[j] = OUT == kOutAcc32 ? 0.f : p.bias[row0 + 4 * (16 * j + ln.n)];
+  }
+  // Every channel group of this wavefront has landed.  (Waiting group by group, with the weights
+  // behind the activations, measured the same: 10.90 against 10.87 us on 64 x 512 -> 512 @14x14.)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // in place: 16 dwords (16 channels x 4 positions) per quad -> 4 cells
+#pragma unroll
+  for (int u = 0; u < BPW; ++u) {
+    const int kg = wave * BPW + u;
+    uint32_t* blk = reinterpret_cast<uint32_t*>(lbase + kg * (kgs * 16));
+    uint32_t r[16];
+    if (lane < qpi) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) r[i] = blk[i * qpi + lane];
+    }
+    // every lane has read before any lane overwrites
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_sched_barrier(0);
+    if (lane < qpi) {
+#pragma unroll
+      for (int b4 = 0; b4 < 4; ++b4) Transpose4x4(r[4 * b4], r[4 * b4 + 1], r[4 * b4 + 2], r[4 * b4 + 3]);
+      uint4* cells = reinterpret_cast<uint4*>(blk) + lane;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) cells[c * qpi] = make_uint4(r[c], r[4 + c], r[8 + c], r[12 + c]);
+    }
+  }
+  __syncthreads();
+
+  // windows: shifted left by sh quads so that fp32 / int32 row pieces start on 64-byte boundaries
+  const int sh = p.align ? ((rho * qpi) & 3) : 0;
+  const int nqt = (qpi + sh) >> 4;            // full windows
+  const int left = qpi + sh - 16 * nqt;       // quads after the last window
+  const int ntail = (left + 3) >> 2;
+  // split between the two wavefronts of the pair, in matrix instructions per k-step:
+  // window x both tiles = 8, window x one tile = 4, tail = 2
+  const int target = (8 * nqt + 2 * ntail) >> 1;
+  const int wa = target >> 3;
+  const bool split = (target - 8 * wa) >= 2 && wa < nqt;
+  constexpr int kElem = OUT == kOutI8 ? 1 : 4;
+  char* orow = static_cast<char*>(p.out) + ((size_t)n * p.M + row0) * hw * kElem;
+  if (half == 0) {
+    if (split) Window<KS, OUT, 1, 0>(xt, kgs, qpi, 16 * wa - sh, wa == 0 && sh > 0, a, rw, p.act, orow, hw, ln);
+    for (int T = 0; T < wa; ++T) Window<KS, OUT, 2, 0>(xt, kgs, qpi, 16 * T - sh, T == 0 && sh > 0, a, rw, p.act, orow, hw, ln);
+  } else {
+    const int first = wa + (split ? 1 : 0);
+    for (int T = nqt - 1; T >= first; --T) Window<KS, OUT, 2, 0>(xt, kgs, qpi, 16 * T - sh, T == 0 && sh > 0, a, rw, p.act, orow, hw, ln);
+    if (split) Window<KS, OUT, 1, 1>(xt, kgs, qpi, 16 * wa - sh, wa == 0 && sh > 0, a, rw, p.act, orow, hw, ln);
+    for (int t = 0; t < ntail; ++t) Tail<KS, OUT>(xt, kgs, qpi, 16 * nqt - sh + 4 * t, a, rw, p.act, orow, hw, ln);
+  }
+}
+
+template <int OUT>
+hipError_t ByKs(const ImageMfmaParams& q, dim3 grid, size_t lds, hipStream_t s) {
+  const dim3 block(512);
+  switch (q.K / 64) {
+    case 2:
+      return LaunchWithLds(ImageMfmaKernel<2, OUT>, grid, block, lds, s, q);
+    case 4:
+      return LaunchWithLds(ImageMfmaKernel<4, OUT>, grid, block, lds, s, q);
+    case 8:
+      return LaunchWithLds(ImageMfmaKernel<8, OUT>, grid, block, lds, s, q);
+    default:
+      return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace
+
+bool ImageMfmaFits(int M, int K, int hw) {
+  if (M <= 0 || M % 128 != 0) return false;
+  if (K != 128 && K != 256 && K != 512) return false;
+  if (hw < 16 || hw > 256 || hw % 4 != 0) return false;
+  const int qpi = hw / 4, kgs = (4 * qpi + 15) / 16 * 16;
+  return 256 + (size_t)(K / 16) * kgs * 16 <= (size_t)kMaxLdsBytes;
+}
+
+hipError_t LaunchImageMfma(int out_kind, const ImageMfmaParams& p, hipStream_t stream) {
+  if (p.batch <= 0) return hipSuccess;
+  if (!ImageMfmaFits(p.M, p.K, p.hw)) return hipErrorInvalidValue;
+  if (reinterpret_cast<uintptr_t>(p.x) % 16 != 0 || reinterpret_cast<uintptr_t>(p.out) % 16 != 0) return hipErrorInvalidValue;
+  ImageMfmaParams q = p;
+  q.qpi = p.hw / 4;
+  q.kgs = (4 * q.qpi + 15) / 16 * 16;  // a channel group's cells start on a 256-byte boundary: conflict-free operand reads
+  q.row_groups = p.M / 128;
+  const int64_t items = (int64_t)p.batch * q.row_groups;
+  if (items > (1 << 28)) return hipErrorInvalidValue;
+  q.items = (int)items;
+  q.per_xcd = (q.items + 7) / 8;
+  q.dma_full = (16 * p.hw) / 1024;
+  q.dma_rem_lanes = ((16 * p.hw) % 1024) / 16;
+  q.align = out_kind != kOutI8;
+  const size_t lds = 256 + (size_t)(p.K / 16) * q.kgs * 16;
+  const dim3 grid(8u * (uint32_t)q.per_xcd);
+  switch (out_kind) {
+    case kOutF32:
+      return ByKs<kOutF32>(q, grid, lds, stream);
+    case kOutI8:
+      return ByKs<kOutI8>(q, grid, lds, stream);
+    case kOutAcc32:
+      return ByKs<kOutAcc32>(q, grid, lds, stream);
+    default:
+      return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace pl

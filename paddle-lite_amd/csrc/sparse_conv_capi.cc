@@ -154,12 +154,19 @@ struct pl_sparse_conv_handle {
   int mfma_i8_wide = 1;
   int mfma_tile_quads = 0;  // 0 = chosen per problem
   int mfma_sub_tiles = 1;   // several tiles per workgroup for <= 64 input channels: 0 never, 1 when enough workgroups remain, 2 always
+  // image MFMA (dense 16x64 tiles, rows of a tile four apart)
+  DevBuf wtiles;
+  // int8 handles prepared with PL_ALGO_AUTO hold several forms and choose per call
+  bool auto_int8 = false;
+  int image_min_items = 128;  // fewest (image, 128-row group) work items for which the image kernel is chosen
+  // row-walk tuning read once at prepare (0 = chosen per problem)
+  int walk_tile = 0, walk_threads = 0, walk_slices = 0;
   // epilogue
   DevBuf scale, bias;
   int padded_rows = 0;
 
   int64_t DeviceBytes() const {
-    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + cw_desc.bytes + cw_idx.bytes + cw_wts.bytes + hw_kidx.bytes + hw_wts.bytes + hw_bias.bytes + wblocks.bytes + kmask.bytes + scale.bytes + bias.bytes);
+    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + cw_desc.bytes + cw_idx.bytes + cw_wts.bytes + hw_kidx.bytes + hw_wts.bytes + hw_bias.bytes + wblocks.bytes + kmask.bytes + wtiles.bytes + scale.bytes + bias.bytes);
   }
 };
 
@@ -371,6 +378,34 @@ int BuildBlockMfma(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
   return PL_OK;
 }
 
+// Device-side form for the image MFMA path: the weight matrix as dense 16x64
+// int8 tiles in matrix-core operand order.  The 16 rows of a tile are four
+// apart (rho, rho + 4, ...): they all start at the same offset inside a
+// 64-byte sector of an fp32 output whose rows are H*W floats long.
+int BuildImageMfma(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
+  const int kss = L.ic / 64;
+  std::vector<int8_t> tiles(static_cast<size_t>(L.oc) * L.ic, 0);
+  auto put = [&](int row, uint32_t c, uint32_t wbits) {
+    const int8_t w = static_cast<int8_t>(wbits & 0xffu);
+    if (w == 0) return;
+    const int rg = row / 128, rl = row % 128;
+    const int rho = rl & 3, m32 = rl >> 2;  // row = rg * 128 + rho + 4 * (16 j + m)
+    const int j = m32 >> 4, m = m32 & 15;
+    const int ks = c >> 6, kk = c & 63;
+    const int lane = m + 16 * (kk >> 4), t = kk & 15;
+    tiles[((((static_cast<size_t>(rg) * 4 + rho) * 2 + j) * kss + ks) * 64 + lane) * 16 + t] = w;
+  };
+  for (const pl::RowGroup& g : L.groups) {
+    for (uint32_t j = 0; j < g.count; ++j) {
+      put(g.row0, L.ic_index[g.first + j], L.w0[g.first + j]);
+      if (g.nrows == 2) put(g.row0 + 1, L.ic_index[g.first + j], L.w1[g.first + j]);
+    }
+  }
+  const hipError_t e = h->wtiles.Upload(tiles.data(), tiles.size());
+  if (e != hipSuccess) return FailHip(e, "uploading the weight tiles");
+  return PL_OK;
+}
+
 int UploadEpilogue(pl_sparse_conv_handle* h, const float* scale, const float* bias) {
   const size_t n = static_cast<size_t>(h->padded_rows);
   if (scale) {
@@ -404,10 +439,7 @@ pl::WalkConfig ChooseWalk(const pl_sparse_conv_handle* h, uint32_t P) {
   if (row_bytes * tp > 64 * 1024) tp = 128;
   while (tp > 16 && row_bytes * tp > static_cast<size_t>(pl::kMaxLdsBytes)) tp >>= 1;
   while (tp > 64 && P <= static_cast<uint32_t>(tp) * 8) tp >>= 1;  // small problems: more tiles
-  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_TILE")) {
-    const int t = std::atoi(e);
-    if (t >= 16 && t <= 256 && (t & (t - 1)) == 0 && row_bytes * t <= static_cast<size_t>(pl::kMaxLdsBytes)) tp = t;
-  }
+  if (h->walk_tile >= 16 && h->walk_tile <= 256 && (h->walk_tile & (h->walk_tile - 1)) == 0 && row_bytes * h->walk_tile <= static_cast<size_t>(pl::kMaxLdsBytes)) tp = h->walk_tile;
   c.tile_pos = tp;
   const size_t lds = row_bytes * tp;
   c.threads = lds > 80 * 1024 ? 1024 : (lds >= 32 * 1024 ? 512 : 256);
@@ -417,14 +449,21 @@ pl::WalkConfig ChooseWalk(const pl_sparse_conv_handle* h, uint32_t P) {
   int slices = static_cast<int>((1024 + tiles - 1) / tiles);
   slices = std::min(slices, std::max(1, h->n_groups / nwaves));
   slices = std::max(1, std::min(slices, 65535));
-  // tuning overrides (power-of-two thread counts only)
-  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_THREADS")) {
-    const int t = std::atoi(e);
-    if (t >= tp && t <= 1024 && (t & (t - 1)) == 0) c.threads = t;
-  }
-  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_SLICES")) slices = std::max(1, std::min(std::atoi(e), std::max(1, h->n_groups)));
+  // tuning overrides read at prepare (power-of-two thread counts only)
+  if (h->walk_threads >= tp && h->walk_threads <= 1024 && (h->walk_threads & (h->walk_threads - 1)) == 0) c.threads = h->walk_threads;
+  if (h->walk_slices > 0) slices = std::max(1, std::min(h->walk_slices, std::max(1, h->n_groups)));
   c.slices = slices;
   return c;
+}
+
+// The algorithm one call uses.  Handles prepared for one algorithm use it;
+// int8 handles prepared with PL_ALGO_AUTO take the image kernel where its
+// shape conditions hold and there are enough (image, row group) work items to
+// occupy the chip, and the block kernel otherwise.
+int AlgoForCall(const pl_sparse_conv_handle* h, int batch, int im_size, bool aligned16) {
+  if (!h->auto_int8) return h->algo;
+  if (h->wtiles.ptr && aligned16 && pl::ImageMfmaFits(h->oc, h->ic, im_size) && static_cast<int64_t>(batch) * (h->oc / 128) >= h->image_min_items) return PL_ALGO_IMAGE_MFMA;
+  return h->algo;
 }
 
 }  // namespace
@@ -454,13 +493,15 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   *out_handle = nullptr;
   if (desc->struct_size != sizeof(pl_sparse_conv_desc)) return Fail(PL_ERR_BAD_ARG, "pl_sparse_conv_desc size mismatch (%u vs %zu)", desc->struct_size, sizeof(pl_sparse_conv_desc));
   if (desc->kind < PL_KIND_FP32 || desc->kind > PL_KIND_FP16) return Fail(PL_ERR_BAD_ARG, "unknown kind %d", desc->kind);
-  if (desc->algo < PL_ALGO_AUTO || desc->algo > PL_ALGO_BLOCK_MFMA) return Fail(PL_ERR_BAD_ARG, "unknown algo %d", desc->algo);
+  if (desc->algo < PL_ALGO_AUTO || desc->algo > PL_ALGO_IMAGE_MFMA) return Fail(PL_ERR_BAD_ARG, "unknown algo %d", desc->algo);
   if (desc->oc <= 0 || desc->ic <= 0 || desc->im_size <= 0) return Fail(PL_ERR_BAD_ARG, "oc, ic and im_size must be positive");
   if (!desc->oc_nonzeros || (desc->n_weights > 0 && (!desc->nonzero_weights || !desc->diffs))) return Fail(PL_ERR_BAD_ARG, "null weight tensors");
   const bool half = desc->kind == PL_KIND_FP16;
   const bool int8 = desc->kind != PL_KIND_FP32 && !half;
   if (int8 && desc->kind != PL_KIND_INT8_ACC32 && !desc->scale) return Fail(PL_ERR_BAD_ARG, "int8 kinds need per-channel scales");
-  if (desc->algo == PL_ALGO_BLOCK_MFMA && !int8) return Fail(PL_ERR_UNSUPPORTED, "the block MFMA algorithm exists for int8 only");
+  if ((desc->algo == PL_ALGO_BLOCK_MFMA || desc->algo == PL_ALGO_IMAGE_MFMA) && !int8) return Fail(PL_ERR_UNSUPPORTED, "the MFMA algorithms exist for int8 only");
+  if (desc->algo == PL_ALGO_IMAGE_MFMA && !pl::ImageMfmaFits(desc->oc, desc->ic, 16))
+    return Fail(PL_ERR_UNSUPPORTED, "the image MFMA algorithm needs oc %% 128 == 0 and ic = 128, 256 or 512 (oc = %d, ic = %d)", desc->oc, desc->ic);
 
   int ndev = 0;
   if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
@@ -492,6 +533,10 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_TILE_QUADS")) h->mfma_tile_quads = std::max(0, std::min(32, std::atoi(e)));
   // tuning switches for experiments; the defaults are what measured best
   if (const char* e = std::getenv("PL_SPARSE_CONV_WG_SLOTS")) h->wg_slots = std::max(1, std::atoi(e));
+  if (const char* e = std::getenv("PL_SPARSE_CONV_IMAGE_MIN_ITEMS")) h->image_min_items = std::max(1, std::atoi(e));
+  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_TILE")) h->walk_tile = std::atoi(e);
+  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_THREADS")) h->walk_threads = std::atoi(e);
+  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_SLICES")) h->walk_slices = std::atoi(e);
   h->kind = desc->kind;
   h->oc = desc->oc;
   h->ic = desc->ic;
@@ -506,6 +551,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   h->padded_rows = CeilDiv(desc->oc, 32) * 32;
 
   int algo = desc->algo;
+  h->auto_int8 = int8 && algo == PL_ALGO_AUTO;
   if (algo == PL_ALGO_AUTO) algo = int8 ? PL_ALGO_BLOCK_MFMA : PL_ALGO_ROW_WALK;
   if (half) {
     // half precision: its own walk; a tile of 16 positions must fit LDS
@@ -525,7 +571,8 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
     return PL_OK;
   }
   if (algo == PL_ALGO_ROW_WALK) {
-    const size_t row_bytes = static_cast<size_t>(int8 ? CeilDiv(desc->ic, 4) : desc->ic) * 4;
+    // fp32 tiles carry one all-zero row behind the channels
+    const size_t row_bytes = static_cast<size_t>(int8 ? CeilDiv(desc->ic, 4) : desc->ic + 1) * 4;
     if (row_bytes * 16 > static_cast<size_t>(pl::kMaxLdsBytes)) {
       delete h;
       return Fail(PL_ERR_UNSUPPORTED, "ic = %d does not fit an LDS tile", desc->ic);
@@ -533,13 +580,17 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   }
   h->algo = algo;
 
-  int rc = algo == PL_ALGO_BLOCK_MFMA ? BuildBlockMfma(L, h) : BuildRowWalk(L, h);
+  const bool mfma_forms = algo == PL_ALGO_BLOCK_MFMA || algo == PL_ALGO_IMAGE_MFMA;
+  int rc = PL_OK;
+  if (algo == PL_ALGO_ROW_WALK) rc = BuildRowWalk(L, h);
+  if (rc == PL_OK && algo == PL_ALGO_BLOCK_MFMA) rc = BuildBlockMfma(L, h);
+  if (rc == PL_OK && (algo == PL_ALGO_IMAGE_MFMA || (h->auto_int8 && pl::ImageMfmaFits(desc->oc, desc->ic, 16)))) rc = BuildImageMfma(L, h);
   if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8) rc = BuildChunkWalk(L, h);
   if (rc == PL_OK) {
-    // the MFMA epilogue always reads a bias; give it zeros when the op has none
+    // the MFMA epilogues always read a bias; give them zeros when the op has none
     std::vector<float> zeros;
     const float* bias = desc->bias;
-    if (!bias && algo == PL_ALGO_BLOCK_MFMA) {
+    if (!bias && mfma_forms) {
       zeros.assign(h->oc, 0.0f);
       bias = zeros.data();
     }
@@ -550,7 +601,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
       scale = ones.data();
     }
     rc = UploadEpilogue(h, int8 ? scale : nullptr, bias);
-    h->has_bias = desc->bias != nullptr || algo == PL_ALGO_BLOCK_MFMA;
+    h->has_bias = desc->bias != nullptr || mfma_forms;
   }
   if (rc != PL_OK) {
     delete h;
@@ -571,6 +622,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
   if (P64 >= (1ll << 31) - 512) return Fail(PL_ERR_UNSUPPORTED, "batch * im_size = %lld exceeds 2^31", static_cast<long long>(P64));
   const uint32_t P = static_cast<uint32_t>(P64);
   const int vec = (im_size % 4 == 0) && (reinterpret_cast<uintptr_t>(x_dev) % 16 == 0) && (reinterpret_cast<uintptr_t>(out_dev) % 16 == 0);
+  const bool aligned16 = reinterpret_cast<uintptr_t>(x_dev) % 16 == 0 && reinterpret_cast<uintptr_t>(out_dev) % 16 == 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipError_t e;
   if (h->half && (im_size % 4 == 0) && (reinterpret_cast<uintptr_t>(x_dev) % 8 == 0) && (reinterpret_cast<uintptr_t>(out_dev) % 8 == 0) && h->walk_chunked > 0 && h->cw_chunks > 0 &&
@@ -623,6 +675,21 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.groups_per_slice = CeilDiv(h->n_groups, slices);
     p.slices = CeilDiv(h->n_groups, p.groups_per_slice);
     e = pl::LaunchHalfWalk(h->semi ? 2 : 1, tp, threads, p, s);
+  } else if (AlgoForCall(h, batch, im_size, aligned16) == PL_ALGO_IMAGE_MFMA) {
+    if (!pl::ImageMfmaFits(h->oc, h->ic, im_size)) return Fail(PL_ERR_UNSUPPORTED, "the image MFMA algorithm needs H*W a multiple of 4 in [16, 256] that fits LDS with %d channels (H*W = %d)", h->ic, im_size);
+    if (reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(out_dev) % 16 != 0) return Fail(PL_ERR_UNSUPPORTED, "the image MFMA algorithm needs 16-byte aligned tensors");
+    pl::ImageMfmaParams p{};
+    p.x = static_cast<const int8_t*>(x_dev);
+    p.out = out_dev;
+    p.wtiles = h->wtiles.ptr;
+    p.scale = static_cast<const float*>(h->scale.ptr);
+    p.bias = static_cast<const float*>(h->bias.ptr);
+    p.M = h->oc;
+    p.K = h->ic;
+    p.hw = im_size;
+    p.batch = batch;
+    p.act = h->act;
+    e = pl::LaunchImageMfma(OutKind(h->kind), p, s);
   } else if (h->algo == PL_ALGO_BLOCK_MFMA) {
     pl::MfmaParams p{};
     p.x = static_cast<const int8_t*>(x_dev);
@@ -746,6 +813,12 @@ int pl_sparse_conv_get_info(const pl_sparse_conv_handle* h, pl_sparse_conv_info*
   info->mfma_blocks = h->blocks_present;
   info->mfma_blocks_total = static_cast<int64_t>(h->row_blocks) * h->ksteps;
   return PL_OK;
+}
+
+int pl_sparse_conv_algo_for(const pl_sparse_conv_handle* h, int32_t batch, int32_t im_size) {
+  if (!h) return Fail(PL_ERR_BAD_ARG, "null handle");
+  if (batch < 0 || im_size <= 0) return Fail(PL_ERR_BAD_ARG, "batch must be >= 0 and im_size > 0");
+  return AlgoForCall(h, batch, im_size, true);
 }
 
 int pl_sparse_conv_set_epilogue(pl_sparse_conv_handle* h, const float* scale, const float* bias, const pl_activation* act) {

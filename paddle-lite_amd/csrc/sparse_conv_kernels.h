@@ -186,6 +186,36 @@ struct MfmaConfig {
 
 hipError_t LaunchBlockMfma(const MfmaConfig& cfg, const MfmaParams& p, hipStream_t stream);
 
+// Image MFMA SpMM (int8, image_mfma_kernels.hip): one workgroup per (image,
+// 128 output rows) with the whole image's activations in LDS.
+struct ImageMfmaParams {
+  const int8_t* x;
+  void* out;
+  // dense 16x64 weight tiles in matrix-core operand order:
+  // [row group of 128][class rho = 0..3][tile j = 0..1][k-step][64 lanes][16 bytes];
+  // lane l of tile (rho, j) holds row rho + 4 (16 j + l % 16), channels 64 ks + 16 (l / 16) .. + 15
+  const void* wtiles;
+  const float* scale;  // output-row order, at least M entries
+  const float* bias;   // likewise (zeros when the op has no bias)
+  int M, K;
+  int hw;
+  int batch;
+  DevAct act;
+  // filled in by the launcher
+  int qpi;             // position quads per image = hw / 4
+  int kgs;             // 16-byte cells per channel group in LDS (a multiple of 16)
+  int row_groups;      // M / 128
+  int items, per_xcd;  // work items (image, row group) in all and per XCD
+  int dma_full, dma_rem_lanes;  // 1 KB pieces of a channel group and the lanes of the last, partial piece
+  int align;           // fp32 / int32 output: windows shifted onto 64-byte sector boundaries
+};
+
+// M a multiple of 128, K = 128, 256 or 512, hw a multiple of 4 in [16, 256]
+// and the image's cells within the LDS of a CU.
+bool ImageMfmaFits(int M, int K, int hw);
+// Needs ImageMfmaFits and 16-byte aligned x / out.
+hipError_t LaunchImageMfma(int out_kind, const ImageMfmaParams& p, hipStream_t stream);
+
 // Largest dynamic LDS size a kernel of this library may be given.
 constexpr int kMaxLdsBytes = 160 * 1024;
 constexpr int kMfmaTilePos = 128;

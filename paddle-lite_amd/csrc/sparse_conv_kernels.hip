@@ -22,9 +22,9 @@
 // Positions are the flattened (image, pixel) index g = n*hw + p, so tiles do
 // not care about image boundaries.
 #include "epilogue.h"
+#include "launch_lds.h"
 #include "sparse_conv_kernels.h"
 
-#include <atomic>
 #include <type_traits>
 
 // This file is compiled as four translation units (in parallel) selected by
@@ -880,25 +880,8 @@ __global__ void __launch_bounds__(256, (KSMAX == 4 ? 4 : 2)) BlockMfmaKernel(con
 #endif  // PL_PART_MFMA_ANY
 
 // ------------------------------------------------------------- launch glue
-// Dynamic LDS above the default limit has to be enabled per kernel and
-// device; remember what was already enabled (one static per instantiation).
-template <typename Kernel, typename Params>
-hipError_t LaunchWithLds(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const Params& p) {
-  if (lds > 48 * 1024) {
-    constexpr int kMaxDevices = 64;
-    static std::atomic<size_t> enabled[kMaxDevices];
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    if (dev < 0 || dev >= kMaxDevices || enabled[dev].load(std::memory_order_acquire) < lds) {
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (e != hipSuccess) return e;
-      if (dev >= 0 && dev < kMaxDevices) enabled[dev].store(lds, std::memory_order_release);
-    }
-  }
-  hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);
-  return hipGetLastError();
-}
+// LaunchWithLds (launch_lds.h) enables dynamic LDS above the default limit per
+// kernel function and device.
 
 #if PL_PART_WALK
 template <bool INT8, int OUT, int NR>

@@ -1,0 +1,121 @@
+"""The image MFMA kernel (one workgroup per image and 128 output rows, whole
+image in LDS) against the CPU oracle through the C ABI: bit-exact for every
+int8 kind.  Shapes cover every class of row alignment (H*W / 4 mod 4 = 0..3),
+one to sixteen window quads left over at the end of a row, images smaller
+than one window, every supported channel count and several row groups."""
+import copy
+import sys
+
+import numpy as np
+import pytest
+
+from helpers import capi, workloads, pla, make_kernel, run_hip, run_oracle, oracle_pack, assert_same
+
+pytestmark = pytest.mark.gpu
+
+AP = pla.ActivationParam
+ACTS = {
+    "none": AP(),
+    "relu": AP("relu"),
+    "relu6": AP("relu6", Relu_clipped_coef=6.0),
+    "leaky": AP("leaky_relu", Leaky_relu_alpha=0.1),
+    "hswish": AP("hard_swish"),
+}
+KINDS = {"acc32": capi.KIND_INT8_ACC32, "fp32out": capi.KIND_INT8_FP32, "int8out": capi.KIND_INT8_INT8}
+
+
+def announce(*what):
+    print("CASE", *what, file=sys.stderr, flush=True)
+
+
+def case_for(kind, batch, ic, oc, h, w, sparsity, paired, act, seed):
+    c = workloads.make_int8("img", batch, ic, oc, h, w, sparsity, paired, act, out_int8=(kind == capi.KIND_INT8_INT8), seed=seed, output_scale=0.05 if kind == capi.KIND_INT8_INT8 else 1.0)
+    c.kind = kind
+    return c
+
+
+# (batch, ic, oc, h, w).  H*W/4 mod 4: 14x14 -> 1, 6x10 -> 3, 8x8 -> 0, 6x9 -> ... (54 is not a multiple of 4, excluded),
+# 10x10 -> 1, 12x14 -> 2, 16x16 -> 0 (largest image), 4x4 -> 0 (smaller than a window), 5x8 -> 2, 4x7 -> 3
+SHAPES = [
+    (3, 512, 128, 14, 14), (2, 256, 256, 6, 10), (2, 128, 128, 8, 8), (1, 512, 384, 10, 10), (2, 256, 128, 12, 14),
+    (1, 512, 128, 16, 16), (3, 128, 256, 4, 4), (2, 256, 128, 5, 8), (2, 128, 128, 4, 7), (1, 512, 128, 9, 12), (9, 256, 128, 2, 10),
+]
+
+
+@pytest.mark.parametrize("kind", sorted(KINDS))
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_image_mfma_bit_exact(shape, kind):
+    announce("image", shape, kind)
+    batch, ic, oc, h, w = shape
+    k = KINDS[kind]
+    for act in (("none",) if kind == "acc32" else ("leaky", "hswish")):
+        case = case_for(k, batch, ic, oc, h, w, 0.85, False, ACTS[act], seed=ic + 3 * oc + h * w)
+        got = run_hip(case, capi.ALGO_IMAGE_MFMA)
+        want = run_oracle(case, oracle_pack(case))
+        assert_same(case, got, want, "image %s %s %s" % (kind, act, shape))
+    if kind == "acc32":
+        ref = np.einsum("mk,bkp->bmp", case.dense.astype(np.int64), case.x.reshape(batch, ic, -1).astype(np.int64)).reshape(got.shape)
+        assert np.array_equal(got.astype(np.int64), ref)
+
+
+@pytest.mark.parametrize("act", sorted(ACTS))
+@pytest.mark.parametrize("out_int8", [False, True], ids=["fp32out", "int8out"])
+@pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
+def test_image_mfma_activations_and_structures(paired, out_int8, act):
+    announce("image acts", paired, out_int8, act)
+    kind = capi.KIND_INT8_INT8 if out_int8 else capi.KIND_INT8_FP32
+    case = case_for(kind, 2, 128, 128, 14, 14, 0.8, paired, ACTS[act], seed=77)
+    got = run_hip(case, capi.ALGO_IMAGE_MFMA, force_semi=paired)
+    want = run_oracle(case, oracle_pack(case, force_semi=paired))
+    assert_same(case, got, want, "image %s" % act)
+
+
+def test_image_mfma_agrees_with_the_other_algorithms_and_no_bias():
+    announce("image vs others")
+    case = case_for(capi.KIND_INT8_FP32, 4, 256, 256, 14, 14, 0.9, False, ACTS["relu"], seed=5)
+    case.bias = None
+    a = run_hip(case, capi.ALGO_IMAGE_MFMA)
+    b = run_hip(case, capi.ALGO_BLOCK_MFMA)
+    c = run_hip(case, capi.ALGO_ROW_WALK)
+    assert np.array_equal(a, b) and np.array_equal(a, c)
+    assert_same(case, a, run_oracle(case, oracle_pack(case)), "no bias")
+
+
+def test_image_mfma_empty_and_dense_rows():
+    announce("image extremes")
+    case = case_for(capi.KIND_INT8_ACC32, 2, 128, 128, 6, 6, 0.5, False, AP(), seed=9)
+    case.dense[5] = 0          # an output row without nonzeros
+    case.dense[64:68] = 127    # fully dense rows of the largest magnitude
+    case.x[0] = -127
+    got = run_hip(case, capi.ALGO_IMAGE_MFMA)
+    ref = np.einsum("mk,bkp->bmp", case.dense.astype(np.int64), case.x.reshape(2, 128, -1).astype(np.int64)).reshape(got.shape)
+    assert np.array_equal(got.astype(np.int64), ref)
+    assert np.all(got[:, 5] == 0)
+
+
+def test_auto_picks_the_image_kernel_only_where_it_applies():
+    announce("image auto")
+    L = capi.lib()
+    case = case_for(capi.KIND_INT8_FP32, 64, 512, 512, 14, 14, 0.85, False, ACTS["leaky"], seed=0)
+    kernel, _ = make_kernel(case, capi.ALGO_AUTO)
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 64, 196) == capi.ALGO_IMAGE_MFMA
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 2, 196) == capi.ALGO_BLOCK_MFMA      # too few work items
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 64, 49) == capi.ALGO_BLOCK_MFMA      # 7x7 is not a multiple of 4
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 64, 28 * 28) == capi.ALGO_BLOCK_MFMA  # does not fit LDS
+    # the same handle serves all of them
+    import torch
+
+    for batch, h, w in ((2, 14, 14), (3, 7, 7)):
+        sub = copy.copy(case)  # same weights, another input size (the oracle's offsets are baked per H*W)
+        sub.x = np.ascontiguousarray(case.x[:batch, :, :h, :w])
+        got = kernel.Run(torch.from_numpy(sub.x).cuda()).cpu().numpy()
+        assert np.array_equal(got, run_oracle(sub))
+    # explicit requests outside the kernel's shapes are refused, not rerouted
+    odd = case_for(capi.KIND_INT8_FP32, 1, 96, 128, 4, 4, 0.5, False, AP(), seed=1)
+    with pytest.raises(capi.SparseConvError) as e:
+        make_kernel(odd, capi.ALGO_IMAGE_MFMA)
+    assert e.value.code == capi.PL_ERR_UNSUPPORTED
+    k2, _ = make_kernel(case_for(capi.KIND_INT8_FP32, 1, 128, 128, 7, 7, 0.5, False, AP(), seed=1), capi.ALGO_IMAGE_MFMA)
+    with pytest.raises(capi.SparseConvError) as e:
+        k2.Run(torch.zeros((1, 128, 7, 7), dtype=torch.int8, device="cuda"))
+    assert e.value.code == capi.PL_ERR_UNSUPPORTED
