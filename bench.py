@@ -24,13 +24,22 @@ LLC_BYTES = 256 << 20  # last-level (Infinity) cache the rotation must exceed
 COPY_CALIBRATION_BYTES = 64 << 20
 
 
+# c3 is the metric of BASELINE.json; the other configurations are reported under their own names
+METRICS = {
+    "c1": "sparse 1x1 conv nnz-GOP/s + % HBM roofline (fp32 unstructured, N=1, 96->192@56x56, 80%)",
+    "c2": "sparse 1x1 conv nnz-GOP/s + % HBM roofline (fp32 semi-structured, N=32, 256->512@28x28, 90%)",
+    "c3": "sparse 1x1 conv nnz-GOP/s + % HBM roofline (int8, N=64, 512->512@14x14, 85%)",
+    "c4": "sparse 1x1 conv nnz-GOP/s + % HBM roofline (int8->int8 semi-structured, N=128, 128->256@56x56, 75%)",
+}
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib", "mobilenet"])
-    ap.add_argument("--algo", default="auto", choices=["auto", "walk", "mfma"])
+    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib", "mobilenet", "density-sweep"])
+    ap.add_argument("--algo", default="auto", choices=["auto", "walk", "mfma", "image"])
     ap.add_argument("--fp16", action="store_true", help="run an fp32 configuration (c1, c2) through the half-precision kernel")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cache-resident", action="store_true", help="reuse one buffer set (reported, never the headline)")
@@ -168,6 +177,66 @@ def run_calib(args):
     return 0
 
 
+def run_density_sweep(args):
+    """Two shapes (the metric shape, and a layer with sixteen times its dense
+    work for the same input and output bytes) at sparsities from 50 to 99 %,
+    zeros placed at random or as whole 32x32 blocks, through every int8
+    algorithm: kernel time per launch (HIP events, rotating buffers) and what
+    PL_ALGO_AUTO chooses.  Every timed kernel's output is compared with the
+    oracle on one image first.  Not the headline metric: printed as its own
+    JSON line."""
+    import numpy as np
+    import torch
+
+    import helpers
+
+    capi, wl = helpers.capi, helpers.workloads
+    L = capi.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    names = {capi.ALGO_ROW_WALK: "row_walk", capi.ALGO_BLOCK_MFMA: "block_mfma", capi.ALGO_IMAGE_MFMA: "image_mfma"}
+    steps = max(50, min(args.steps, 300))
+    rows = []
+    for shape in ("metric", "wide"):
+        batch, ic, oc, hw = wl.DENSITY_SHAPES[shape]
+        set_bytes = batch * hw * hw * (ic + 4 * oc)
+        n_sets = int(LLC_BYTES * 1.25 // set_bytes) + 1
+        xs = outs = None
+        for blocked in (False, True):
+            for sparsity in (0.50, 0.70, 0.85, 0.90, 0.95, 0.98, 0.99):
+                case = wl.config_density(shape, sparsity, blocked)
+                if xs is None:
+                    x0 = torch.from_numpy(case.x).cuda()
+                    xs = [x0] + [x0.clone() for _ in range(n_sets - 1)]
+                    outs = [torch.empty((batch, oc, hw, hw), dtype=torch.float32, device="cuda") for _ in range(n_sets)]
+                    xp = (C.c_void_p * n_sets)(*[t.data_ptr() for t in xs])
+                    op = (C.c_void_p * n_sets)(*[t.data_ptr() for t in outs])
+                want = helpers.run_oracle(case, x=case.x[:1])
+                row = {"shape": "N=%d %d->%d @%dx%d" % (batch, ic, oc, hw, hw), "sparsity": sparsity, "zeros": "blocks" if blocked else "random", "nnz": case.nnz, "kernel_us": {}}
+                for a in (capi.ALGO_ROW_WALK, capi.ALGO_BLOCK_MFMA, capi.ALGO_IMAGE_MFMA, capi.ALGO_AUTO):
+                    try:
+                        kernel, _ = helpers.make_kernel(case, algo=a)
+                    except capi.SparseConvError:
+                        continue  # the shape is outside this algorithm's range
+                    if a == capi.ALGO_AUTO:
+                        info = kernel.info()
+                        row["auto"] = names[capi.check(L.pl_sparse_conv_algo_for(kernel._handle, batch, hw * hw))]
+                        row["blocks_present"] = [info["mfma_blocks"], info["mfma_blocks_total"]]
+                        continue
+                    capi.check(L.pl_sparse_conv_run_sequence(kernel._handle, xp, op, n_sets, batch, hw * hw, n_sets + 10, C.c_void_p(stream), None))
+                    torch.cuda.synchronize()
+                    assert np.array_equal(outs[0][:1].cpu().numpy(), want), "%s differs from the oracle at %s" % (names[a], row)
+                    ms = C.c_float(0.0)
+                    capi.check(L.pl_sparse_conv_run_sequence(kernel._handle, xp, op, n_sets, batch, hw * hw, steps, C.c_void_p(stream), C.byref(ms)))
+                    row["kernel_us"][names[a]] = round(ms.value * 1e3 / steps, 2)
+                row["fastest"] = min(row["kernel_us"], key=row["kernel_us"].get)
+                rows.append(row)
+        del xs, outs
+        torch.cuda.empty_cache()
+    print(json.dumps({"metric": "int8 sparse 1x1 conv: kernel us per launch by algorithm, sparsity and zero structure", "unit": "us", "n_gpus": 1, "steps": steps, "data": "synthetic",
+                      "config": {"workload": "density_sweep", "parity_checked": True}, "rows": rows}))
+    return 0
+
+
 def run_c5(args):
     """MobileNetV1-1.0 pointwise stack (13 layers, batch 64, int8 -> int8, 90 %
     unstructured zeros, relu) timed as one sequence of 13 launches per step.
@@ -188,6 +257,8 @@ def run_c5(args):
     total_ops = total_bytes = 0.0
     for i in range(13):
         case = wl.config5_layer(i)
+        if args.algo == "image":
+            raise SystemExit("--algo image applies to single layers; the stack holds shapes outside the image kernel's range (use auto)")
         kernel, weights = helpers.make_kernel(case, algo={"auto": capi.ALGO_AUTO, "walk": capi.ALGO_ROW_WALK, "mfma": capi.ALGO_BLOCK_MFMA}[args.algo])
         ic, oc, hw = wl.MOBILENET_V1_POINTWISE[i]
         chained = prev_out is not None and tuple(prev_out.shape[1:]) == (ic, hw, hw)
@@ -386,6 +457,8 @@ def main():
         sys.stderr.write("bench.py needs a GPU\n")
         return 2
     torch.cuda.set_device(0)
+    if args.config == "density-sweep":
+        return run_density_sweep(args)
     if args.config == "c5":
         return run_c5(args)
     if args.config == "calib":
@@ -401,7 +474,7 @@ def main():
         case.x = case.x.astype(np.float16)
         case.name += "_fp16"
         args.no_cpu_baseline = True  # the CPU baselines are fp32 / int8 paths
-    algo = {"auto": capi.ALGO_AUTO, "walk": capi.ALGO_ROW_WALK, "mfma": capi.ALGO_BLOCK_MFMA}[args.algo]
+    algo = {"auto": capi.ALGO_AUTO, "walk": capi.ALGO_ROW_WALK, "mfma": capi.ALGO_BLOCK_MFMA, "image": capi.ALGO_IMAGE_MFMA}[args.algo]
     kernel, weights = helpers.make_kernel(case, algo=algo)
     info = kernel.info()
     ops = case.algorithmic_ops()
@@ -472,10 +545,29 @@ def main():
         copy_gbs = 2.0 * (1 << 30) * 10 / (c0.elapsed_time(c1) * 1e-3) / 1e9
         del src, dst
     achieved = nbytes / (kernel_ms * 1e-3) / 1e9
-    algo_name = {capi.ALGO_ROW_WALK: "row_walk", capi.ALGO_BLOCK_MFMA: "block_mfma"}[info["algo"]]
+    algo_names = {capi.ALGO_ROW_WALK: "row_walk", capi.ALGO_BLOCK_MFMA: "block_mfma", capi.ALGO_IMAGE_MFMA: "image_mfma"}
+    algo_name = algo_names[capi.check(L.pl_sparse_conv_algo_for(kernel._handle, case.batch, case.im_size))]
     traffic, traffic_detail = measured_traffic(case.name, algo_name)
+    # int8: the same launch through every algorithm the shape allows (same rotating buffers, 300 launches each)
+    per_algo = None
+    if case.kind in (capi.KIND_INT8_FP32, capi.KIND_INT8_INT8):
+        per_algo = {algo_name: round(kernel_ms * 1e3, 3)}
+        for a, name in sorted(algo_names.items()):
+            if name in per_algo:
+                continue
+            try:
+                other, _ = helpers.make_kernel(case, algo=a)
+            except capi.SparseConvError:
+                continue  # this shape is outside the algorithm's range
+            if L.pl_sparse_conv_run_sequence(other._handle, xp, op, n_sets, case.batch, case.im_size, 50, C.c_void_p(stream), None) < 0:
+                continue
+            torch.cuda.synchronize()
+            assert np.array_equal(outs[0][:nchk].cpu().numpy(), want), "%s output differs from the oracle" % name
+            ms_o = C.c_float(0.0)
+            capi.check(L.pl_sparse_conv_run_sequence(other._handle, xp, op, n_sets, case.batch, case.im_size, 300, C.c_void_p(stream), C.byref(ms_o)))
+            per_algo[name] = round(ms_o.value * 1e3 / 300, 3)
     line = {
-        "metric": "sparse 1x1 conv nnz-GOP/s + % HBM roofline (int8, N=64, 512->512@14x14, 85%)",
+        "metric": METRICS[args.config] + (" (half-precision kernel)" if args.fp16 else ""),
         "value": ops * args.steps / wall / 1e9,
         "unit": "nnz-GOP/s",
         "n_gpus": 1,
@@ -514,6 +606,7 @@ def main():
             "measured_copy_GBs": copy_gbs,
             "frac_of_measured_copy": achieved / copy_gbs if copy_gbs else None,
             "cache_resident_kernel_us": cache_resident_us,
+            "kernel_us_by_algorithm": per_algo,
         },
     }
     if args.copy_calibration:

@@ -84,6 +84,26 @@ def make_int8(name, batch, ic, oc, h, w, sparsity, paired, act, out_int8, seed=0
     return Case(name, kind, x, dense, bias, act, weight_scale=ws, input_scale=input_scale, output_scale=output_scale, paired=paired)
 
 
+DENSITY_SHAPES = {"metric": (64, 512, 512, 14), "wide": (16, 2048, 2048, 14)}
+
+
+def config_density(shape, sparsity, blocked, seed=0):
+    """int8 -> fp32 with leaky_relu at a chosen sparsity on one of
+    DENSITY_SHAPES (batch, ic, oc, h = w): "metric" is the metric shape, "wide"
+    a layer with sixteen times its dense work for the same input and output
+    bytes.  blocked: zeros come as whole 32x32 blocks of the weight matrix (a
+    Bernoulli mask over the grid of blocks, kept blocks fully dense) instead
+    of single weights."""
+    batch, ic, oc, hw = DENSITY_SHAPES[shape]
+    c = make_int8("density_%s_%02d_%s" % (shape, round(sparsity * 100), "blocked" if blocked else "random"), batch, ic, oc, hw, hw, 0.0 if blocked else sparsity, False,
+                  ActivationParam("leaky_relu", Leaky_relu_alpha=0.1), out_int8=False, seed=seed)
+    if blocked:
+        rng = np.random.RandomState(seed + 1000)
+        keep = rng.random_sample((oc // 32, ic // 32)) >= sparsity
+        c.dense = (c.dense * np.kron(keep, np.ones((32, 32), dtype=bool))).astype(np.int8)
+    return c
+
+
 def config1(batch=1):
     """fp32 unstructured, 1x96x56x56 -> 192, 80 % zeros, relu."""
     return make_fp32("c1_fp32_unstructured", batch, 96, 192, 56, 56, 0.80, False, ActivationParam("relu"), seed=0, w_sigma=0.1)

@@ -119,3 +119,31 @@ def test_auto_picks_the_image_kernel_only_where_it_applies():
     with pytest.raises(capi.SparseConvError) as e:
         k2.Run(torch.zeros((1, 128, 7, 7), dtype=torch.int8, device="cuda"))
     assert e.value.code == capi.PL_ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("kind", ["acc32", "fp32out", "int8out"])
+def test_mixed_empty_sparse_and_dense_blocks_all_algorithms(kind):
+    """A weight matrix whose 32x32 blocks are empty, 5 % filled or fully dense
+    in equal parts (plus one all-zero row block and one all-zero k-step):
+    every int8 algorithm against the oracle, and against each other."""
+    announce("mixed blocks", kind)
+    k = KINDS[kind]
+    case = case_for(k, 3, 256, 256, 14, 14, 0.0, False, ACTS["none" if kind == "acc32" else "relu6"], seed=21)
+    rng = np.random.RandomState(4)
+    kinds = rng.randint(0, 3, size=(8, 8))  # 0 empty, 1 sparse, 2 dense
+    kinds[3, :] = 0  # an empty row block
+    kinds[:, 5] = 0  # a channel block no row uses
+    mask = np.zeros((256, 256), dtype=bool)
+    for bi in range(8):
+        for bj in range(8):
+            blk = {0: np.zeros((32, 32), bool), 1: rng.random_sample((32, 32)) < 0.05, 2: np.ones((32, 32), bool)}[int(kinds[bi, bj])]
+            mask[32 * bi:32 * bi + 32, 32 * bj:32 * bj + 32] = blk
+    case.dense = (case.dense * mask).astype(np.int8)
+    want = run_oracle(case, oracle_pack(case))
+    results = {}
+    for name, algo in (("walk", capi.ALGO_ROW_WALK), ("block", capi.ALGO_BLOCK_MFMA), ("image", capi.ALGO_IMAGE_MFMA), ("auto", capi.ALGO_AUTO)):
+        results[name] = run_hip(case, algo)
+        assert_same(case, results[name], want, "mixed blocks %s %s" % (kind, name))
+    kernel, _ = make_kernel(case, capi.ALGO_BLOCK_MFMA)
+    info = kernel.info()
+    assert info["mfma_blocks"] == int(np.count_nonzero([[mask[32 * i:32 * i + 32, 32 * j:32 * j + 32].any() for j in range(8)] for i in range(8)])) < info["mfma_blocks_total"] == 64
