@@ -142,6 +142,7 @@ struct pl_sparse_conv_handle {
   DevBuf cw_desc, cw_idx, cw_wts;
   int cw_chunks = 0, cw_slices = 0;
   int walk_chunked = 1;  // 0 never, 1 when the problem is large enough, 2 whenever the shape allows
+  bool walk_plain_fits = true;  // false: more channels than the plain walk's LDS tile holds, only the chunked walk can run
   // half-precision row walk
   bool half = false;
   pl::DevActH act_h{};
@@ -574,8 +575,13 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
     // fp32 tiles carry one all-zero row behind the channels
     const size_t row_bytes = static_cast<size_t>(int8 ? CeilDiv(desc->ic, 4) : desc->ic + 1) * 4;
     if (row_bytes * 16 > static_cast<size_t>(pl::kMaxLdsBytes)) {
-      delete h;
-      return Fail(PL_ERR_UNSUPPORTED, "ic = %d does not fit an LDS tile", desc->ic);
+      // the whole-K tile of the plain walk does not fit LDS; the fp32 walk over
+      // channel chunks needs no such tile and serves the shapes it supports
+      if (int8) {
+        delete h;
+        return Fail(PL_ERR_UNSUPPORTED, "ic = %d does not fit an LDS tile", desc->ic);
+      }
+      h->walk_plain_fits = false;
     }
   }
   h->algo = algo;
@@ -726,8 +732,10 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     c.sub_tiles = h->mfma_sub_tiles;
     if (h->mfma_tile_quads > 0) c.tile_quads = h->mfma_tile_quads;
     e = pl::LaunchBlockMfma(c, p, s);
-  } else if (!h->int8 && vec && h->walk_chunked > 0 && h->cw_chunks > 0 &&
-             (h->walk_chunked == 2 || (h->ic > 128 && static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kChunkWalkTile)) * h->cw_slices >= 256))) {
+  } else if (!h->int8 && !h->walk_plain_fits && !vec) {
+    return Fail(PL_ERR_UNSUPPORTED, "fp32 with ic = %d runs as a walk over channel chunks, which needs H*W %% 4 == 0 and 16-byte aligned tensors (H*W = %d)", h->ic, im_size);
+  } else if (!h->int8 && vec && h->cw_chunks > 0 &&
+             (!h->walk_plain_fits || (h->walk_chunked > 0 && (h->walk_chunked == 2 || (h->ic > 128 && static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kChunkWalkTile)) * h->cw_slices >= 256))))) {
     // fp32 with many channels and enough work for every CU: walk over
     // channel chunks (256 positions per list fetch)
     pl::ChunkWalkParams p{};

@@ -33,6 +33,22 @@ std::vector<float> PerChannelScales(const operators::SparseConvParam& param) {
   if (s.size() == 1) s.resize(oc, s[0]);
   return s;
 }
+
+// The device kernels compute a 1x1 / stride 1 / pad 0 / dilation 1 / group 1
+// convolution and size their reads from the output's H*W.  The detect pass
+// only creates the op under these conditions
+// (lite/core/optimizer/mir/sparse_conv_detect_pass.cc:596-640), but an op
+// description loaded from a model file can say anything, and the op's own
+// InferShape honours strides and paddings: refuse what would make the kernel
+// read outside the input.
+void CheckGeometry(const operators::SparseConvParam& param) {
+  for (int s : param.strides) CHECK_EQ(s, 1) << "sparse_conv2d(kHIP): strides must be 1";
+  CHECK(param.paddings != nullptr && param.dilations != nullptr) << "sparse_conv2d(kHIP): paddings / dilations unset";
+  for (int p : *param.paddings) CHECK_EQ(p, 0) << "sparse_conv2d(kHIP): paddings must be 0";
+  for (int d : *param.dilations) CHECK_EQ(d, 1) << "sparse_conv2d(kHIP): dilations must be 1";
+  CHECK_EQ(param.groups, 1) << "sparse_conv2d(kHIP): groups must be 1";
+  CHECK_EQ(param.x->dims().size(), 4u) << "sparse_conv2d(kHIP): Input must be NCHW";
+}
 }  // namespace
 
 void SetSparseConvReferenceQuirks(bool on) { g_reference_quirks = on; }
@@ -47,7 +63,9 @@ template <PrecisionType P, PrecisionType O>
 void SparseConvCompute<P, O>::Upload(int kind) {
   auto& param = this->template Param<param_t>();
   CHECK(param.x && param.nonzero_weights && param.oc_nonzeros && param.diffs) << "sparse_conv2d: unset input";
+  CheckGeometry(param);
   const DDim& xd = param.x->dims();
+  ic_ = xd[1];
   pl_sparse_conv_desc d{};
   d.struct_size = sizeof(d);
   d.kind = kind;
@@ -135,8 +153,12 @@ void SparseConvCompute<P, O>::Run() {
   auto& ctx = this->ctx_->template As<HIPContext>();
   CHECK(handle_ != nullptr) << "PrepareForRun was not called";
   CHECK(param.x->target() == TargetType::kHIP) << "sparse_conv2d(kHIP): Input must live on the device (io_copy missing?)";
+  CheckGeometry(param);
   const DDim& xd = param.x->dims();
   const DDim& od = param.output->dims();
+  CHECK_EQ(od.size(), 4u) << "sparse_conv2d(kHIP): Output must be NCHW";
+  CHECK_EQ(xd[1], ic_) << "sparse_conv2d(kHIP): Input has " << xd[1] << " channels, the weights were prepared for " << ic_;
+  CHECK(xd[0] == od[0] && xd[2] * xd[3] == od[2] * od[3]) << "sparse_conv2d(kHIP): Input and Output differ in batch or H*W";
   const int batch = static_cast<int>(xd[0]);
   const int im_size = static_cast<int>(od[2] * od[3]);
   void* out = (O == PRECISION(kFloat)) ? static_cast<void*>(param.output->template mutable_data<float>(TargetType::kHIP))

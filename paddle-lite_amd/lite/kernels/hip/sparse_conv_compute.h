@@ -36,6 +36,7 @@ class SparseConvCompute : public KernelLite<TARGET(kHIP), Ptype> {
   bool flag_trans_bias_{false};
   std::vector<float> w_scale_;
   pl_sparse_conv_handle* handle_{nullptr};
+  int64_t ic_{0};  // input channels the weights were prepared for
 };
 
 // The reference divides the int8-output leaky_relu slope by the output scale

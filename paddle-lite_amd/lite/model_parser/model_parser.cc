@@ -75,6 +75,18 @@ PrecisionType ToPrecision(int var_type) {
   }
 }
 
+size_t ElementBytes(PrecisionType p) {
+  switch (p) {
+    case PrecisionType::kBool:
+    case PrecisionType::kInt8:
+    case PrecisionType::kUInt8: return 1;
+    case PrecisionType::kInt16:
+    case PrecisionType::kFP16: return 2;
+    case PrecisionType::kInt64: return 8;
+    default: return 4;
+  }
+}
+
 // ------------------------------------------------------------- topology
 Builder::Ref WriteAttr(Builder* b, const std::string& name, const std::any& value) {
   const std::type_info& t = value.type();
@@ -246,9 +258,20 @@ void FillTensor(const Table& param, Scope* scope) {
   if (!t.valid() || !t.Has(slot::kParamData)) throw FormatError("parameter " + name + " has no data");
   const auto dim = t.Vector<int64_t>(slot::kParamDim);
   const auto data = t.Vector<uint8_t>(slot::kParamData);
+  // the dimensions must describe exactly the bytes that are there: kernels size
+  // their reads from the dimensions
+  const PrecisionType precision = ToPrecision(t.Scalar<int32_t>(slot::kParamDataType, 0));
+  const std::vector<int64_t> dims = dim.ToVector();
+  uint64_t numel = 1;
+  for (int64_t d : dims) {
+    if (d < 0 || (d > 0 && numel > (uint64_t{1} << 40) / static_cast<uint64_t>(d))) throw FormatError("parameter " + name + " has illegal dimensions");
+    numel *= static_cast<uint64_t>(d);
+  }
+  if (numel * ElementBytes(precision) != data.size())
+    throw FormatError("parameter " + name + ": dimensions describe " + std::to_string(numel * ElementBytes(precision)) + " bytes, the record holds " + std::to_string(data.size()));
   Tensor* tensor = scope->Var(name)->GetMutable<Tensor>();
-  tensor->Resize(dim.ToVector());
-  tensor->set_precision(ToPrecision(t.Scalar<int32_t>(slot::kParamDataType, 0)));
+  tensor->Resize(dims);
+  tensor->set_precision(precision);
   void* dst = tensor->mutable_data(TargetType::kHost, data.size());
   if (data.size()) std::memcpy(dst, data.bytes(), data.size());
   tensor->set_persistable(true);

@@ -36,6 +36,17 @@ static int g_failures = 0;
     }                                                                  \
   } while (0)
 
+// true when f() raises a FatalError whose text contains `what`
+template <typename F>
+static bool ThrowsWith(const char* what, F f) {
+  try {
+    f();
+  } catch (const FatalError& e) {
+    return std::string(e.what()).find(what) != std::string::npos;
+  }
+  return false;
+}
+
 template <typename F>
 static bool Throws(F f) {
   try {
@@ -338,6 +349,31 @@ static void RegistryAndErrorPaths() {
     EXPECT(ks.size() == 1);
     EXPECT(Throws([&] { ks[0]->Launch(); }));
   }
+  // An op description that is not 1x1 / stride 1 / pad 0 / dilation 1 / group 1 (only a model file can
+  // carry one: the pass never creates it) is refused by the kHIP kernel before any device work: its
+  // output would be larger than the input the kernel reads.
+  auto refused = [&](const char* what, std::function<void(OpInfo*)> edit) {
+    Scope s;
+    std::vector<float> w2;
+    Problem q{1, 8, 4, 4, 4, 0.6f, false, false, false, false, "", 5};
+    std::vector<OpInfo> o{MakeConv(q, &s, &w2, &is, &os)};
+    mir::SparseConvDetectPass ps;
+    ps.SetSparseThreshold(0.0f);
+    EXPECT(ps.Apply(&o, &s) == 1);
+    edit(&o[0]);
+    auto sp = LiteOpRegistry::Global().Create("sparse_conv2d");
+    EXPECT(sp->Attach(o[0], &s) && sp->InferShape());
+    auto ks = sp->CreateKernels({paddle::lite_api::Place(TARGET(kHIP), PRECISION(kFloat), DATALAYOUT(kNCHW))}, "sparse_conv2d/def");
+    EXPECT(ks.size() == 1);
+    if (!ThrowsWith(what, [&] { ks[0]->Launch(); })) {
+      std::printf("  FAILED: the kHIP kernel accepted an op with %s\n", what);
+      ++g_failures;
+    }
+  };
+  refused("paddings must be 0", [](OpInfo* o) { o->SetAttr<std::vector<int>>("paddings", {1, 1}); });
+  refused("strides must be 1", [](OpInfo* o) { o->SetAttr<std::vector<int>>("strides", {2, 2}); });
+  refused("dilations must be 1", [](OpInfo* o) { o->SetAttr<std::vector<int>>("dilations", {2, 2}); });
+  refused("groups must be 1", [](OpInfo* o) { o->SetAttr<int>("groups", 2); });
 }
 
 // The precision changes either side of an int8 convolution: op attach /

@@ -287,3 +287,23 @@ def test_error_paths_return_codes():
     assert L.pl_sparse_conv_run(h, None, None, 1, 4, None) == capi.PL_ERR_BAD_ARG
     assert L.pl_sparse_conv_run(h, None, None, 0, 4, None) == capi.PL_OK  # empty batch
     L.pl_sparse_conv_destroy(h)
+
+
+def test_fp32_more_channels_than_the_plain_walks_lds_tile():
+    """The plain fp32 walk keeps all channels of 16 positions (plus a zero row)
+    in LDS: 2559 channels fit, 2560 do not.  Beyond that the walk over channel
+    chunks serves the shapes it supports (H*W a multiple of 4, aligned
+    tensors); other shapes are refused at the call, not at prepare."""
+    import torch
+
+    announce("fp32 large K")
+    for ic, h, w, ok in ((2559, 3, 3, True), (2560, 3, 3, False), (2560, 4, 4, True), (3000, 2, 6, True), (3000, 5, 5, False)):
+        case = small_case(capi.KIND_FP32, 2, ic, 24, h, w, 0.9, False, ACTS["relu"], seed=ic + h)
+        kernel, _ = make_kernel(case, capi.ALGO_ROW_WALK)  # prepare succeeds in every case
+        if ok:
+            got = run_hip(case, kernel=kernel)
+            assert_same(case, got, run_oracle(case, oracle_pack(case)), "fp32 ic=%d %dx%d" % (ic, h, w))
+        else:
+            with pytest.raises(capi.SparseConvError) as e:
+                kernel.Run(torch.from_numpy(case.x).cuda())
+            assert e.value.code == capi.PL_ERR_UNSUPPORTED

@@ -101,3 +101,31 @@ def test_truncated_fixture_is_refused(tool, tmp_path):
         f.write(data[: len(data) - 7])
     rc, out = run(tool, "dump", cut)
     assert rc == 1 and out.startswith("error:")
+
+
+def test_dimensions_that_overstate_the_data_are_refused(tool, tmp_path):
+    """A parameter record whose dimensions claim more elements than its data
+    holds must not load: kernels size their reads from the dimensions."""
+    with open(os.path.join(GOLDEN, "ref_example_v2.nb"), "rb") as f:
+        data = bytearray(f.read())
+    # the dimension vector [9] of the int8 tensor conv2_w_nonzeros_output: length 1, then one int64
+    pat = (1).to_bytes(4, "little") + (9).to_bytes(8, "little")
+    hits = []
+    at = data.find(pat)
+    while at >= 0:
+        hits.append(at)
+        at = data.find(pat, at + 1)
+    assert hits, "no vector [9] in the fixture"
+    # the same vector also occurs as the variable's shape in the topology; exactly one occurrence is the
+    # parameter record's, and raising it must be refused
+    refused = 0
+    for i, at in enumerate(hits):
+        patched = bytearray(data)
+        patched[at + 4:at + 12] = (10).to_bytes(8, "little")
+        bad = str(tmp_path / ("overstated%d.nb" % i))
+        with open(bad, "wb") as f:
+            f.write(patched)
+        rc, out = run(tool, "dump", bad)
+        if rc == 1 and out.startswith("error:") and "dimensions describe 10 bytes, the record holds 9" in out:
+            refused += 1
+    assert refused == 1
