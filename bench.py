@@ -128,6 +128,24 @@ def cpu_baseline(case, packed, budget_s=12.0):
         "ms": best * 1e3,
         "sample": "full batch, best of %d, exact-accumulating blocked per-image GEMM with OpenMP" % reps,
     }
+    # the reference's own x86 dense conv2d 1x1 (int8 -> fp32 only: its GEMM is in-tree; the fp32 path needs
+    # MKL).  Timing only: its 16-bit pair sums saturate on full-range inputs.
+    if case.kind == helpers.capi.KIND_INT8_FP32 and O.have_ref_x86_gemm():
+        ws = np.asarray(case.weight_scale, np.float32)
+        relu = {O.ACT_RELU: (1, 1.0), O.ACT_RELU6: (2, act.relu6_coef), O.ACT_LEAKY_RELU: (3, act.leaky_alpha)}.get(act.type, (0, 1.0))
+        legs = {}
+        for name, th in (("serial", 1), ("all_cores", threads)):
+            reps = 1
+            O.ref_x86_conv1x1_s8_f32(case.x[:max(1, th)], case.dense, ws, case.input_scale, bias, relu[0], relu[1], 1, th)
+            while True:
+                _, secs = O.ref_x86_conv1x1_s8_f32(case.x, case.dense, ws, case.input_scale, bias, relu[0], relu[1], reps, th)
+                if secs > 2.0 or reps >= 64:
+                    break
+                reps *= 2
+            legs[name] = {"value": ops_img * case.batch * reps / secs / 1e9, "unit": "nnz-GOP/s", "dense_GOPs": 2.0 * oc * ic * hw * case.batch * reps / secs / 1e9, "cores": th, "kind": "reference",
+                          "ms_per_batch": secs * 1e3 / reps,
+                          "sample": "%d passes over the batch, generate_gemm_s8u8_x86_kern<float>::compute per image as Conv2dCompute<kInt8,kFloat>::Run calls it%s" % (reps, "" if th == 1 else "; images dealt to OpenMP threads (an extension: the reference's loop over images is serial)")}
+        naive["x86_dense_reference"] = legs
     del packed
     return naive
 

@@ -373,3 +373,82 @@ def dense_conv1x1(out_kind, w_dense, x, scale=None, bias=None, act=None,
                                    _p(scale), _p(out), batch, M, K, N,
                                    C.byref(act) if act else None, int(threads))
     return out, used
+
+
+# ------------------------------------------------- reference packers / x86 GEMM
+_REF_PACKERS_PATH = os.path.join(_HERE, "_ref", "libref_packers.so")
+_REF_X86_GEMM_PATH = os.path.join(_HERE, "_ref", "libref_x86_gemm.so")
+
+
+def have_ref_packers():
+    return os.path.exists(_REF_PACKERS_PATH)
+
+
+def have_ref_x86_gemm():
+    return os.path.exists(_REF_X86_GEMM_PATH)
+
+
+def _ref_lib(path):
+    if path not in _ref:
+        _ref[path] = C.CDLL(path)
+    return _ref[path]
+
+
+def ref_count_zeros_pad4(w):
+    """The reference's ComputeSparseZeros (lite/tests/math/conv_ut.h:183-207)."""
+    w = _c(w)
+    nb = C.c_int(0)
+    z = _ref_lib(_REF_PACKERS_PATH).ref_count_zeros_pad4(_dtype_code(w), _p(w), w.shape[0], w.shape[1], C.byref(nb))
+    return z, nb.value
+
+
+def ref_count_semi(w):
+    """The reference's ComputeSemiSparseZeros (conv_ut.h:209-274)."""
+    w = _c(w)
+    cn, cc, cb, fs = C.c_int(0), C.c_int(0), C.c_int(0), C.c_int(0)
+    z = _ref_lib(_REF_PACKERS_PATH).ref_count_semi(_dtype_code(w), _p(w), w.shape[0], w.shape[1], C.byref(cn), C.byref(cc), C.byref(cb), C.byref(fs))
+    return dict(zeros=z, count_nonzeroes=cn.value, count_channels=cc.value, count_blocks=cb.value, flag_semi=fs.value)
+
+
+def ref_pack(w, im_size, layout):
+    """The reference's ComputeSparseWeight (both overloads) /
+    ComputeSemiSparseWeight (conv_ut.h:276-538) on a dense [M, K] matrix; the
+    output sizes are what its tests allocate (conv_ut.h counting passes)."""
+    w = _c(w)
+    M, K = w.shape
+    if layout == LAYOUT_PADDED:
+        _, n_w = ref_count_zeros_pad4(w)
+        n_d = n_w
+    elif layout == LAYOUT_UNPADDED:
+        n_w = n_d = int(np.count_nonzero(w))
+    else:
+        c = ref_count_semi(w)
+        if not c["flag_semi"]:
+            raise ValueError("the reference packs semi-structured only where its block rule fires")
+        n_w, n_d = c["count_nonzeroes"], c["count_blocks"]
+    nz = np.zeros(max(n_w, 1), dtype=w.dtype)[:n_w]
+    oc = np.zeros(M, dtype=np.uint32)
+    df = np.zeros(max(n_d, 1), dtype=np.int32)[:n_d]
+    code = {LAYOUT_UNPADDED: 0, LAYOUT_PADDED: 1, LAYOUT_SEMI: 2}[layout]
+    fn = _ref_lib(_REF_PACKERS_PATH).ref_pack
+    fn.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int64]
+    first_ic = fn(_dtype_code(w), code, _p(w), M, K, int(im_size), _p(nz), n_w, _p(oc), _p(df), n_d)
+    if first_ic < 0:
+        raise ValueError("the reference packer refused the matrix")
+    return Packed(layout, nz, oc, df, first_ic, int(layout == LAYOUT_SEMI), M, K, int(im_size))
+
+
+def ref_x86_conv1x1_s8_f32(x, w_dense, weight_scale, input_scale, bias=None, relu_type=0, relu_alpha=1.0, reps=1, threads=1):
+    """The reference's x86 int8 GEMM run like its dense conv2d kernel runs a
+    1x1 convolution (lite/kernels/x86/conv_compute.cc:215-340).  Returns
+    (out, seconds spent in the compute calls)."""
+    x, w_dense = _c(x, np.int8), _c(w_dense, np.int8)
+    ws, bias = _c(weight_scale, np.float32), _c(bias, np.float32)
+    batch, K, N = x.shape[0], x.shape[1], int(np.prod(x.shape[2:]))
+    M = w_dense.shape[0]
+    out = np.zeros((batch, M) + x.shape[2:], dtype=np.float32)
+    fn = _ref_lib(_REF_X86_GEMM_PATH).ref_x86_conv1x1_s8_f32
+    fn.restype = C.c_double
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_int]
+    secs = fn(_p(x), _p(out), batch, M, N, K, _p(w_dense), _p(ws), float(input_scale), _p(bias), int(relu_type), float(relu_alpha), int(reps), int(threads))
+    return out, secs
