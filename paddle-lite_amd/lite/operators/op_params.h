@@ -15,9 +15,9 @@ namespace paddle {
 namespace lite {
 namespace operators {
 
-struct ParamBase {
-  virtual ~ParamBase() = default;
-};
+// An empty base as in the reference (lite/operators/op_params.h:36): the
+// parameter structs carry no virtual table, their first field sits at offset 0.
+struct ParamBase {};
 
 struct ActivationParam : ParamBase {
   const lite::Tensor* X{};
