@@ -95,6 +95,7 @@ MODEL_TOOL_BIN = os.path.join(ROOT, "tests", "cpp", "model_file_tool")
 LITE_SOURCES = [
     "core/tensor.cc",
     "core/op_lite.cc",
+    "core/optimizer/mir/graph.cc",
     "core/optimizer/mir/sparse_conv_detect_pass.cc",
     "core/optimizer/mir/int8_chain_pass.cc",
     "model_parser/model_parser.cc",

@@ -1,5 +1,6 @@
 #include "lite/core/optimizer/mir/int8_chain_pass.h"
 
+#include <algorithm>
 #include <map>
 
 #include "lite/core/op_registry.h"
@@ -9,10 +10,13 @@ namespace lite {
 namespace mir {
 namespace {
 
+// Where the value of a variable can be read from: the host tensor (feeds),
+// the fp32 tensor on the device, and int8 tensors on the device, one per
+// quantisation scale that a consumer asked for.
 struct VarState {
-  bool on_device = false;
-  bool int8 = false;
-  std::string name;  // variable that currently holds the value
+  std::string host;
+  std::string dev_fp32;
+  std::map<float, std::string> dev_int8;
 };
 
 bool IsInt8Op(const OpInfo& op) { return op.HasAttr("enable_int8") && op.GetAttr<bool>("enable_int8"); }
@@ -41,61 +45,84 @@ ProgramStep Calib(const std::string& from, const std::string& to, float scale, b
 }  // namespace
 
 std::vector<ProgramStep> Int8ChainPass::Apply(const std::vector<OpInfo>& ops, const std::vector<std::string>& feeds, const std::vector<std::string>& fetches, Scope* scope) const {
+  const Graph graph(ops, *scope);
+  return Apply(graph, feeds, fetches, scope);
+}
+
+std::vector<ProgramStep> Int8ChainPass::Apply(const Graph& graph, const std::vector<std::string>& feeds, const std::vector<std::string>& fetches, Scope* scope) const {
   std::vector<ProgramStep> steps;
   std::map<std::string, VarState> vars;
   for (const std::string& f : feeds) {
     CHECK(scope->FindVar(f) != nullptr) << "feed " << f << " is not in the scope";
-    vars[f] = VarState{false, false, f};
+    vars[f].host = f;
   }
   auto is_fetch = [&](const std::string& v) { return std::find(fetches.begin(), fetches.end(), v) != fetches.end(); };
 
+  const std::vector<OpInfo> ops = graph.TopologicalOps();
   for (size_t i = 0; i < ops.size(); ++i) {
     OpInfo op = ops[i];
     const bool depthwise = op.Type() == "depthwise_conv2d";
-    CHECK(op.Type() == "sparse_conv2d" || depthwise) << "this pass handles chains of sparse_conv2d and depthwise_conv2d, got " << op.Type();
+    CHECK(op.Type() == "sparse_conv2d" || depthwise) << "this pass handles graphs of sparse_conv2d and depthwise_conv2d, got " << op.Type();
     const bool int8 = IsInt8Op(op);
     CHECK(int8 || !depthwise) << "depthwise_conv2d has int8 kernels only on this target";
     const std::string in = op.Input("Input").front();
     const std::string out = op.Output("Output").front();
     CHECK(vars.count(in) != 0) << "input " << in << " of op " << i << " has no producer and is not fed";
 
-    // output type: int8 only if the value is consumed, only by int8 ops, and
-    // not wanted by the caller
+    // Output type (static_kernel_pick_pass.cc:97-135): int8 only if the
+    // value is consumed, by int8 ops only, and not wanted by the caller; the
+    // output scale is then the consumers' input scale.  Consumers that
+    // disagree on that scale cannot share one int8 tensor: the op then
+    // produces fp32 and each consumer gets its own calib.
     bool out_int8 = int8 && !is_fetch(out);
     bool consumed = false;
     float consumer_scale = 1.f;
-    for (size_t j = i + 1; j < ops.size() && out_int8; ++j) {
-      if (ops[j].Input("Input").front() != out) continue;
-      if (!IsInt8Op(ops[j])) {
-        out_int8 = false;
+    for (const Graph::Node* consumer : graph.Consumers(out)) {
+      if (!out_int8) break;
+      const OpInfo& c = consumer->op;
+      if (!c.HasInput("Input") || c.Input("Input").front() != out || !IsInt8Op(c)) {
+        out_int8 = false;  // read as something else than an int8 activation
         break;
       }
-      CHECK(ops[j].HasInputScale("Input0_scale", true)) << "int8 consumer without an input scale";
-      if (!consumed) consumer_scale = ops[j].GetInputScale("Input0_scale", true)[0];
+      CHECK(c.HasInputScale("Input0_scale", true)) << "int8 consumer without an input scale";
+      const float sc = c.GetInputScale("Input0_scale", true)[0];
+      if (consumed && sc != consumer_scale) out_int8 = false;
+      consumer_scale = sc;
       consumed = true;
     }
     out_int8 = out_int8 && consumed;
     if (out_int8) op.SetOutputScale("Output0_scale", {consumer_scale}, true);
 
-    // bring the input where and how the kernel declares it
-    VarState cur = vars[in];
-    if (!cur.on_device) {
-      const std::string dev = cur.name + "/hip";
-      steps.push_back(IoCopy(cur.name, dev, true));
-      cur.on_device = true;
-      cur.name = dev;
-    }
-    if (int8 && !cur.int8) {
+    // bring the input where and how the kernel declares it; later consumers
+    // of the same variable reuse the copies and casts made here
+    VarState& cur = vars[in];
+    std::string src;
+    if (int8) {
       CHECK(op.HasInputScale("Input0_scale", true)) << "int8 op without an input scale";
-      const std::string q = cur.name + "/int8";
-      steps.push_back(Calib(cur.name, q, op.GetInputScale("Input0_scale", true)[0], true));
-      cur.int8 = true;
-      cur.name = q;
-    } else if (!int8 && cur.int8) {
-      LOG(FATAL) << "an fp32 op consumes the int8 output of op " << in << ": the output-type rule forbids it";
+      const float sc = op.GetInputScale("Input0_scale", true)[0];
+      auto q = cur.dev_int8.find(sc);
+      if (q == cur.dev_int8.end()) {
+        CHECK(cur.dev_int8.empty() || !cur.dev_fp32.empty() || !cur.host.empty())
+            << "variable " << in << " exists as int8 with another scale only: the output-type rule forbids it";
+        if (cur.dev_fp32.empty()) {
+          CHECK(!cur.host.empty()) << "variable " << in << " has no fp32 form to quantise";
+          cur.dev_fp32 = cur.host + "/hip";
+          steps.push_back(IoCopy(cur.host, cur.dev_fp32, true));
+        }
+        const std::string name = cur.dev_fp32 + (cur.dev_int8.empty() ? "/int8" : "/int8_" + std::to_string(cur.dev_int8.size()));
+        steps.push_back(Calib(cur.dev_fp32, name, sc, true));
+        q = cur.dev_int8.emplace(sc, name).first;
+      }
+      src = q->second;
+    } else {
+      if (cur.dev_fp32.empty()) {
+        CHECK(!cur.host.empty()) << "an fp32 op consumes variable " << in << ", which exists as int8 only: the output-type rule forbids it";
+        cur.dev_fp32 = cur.host + "/hip";
+        steps.push_back(IoCopy(cur.host, cur.dev_fp32, true));
+      }
+      src = cur.dev_fp32;
     }
-    vars[in] = cur;  // later consumers of the same variable reuse the casts
-    op.SetInput("Input", {cur.name});
+    op.SetInput("Input", {src});
 
     ProgramStep s;
     s.op = op;
@@ -104,13 +131,19 @@ std::vector<ProgramStep> Int8ChainPass::Apply(const std::vector<OpInfo>& ops, co
                          : std::string("sparse_conv2d/") + (!int8 ? "def" : (out_int8 ? "int8_int8_out" : "int8_fp32_out"));
     s.place = lite_api::Place(TARGET(kHIP), int8 ? PRECISION(kInt8) : PRECISION(kFloat), DATALAYOUT(kNCHW));
     steps.push_back(s);
-    vars[out] = VarState{true, out_int8, out};
+    VarState& produced = vars[out];
+    if (out_int8) {
+      produced.dev_int8[consumer_scale] = out;
+    } else {
+      produced.dev_fp32 = out;
+    }
   }
   for (const std::string& f : fetches) {
     CHECK(vars.count(f) != 0) << "fetch " << f << " is never produced";
     const VarState& v = vars[f];
-    CHECK(!v.int8) << "a fetched variable is fp32 by the output-type rule";
-    if (v.on_device) steps.push_back(IoCopy(v.name, f + "/host", false));
+    if (!v.host.empty()) continue;  // a feed wanted back: already on the host
+    CHECK(!v.dev_fp32.empty()) << "a fetched variable is fp32 by the output-type rule";
+    steps.push_back(IoCopy(v.dev_fp32, f + "/host", false));
   }
   return steps;
 }

@@ -1,6 +1,6 @@
 // What the reference's optimiser does around quantised ops, restated for a
-// linear list of sparse_conv2d and int8 depthwise_conv2d ops that all run on
-// TARGET(kHIP):
+// graph of sparse_conv2d and int8 depthwise_conv2d ops that all run on
+// TARGET(kHIP) (a variable may have several consumers):
 //  * the output-type rule of static_kernel_pick_pass
 //    (lite/core/optimizer/mir/static_kernel_pick_pass.cc:97-135): an op with
 //    enable_int8 produces int8 only if every consumer of its output has
@@ -24,6 +24,7 @@
 #include "lite/core/kernel.h"
 #include "lite/core/op_desc.h"
 #include "lite/core/op_lite.h"
+#include "lite/core/optimizer/mir/graph.h"
 #include "lite/core/scope.h"
 
 namespace paddle {
@@ -42,6 +43,8 @@ class Int8ChainPass {
   // `feeds`: fp32 host tensors in `scope`.  `fetches`: variables wanted back
   // on the host as fp32; the host copy of "v" is named "v/host".
   std::vector<ProgramStep> Apply(const std::vector<OpInfo>& ops, const std::vector<std::string>& feeds, const std::vector<std::string>& fetches, Scope* scope) const;
+  // The same on a graph (consumers are read from its links, steps come out in topological order).
+  std::vector<ProgramStep> Apply(const Graph& graph, const std::vector<std::string>& feeds, const std::vector<std::string>& fetches, Scope* scope) const;
 };
 
 // Creates the op and the kernel of every step once, then launches them in

@@ -1,5 +1,7 @@
 #include "lite/core/optimizer/mir/sparse_conv_detect_pass.h"
 
+#include "lite/core/optimizer/mir/graph.h"
+
 #include "pl_sparse_conv.h"
 #include "lite/core/tensor.h"
 
@@ -35,8 +37,16 @@ Counts Analyse(int dtype, const void* w, int oc, int ic) {
 }  // namespace
 
 int SparseConvDetectPass::Apply(std::vector<OpInfo>* ops, Scope* scope) const {
+  Graph graph(*ops, *scope);
+  const int replaced = Apply(&graph, scope);
+  *ops = graph.TopologicalOps();
+  return replaced;
+}
+
+int SparseConvDetectPass::Apply(Graph* graph, Scope* scope) const {
   int replaced = 0;
-  for (OpInfo& conv : *ops) {
+  for (Graph::Node* node : graph->OpNodes()) {
+    OpInfo& conv = node->op;
     if (conv.Type() != "conv2d") continue;
     const std::string x = conv.Input("Input").front();
     const std::string w = conv.Input("Filter").front();
@@ -96,8 +106,22 @@ int SparseConvDetectPass::Apply(std::vector<OpInfo>* ops, Scope* scope) const {
     sparse.CopyAttrsFrom(conv);
     sparse.SetAttr<int>("first_ic", first_ic);
     sparse.SetAttr<int>("flag_semi", c.flag_semi);
-    conv = sparse;
-    scope->Erase(w);  // the dense filter is dropped with its node (:835-845)
+
+    // The rewrite on the graph (:828-857): the conv node goes, the sparse op
+    // node takes over its links to the activation, the bias and the output,
+    // the three new weight variables are linked in, and the dense filter's
+    // node is dropped.  A filter that another op still reads keeps its node
+    // and its tensor (the reference removes the node regardless and would
+    // leave that op with a dangling link).
+    const int order = node->order;
+    Graph::Node* filter = graph->Var(w);
+    graph->RemoveNode(node);  // `conv` is gone from here on
+    for (const char* weight : {"_nonzeros_output", "_oc_nonzeros", "_ic_diffs"}) graph->RetrieveVarNode(w + weight, true);
+    graph->CreateOpNode(sparse, order);
+    if (filter != nullptr && filter->outlinks.empty() && filter->inlinks.empty()) {
+      graph->RemoveNode(filter);
+      scope->Erase(w);
+    }
     ++replaced;
   }
   return replaced;

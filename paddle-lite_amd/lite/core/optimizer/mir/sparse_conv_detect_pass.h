@@ -1,8 +1,8 @@
-// sparse_conv_detect_pass on a linear op list: rewrites every eligible
-// conv2d (1x1, stride 1, pad 0, group 1, fp32 or int8 weights, enough zeros)
-// into sparse_conv2d and creates its three weight tensors
-// (reference: lite/core/optimizer/mir/sparse_conv_detect_pass.{h,cc}; there
-// the same rewrite runs on the SSA graph and is bound to TARGET(kARM) only).
+// sparse_conv_detect_pass: rewrites every eligible conv2d (1x1, stride 1,
+// pad 0, group 1, fp32 or int8 weights, enough zeros) of a graph into
+// sparse_conv2d and creates its three weight tensors
+// (reference: lite/core/optimizer/mir/sparse_conv_detect_pass.{h,cc}, bound
+// to TARGET(kARM) only there).
 #pragma once
 
 #include <string>
@@ -15,6 +15,8 @@
 namespace paddle {
 namespace lite {
 namespace mir {
+
+class Graph;
 
 class SparseConvDetectPass {
  public:
@@ -34,7 +36,14 @@ class SparseConvDetectPass {
   // Targets the pass runs for; the reference binds kARM, this build adds kHIP.
   static bool BoundTo(lite_api::TargetType t) { return t == lite_api::TargetType::kARM || t == lite_api::TargetType::kHIP; }
 
-  // Rewrites ops in place; returns how many conv2d ops were replaced.
+  // The rewrite on the graph, as the reference runs it
+  // (sparse_conv_detect_pass.cc:596-857): every eligible conv2d node is
+  // replaced by a sparse_conv2d node that takes over its links, the three new
+  // weight variables are linked in and the dense filter's node is dropped.
+  // Returns how many conv2d ops were replaced.
+  int Apply(Graph* graph, Scope* scope) const;
+  // Convenience for a list of ops: builds the graph, applies the pass and
+  // writes the ops back in topological order (list order for a chain).
   int Apply(std::vector<OpInfo>* ops, Scope* scope) const;
 
  private:

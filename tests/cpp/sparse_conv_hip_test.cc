@@ -7,6 +7,7 @@
 //
 //   sparse_conv_hip_test --cpu   registry, op, pass and error paths (no device)
 //   sparse_conv_hip_test --gpu   the above plus execution on the device
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -16,6 +17,7 @@
 #include <vector>
 
 #include "lite/core/op_registry.h"
+#include "lite/core/optimizer/mir/graph.h"
 #include "lite/core/optimizer/mir/int8_chain_pass.h"
 #include "lite/core/optimizer/mir/sparse_conv_detect_pass.h"
 #include "lite/kernels/hip/sparse_conv_compute.h"
@@ -663,6 +665,179 @@ static Tensor RunSparseOnDevice(OpInfo info, Scope* scope, PrecisionType prec, c
   return y_host;
 }
 
+// A graph with a branch: one int8 layer whose output feeds an int8 layer and
+// an fp32 layer.  The output-type rule (static_kernel_pick_pass.cc:97-135)
+// keeps the producer's output fp32 ("int8 out only if all consumers are
+// int8"), the int8 consumer gets a calib, the fp32 consumer reads the fp32
+// tensor; on the device both fetched outputs equal the oracle's.  Also: int8
+// consumers that disagree on their input scale, a filter shared by two convs,
+// and the graph bookkeeping of the detect pass.
+static void BranchingGraph(bool run_on_device) {
+  std::printf("branching graph\n");
+  std::fflush(stdout);
+  const int batch = 2, hh = 6, ww = 6, hw = hh * ww;
+  const int c0 = 48, c1 = 64, c2 = 40, c3 = 24;
+  const float s0 = 0.02f, s1 = 0.05f;
+  Scope scope;
+  std::mt19937 gen(99);
+  std::uniform_real_distribution<float> uni(0.f, 1.f);
+  std::normal_distribution<float> nrm(0.f, 1.f);
+  Tensor* a0 = scope.NewTensor("a0");
+  a0->Resize({batch, c0, hh, ww});
+  float* a0d = a0->mutable_data<float>(TargetType::kHost);
+  for (int64_t i = 0; i < a0->numel(); ++i) a0d[i] = uni(gen) * 2.f - 1.f;
+  struct Layer {
+    std::vector<int8_t> w8;
+    std::vector<float> wf, ws, bias;
+  };
+  auto make = [&](const std::string& n, const std::string& in, const std::string& out, int ic, int oc, bool int8, float in_scale, Layer* L) {
+    Tensor* w = scope.NewTensor("w" + n);
+    w->Resize({oc, ic, 1, 1});
+    if (int8) {
+      int8_t* wd = w->mutable_data<int8_t>(TargetType::kHost);
+      for (int64_t i = 0; i < w->numel(); ++i) {
+        int v = static_cast<int>(uni(gen) * 127.f) + 1;
+        if (uni(gen) < 0.5f) v = -v;
+        wd[i] = uni(gen) >= 0.7f ? static_cast<int8_t>(v) : 0;
+      }
+      L->w8.assign(wd, wd + w->numel());
+    } else {
+      float* wd = w->mutable_data<float>(TargetType::kHost);
+      for (int64_t i = 0; i < w->numel(); ++i) wd[i] = uni(gen) >= 0.7f ? nrm(gen) * 0.1f : 0.f;
+      L->wf.assign(wd, wd + w->numel());
+    }
+    Tensor* b = scope.NewTensor("b" + n);
+    b->Resize({oc});
+    float* bd = b->mutable_data<float>(TargetType::kHost);
+    L->bias.resize(oc);
+    for (int i = 0; i < oc; ++i) L->bias[i] = bd[i] = nrm(gen) * 0.1f;
+    L->ws.resize(oc);
+    for (float& v : L->ws) v = 0.001f + 0.004f * uni(gen);
+    OpInfo conv("conv2d");
+    conv.SetInput("Input", {in});
+    conv.SetInput("Filter", {"w" + n});
+    conv.SetInput("Bias", {"b" + n});
+    conv.SetOutput("Output", {out});
+    scope.NewTensor(out);
+    conv.SetAttr<std::vector<int>>("strides", {1, 1});
+    conv.SetAttr<std::vector<int>>("paddings", {0, 0});
+    conv.SetAttr<std::vector<int>>("dilations", {1, 1});
+    conv.SetAttr<int>("groups", 1);
+    conv.SetAttr<bool>("with_act", true);
+    conv.SetAttr<std::string>("act_type", "relu");
+    if (int8) {
+      conv.SetAttr<bool>("enable_int8", true);
+      conv.SetInputScale("Input0_scale", {in_scale}, true);
+      conv.SetInputScale("Filter0_scale", L->ws, true);
+      conv.SetOutputScale("Output0_scale", {1.f}, true);
+    }
+    return conv;
+  };
+  Layer A, B, Cc;
+  std::vector<OpInfo> ops;
+  ops.push_back(make("A", "a0", "a1", c0, c1, true, s0, &A));
+  ops.push_back(make("B", "a1", "yb", c1, c2, true, s1, &B));
+  ops.push_back(make("C", "a1", "yc", c1, c3, false, 1.f, &Cc));
+  scope.FindMutableTensor("a1")->Resize({batch, c1, hh, ww});
+
+  mir::Graph graph(ops, scope);
+  const mir::Graph& cgraph = graph;
+  EXPECT(graph.OpNodes().size() == 3 && cgraph.Consumers("a1").size() == 2 && cgraph.Producer("a1") == cgraph.OpNodes()[0]);
+  EXPECT(graph.Var("wA") != nullptr);
+  mir::SparseConvDetectPass detect;
+  detect.SetSparseThreshold(0.5f);
+  EXPECT(detect.Apply(&graph, &scope) == 3);
+  // the conv nodes are gone, the sparse ops hold their links, the dense filters left graph and scope
+  EXPECT(graph.OpNodes().size() == 3 && cgraph.Consumers("a1").size() == 2);
+  for (const auto* n : cgraph.OpNodes()) EXPECT(n->op.Type() == "sparse_conv2d" && n->inlinks.size() == 5 && n->outlinks.size() == 1);
+  EXPECT(graph.Var("wA") == nullptr && scope.FindVar("wA") == nullptr && graph.Var("wA_ic_diffs") != nullptr && graph.Var("wA_ic_diffs")->is_weight);
+  EXPECT(cgraph.Producer("a1") != nullptr && cgraph.Producer("a1")->op.Type() == "sparse_conv2d" && cgraph.Producer("a0") == nullptr);
+
+  mir::Int8ChainPass chain;
+  std::vector<mir::ProgramStep> steps = chain.Apply(cgraph, {"a0"}, {"yb", "yc"}, &scope);
+  // io_copy a0, calib a0, A (fp32 out), calib a1 for B, B, C, two fetches
+  EXPECT(steps.size() == 8);
+  if (steps.size() == 8) {
+    EXPECT(steps[2].kernel == "sparse_conv2d/int8_fp32_out");
+    EXPECT(steps[3].kernel == "calib/fp32_to_int8" && steps[3].op.GetAttr<float>("scale") == s1 && steps[3].op.Input("Input").front() == "a1");
+    EXPECT(steps[4].kernel == "sparse_conv2d/int8_fp32_out" && steps[4].op.Input("Input").front() == "a1/int8");
+    EXPECT(steps[5].kernel == "sparse_conv2d/def" && steps[5].op.Input("Input").front() == "a1");
+    EXPECT(steps[6].kernel == "io_copy/device_to_host" && steps[7].kernel == "io_copy/device_to_host");
+  }
+  // the same with the fp32 consumer first in the list: the int8 consumer still gets its calib
+  {
+    std::vector<OpInfo> reordered = cgraph.TopologicalOps();
+    std::swap(reordered[1], reordered[2]);
+    auto st = chain.Apply(reordered, {"a0"}, {"yb", "yc"}, &scope);
+    EXPECT(st.size() == 8 && st[3].kernel == "sparse_conv2d/def" && st[4].kernel == "calib/fp32_to_int8" && st[5].kernel == "sparse_conv2d/int8_fp32_out");
+  }
+  // two int8 consumers that agree on the scale share an int8 output; if they disagree the producer
+  // keeps fp32 and each gets its own calib
+  {
+    std::vector<OpInfo> two = cgraph.TopologicalOps();
+    two[2] = two[1];
+    two[2].SetOutput("Output", {"yb2"});
+    auto st = chain.Apply(two, {"a0"}, {"yb", "yb2"}, &scope);
+    EXPECT(st.size() == 7 && st[2].kernel == "sparse_conv2d/int8_int8_out" && st[2].op.GetOutputScale("Output0_scale", true)[0] == s1 && st[3].op.Input("Input").front() == "a1" &&
+           st[4].op.Input("Input").front() == "a1");
+    two[2].SetInputScale("Input0_scale", {0.07f}, true);
+    st = chain.Apply(two, {"a0"}, {"yb", "yb2"}, &scope);
+    EXPECT(st.size() == 9 && st[2].kernel == "sparse_conv2d/int8_fp32_out" && st[3].kernel == "calib/fp32_to_int8" && st[5].kernel == "calib/fp32_to_int8" &&
+           st[3].op.GetAttr<float>("scale") == s1 && st[5].op.GetAttr<float>("scale") == 0.07f && st[3].op.Output("Out").front() != st[5].op.Output("Out").front());
+  }
+  // a filter read by two convs stays in the graph and in the scope while one of them still reads it
+  {
+    Scope s2;
+    std::vector<float> w2;
+    float is, os;
+    Problem q{1, 8, 4, 4, 4, 0.7f, false, false, false, false, "", 6};
+    OpInfo c1op = MakeConv(q, &s2, &w2, &is, &os);
+    OpInfo c2op = c1op;
+    c2op.SetOutput("Output", {"y2"});
+    s2.NewTensor("y2");
+    c2op.SetAttr<std::vector<int>>("strides", {2, 2});  // not eligible: keeps reading the dense filter
+    std::vector<OpInfo> shared{c1op, c2op};
+    mir::SparseConvDetectPass ps;
+    ps.SetSparseThreshold(0.5f);
+    EXPECT(ps.Apply(&shared, &s2) == 1);
+    EXPECT(shared[0].Type() == "sparse_conv2d" && shared[1].Type() == "conv2d" && s2.FindVar("conv_w") != nullptr);
+  }
+  // a variable written twice is refused
+  {
+    std::vector<OpInfo> twice = cgraph.TopologicalOps();
+    twice[2].SetOutput("Output", {"yb"});
+    EXPECT(Throws([&] { mir::Graph g(twice, scope); }));
+  }
+  if (!run_on_device) return;
+
+  mir::HipProgram program(steps, &scope);
+  program.Run();
+  const Tensor* yb = scope.FindMutableTensor("yb/host");
+  const Tensor* yc = scope.FindMutableTensor("yc/host");
+  EXPECT(yb != nullptr && yb->dims() == DDim({batch, c2, hh, ww}) && yc != nullptr && yc->dims() == DDim({batch, c3, hh, ww}));
+  // oracle: A int8 -> fp32, then B on the requantised tensor and C (fp32 weights) on the fp32 one
+  std::vector<int8_t> q0(a0->numel());
+  plo_fp32_to_int8(a0d, q0.data(), s0, a0->numel());
+  plo_act act{1, 6.f, 0.1f, 6.f, 3.f, 6.f};
+  std::vector<float> ms(c1), mb(c1), a1(static_cast<size_t>(batch) * c1 * hw);
+  EXPECT(plo_merge_params(1, c1, A.ws.data(), c1, s0, 1.f, A.bias.data(), ms.data(), mb.data(), &act) == 0);
+  plo_dense_conv1x1(1, A.w8.data(), q0.data(), A.bias.data(), ms.data(), a1.data(), batch, c1, c0, hw, &act, 1);
+  std::vector<int8_t> q1(a1.size());
+  plo_fp32_to_int8(a1.data(), q1.data(), s1, static_cast<int64_t>(a1.size()));
+  std::vector<float> msb(c2), mbb(c2), want_b(static_cast<size_t>(batch) * c2 * hw), want_c(static_cast<size_t>(batch) * c3 * hw);
+  plo_act act_b{1, 6.f, 0.1f, 6.f, 3.f, 6.f};
+  EXPECT(plo_merge_params(1, c2, B.ws.data(), c2, s1, 1.f, B.bias.data(), msb.data(), mbb.data(), &act_b) == 0);
+  plo_dense_conv1x1(1, B.w8.data(), q1.data(), B.bias.data(), msb.data(), want_b.data(), batch, c2, c1, hw, &act_b, 1);
+  plo_dense_conv1x1(0, Cc.wf.data(), a1.data(), Cc.bias.data(), nullptr, want_c.data(), batch, c3, c1, hw, &act, 1);
+  if (yb) EXPECT(std::memcmp(want_b.data(), yb->raw_data(), want_b.size() * 4) == 0);
+  if (yc) {
+    const float* g = yc->data<float>();
+    double worst = 0;
+    for (size_t i = 0; i < want_c.size(); ++i) worst = std::max(worst, std::fabs(static_cast<double>(g[i]) - want_c[i]) / std::max(1.0, std::fabs(static_cast<double>(want_c[i]))));
+    EXPECT(worst < 1e-5);
+  }
+}
+
 // The optimised-model file: what the detect pass produced is written as a
 // "<name>.nb" file, read back into an empty scope, and the loaded
 // sparse_conv2d gives the same output bytes as the one that was saved.
@@ -1067,6 +1242,7 @@ int main(int argc, char** argv) {
   for (const Problem& p : problems) RunProblem(p, gpu);
   CalibChain(gpu);
   Int8Chain(gpu);
+  BranchingGraph(gpu);
   HalfPrecision(gpu);
   ModelFile(gpu);
   Depthwise(gpu);
