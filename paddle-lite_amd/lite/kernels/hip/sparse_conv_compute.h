@@ -3,9 +3,11 @@
 // gfx950 library behind Run().
 #pragma once
 
+#include <string>
 #include <vector>
 
 #include "lite/core/kernel.h"
+#include "lite/core/profile/profiler.h"
 #include "lite/operators/op_params.h"
 
 struct pl_sparse_conv_handle;
@@ -29,6 +31,12 @@ class SparseConvCompute : public KernelLite<TARGET(kHIP), Ptype> {
 
   const std::vector<float>& merged_scales() const { return w_scale_; }
 
+  // The math entry point and algorithm of the last Run(), for the profiler
+  // (the ARM class reports "sparse_conv_fp32_pipelined" etc. through
+  // KERNEL_FUNC_NAME, lite/kernels/arm/sparse_conv_compute.h:34-43).
+  void SetProfileRuntimeKernelInfo(paddle::lite::profile::OpCharacter* ch) const { ch->kernel_func_name = kernel_func_name_; }
+  const std::string& kernel_func_name() const { return kernel_func_name_; }
+
  private:
   void Upload(int kind);
 
@@ -37,6 +45,7 @@ class SparseConvCompute : public KernelLite<TARGET(kHIP), Ptype> {
   std::vector<float> w_scale_;
   pl_sparse_conv_handle* handle_{nullptr};
   int64_t ic_{0};  // input channels the weights were prepared for
+  std::string kernel_func_name_{"NotImplForSparseConv"};
 };
 
 // The reference divides the int8-output leaky_relu slope by the output scale

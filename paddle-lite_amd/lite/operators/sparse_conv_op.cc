@@ -125,6 +125,24 @@ bool SparseConvOp::AttachImpl(const cpp::OpDesc& d, Scope* scope) {
   return true;
 }
 
+void SparseConvOp::GetOpRuntimeInfo(paddle::lite::profile::OpCharacter* ch) const {
+  // names as lite_api::ActivationTypeToStr prints them (lite/api/paddle_place.cc:48-69), including
+  // the table's shift against the enum from position 6 on (hard_swish = 10 prints as "Abs")
+  static const char* const kActNames[] = {"unk", "Relu", "Relu6", "PRelu", "LeakyRelu", "Sigmoid", "Silu", "Tanh", "Swish", "Exp", "Abs", "HardSwish", "Reciprocal", "ThresholdedRelu", "Elu", "HardSigmoid", "log"};
+  const DDim& filter_dims = param_.oc_nonzeros->dims();
+  const DDim& input_dims = param_.x->dims();
+  const DDim& output_dims = param_.output->dims();
+  ch->op_type = "sparse_conv2d";
+  ch->input_shape = ch->DimToStr(input_dims);
+  ch->output_shape = ch->DimToStr(output_dims);
+  ch->filter_shape = ch->DimToStr(filter_dims) + "x" + std::to_string(input_dims[1]) + "x1x1";
+  const int act = static_cast<int>(param_.activation_param.active_type);
+  CHECK(act >= 0 && act < static_cast<int>(sizeof(kActNames) / sizeof(kActNames[0]))) << "unknown activation type " << act;
+  ch->remark = std::string("1x1p") + std::to_string((*param_.paddings)[0]) + "s" + std::to_string(param_.strides[0]) + "g" + std::to_string(param_.groups) + "d" + std::to_string((*param_.dilations)[0]) +
+               (param_.bias ? "Bias" : "") + kActNames[act];
+  ch->macs = Macs();
+}
+
 float SparseConvOp::Macs() const {
   return 2.f * param_.output->dims().production() * param_.x->dims()[1] / param_.groups;
 }

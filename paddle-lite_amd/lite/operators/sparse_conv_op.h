@@ -6,6 +6,7 @@
 #include <string>
 
 #include "lite/core/op_lite.h"
+#include "lite/core/profile/profiler.h"
 #include "lite/operators/op_params.h"
 
 namespace paddle {
@@ -26,6 +27,11 @@ class SparseConvOp : public OpLite {
   // Dense-counted multiply-accumulate operations, as the reference reports
   // them to its profiler (sparse_conv_op.h:41-63).
   float Macs() const;
+  // What the op tells the profiler about one run: shapes, the
+  // "1x1p<pad>s<stride>g<groups>d<dilation>[Bias]<Activation>" remark and the
+  // dense-counted operations (sparse_conv_op.h:41-63; compiled there under
+  // LITE_WITH_PROFILE only).
+  void GetOpRuntimeInfo(paddle::lite::profile::OpCharacter* ch) const;
   const SparseConvParam& param() const { return param_; }
 
  private:

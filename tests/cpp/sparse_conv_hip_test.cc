@@ -180,6 +180,20 @@ static void RunProblem(const Problem& p, bool run_on_device) {
   EXPECT(op->InferShape());
   Tensor* y = scope.FindMutableTensor("y");
   EXPECT(y->dims() == DDim({p.batch, p.oc, p.h, p.w}));
+  {
+    // what the op reports to the profiler (sparse_conv_op.h:41-63)
+    paddle::lite::profile::OpCharacter ch;
+    static_cast<operators::SparseConvOp*>(op.get())->GetOpRuntimeInfo(&ch);
+    const std::string dims = std::to_string(p.batch) + "x";
+    EXPECT(ch.input_shape == dims + std::to_string(p.ic) + "x" + std::to_string(p.h) + "x" + std::to_string(p.w));
+    EXPECT(ch.output_shape == dims + std::to_string(p.oc) + "x" + std::to_string(p.h) + "x" + std::to_string(p.w));
+    EXPECT(ch.filter_shape == std::to_string(p.oc) + "x" + std::to_string(p.ic) + "x1x1");
+    // the reference's name table has "Silu" inserted at position 6 while its enum has not
+    // (lite/api/paddle_place.cc:48-69 against paddle_place.h:122-148): kHardSwish = 10 prints as "Abs"
+    const std::string act = p.act == "relu" ? "Relu" : p.act == "relu6" ? "Relu6" : p.act == "leaky_relu" ? "LeakyRelu" : p.act == "hard_swish" ? "Abs" : "unk";
+    EXPECT(ch.remark == std::string("1x1p0s1g1d1") + (p.bias ? "Bias" : "") + act);
+    EXPECT(ch.macs == 2.f * p.batch * p.oc * p.h * p.w * p.ic);
+  }
 
   const PrecisionType prec = p.int8 ? PRECISION(kInt8) : PRECISION(kFloat);
   const std::string alias = !p.int8 ? "def" : (p.out_int8 ? "int8_int8_out" : "int8_fp32_out");
@@ -207,6 +221,13 @@ static void RunProblem(const Problem& p, bool run_on_device) {
   k->Launch();
   k->Launch();  // second epoch: no PrepareForRun
   k->mutable_context_as<HIPContext>()->Sync();
+  {
+    paddle::lite::profile::OpCharacter ch;
+    if (!p.int8) static_cast<kernels::hip::SparseConvCompute<PRECISION(kFloat), PRECISION(kFloat)>*>(k)->SetProfileRuntimeKernelInfo(&ch);
+    else if (p.out_int8) static_cast<kernels::hip::SparseConvCompute<PRECISION(kInt8), PRECISION(kInt8)>*>(k)->SetProfileRuntimeKernelInfo(&ch);
+    else static_cast<kernels::hip::SparseConvCompute<PRECISION(kInt8), PRECISION(kFloat)>*>(k)->SetProfileRuntimeKernelInfo(&ch);
+    EXPECT(ch.kernel_func_name == (p.int8 ? "pl_sparse_conv_run/block_mfma" : "pl_sparse_conv_run/row_walk"));
+  }
   EXPECT(y->target() == TARGET(kHIP));
   Tensor y_host;
   y_host.CopyDataFrom(*y, TargetType::kHost);
