@@ -86,16 +86,24 @@ __device__ __forceinline__ void ChunkWalkBody(const ChunkWalkParams& p, uint32_t
   const float* xcol = static_cast<const float*>(p.x) + (size_t)n * p.K * p.hw + pp;
   const uint32_t* xlane = tile + 4 * lane;  // the lane's four positions of LDS row 0
 
+  // The next chunk travels from memory into registers while the current one
+  // is walked (the walk itself issues no vector memory instruction, so it
+  // never waits for these loads); the registers are written to LDS once every
+  // wavefront has finished with the current chunk.
+  uint4 v[kChunk / kWaves];
+  auto fetch = [&](int chunk) {
+    const int c0 = chunk * kChunk;
+#pragma unroll
+    for (int u = 0; u < kChunk / kWaves; ++u) {
+      const int ch = min(c0 + r0 + kWaves * u, p.K - 1);
+      v[u] = *reinterpret_cast<const uint4*>(xcol + (size_t)ch * p.hw);
+    }
+  };
+  fetch(0);
   for (int chunk = 0; chunk < p.n_chunks; ++chunk) {
     if (chunk > 0) __syncthreads();  // the previous chunk is read until every wavefront has walked it
     {
       const int c0 = chunk * kChunk;
-      uint4 v[kChunk / kWaves];
-#pragma unroll
-      for (int u = 0; u < kChunk / kWaves; ++u) {
-        const int ch = min(c0 + r0 + kWaves * u, p.K - 1);
-        v[u] = *reinterpret_cast<const uint4*>(xcol + (size_t)ch * p.hw);
-      }
 #pragma unroll
       for (int u = 0; u < kChunk / kWaves; ++u) {
         const int kl = r0 + kWaves * u;
@@ -106,29 +114,40 @@ __device__ __forceinline__ void ChunkWalkBody(const ChunkWalkParams& p, uint32_t
       if (chunk == 0 && tid < kTile / 4) *reinterpret_cast<uint4*>(tile + (size_t)kChunk * kTile + 4 * tid) = make_uint4(0, 0, 0, 0);
     }
     __syncthreads();
+    if (chunk + 1 < p.n_chunks) fetch(chunk + 1);
 
     const ConstWords dw = descp + ((size_t)((slice * p.n_chunks + chunk) * kWaves + wave) * G) * 2;
 #pragma unroll
     for (int gi = 0; gi < G; ++gi) {
-      const uint32_t first = dw[2 * gi], batches = dw[2 * gi + 1];
+      const uint32_t first = dw[2 * gi], entries = dw[2 * gi + 1];
       const ConstWords ip = idxp + first;
       const ConstWords wp = wtsp + (size_t)first * (4 * NR);
+      auto entry = [&](uint32_t kl, uint32_t w0, uint32_t w1) {
+        const uint4 xv = *reinterpret_cast<const uint4*>(xlane + (size_t)kl * kTile);
+        const float x4[4] = {__uint_as_float(xv.x), __uint_as_float(xv.y), __uint_as_float(xv.z), __uint_as_float(xv.w)};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[gi][0][j] = __builtin_fmaf(x4[j], __uint_as_float(w0), acc[gi][0][j]);
+          if (NR == 2) acc[gi][NR - 1][j] = __builtin_fmaf(x4[j], __uint_as_float(w1), acc[gi][NR - 1][j]);
+        }
+      };
+      const uint32_t batches = entries >> 2, rem = entries & 3u;
       for (uint32_t b = 0; b < batches; ++b) {
         const uint32_t packed = ip[b];
         uint32_t w[4 * NR];
 #pragma unroll
         for (int i = 0; i < 4 * NR; ++i) w[i] = wp[(size_t)b * (4 * NR) + i];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const uint32_t kl = (packed >> (8 * e)) & 0xffu;
-          const uint4 xv = *reinterpret_cast<const uint4*>(xlane + (size_t)kl * kTile);
-          const float x4[4] = {__uint_as_float(xv.x), __uint_as_float(xv.y), __uint_as_float(xv.z), __uint_as_float(xv.w)};
+        for (int e = 0; e < 4; ++e) entry((packed >> (8 * e)) & 0xffu, w[e * NR], w[e * NR + NR - 1]);
+      }
+      if (rem != 0) {  // the last, partly filled batch: only its real entries
+        const uint32_t packed = ip[batches];
+        uint32_t w[3 * NR];
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            acc[gi][0][j] = __builtin_fmaf(x4[j], __uint_as_float(w[e * NR]), acc[gi][0][j]);
-            if (NR == 2) acc[gi][NR - 1][j] = __builtin_fmaf(x4[j], __uint_as_float(w[e * NR + NR - 1]), acc[gi][NR - 1][j]);
-          }
-        }
+        for (int i = 0; i < 3 * NR; ++i) w[i] = wp[(size_t)batches * (4 * NR) + i];
+        entry(packed & 0xffu, w[0], w[NR - 1]);
+        if (rem > 1) entry((packed >> 8) & 0xffu, w[NR], w[NR + NR - 1]);
+        if (rem > 2) entry((packed >> 16) & 0xffu, w[2 * NR], w[2 * NR + NR - 1]);
       }
     }
   }
@@ -186,13 +205,17 @@ hipError_t LaunchBig(K kernel, dim3 grid, dim3 block, size_t lds, hipStream_t s,
 
 hipError_t LaunchChunkWalk(int nrows, const ChunkWalkParams& p, hipStream_t stream) {
   if (p.P == 0 || p.n_groups == 0) return hipSuccess;
-  if (p.hw % 4 != 0 || p.n_chunks < 1 || p.slices < 1) return hipErrorInvalidValue;
+  if (p.hw % 4 != 0 || p.n_chunks < 1 || p.slices < 1 || (p.groups_per_wave != 4 && p.groups_per_wave != 8)) return hipErrorInvalidValue;
   ChunkWalkParams q = p;
   q.tiles = (int)((p.P + kTile - 1) / kTile);
   const size_t lds = (size_t)(kChunk + 1) * kTile * 4;
   dim3 grid(8u * (uint32_t)q.slices * (((uint32_t)q.tiles + 7) / 8)), block(64 * kWaves);
-  if (nrows == 2) return LaunchBig(ChunkWalkKernel<2, kChunkWalkGroups>, grid, block, lds, stream, q);
-  return LaunchBig(ChunkWalkKernel<1, kChunkWalkGroups>, grid, block, lds, stream, q);
+  if (p.groups_per_wave == 4) {
+    if (nrows == 2) return LaunchBig(ChunkWalkKernel<2, 4>, grid, block, lds, stream, q);
+    return LaunchBig(ChunkWalkKernel<1, 4>, grid, block, lds, stream, q);
+  }
+  if (nrows == 2) return LaunchBig(ChunkWalkKernel<2, 8>, grid, block, lds, stream, q);
+  return LaunchBig(ChunkWalkKernel<1, 8>, grid, block, lds, stream, q);
 }
 
 }  // namespace pl

@@ -164,14 +164,12 @@ __device__ __forceinline__ void DwItem(const DwConvParams& p, uint32_t plane, in
     const size_t row_at = ((size_t)plane * (uint32_t)p.oh + (uint32_t)oy) * (uint32_t)p.ow + (uint32_t)ox0;
     if (OUT == kOutI8) {
       uint32_t packed[CG];
-      int last[CG];  // third value of each group: a tail of three outputs stores it as a byte
 #pragma unroll
       for (int q4 = 0; q4 < CG; ++q4) {
-        int q[4];
+        float q[4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) q[k] = ActQuantI8<ACT>(__builtin_fmaf((float)acc[o][4 * q4 + k], s, b), p.act);
-        packed[q4] = PackI8x4(q[0], q[1], q[2], q[3]);
-        last[q4] = q[2];
+        for (int k = 0; k < 4; ++k) q[k] = ActQuantF<ACT>(__builtin_fmaf((float)acc[o][4 * q4 + k], s, b), p.act);
+        packed[q4] = TruncPackI8x4(q[0], q[1], q[2], q[3]);
       }
       int8_t* dst = static_cast<int8_t*>(p.out) + row_at;
       // global memory takes dword and short stores at any byte address
@@ -192,7 +190,7 @@ __device__ __forceinline__ void DwItem(const DwConvParams& p, uint32_t plane, in
           } else {
             if (n_out >= 2) *reinterpret_cast<uint16_t*>(dst + 4 * q4) = (uint16_t)packed[q4];
             if (n_out == 1) dst[4 * q4] = (int8_t)packed[q4];
-            if (n_out == 3) dst[4 * q4 + 2] = (int8_t)last[q4];
+            if (n_out == 3) dst[4 * q4 + 2] = (int8_t)(packed[q4] >> 16);
           }
         }
       }

@@ -66,17 +66,19 @@ __device__ __forceinline__ void DispatchAct(int type, F&& f) {
 // max(v, -127), round half away from zero, min(., 127).  The bounds are
 // integers, so clamping first gives the same result; rounding half away from
 // zero is the truncated sum with the largest float below one half (adding one
-// half itself would carry 0.49999997 up to 1).
-__device__ __forceinline__ int QuantizeI8(float v) {
+// half itself would carry 0.49999997 up to 1).  QuantizeF is that sum, the
+// float whose truncation is the int8 value.
+__device__ __forceinline__ float QuantizeF(float v) {
   v = __builtin_amdgcn_fmed3f(v, -127.0f, 127.0f);
-  return static_cast<int>(v + __builtin_copysignf(0x1.fffffep-2f, v));
+  return v + __builtin_copysignf(0x1.fffffep-2f, v);
 }
+__device__ __forceinline__ int QuantizeI8(float v) { return static_cast<int>(QuantizeF(v)); }
 
-// Activation and quantisation of one value.  relu followed by the clamp is
-// one median, and its result has no sign to copy.
+// Activation and quantisation of one value, up to the truncation.  relu
+// followed by the clamp is one median, and its result has no sign to copy.
 template <int ACT>
-__device__ __forceinline__ int ActQuantI8(float v, const DevAct& a) {
-  if (ACT == 1) return static_cast<int>(__builtin_amdgcn_fmed3f(v, 0.0f, 127.0f) + 0x1.fffffep-2f);
+__device__ __forceinline__ float ActQuantF(float v, const DevAct& a) {
+  if (ACT == 1) return __builtin_amdgcn_fmed3f(v, 0.0f, 127.0f) + 0x1.fffffep-2f;
   if (ACT == 2) {
     // relu6 followed by the clamp is one median over the intersected bounds
     // (wave-uniform, computed once), and the sign of its result is the sign
@@ -85,10 +87,51 @@ __device__ __forceinline__ int ActQuantI8(float v, const DevAct& a) {
     const float lo127 = fmaxf(fminf(0.0f, hi), -127.0f);
     const float hi127 = fmaxf(fminf(hi, 127.0f), lo127);
     const float half = hi >= 0.0f ? 0x1.fffffep-2f : -0x1.fffffep-2f;
-    return static_cast<int>(__builtin_amdgcn_fmed3f(v, lo127, hi127) + half);
+    return __builtin_amdgcn_fmed3f(v, lo127, hi127) + half;
   }
-  if (ACT < 0) return QuantizeI8(Activate(v, a));
-  return QuantizeI8(ActivateT<(ACT < 0 ? 0 : ACT)>(v, a));
+  if (ACT < 0) return QuantizeF(Activate(v, a));
+  return QuantizeF(ActivateT<(ACT < 0 ? 0 : ACT)>(v, a));
+}
+template <int ACT>
+__device__ __forceinline__ int ActQuantI8(float v, const DevAct& a) {
+  return static_cast<int>(ActQuantF<ACT>(v, a));
+}
+
+// Truncates eight floats to integers and packs their low bytes into two
+// dwords (a0 in byte 0 of the first).  The conversion writes its byte straight
+// into the destination register (sub-dword destination select), so no separate
+// packing instruction is needed.  An instruction that writes part of a
+// register must not be followed directly by one that reads that register: the
+// two dwords are filled alternately and a wait state closes the sequence.
+__device__ __forceinline__ void TruncPackI8x8(float a0, float a1, float a2, float a3, float b0, float b1, float b2, float b3, uint32_t& a, uint32_t& b) {
+  asm("v_cvt_i32_f32_sdwa %0, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"
+      "v_cvt_i32_f32_sdwa %1, %6 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"
+      "v_cvt_i32_f32_sdwa %0, %3 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+      "v_cvt_i32_f32_sdwa %1, %7 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+      "v_cvt_i32_f32_sdwa %0, %4 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+      "v_cvt_i32_f32_sdwa %1, %8 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+      "v_cvt_i32_f32_sdwa %0, %5 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+      "v_cvt_i32_f32_sdwa %1, %9 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+      "s_nop 0"
+      : "=&v"(a), "=&v"(b)
+      : "v"(a0), "v"(a1), "v"(a2), "v"(a3), "v"(b0), "v"(b1), "v"(b2), "v"(b3));
+}
+
+// The same for four floats and one dword; a wait state separates each
+// conversion from the next one, which reads the register it completes.
+__device__ __forceinline__ uint32_t TruncPackI8x4(float a0, float a1, float a2, float a3) {
+  uint32_t a;
+  asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD\n\t"
+      "s_nop 0\n\t"
+      "v_cvt_i32_f32_sdwa %0, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+      "s_nop 0\n\t"
+      "v_cvt_i32_f32_sdwa %0, %3 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+      "s_nop 0\n\t"
+      "v_cvt_i32_f32_sdwa %0, %4 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD\n\t"
+      "s_nop 0"
+      : "=&v"(a)
+      : "v"(a0), "v"(a1), "v"(a2), "v"(a3));
+  return a;
 }
 
 // Low bytes of four quantized values as one dword (a in byte 0).

@@ -37,9 +37,9 @@ namespace pl {
 namespace {
 
 using epilogue::ActivateT;
-using epilogue::ActQuantI8;
+using epilogue::ActQuantF;
 using epilogue::DispatchAct;
-using epilogue::PackI8x4;
+using epilogue::TruncPackI8x4;
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -83,7 +83,7 @@ template <int OUT, int ACT>
 __device__ __forceinline__ u4 Finish4(int a0, int a1, int a2, int a3, float s, float b, const DevAct& act) {
   if (OUT == kOutAcc32) return u4{(uint32_t)a0, (uint32_t)a1, (uint32_t)a2, (uint32_t)a3};
   const float v0 = __builtin_fmaf((float)a0, s, b), v1 = __builtin_fmaf((float)a1, s, b), v2 = __builtin_fmaf((float)a2, s, b), v3 = __builtin_fmaf((float)a3, s, b);
-  if (OUT == kOutI8) return u4{PackI8x4(ActQuantI8<ACT>(v0, act), ActQuantI8<ACT>(v1, act), ActQuantI8<ACT>(v2, act), ActQuantI8<ACT>(v3, act)), 0u, 0u, 0u};
+  if (OUT == kOutI8) return u4{TruncPackI8x4(ActQuantF<ACT>(v0, act), ActQuantF<ACT>(v1, act), ActQuantF<ACT>(v2, act), ActQuantF<ACT>(v3, act)), 0u, 0u, 0u};
   return u4{__float_as_uint(ActivateT<ACT>(v0, act)), __float_as_uint(ActivateT<ACT>(v1, act)), __float_as_uint(ActivateT<ACT>(v2, act)), __float_as_uint(ActivateT<ACT>(v3, act))};
 }
 

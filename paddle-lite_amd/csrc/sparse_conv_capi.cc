@@ -141,6 +141,7 @@ struct pl_sparse_conv_handle {
   // fp32 row walk over channel chunks (built beside the plain form)
   DevBuf cw_desc, cw_idx, cw_wts;
   int cw_chunks = 0, cw_slices = 0;
+  int cw_groups = 8;  // row groups per wavefront of the fp32 walk over channel chunks: 8, or 4 on request
   int walk_chunked = 1;  // 0 never, 1 when the problem is large enough, 2 whenever the shape allows
   bool walk_plain_fits = true;  // false: more channels than the plain walk's LDS tile holds, only the chunked walk can run
   // half-precision row walk
@@ -289,9 +290,13 @@ int UploadHalfBias(pl_sparse_conv_handle* h, const float* bias) {
 // lies in the chunk, in index order, padded with zero-weight entries that
 // point at the tile's zero row.
 // half: one weight dword per entry, the two rows' binary16 patterns in its halves
+// fp32: the descriptor counts entries (the last batch of a list is walked up
+// to its last real entry) and a wavefront owns h->cw_groups row groups; half:
+// it counts batches and a wavefront owns kChunkWalkGroups.
 int BuildChunkWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h, bool half = false) {
   const int nr = L.semi ? 2 : 1;
-  const int per_slice = pl::kChunkWalkWaves * pl::kChunkWalkGroups;
+  const int groups_per_wave = half ? pl::kChunkWalkGroups : h->cw_groups;
+  const int per_slice = pl::kChunkWalkWaves * groups_per_wave;
   const int n_groups = static_cast<int>(L.groups.size());
   const int slices = CeilDiv(n_groups, per_slice);
   const int chunks = CeilDiv(L.ic, pl::kChunkWalkChunk);
@@ -305,7 +310,7 @@ int BuildChunkWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h, bool ha
         d[0] = static_cast<uint32_t>(idx.size());
         if (g >= n_groups) continue;
         const pl::RowGroup& rg = L.groups[g];
-        uint32_t packed = 0;
+        uint32_t packed = 0, entries = 0;
         int fill = 0;
         auto flush = [&]() {
           for (; fill < 4; ++fill) {  // padding entries: zero row, zero weights
@@ -319,6 +324,7 @@ int BuildChunkWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h, bool ha
         for (uint32_t j = 0; j < rg.count; ++j) {
           const uint32_t k = L.ic_index[rg.first + j];
           if (static_cast<int>(k / pl::kChunkWalkChunk) != c) continue;
+          ++entries;
           packed |= (k % pl::kChunkWalkChunk) << (8 * fill);
           if (half) {
             float w0, w1 = 0.f;
@@ -332,7 +338,7 @@ int BuildChunkWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h, bool ha
           if (++fill == 4) flush();
         }
         if (fill > 0) flush();
-        d[1] = static_cast<uint32_t>(idx.size()) - d[0];
+        d[1] = half ? static_cast<uint32_t>(idx.size()) - d[0] : entries;
       }
     }
   }
@@ -538,6 +544,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_TILE")) h->walk_tile = std::atoi(e);
   if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_THREADS")) h->walk_threads = std::atoi(e);
   if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_SLICES")) h->walk_slices = std::atoi(e);
+  if (const char* e = std::getenv("PL_SPARSE_CONV_CHUNK_WALK_GROUPS")) h->cw_groups = std::atoi(e) == 4 ? 4 : 8;
   h->kind = desc->kind;
   h->oc = desc->oc;
   h->ic = desc->ic;
@@ -749,6 +756,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.n_groups = h->n_groups;
     p.n_chunks = h->cw_chunks;
     p.slices = h->cw_slices;
+    p.groups_per_wave = h->cw_groups;
     p.M = h->oc;
     p.K = h->ic;
     p.hw = im_size;

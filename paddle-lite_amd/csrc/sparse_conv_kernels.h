@@ -67,8 +67,8 @@ hipError_t LaunchRowWalk(const WalkConfig& cfg, const WalkParams& p, hipStream_t
 
 // fp32 row walk over channel chunks (chunk_walk_kernels.hip): a workgroup of
 // kChunkWalkWaves wavefronts takes kChunkWalkTile positions and a slice of
-// kChunkWalkWaves * kChunkWalkGroups row groups, and stages kChunkWalkChunk
-// channels at a time.
+// kChunkWalkWaves * groups_per_wave row groups (4 or 8; the half-precision
+// walk always kChunkWalkGroups), and stages kChunkWalkChunk channels at a time.
 constexpr int kChunkWalkTile = 256;
 constexpr int kChunkWalkChunk = 64;
 constexpr int kChunkWalkWaves = 8;
@@ -78,13 +78,14 @@ struct ChunkWalkParams {
   const void* x;
   void* out;
   const DevGroup* groups;  // row0 / nrows of every row group
-  // [slice][chunk][wave][group of the wave]: first batch, number of batches
+  // [slice][chunk][wave][group of the wave]: first batch, number of entries
   const uint32_t* desc;
   const uint32_t* idx;     // per batch of four entries: four chunk-local channels, 8 bits each (kChunkWalkChunk = zero row)
   const uint32_t* wts;     // per batch: 4 entries x nrows float bit patterns
   const float* bias;       // may be null
   int n_groups;
   int n_chunks, slices;
+  int groups_per_wave;     // 4 or 8, as the descriptors were built
   int M, K;
   int hw;
   uint32_t P;

@@ -221,7 +221,7 @@ __device__ __forceinline__ void StoreRow(const WalkParams& p, int row, uint32_t 
     } else if (OUT == kOutI8) {
       int8_t* dst = static_cast<int8_t*>(p.out) + idx;
       if (PPL == 4) {
-        StreamStore(PackI8x4(QuantizeI8(v[0]), QuantizeI8(v[1]), QuantizeI8(v[2]), QuantizeI8(v[3])), dst);
+        StreamStore(TruncPackI8x4(QuantizeF(v[0]), QuantizeF(v[1]), QuantizeF(v[2]), QuantizeF(v[3])), dst);
       } else {
 #pragma unroll
         for (int j = 0; j < PPL; ++j) dst[j] = static_cast<int8_t>(QuantizeI8(v[j]));
@@ -534,14 +534,19 @@ __device__ __forceinline__ void MfmaEpilogueI8Wide(const MfmaParams& p, const v1
   const int row_base = rb * 32 + 4 * (lane >> 5);
   const int j = lane & 31;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int ro = 8 * (r >> 2) + (r & 3);
-    const float s = rc.s[r], b = rc.b[r];
-    int q[4];
+  for (int r = 0; r < 16; r += 2) {  // two rows at a time: their bytes are packed by the conversions themselves
+    float f[2][4];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) q[c] = ActQuantI8<ACT>(__builtin_fmaf((float)acc[c][r], s, b), p.act);
-    const uint32_t w = PackI8x4(q[0], q[1], q[2], q[3]);
-    stage[(4 * (lane >> 5) + ro) * 32 + j] = w;  // row-local index 0..31, 32 dwords per row
+    for (int h = 0; h < 2; ++h) {
+      const float s = rc.s[r + h], b = rc.b[r + h];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) f[h][c] = ActQuantF<ACT>(__builtin_fmaf((float)acc[c][r + h], s, b), p.act);
+    }
+    uint32_t w0, w1;
+    TruncPackI8x8(f[0][0], f[0][1], f[0][2], f[0][3], f[1][0], f[1][1], f[1][2], f[1][3], w0, w1);
+    const int ro = 8 * (r >> 2) + (r & 3);  // r is even: row r + 1 is ro + 1
+    stage[(4 * (lane >> 5) + ro) * 32 + j] = w0;  // row-local index 0..31, 32 dwords per row
+    stage[(4 * (lane >> 5) + ro + 1) * 32 + j] = w1;
   }
   // the same wavefront reads back: its LDS operations complete in order
   char* obase = static_cast<char*>(p.out) + ((size_t)n * p.M + (size_t)rb * 32) * p.hw + pp;

@@ -155,7 +155,7 @@ def test_fp32_within_tolerance(shape, paired, act):
 # staged at a time); forced here, the library picks it by itself only for
 # large problems.  Needs H*W % 4 == 0.  (batch, ic, oc, h, w): one chunk and
 # several, a channel count off the chunk grid, more row groups than one slice
-# holds (64), an odd row count, a tile that spans images.
+# holds (32 or 64), an odd row count, a tile that spans images.
 CHUNKED_SHAPES = [(2, 64, 64, 4, 4), (1, 96, 48, 8, 6), (3, 130, 67, 4, 5), (1, 300, 150, 16, 16), (5, 70, 33, 2, 2), (2, 257, 20, 12, 12)]
 
 
@@ -170,6 +170,10 @@ def test_fp32_chunked_walk(shape, paired, act, monkeypatch):
     monkeypatch.setenv("PL_SPARSE_CONV_WALK_CHUNKED", "2")
     got = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired)
     assert_same(case, got, want, "fp32 chunked %s %s" % (act, shape))
+    # four row groups per wavefront instead of eight: the same bits
+    monkeypatch.setenv("PL_SPARSE_CONV_CHUNK_WALK_GROUPS", "4")
+    assert np.array_equal(got, run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired))
+    monkeypatch.delenv("PL_SPARSE_CONV_CHUNK_WALK_GROUPS")
     # and the plain walk gives the same bits (same order of fused multiply-adds)
     monkeypatch.setenv("PL_SPARSE_CONV_WALK_CHUNKED", "0")
     plain = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired)
