@@ -153,6 +153,8 @@ struct pl_sparse_conv_handle {
   int64_t blocks_present = 0;
   DevBuf wblocks, kmask;
   int wg_slots = 512;       // workgroups resident at once (2 per CU)
+  int wg_slots_default = 512;  // the same before any override: twice the device's CU count
+  int mfma_stream = 1;      // streaming block MFMA: 0 never, 1 when the shape suits it, 2 whenever the shape allows
   int mfma_i8_wide = 1;
   int mfma_tile_quads = 0;  // 0 = chosen per problem
   int mfma_sub_tiles = 1;   // several tiles per workgroup for <= 64 input channels: 0 never, 1 when enough workgroups remain, 2 always
@@ -534,12 +536,14 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   if (!h) return Fail(PL_ERR_BAD_ARG, "out of host memory");
   h->device = dev;
   h->wg_slots = 2 * std::max(1, prop.multiProcessorCount);
+  h->wg_slots_default = h->wg_slots;
   if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_I8_WIDE")) h->mfma_i8_wide = std::atoi(e) != 0;
   if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_CHUNKED")) h->walk_chunked = std::max(0, std::min(2, std::atoi(e)));
   if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_SUB_TILES")) h->mfma_sub_tiles = std::max(0, std::min(2, std::atoi(e)));
   if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_TILE_QUADS")) h->mfma_tile_quads = std::max(0, std::min(32, std::atoi(e)));
   // tuning switches for experiments; the defaults are what measured best
   if (const char* e = std::getenv("PL_SPARSE_CONV_WG_SLOTS")) h->wg_slots = std::max(1, std::atoi(e));
+  if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_STREAM")) h->mfma_stream = std::max(0, std::min(2, std::atoi(e)));
   if (const char* e = std::getenv("PL_SPARSE_CONV_IMAGE_MIN_ITEMS")) h->image_min_items = std::max(1, std::atoi(e));
   if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_TILE")) h->walk_tile = std::atoi(e);
   if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_THREADS")) h->walk_threads = std::atoi(e);
@@ -736,6 +740,8 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
       c.tile_quads = static_cast<int>(std::min<int64_t>(32, std::max<int64_t>(8, (quads + target_tiles - 1) / target_tiles)));
     }
     c.i8_wide_stores = h->mfma_i8_wide;
+    c.stream = h->mfma_stream;
+    c.cus = std::max(1, h->wg_slots_default / 2);
     c.sub_tiles = h->mfma_sub_tiles;
     if (h->mfma_tile_quads > 0) c.tile_quads = h->mfma_tile_quads;
     e = pl::LaunchBlockMfma(c, p, s);

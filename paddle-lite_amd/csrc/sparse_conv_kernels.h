@@ -175,6 +175,10 @@ struct MfmaParams {
   int sub_tiles;           // tiles per workgroup (1, 2 or 4)
   int row_groups;          // groups of four row blocks
   int i8_stage;            // int8 output is regrouped through LDS for 16-byte stores
+  // streaming variant (tiles cut per image, workgroups walk over tiles)
+  int stream_tpi;          // tiles per image
+  int stream_tiles;        // batch * stream_tpi
+  int stream_lanes;        // workgroups per XCD and row group = tile stride of a workgroup
 };
 
 struct MfmaConfig {
@@ -183,6 +187,8 @@ struct MfmaConfig {
   int tile_quads;      // 1..32 position quads per workgroup tile
   int sub_tiles;       // several tiles per workgroup for at most 64 input channels: 0 never, 1 when enough workgroups remain, 2 always
   int i8_wide_stores;  // int8 output: regroup through LDS into 16-byte stores
+  int stream;          // streaming variant for large maps with 128 / 256 channels: 0 never, 1 when the shape suits it, 2 whenever the shape allows
+  int cus;             // compute units of the device
 };
 
 hipError_t LaunchBlockMfma(const MfmaConfig& cfg, const MfmaParams& p, hipStream_t stream);

@@ -867,6 +867,193 @@ __device__ __forceinline__ void MfmaBody(const MfmaParams& p, uint4* xt) {
   PL_PHASE_MARK(6);
 }
 
+// ------------------------------------------------------ streaming block MFMA
+// Large feature maps with 128 or 256 input channels (K = 32 * KSMAX, H*W a
+// multiple of 16, whole row groups).  The grid is as large as the chip holds
+// at once; a workgroup keeps one row group (its weight blocks stay in
+// registers) and walks over tiles of its XCD's range.  While the epilogue of
+// one tile runs (the vector-ALU bound part for int8 output) the activations
+// of the workgroup's next tile are already on their way into registers:
+//   barrier | loads(next) | epilogue + stores(current) | commit(next) | barrier | multiply(next)
+// Loads, stores and the commit sit in one straight-line block, so the commit
+// waits for exactly the loads (the stores issued after them may still be in
+// flight).  Tiles are cut per image (the last tile of an image may hold fewer
+// quads): every tile then takes the same path, and the lanes behind the last
+// quad repeat it (same loads, same results, same store addresses).
+struct StreamTile {
+  uint32_t n;    // image
+  uint32_t pp0;  // first position of the tile in its image
+  int jv;        // quads of the tile that exist (a multiple of 4, at most 32)
+};
+
+__device__ __forceinline__ StreamTile LocateStreamTile(const MfmaParams& p, int t) {
+  StreamTile s;
+  s.n = (uint32_t)t / (uint32_t)p.stream_tpi;
+  const uint32_t k = (uint32_t)t - s.n * (uint32_t)p.stream_tpi;
+  s.pp0 = 128u * k;
+  s.jv = min(32, p.qpi - 32 * (int)k);
+  return s;
+}
+
+// acc = A (the wavefront's 32 rows) x B (the tile in LDS) over all k-steps.
+template <int KSMAX>
+__device__ __forceinline__ void StreamMultiply(v16i (&acc)[4], const v4i (&a)[KSMAX], const uint4* bbase, uint32_t kmask) {
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[c][i] = 0;
+  if (kmask == (1u << KSMAX) - 1u) {
+    // every block present: no branches, the cells of the next k-step are
+    // read while this one is multiplied
+    uint4 bq[2][4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) bq[0][c] = bbase[c * 32];
+#pragma unroll
+    for (int i = 0; i < KSMAX; ++i) {
+      if (i + 1 < KSMAX) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) bq[(i + 1) & 1][c] = bbase[(size_t)(2 * (i + 1)) * kMfmaTilePos + c * 32];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const uint4 q = bq[i & 1][c];
+        acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], v4i{(int)q.x, (int)q.y, (int)q.z, (int)q.w}, acc[c], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < KSMAX; ++i) {
+    if (kmask & (1u << i)) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const uint4 bq = bbase[(size_t)(2 * i) * kMfmaTilePos + c * 32];
+        acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], v4i{(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w}, acc[c], 0, 0, 0);
+      }
+    }
+  }
+}
+
+// Epilogue of one tile.  rcs: the row group's 128 scales followed by its 128
+// biases in LDS; stage: the wavefront's 4 KB (int8 output only).
+template <int OUT, int ACT>
+__device__ __forceinline__ void StreamEpilogue(const MfmaParams& p, const v16i (&acc)[4], const float* rcs, uint32_t* stage, int wave, int rb, int lane, const StreamTile& s) {
+  const int j = lane & 31, half = lane >> 5;
+  const float* rs = rcs + wave * 32 + 4 * half;
+  if (OUT == kOutI8) {
+#pragma unroll
+    for (int g4 = 0; g4 < 4; ++g4) {
+      const float4 sv = *reinterpret_cast<const float4*>(rs + 8 * g4);
+      const float4 bv = *reinterpret_cast<const float4*>(rs + 128 + 8 * g4);
+      const float sc[4] = {sv.x, sv.y, sv.z, sv.w}, bi[4] = {bv.x, bv.y, bv.z, bv.w};
+#pragma unroll
+      for (int i = 0; i < 4; i += 2) {
+        float f[2][4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int c = 0; c < 4; ++c) f[h][c] = ActQuantF<ACT>(__builtin_fmaf((float)acc[c][4 * g4 + i + h], sc[i + h], bi[i + h]), p.act);
+        uint32_t w0, w1;
+        TruncPackI8x8(f[0][0], f[0][1], f[0][2], f[0][3], f[1][0], f[1][1], f[1][2], f[1][3], w0, w1);
+        const int ro = 4 * half + 8 * g4 + i;  // row of the block; 32 dwords per row
+        stage[ro * 32 + j] = w0;
+        stage[(ro + 1) * 32 + j] = w1;
+      }
+    }
+    // the same wavefront reads back: its LDS operations complete in order
+    char* obase = static_cast<char*>(p.out) + (uint32_t)((s.n * (uint32_t)p.M + (uint32_t)rb * 32u) * (uint32_t)p.hw + s.pp0);
+    const int chunk = min(lane & 7, (s.jv >> 2) - 1);  // 16 positions; chunks behind the tile's end repeat its last one
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 8 * i + (lane >> 3);
+      const uint4 v = *reinterpret_cast<const uint4*>(stage + row * 32 + chunk * 4);
+      StreamStore(make_int4((int)v.x, (int)v.y, (int)v.z, (int)v.w), obase + (uint32_t)row * (uint32_t)p.hw + chunk * 16);
+    }
+  } else {
+    const int jc = min(j, s.jv - 1);
+    char* lane_base = static_cast<char*>(p.out) + (uint32_t)(((s.n * (uint32_t)p.M + (uint32_t)rb * 32u + 4u * half) * (uint32_t)p.hw + s.pp0 + 4u * jc) * 4u);
+#pragma unroll
+    for (int g4 = 0; g4 < 4; ++g4) {
+      const float4 sv = *reinterpret_cast<const float4*>(rs + 8 * g4);
+      const float4 bv = *reinterpret_cast<const float4*>(rs + 128 + 8 * g4);
+      const float sc[4] = {sv.x, sv.y, sv.z, sv.w}, bi[4] = {bv.x, bv.y, bv.z, bv.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) v[c] = ActivateT<ACT>(__builtin_fmaf((float)acc[c][4 * g4 + i], sc[i], bi[i]), p.act);
+        StreamStore(make_float4(v[0], v[1], v[2], v[3]), lane_base + (size_t)(8 * g4 + i) * (size_t)p.hw * 4u);
+      }
+    }
+  }
+}
+
+template <int KSMAX, int OUT, int ACT>
+__device__ __forceinline__ void StreamBody(const MfmaParams& p, uint4* xt) {
+  const int tid = threadIdx.x, lane = tid & 63, j = tid & 31, kg0 = tid >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int group = slot % p.row_groups, tl = slot / p.row_groups;
+  const int lo = (int)(((int64_t)xcd * p.stream_tiles) >> 3), hi = (int)(((int64_t)(xcd + 1) * p.stream_tiles) >> 3);
+  int t = lo + tl;
+  if (t >= hi) return;
+  const int rb = group * 4 + wave;
+  const uint32_t kmask = p.kmask[(size_t)rb * p.kmask_words] & ((1u << KSMAX) - 1u);
+  v4i a[KSMAX];
+#pragma unroll
+  for (int ks = 0; ks < KSMAX; ++ks) a[ks] = static_cast<const v4i*>(p.wblocks)[((size_t)rb * p.ksteps + ks) * 64 + lane];
+  // LDS: activation tile | the row group's scales and biases | int8 staging
+  float* rcs = reinterpret_cast<float*>(xt + (size_t)2 * KSMAX * kMfmaTilePos);
+  uint32_t* stage = reinterpret_cast<uint32_t*>(rcs + 256) + wave * 1024;
+  if (tid < 128) {
+    rcs[tid] = p.scale[group * 128 + tid];
+    rcs[128 + tid] = p.bias[group * 128 + tid];
+  }
+  constexpr int kPasses = KSMAX / 4;
+  uint32_t r[kPasses][16];
+  const QuadInfo none = {0u, 0u, 4};
+  auto issue = [&](const StreamTile& s) {
+    const QuadInfo q = {s.n, s.pp0 + 4u * (uint32_t)min(j, s.jv - 1), 4};
+#pragma unroll
+    for (int u = 0; u < kPasses; ++u) LoadX<true>(r[u], p, q, 8 * u, kg0);
+  };
+  auto commit = [&]() {
+#pragma unroll
+    for (int u = 0; u < kPasses; ++u) CommitX<true>(r[u], xt, p, none, true, true, 8 * u, kg0, j);
+  };
+  const uint4* bbase = xt + (size_t)(lane >> 5) * kMfmaTilePos + (lane & 31);
+  v16i acc[4];
+  StreamTile cur = LocateStreamTile(p, t);
+  issue(cur);
+  commit();
+  __syncthreads();
+  StreamMultiply<KSMAX>(acc, a, bbase, kmask);
+  for (t += p.stream_lanes; t < hi; t += p.stream_lanes) {
+    const StreamTile next = LocateStreamTile(p, t);
+    __syncthreads();  // every wavefront has read the current tile
+    issue(next);
+    __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the epilogue
+    StreamEpilogue<OUT, ACT>(p, acc, rcs, stage, wave, rb, lane, cur);
+    __builtin_amdgcn_sched_barrier(0);
+    commit();
+    __syncthreads();
+    StreamMultiply<KSMAX>(acc, a, bbase, kmask);
+    cur = next;
+  }
+  StreamEpilogue<OUT, ACT>(p, acc, rcs, stage, wave, rb, lane, cur);
+}
+
+template <int KSMAX, int OUT>
+__global__ void __launch_bounds__(256, (KSMAX == 4 ? 3 : 2)) StreamMfmaKernel(const MfmaParams p) {
+  extern __shared__ uint4 xt[];
+  DispatchAct(p.act.type, [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
+    StreamBody<KSMAX, OUT, ACT>(p, xt);
+  });
+}
+
 // At least two workgroups per CU (two wavefronts per SIMD): caps the kernel
 // at 256 VGPRs.
 template <int KSMAX, int OUT>
@@ -934,6 +1121,12 @@ hipError_t MfmaByKs(int ks_max, const MfmaParams& p, dim3 grid, dim3 block, size
       return hipErrorInvalidValue;
   }
 }
+template <int OUT>
+hipError_t StreamByKs(const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
+  if (p.ksteps == 4) return LaunchWithLds(StreamMfmaKernel<4, OUT>, grid, block, lds, s, p);
+  if (p.ksteps == 8) return LaunchWithLds(StreamMfmaKernel<8, OUT>, grid, block, lds, s, p);
+  return hipErrorInvalidValue;
+}
 #endif  // PL_PART_MFMA_ANY
 
 }  // namespace
@@ -943,12 +1136,16 @@ hipError_t MfmaByKs(int ks_max, const MfmaParams& p, dim3 grid, dim3 block, size
 hipError_t LaunchMfmaF32(int ks_max, const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s);
 hipError_t LaunchMfmaI8(int ks_max, const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s);
 hipError_t LaunchMfmaAcc32(int ks_max, const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s);
+hipError_t LaunchStreamF32(const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s);
+hipError_t LaunchStreamI8(const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s);
 
 #if PL_PART_MFMA_F32
 hipError_t LaunchMfmaF32(int ks_max, const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s) { return MfmaByKs<kOutF32>(ks_max, p, grid, block, lds, s); }
+hipError_t LaunchStreamF32(const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s) { return StreamByKs<kOutF32>(p, grid, block, lds, s); }
 #endif
 #if PL_PART_MFMA_I8
 hipError_t LaunchMfmaI8(int ks_max, const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s) { return MfmaByKs<kOutI8>(ks_max, p, grid, block, lds, s); }
+hipError_t LaunchStreamI8(const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s) { return StreamByKs<kOutI8>(p, grid, block, lds, s); }
 #endif
 #if PL_PART_MFMA_ACC32
 hipError_t LaunchMfmaAcc32(int ks_max, const MfmaParams& p, dim3 grid, dim3 block, size_t lds, hipStream_t s) { return MfmaByKs<kOutAcc32>(ks_max, p, grid, block, lds, s); }
@@ -994,6 +1191,25 @@ hipError_t LaunchBlockMfma(const MfmaConfig& cfg, const MfmaParams& p, hipStream
   q.tile_quads = cfg.tile_quads;
   uint32_t tiles = (q.total_quads + cfg.tile_quads - 1) / cfg.tile_quads;
   q.row_groups = (p.row_blocks + 3) / 4;
+  // Streaming variant: large maps with 128 or 256 channels, whole row groups,
+  // 16-byte row pieces, tiles cut per image with at most 5 % of the quads of
+  // the per-image tiling empty, and several tiles for every resident workgroup.
+  if (cfg.stream && (cfg.out_kind == kOutI8 || cfg.out_kind == kOutF32) && (p.ksteps == 4 || p.ksteps == 8) && p.K == 32 * p.ksteps && cfg.ks_max == p.ksteps &&
+      p.hw % 16 == 0 && p.small && p.row_blocks % 4 == 0 && p.M == 32 * p.row_blocks && cfg.tile_quads == 32 && reinterpret_cast<uintptr_t>(p.out) % 16 == 0) {
+    const int tpi = (q.qpi + 31) / 32;
+    const int64_t stream_tiles = (int64_t)(p.P / (uint32_t)p.hw) * tpi;
+    const int per_cu = p.ksteps == 4 ? 3 : 2;  // resident workgroups per CU, by registers
+    int lanes = std::max(1, cfg.cus * per_cu / 8 / q.row_groups);
+    if (stream_tiles < (1ll << 30) && (cfg.stream == 2 || (tpi * 32 * 100 <= q.qpi * 105 && stream_tiles >= (int64_t)8 * lanes * 4))) {
+      lanes = (int)std::min<int64_t>(lanes, (stream_tiles + 7) / 8);
+      q.stream_tpi = tpi;
+      q.stream_tiles = (int)stream_tiles;
+      q.stream_lanes = lanes;
+      size_t slds = (size_t)2 * p.ksteps * kMfmaTilePos * 16 + 1024 + (cfg.out_kind == kOutI8 ? 16384 : 0);
+      dim3 sgrid(8u * (uint32_t)q.row_groups * (uint32_t)lanes), sblock(256);
+      return cfg.out_kind == kOutI8 ? LaunchStreamI8(q, sgrid, sblock, slds, stream) : LaunchStreamF32(q, sgrid, sblock, slds, stream);
+    }
+  }
   // at most 64 input channels: a workgroup takes 4 / ksteps tiles at once
   // (every row group must have 1, 2 or 4 row blocks, and enough workgroups
   // must remain to fill the chip)
