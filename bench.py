@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib", "mobilenet", "density-sweep"])
+    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib", "mobilenet", "density-sweep", "floors"])
     ap.add_argument("--algo", default="auto", choices=["auto", "walk", "mfma", "image"])
     ap.add_argument("--fp16", action="store_true", help="run an fp32 configuration (c1, c2) through the half-precision kernel")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -273,6 +273,73 @@ def run_density_sweep(args):
     return 0
 
 
+def run_floors(args):
+    """What the device needs for the launch and the memory traffic of the
+    metric shape (64 x 512 -> 512 @14x14, int8 -> fp32) without the
+    arithmetic: the probes of paddle-lite_amd/csrc/probe_kernels.hip on the
+    image kernel's grid and rotating buffers, next to the image kernel itself.
+    Not the headline metric: printed as its own JSON line."""
+    import torch
+
+    import helpers
+
+    capi, wl = helpers.capi, helpers.workloads
+    here = os.path.dirname(os.path.abspath(__file__))
+    path = os.path.join(here, "paddle-lite_amd", "lib", "libpl_probe.so")
+    if not os.path.exists(path):
+        sys.stderr.write("the floor probes are not built: run __graft_entry__.build()\n")
+        return 2
+    P = C.CDLL(path)
+    P.pl_probe_floor.restype = C.c_int
+    P.pl_probe_floor.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_float)]
+    case = wl.CONFIGS["c3"]()
+    kernel, weights = helpers.make_kernel(case, algo=capi.ALGO_AUTO)
+    batch, ic, oc, hw = case.batch, case.dense.shape[1], case.dense.shape[0], case.im_size
+    set_bytes = case.x.nbytes + batch * oc * hw * 4
+    n_sets = int(LLC_BYTES * 1.25 // set_bytes) + 1
+    x0 = torch.from_numpy(case.x).cuda()
+    xs = [x0] + [x0.clone() for _ in range(n_sets - 1)]
+    outs = [torch.empty((batch, oc) + tuple(case.x.shape[2:]), dtype=torch.float32, device="cuda") for _ in range(n_sets)]
+    xp = (C.c_void_p * n_sets)(*[t.data_ptr() for t in xs])
+    op = (C.c_void_p * n_sets)(*[t.data_ptr() for t in outs])
+    stream = torch.cuda.current_stream().cuda_stream
+    L = capi.lib()
+    steps = max(200, args.steps)
+
+    def probe(kind, n):
+        ms = C.c_float(0.0)
+        rc = P.pl_probe_floor(kind, xp, op, n_sets, batch, ic, oc, hw, n, C.c_void_p(stream), C.byref(ms))
+        if rc != 0:
+            raise RuntimeError("pl_probe_floor(%d) failed with HIP error %d" % (kind, rc))
+        return ms.value * 1e3 / n
+
+    def image(n):
+        ms = C.c_float(0.0)
+        capi.check(L.pl_sparse_conv_run_sequence(kernel._handle, xp, op, n_sets, batch, hw, n, C.c_void_p(stream), C.byref(ms)))
+        return ms.value * 1e3 / n
+
+    settle(lambda: image(200))
+    names = ["empty", "write", "stream", "load", "load_write", "load_transpose_write"]
+    rows = {}
+    for rep_i in range(3):  # three rounds, the best of each
+        for k, name in enumerate(names):
+            probe(k, 100)
+            us = probe(k, steps)
+            rows[name] = round(min(us, rows.get(name, 1e9)), 2)
+        image(100)
+        rows["image_mfma_kernel"] = round(min(image(steps), rows.get("image_mfma_kernel", 1e9)), 2)
+    nbytes = case.algorithmic_bytes(weights)
+    print(json.dumps({
+        "metric": "launch and memory floors of the metric shape: us per launch",
+        "unit": "us", "n_gpus": 1, "steps": steps, "data": "synthetic",
+        "config": {"workload": "floors_c3_shape", "shape": "N=%d %d->%d @%dx%d" % (batch, ic, oc, case.x.shape[2], case.x.shape[3]), "buffer_sets": n_sets, "grid": "%d workgroups x 512 threads (stream: 2048 x 256)" % (batch * oc // 128),
+                   "input_MB": case.x.nbytes / 1e6, "output_MB": batch * oc * hw * 4 / 1e6},
+        "us_per_launch": rows,
+        "frac_of_8TBs_if_the_kernel_ran_at": {k: round(nbytes / (v * 1e-6) / 1e9 / HBM_PEAK_GBS, 3) for k, v in rows.items() if k != "empty" and k != "load"},
+    }))
+    return 0
+
+
 def run_c5(args):
     """MobileNetV1-1.0 pointwise stack (13 layers, batch 64, int8 -> int8, 90 %
     unstructured zeros, relu) timed as one sequence of 13 launches per step.
@@ -497,6 +564,8 @@ def main():
     torch.cuda.set_device(0)
     if args.config == "density-sweep":
         return run_density_sweep(args)
+    if args.config == "floors":
+        return run_floors(args)
     if args.config == "c5":
         return run_c5(args)
     if args.config == "calib":
