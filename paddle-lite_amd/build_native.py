@@ -32,6 +32,7 @@ SOURCES = [
     ("sparse_conv_capi.cc", "sparse_conv_capi.o", []),
     ("calib_kernels.hip", "calib_kernels.o", []),
     ("chunk_walk_kernels.hip", "chunk_walk_kernels.o", []),
+    ("tile_walk_kernels.hip", "tile_walk_kernels.o", []),
     ("fp16_walk_kernels.hip", "fp16_walk_kernels.o", []),
     ("dwconv_kernels.hip", "dwconv_kernels.o", []),
     ("image_mfma_kernels.hip", "image_mfma_kernels.o", []),

@@ -141,6 +141,10 @@ struct pl_sparse_conv_handle {
   // fp32 row walk over channel chunks (built beside the plain form)
   DevBuf cw_desc, cw_idx, cw_wts;
   int cw_chunks = 0, cw_slices = 0;
+  // fp32 tile walk (whole tile and lists in LDS)
+  DevBuf tw_stream, tw_first, tw_desc;
+  int tw_groups_per_stream = 0;  // 0: not built
+  int walk_tiled = 1;            // 0 never, 1 when the problem suits it, 2 whenever the shape allows
   int cw_groups = 8;  // row groups per wavefront of the fp32 walk over channel chunks: 8, or 4 on request
   int walk_chunked = 1;  // 0 never, 1 when the problem is large enough, 2 whenever the shape allows
   bool walk_plain_fits = true;  // false: more channels than the plain walk's LDS tile holds, only the chunked walk can run
@@ -353,6 +357,79 @@ int BuildChunkWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h, bool ha
   return PL_OK;
 }
 
+// Device-side form for the fp32 tile walk: the row groups are dealt to
+// kTileWalkWaves list streams (longest list first, each to the stream with the
+// least work so far); a stream is the concatenation of its groups' batches of
+// four entries as records of byte offsets and weights.
+int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_handle* h) {
+  h->tw_groups_per_stream = 0;
+  if (pl::TileWalkLdsBytes(L.ic) > static_cast<size_t>(pl::kMaxLdsBytes)) return PL_OK;  // too many channels for one tile: other walks
+  const int nr = L.semi ? 2 : 1;
+  const int streams = pl::kTileWalkWaves;
+  const int n_groups = static_cast<int>(L.groups.size());
+  std::vector<int> order(n_groups);
+  for (int g = 0; g < n_groups; ++g) order[g] = g;
+  std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return L.groups[a].count > L.groups[b].count; });
+  std::vector<std::vector<int>> members(streams);
+  std::vector<int64_t> load(streams, 0);
+  for (int g : order) {
+    int best = 0;
+    for (int s2 = 1; s2 < streams; ++s2)
+      if (load[s2] < load[best]) best = s2;
+    members[best].push_back(g);
+    load[best] += (L.groups[g].count + 3) / 4 + 2;  // batches, plus the group's epilogue
+  }
+  const uint32_t rec_words = 4 + 4 * nr;
+  const uint32_t chunk_words = pl::kTileWalkChunkBytes / 4;
+  const uint32_t recs_per_chunk = chunk_words / rec_words;
+  const uint32_t zero_row = static_cast<uint32_t>(L.ic) * pl::kTileWalkTile * 4;
+  std::vector<uint32_t> stream, first(streams, 0), counts(streams, 0);
+  for (int s2 = 0; s2 < streams; ++s2) {
+    first[s2] = static_cast<uint32_t>(stream.size() / chunk_words);
+    counts[s2] = static_cast<uint32_t>(members[s2].size());
+    uint32_t recs = 0;
+    auto pad_chunk = [&]() {
+      while (stream.size() % chunk_words != 0) stream.push_back(0u);
+    };
+    auto put = [&](const uint32_t* rec) {
+      if (recs == recs_per_chunk) {  // records do not straddle chunks
+        pad_chunk();
+        recs = 0;
+      }
+      stream.insert(stream.end(), rec, rec + rec_words);
+      ++recs;
+    };
+    for (int g : members[s2]) {
+      const pl::RowGroup& rg = L.groups[g];
+      uint32_t rec[12] = {0};
+      rec[0] = static_cast<uint32_t>(rg.row0) | (static_cast<uint32_t>(rg.nrows) << 24);
+      rec[1] = rg.count;
+      if (bias) {
+        std::memcpy(&rec[2], &bias[rg.row0], 4);
+        if (rg.nrows == 2) std::memcpy(&rec[3], &bias[rg.row0 + 1], 4);
+      }
+      put(rec);
+      for (uint32_t e0 = 0; e0 < rg.count; e0 += 4) {
+        for (uint32_t e = 0; e < 4; ++e) {
+          const bool real = e0 + e < rg.count;
+          rec[e] = real ? L.ic_index[rg.first + e0 + e] * pl::kTileWalkTile * 4 : zero_row;
+          rec[4 + e * nr] = real ? L.w0[rg.first + e0 + e] : 0u;
+          if (nr == 2) rec[4 + e * nr + 1] = real ? L.w1[rg.first + e0 + e] : 0u;
+        }
+        put(rec);
+      }
+    }
+    pad_chunk();
+    stream.insert(stream.end(), chunk_words, 0u);  // the spare chunk the prefetch may touch
+  }
+  hipError_t e = h->tw_stream.Upload(stream.data(), stream.size() * sizeof(uint32_t));
+  if (e == hipSuccess) e = h->tw_first.Upload(first.data(), first.size() * sizeof(uint32_t));
+  if (e == hipSuccess) e = h->tw_desc.Upload(counts.data(), counts.size() * sizeof(uint32_t));
+  if (e != hipSuccess) return FailHip(e, "uploading the tile-walk list streams");
+  h->tw_groups_per_stream = 1;
+  return PL_OK;
+}
+
 // Device-side form for the block MFMA path: the weight matrix as dense
 // 32x32 int8 blocks in matrix-core operand order, plus the mask of blocks
 // that hold a nonzero.
@@ -538,6 +615,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   h->wg_slots = 2 * std::max(1, prop.multiProcessorCount);
   h->wg_slots_default = h->wg_slots;
   if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_I8_WIDE")) h->mfma_i8_wide = std::atoi(e) != 0;
+  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_TILED")) h->walk_tiled = std::max(0, std::min(2, std::atoi(e)));
   if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_CHUNKED")) h->walk_chunked = std::max(0, std::min(2, std::atoi(e)));
   if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_SUB_TILES")) h->mfma_sub_tiles = std::max(0, std::min(2, std::atoi(e)));
   if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_TILE_QUADS")) h->mfma_tile_quads = std::max(0, std::min(32, std::atoi(e)));
@@ -603,6 +681,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   if (rc == PL_OK && algo == PL_ALGO_BLOCK_MFMA) rc = BuildBlockMfma(L, h);
   if (rc == PL_OK && (algo == PL_ALGO_IMAGE_MFMA || (h->auto_int8 && pl::ImageMfmaFits(desc->oc, desc->ic, 16)))) rc = BuildImageMfma(L, h);
   if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8) rc = BuildChunkWalk(L, h);
+  if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8 && !half) rc = BuildTileWalk(L, desc->bias, h);
   if (rc == PL_OK) {
     // the MFMA epilogues always read a bias; give them zeros when the op has none
     std::vector<float> zeros;
@@ -745,6 +824,23 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     c.sub_tiles = h->mfma_sub_tiles;
     if (h->mfma_tile_quads > 0) c.tile_quads = h->mfma_tile_quads;
     e = pl::LaunchBlockMfma(c, p, s);
+  } else if (!h->int8 && !h->half && vec && h->tw_groups_per_stream > 0 && h->walk_tiled > 0 &&
+             (h->walk_tiled == 2 || 2 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kTileWalkTile)) >= h->wg_slots_default / 2)) {
+    // fp32 with enough 128-position tiles for at least half of the CUs: the
+    // walk with the tile and the lists in LDS
+    pl::TileWalkParams p{};
+    p.x = static_cast<const float*>(x_dev);
+    p.out = static_cast<float*>(out_dev);
+    p.stream = h->tw_stream.ptr;
+    p.stream_first = static_cast<const uint32_t*>(h->tw_first.ptr);
+    p.stream_groups = static_cast<const uint32_t*>(h->tw_desc.ptr);
+    p.n_groups = h->n_groups;
+    p.M = h->oc;
+    p.K = h->ic;
+    p.hw = im_size;
+    p.P = P;
+    p.act = h->act;
+    e = pl::LaunchTileWalk(h->semi ? 2 : 1, p, s);
   } else if (!h->int8 && !h->walk_plain_fits && !vec) {
     return Fail(PL_ERR_UNSUPPORTED, "fp32 with ic = %d runs as a walk over channel chunks, which needs H*W %% 4 == 0 and 16-byte aligned tensors (H*W = %d)", h->ic, im_size);
   } else if (!h->int8 && vec && h->cw_chunks > 0 &&

@@ -96,6 +96,40 @@ struct ChunkWalkParams {
 // Needs hw % 4 == 0 and 16-byte aligned x / out.
 hipError_t LaunchChunkWalk(int nrows, const ChunkWalkParams& p, hipStream_t stream);
 
+// fp32 walk with the whole tile and the index lists in LDS
+// (tile_walk_kernels.hip): a workgroup of kTileWalkWaves wavefronts takes
+// kTileWalkTile positions with all input channels; wavefront s walks the row
+// groups of list stream s.
+constexpr int kTileWalkTile = 128;
+constexpr int kTileWalkWaves = 16;
+constexpr int kTileWalkChunkBytes = 1536;  // piece of a list stream held in LDS per wavefront
+
+struct TileWalkParams {
+  const float* x;
+  float* out;
+  // List streams, kTileWalkChunkBytes at a time, as records of 16 + 16 * nrows
+  // bytes.  A row group is a header record (first row | rows << 24, entries,
+  // bias bit patterns of its rows) followed by one record per batch of four
+  // entries: four byte offsets of channel rows in the tile (channel *
+  // kTileWalkTile * 4; unused slots of the last batch point at the zero row
+  // behind the last channel), then 4 x nrows float bit patterns (entry-major).
+  // Records do not straddle chunks; every stream ends with one spare chunk.
+  const void* stream;
+  const uint32_t* stream_first;   // [kTileWalkWaves] first chunk of every stream
+  const uint32_t* stream_groups;  // [kTileWalkWaves] row groups in every stream
+  int n_groups;
+  int M, K;
+  int hw;
+  uint32_t P;
+  DevAct act;
+  int tiles;                     // filled in by the launcher
+};
+
+// LDS the kernel needs for K input channels.
+size_t TileWalkLdsBytes(int K);
+// Needs hw % 4 == 0 and 16-byte aligned x / out.
+hipError_t LaunchTileWalk(int nrows, const TileWalkParams& p, hipStream_t stream);
+
 // Half-precision row walk (fp16_walk_kernels.hip).  Activation constants as
 // binary16 bit patterns.
 struct DevActH {

@@ -1,0 +1,211 @@
+// fp32 walk with the whole tile and the index lists in LDS.
+//
+// The other fp32 walks read index lists and weights through the scalar data
+// cache, whose fill rate bounds them (a list set of 70 - 100 KB per tile
+// streams through a 16 KB cache; the scalar path delivers about one byte per
+// clock and CU).  Here a workgroup of sixteen wavefronts keeps all input
+// channels of 128 positions in LDS, and every wavefront streams the lists of
+// its row groups through a private 1.5 KB LDS buffer: the next piece of the
+// stream is fetched into registers with ordinary vector loads (24 bytes per
+// lane) while the current one is walked, and list records are read from LDS
+// with the same address in every lane.  Per entry: one 8-byte LDS read of
+// the activations (two positions per lane), the entry's share of three
+// 16-byte record reads, one address add and four fused multiply-adds.  A row
+// group's header (rows, list length, bias) travels in the stream too, so the
+// walk issues no scalar memory load.
+// Outputs of a row group are stored as soon as its list ends, so the stores
+// spread over the whole walk.  The order of the fused multiply-adds of one
+// output is the index order and the accumulator starts at the bias, as in the
+// other walks (same bits).
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <type_traits>
+
+#include "epilogue.h"
+#include "launch_lds.h"
+#include "sparse_conv_kernels.h"
+
+namespace pl {
+namespace {
+
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef const __attribute__((address_space(4))) uint32_t* ConstWords;
+typedef const __attribute__((address_space(4))) float* ConstFloats;
+
+using epilogue::ActivateT;
+using epilogue::DispatchAct;
+
+constexpr int kTP = kTileWalkTile;      // positions per workgroup
+constexpr int kWaves = kTileWalkWaves;  // wavefronts per workgroup = list streams
+constexpr int kChunkBytes = kTileWalkChunkBytes;
+
+// Workgroup id -> tile: each XCD (linear id mod 8) owns a contiguous range of tiles.
+__device__ __forceinline__ int XcdTile(int tiles) {
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int first = (xcd * tiles) >> 3, last = ((xcd + 1) * tiles) >> 3;
+  const int t = first + slot;
+  return t < last ? t : -1;
+}
+
+template <int NR, int ACT>
+__device__ __forceinline__ void TileWalkBody(const TileWalkParams& p, float* tile) {
+  constexpr int kRecBytes = NR == 2 ? 48 : 32;  // four byte offsets, then 4 * NR weights
+  constexpr int kRecs = kChunkBytes / kRecBytes;
+  const int tile_id = XcdTile(p.tiles);
+  if (tile_id < 0) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t tile0 = (uint32_t)tile_id * (uint32_t)kTP;
+  char* tile_bytes = reinterpret_cast<char*>(tile);
+  char* lbuf = tile_bytes + (size_t)(p.K + 1) * kTP * 4 + wave * kChunkBytes;
+
+  // the wavefront's list stream: chunks of kChunkBytes, lane i holds bytes
+  // [16 i, 16 i + 16) and [1024 + 8 i, 1024 + 8 i + 8) of a chunk
+  const char* sp = reinterpret_cast<const char*>(p.stream) + (size_t)((ConstWords)p.stream_first)[wave] * kChunkBytes;
+  u4 pa = *reinterpret_cast<const u4*>(sp + 16 * lane);
+  u2 pb = *reinterpret_cast<const u2*>(sp + 1024 + 8 * lane);
+
+  // staging: 32 threads per channel row (four positions each), 32 rows per pass
+  {
+    const int c4 = tid & 31, r0 = tid >> 5;
+    const uint32_t gpos = tile0 + 4u * (uint32_t)c4;
+    const bool live = gpos < p.P;
+    const uint32_t n = live ? gpos / (uint32_t)p.hw : 0u;
+    const uint32_t pp = live ? gpos % (uint32_t)p.hw : 0u;
+    const float* xcol = p.x + (size_t)n * p.K * p.hw + pp;
+    for (int k0 = 0; k0 < p.K; k0 += 128) {
+      uint4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int k = min(k0 + r0 + 32 * u, p.K - 1);
+        v[u] = *reinterpret_cast<const uint4*>(xcol + (size_t)k * p.hw);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int k = k0 + r0 + 32 * u;
+        if (k < p.K) *reinterpret_cast<uint4*>(tile_bytes + ((size_t)k * kTP + 4 * c4) * 4) = live ? v[u] : make_uint4(0, 0, 0, 0);
+      }
+    }
+    // row K is all zero: the target of list padding entries
+    if (tid < kTP / 4) *reinterpret_cast<uint4*>(tile_bytes + ((size_t)p.K * kTP + 4 * tid) * 4) = make_uint4(0, 0, 0, 0);
+  }
+  __syncthreads();
+
+  const uint32_t lane8 = 8u * (uint32_t)lane;
+  const uint32_t gpos = tile0 + 2u * (uint32_t)lane;
+  const bool store_on = gpos < p.P;
+  const uint32_t on = store_on ? gpos / (uint32_t)p.hw : 0u, opp = store_on ? gpos % (uint32_t)p.hw : 0u;
+  float* obase = p.out + (size_t)on * p.M * p.hw + opp;
+
+  int rec = kRecs;  // records of the current chunk already walked: the first chunk is still in registers
+  int chunk = 0;
+  // next record of the stream; at the end of a chunk the prefetched one becomes
+  // the current one (only this wavefront reads the buffer, and its LDS
+  // operations execute in order) and the one after it is requested
+  auto next = [&]() -> const char* {
+    if (rec == kRecs) {
+      *reinterpret_cast<u4*>(lbuf + 16 * lane) = pa;
+      *reinterpret_cast<u2*>(lbuf + 1024 + 8 * lane) = pb;
+      ++chunk;
+      const char* np = sp + (size_t)chunk * kChunkBytes;  // the stream ends with one spare chunk
+      pa = *reinterpret_cast<const u4*>(np + 16 * lane);
+      pb = *reinterpret_cast<const u2*>(np + 1024 + 8 * lane);
+      rec = 0;
+    }
+    return lbuf + (rec++) * kRecBytes;
+  };
+  const int n_groups = (int)((ConstWords)p.stream_groups)[wave];
+  for (int j = 0; j < n_groups; ++j) {
+    // header record of the row group: first row | rows << 24, entries, bias bits of its rows
+    const u4 hdr = *reinterpret_cast<const u4*>(next());
+    const int row0 = __builtin_amdgcn_readfirstlane((int)(hdr.x & 0xffffffu)), nrows = __builtin_amdgcn_readfirstlane((int)(hdr.x >> 24));
+    const uint32_t entries = (uint32_t)__builtin_amdgcn_readfirstlane((int)hdr.y);
+    float acc[NR][2];
+    acc[0][0] = acc[0][1] = __uint_as_float(hdr.z);
+    if (NR == 2) acc[NR - 1][0] = acc[NR - 1][1] = __uint_as_float(hdr.w);
+    auto entry = [&](uint32_t off, float w0, float w1) {
+      const v2f x = *reinterpret_cast<const v2f*>(tile_bytes + (off + lane8));
+      acc[0][0] = __builtin_fmaf(x[0], w0, acc[0][0]);
+      acc[0][1] = __builtin_fmaf(x[1], w0, acc[0][1]);
+      if (NR == 2) {
+        acc[NR - 1][0] = __builtin_fmaf(x[0], w1, acc[NR - 1][0]);
+        acc[NR - 1][1] = __builtin_fmaf(x[1], w1, acc[NR - 1][1]);
+      }
+    };
+    auto weights = [&](const char* r, float (&w)[4 * NR]) {
+      const u4 wa = *reinterpret_cast<const u4*>(r + 16);
+      w[0] = __uint_as_float(wa.x), w[1] = __uint_as_float(wa.y), w[2] = __uint_as_float(wa.z), w[3] = __uint_as_float(wa.w);
+      if (NR == 2) {
+        const u4 wb = *reinterpret_cast<const u4*>(r + (NR == 2 ? 32 : 16));
+        w[4 * NR - 4] = __uint_as_float(wb.x), w[4 * NR - 3] = __uint_as_float(wb.y), w[4 * NR - 2] = __uint_as_float(wb.z), w[4 * NR - 1] = __uint_as_float(wb.w);
+      }
+    };
+    const uint32_t batches = entries >> 2, rem = entries & 3u;
+    for (uint32_t b = 0; b < batches; ++b) {
+      const char* r = next();
+      const u4 off = *reinterpret_cast<const u4*>(r);
+      float w[4 * NR];
+      weights(r, w);
+      v2f x[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[e] = *reinterpret_cast<const v2f*>(tile_bytes + (off[e] + lane8));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        acc[0][0] = __builtin_fmaf(x[e][0], w[e * NR], acc[0][0]);
+        acc[0][1] = __builtin_fmaf(x[e][1], w[e * NR], acc[0][1]);
+        if (NR == 2) {
+          acc[NR - 1][0] = __builtin_fmaf(x[e][0], w[e * NR + NR - 1], acc[NR - 1][0]);
+          acc[NR - 1][1] = __builtin_fmaf(x[e][1], w[e * NR + NR - 1], acc[NR - 1][1]);
+        }
+      }
+    }
+    if (rem != 0) {  // the last, partly filled batch: only its real entries
+      const char* r = next();
+      const u4 off = *reinterpret_cast<const u4*>(r);
+      float w[4 * NR];
+      weights(r, w);
+      entry(off[0], w[0], w[NR - 1]);
+      if (rem > 1) entry(off[1], w[NR], w[NR + NR - 1]);
+      if (rem > 2) entry(off[2], w[2 * NR], w[2 * NR + NR - 1]);
+    }
+    if (store_on) {
+#pragma unroll
+      for (int rr = 0; rr < NR; ++rr) {
+        if (rr < nrows) {
+          const v2f o = {ActivateT<ACT>(acc[rr][0], p.act), ActivateT<ACT>(acc[rr][1], p.act)};
+          __builtin_nontemporal_store(o, reinterpret_cast<v2f*>(obase + (size_t)(row0 + rr) * p.hw));
+        }
+      }
+    }
+  }
+}
+
+template <int NR>
+__global__ void __launch_bounds__(64 * kTileWalkWaves) TileWalkKernel(const TileWalkParams p) {
+  extern __shared__ float tile_lds[];
+  DispatchAct(p.act.type, [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
+    TileWalkBody<NR, ACT>(p, tile_lds);
+  });
+}
+
+}  // namespace
+
+size_t TileWalkLdsBytes(int K) { return (size_t)(K + 1) * kTP * 4 + (size_t)kWaves * kChunkBytes; }
+
+hipError_t LaunchTileWalk(int nrows, const TileWalkParams& p, hipStream_t stream) {
+  if (p.P == 0 || p.n_groups == 0) return hipSuccess;
+  if (p.hw % 4 != 0) return hipErrorInvalidValue;
+  const size_t lds = TileWalkLdsBytes(p.K);
+  if (lds > (size_t)kMaxLdsBytes) return hipErrorInvalidValue;
+  TileWalkParams q = p;
+  q.tiles = (int)((p.P + kTP - 1) / kTP);
+  dim3 grid(8u * (((uint32_t)q.tiles + 7) / 8)), block(64 * kWaves);
+  if (nrows == 2) return LaunchWithLds(TileWalkKernel<2>, grid, block, lds, stream, q);
+  return LaunchWithLds(TileWalkKernel<1>, grid, block, lds, stream, q);
+}
+
+}  // namespace pl

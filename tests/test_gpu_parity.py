@@ -180,6 +180,34 @@ def test_fp32_chunked_walk(shape, paired, act, monkeypatch):
     assert np.array_equal(got, plain)
 
 
+# fp32 walk with the whole tile and the index lists in LDS (128 positions and
+# sixteen list streams per workgroup); forced here, the library picks it by
+# itself for large problems.  Needs H*W % 4 == 0 and at most 264 channels.
+# (batch, ic, oc, h, w): fewer row groups than streams, more, an odd row
+# count, a tile that spans images, a last tile that is not full, the largest
+# channel count, lists longer than one LDS piece.
+TILED_SHAPES = [(2, 64, 8, 4, 4), (1, 96, 48, 8, 6), (3, 130, 67, 4, 5), (1, 264, 150, 16, 16), (5, 70, 33, 2, 2), (2, 257, 20, 12, 12), (3, 256, 96, 10, 10)]
+
+
+@pytest.mark.parametrize("act", ["none", "relu6", "hswish"])
+@pytest.mark.parametrize("shape", TILED_SHAPES, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
+def test_fp32_tiled_walk(shape, paired, act, monkeypatch):
+    announce("fp32 tiled", shape, paired, act)
+    batch, ic, oc, h, w = shape
+    sparsity = 0.3 if ic == 256 else 0.75  # the dense case: lists of ~180 entries, several LDS pieces per stream
+    case = small_case(capi.KIND_FP32, batch, ic, oc, h, w, sparsity, paired, ACTS[act], seed=ic + 3 * oc)
+    want = run_oracle(case, oracle_pack(case, force_semi=paired))
+    monkeypatch.setenv("PL_SPARSE_CONV_WALK_TILED", "2")
+    got = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired)
+    assert_same(case, got, want, "fp32 tiled %s %s" % (act, shape))
+    # and the plain walk gives the same bits (same order of fused multiply-adds)
+    monkeypatch.setenv("PL_SPARSE_CONV_WALK_TILED", "0")
+    monkeypatch.setenv("PL_SPARSE_CONV_WALK_CHUNKED", "0")
+    plain = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired)
+    assert np.array_equal(got, plain)
+
+
 def test_no_bias_and_single_scale():
     announce("nobias")
     for kind in (capi.KIND_FP32, capi.KIND_INT8_FP32, capi.KIND_INT8_INT8):
