@@ -173,7 +173,12 @@ __device__ __forceinline__ void Tail(const uint4* __restrict__ xt, int kgs, int 
   });
 }
 
-template <int KS, int OUT>
+// QPI: quads per image when known at compile time (49 = 14 x 14 maps), else 0.
+// With the constant, the LDS offsets of the regrouping and of the operand
+// reads become immediates (64 x 512 -> 512 @14x14: 10.8 -> 10.4 us); the image
+// size in bytes stays a run-time value on purpose (as a constant it changed the
+// schedule of the direct loads and the stores and cost more than it saved).
+template <int KS, int OUT, int QPI>
 __global__ void __launch_bounds__(512) ImageMfmaKernel(const ImageMfmaParams p) {
   extern __shared__ uint4 lds_raw[];
   // shifted windows read up to three cells in front of a row of cells
@@ -184,7 +189,7 @@ __global__ void __launch_bounds__(512) ImageMfmaKernel(const ImageMfmaParams p) 
   if (item >= p.items) return;
   const int n = item / p.row_groups, rg = item - n * p.row_groups;
   const int rho = wave & 3, half = wave >> 2;
-  const int qpi = p.qpi, kgs = p.kgs, hw = p.hw;
+  const int qpi = QPI ? QPI : p.qpi, kgs = QPI ? (4 * QPI + 15) / 16 * 16 : p.kgs, hw = p.hw;
   constexpr int NKG = 4 * KS, BPW = NKG / 8;
   static_assert(NKG % 8 == 0, "channel groups are dealt evenly to the eight wavefronts");
 
@@ -241,11 +246,28 @@ __global__ void __launch_bounds__(512) ImageMfmaKernel(const ImageMfmaParams p) 
     __builtin_amdgcn_s_waitcnt(0xc07f);
     __builtin_amdgcn_sched_barrier(0);
     if (lane < qpi) {
+      // Two stages of byte permutes.  The second stage is done cell by cell so
+      // that the four dwords of a cell (one per block of four channels) are
+      // produced next to each other, where the 16-byte store wants them.
+      uint32_t lo[4][2], hi[4][2];
 #pragma unroll
-      for (int b4 = 0; b4 < 4; ++b4) Transpose4x4(r[4 * b4], r[4 * b4 + 1], r[4 * b4 + 2], r[4 * b4 + 3]);
+      for (int b4 = 0; b4 < 4; ++b4) {
+        lo[b4][0] = __builtin_amdgcn_perm(r[4 * b4 + 1], r[4 * b4], 0x05010400u);      // positions 0, 1 of channels 4 b4, 4 b4 + 1
+        hi[b4][0] = __builtin_amdgcn_perm(r[4 * b4 + 1], r[4 * b4], 0x07030602u);      // positions 2, 3
+        lo[b4][1] = __builtin_amdgcn_perm(r[4 * b4 + 3], r[4 * b4 + 2], 0x05010400u);  // the same of channels 4 b4 + 2, 4 b4 + 3
+        hi[b4][1] = __builtin_amdgcn_perm(r[4 * b4 + 3], r[4 * b4 + 2], 0x07030602u);
+      }
       uint4* cells = reinterpret_cast<uint4*>(blk) + lane;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) cells[c * qpi] = make_uint4(r[c], r[4 + c], r[8 + c], r[12 + c]);
+      for (int c = 0; c < 4; ++c) {
+        const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+        uint4 cell;
+        cell.x = __builtin_amdgcn_perm((c & 2) ? hi[0][1] : lo[0][1], (c & 2) ? hi[0][0] : lo[0][0], sel);
+        cell.y = __builtin_amdgcn_perm((c & 2) ? hi[1][1] : lo[1][1], (c & 2) ? hi[1][0] : lo[1][0], sel);
+        cell.z = __builtin_amdgcn_perm((c & 2) ? hi[2][1] : lo[2][1], (c & 2) ? hi[2][0] : lo[2][0], sel);
+        cell.w = __builtin_amdgcn_perm((c & 2) ? hi[3][1] : lo[3][1], (c & 2) ? hi[3][0] : lo[3][0], sel);
+        cells[c * qpi] = cell;
+      }
     }
   }
   __syncthreads();
@@ -276,13 +298,25 @@ __global__ void __launch_bounds__(512) ImageMfmaKernel(const ImageMfmaParams p) 
 template <int OUT>
 hipError_t ByKs(const ImageMfmaParams& q, dim3 grid, size_t lds, hipStream_t s) {
   const dim3 block(512);
+  if (q.qpi == 49) {
+    switch (q.K / 64) {
+      case 2:
+        return LaunchWithLds(ImageMfmaKernel<2, OUT, 49>, grid, block, lds, s, q);
+      case 4:
+        return LaunchWithLds(ImageMfmaKernel<4, OUT, 49>, grid, block, lds, s, q);
+      case 8:
+        return LaunchWithLds(ImageMfmaKernel<8, OUT, 49>, grid, block, lds, s, q);
+      default:
+        return hipErrorInvalidValue;
+    }
+  }
   switch (q.K / 64) {
     case 2:
-      return LaunchWithLds(ImageMfmaKernel<2, OUT>, grid, block, lds, s, q);
+      return LaunchWithLds(ImageMfmaKernel<2, OUT, 0>, grid, block, lds, s, q);
     case 4:
-      return LaunchWithLds(ImageMfmaKernel<4, OUT>, grid, block, lds, s, q);
+      return LaunchWithLds(ImageMfmaKernel<4, OUT, 0>, grid, block, lds, s, q);
     case 8:
-      return LaunchWithLds(ImageMfmaKernel<8, OUT>, grid, block, lds, s, q);
+      return LaunchWithLds(ImageMfmaKernel<8, OUT, 0>, grid, block, lds, s, q);
     default:
       return hipErrorInvalidValue;
   }

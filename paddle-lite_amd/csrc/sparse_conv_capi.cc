@@ -825,9 +825,11 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     if (h->mfma_tile_quads > 0) c.tile_quads = h->mfma_tile_quads;
     e = pl::LaunchBlockMfma(c, p, s);
   } else if (!h->int8 && !h->half && vec && h->tw_groups_per_stream > 0 && h->walk_tiled > 0 &&
-             (h->walk_tiled == 2 || 2 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kTileWalkTile)) >= h->wg_slots_default / 2)) {
-    // fp32 with enough 128-position tiles for at least half of the CUs: the
-    // walk with the tile and the lists in LDS
+             (h->walk_tiled == 2 || 32 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kTileWalkTile)) >= 5 * h->wg_slots_default)) {
+    // fp32 with 128-position tiles for at least 5/16 of the CUs (a tile takes
+    // about 24 us whatever their number; measured crossover against the other
+    // walks between 49 and 98 tiles on 256 CUs): the walk with the tile and
+    // the lists in LDS
     pl::TileWalkParams p{};
     p.x = static_cast<const float*>(x_dev);
     p.out = static_cast<float*>(out_dev);
