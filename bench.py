@@ -24,7 +24,7 @@ LLC_BYTES = 256 << 20  # last-level (Infinity) cache the rotation must exceed
 COPY_CALIBRATION_BYTES = 64 << 20
 
 
-# c3 is the metric of BASELINE.json; the other configurations are reported under their own names
+# c3 is the headline metric; the other configurations are reported under their own names
 METRICS = {
     "c1": "sparse 1x1 conv nnz-GOP/s + % HBM roofline (fp32 unstructured, N=1, 96->192@56x56, 80%)",
     "c2": "sparse 1x1 conv nnz-GOP/s + % HBM roofline (fp32 semi-structured, N=32, 256->512@28x28, 90%)",

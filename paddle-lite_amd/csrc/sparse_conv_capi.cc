@@ -143,7 +143,7 @@ struct pl_sparse_conv_handle {
   int cw_chunks = 0, cw_slices = 0;
   // fp32 tile walk (whole tile and lists in LDS)
   DevBuf tw_stream, tw_first, tw_desc;
-  int tw_groups_per_stream = 0;  // 0: not built
+  int tw_built = 0;  // list streams of the tile walk uploaded
   int walk_tiled = 1;            // 0 never, 1 when the problem suits it, 2 whenever the shape allows
   int cw_groups = 8;  // row groups per wavefront of the fp32 walk over channel chunks: 8, or 4 on request
   int walk_chunked = 1;  // 0 never, 1 when the problem is large enough, 2 whenever the shape allows
@@ -362,7 +362,7 @@ int BuildChunkWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h, bool ha
 // least work so far); a stream is the concatenation of its groups' batches of
 // four entries as records of byte offsets and weights.
 int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_handle* h) {
-  h->tw_groups_per_stream = 0;
+  h->tw_built = 0;
   if (pl::TileWalkLdsBytes(L.ic) > static_cast<size_t>(pl::kMaxLdsBytes)) return PL_OK;  // too many channels for one tile: other walks
   const int nr = L.semi ? 2 : 1;
   const int streams = pl::kTileWalkWaves;
@@ -426,7 +426,7 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
   if (e == hipSuccess) e = h->tw_first.Upload(first.data(), first.size() * sizeof(uint32_t));
   if (e == hipSuccess) e = h->tw_desc.Upload(counts.data(), counts.size() * sizeof(uint32_t));
   if (e != hipSuccess) return FailHip(e, "uploading the tile-walk list streams");
-  h->tw_groups_per_stream = 1;
+  h->tw_built = 1;
   return PL_OK;
 }
 
@@ -824,7 +824,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     c.sub_tiles = h->mfma_sub_tiles;
     if (h->mfma_tile_quads > 0) c.tile_quads = h->mfma_tile_quads;
     e = pl::LaunchBlockMfma(c, p, s);
-  } else if (!h->int8 && !h->half && vec && h->tw_groups_per_stream > 0 && h->walk_tiled > 0 &&
+  } else if (!h->int8 && !h->half && vec && h->tw_built != 0 && h->walk_tiled > 0 &&
              (h->walk_tiled == 2 || 32 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kTileWalkTile)) >= 5 * h->wg_slots_default)) {
     // fp32 with 128-position tiles for at least 5/16 of the CUs (a tile takes
     // about 24 us whatever their number; measured crossover against the other
