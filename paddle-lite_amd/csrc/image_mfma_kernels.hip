@@ -207,6 +207,12 @@ __global__ void __launch_bounds__(512) ImageMfmaKernel(const ImageMfmaParams p) 
     if (lane < p.dma_rem_lanes)
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + p.dma_full * 1024), (__attribute__((address_space(3))) void*)(dst + p.dma_full * 1024), 16, 0, 0);
   }
+  // Every channel group of this wavefront has landed.  (The builtin, not an assembly statement: the
+  // compiler then knows that no direct load is in flight any more and puts no wait of its own in front
+  // of the LDS accesses below.)
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+  // The weights, scales and biases are requested now and arrive while the activations are regrouped:
+  // LDS operations wait for direct loads that may still be in flight, not for ordinary ones.
   // weights of the wavefront's two row tiles, all channels
   v4i a[2][KS];
   const v4i* wt = static_cast<const v4i*>(p.wtiles) + ((size_t)(rg * 4 + rho) * 2 * KS) * 64 + lane;
@@ -229,9 +235,6 @@ __global__ void __launch_bounds__(512) ImageMfmaKernel(const ImageMfmaParams p) 
     rw.sct[j] = OUT == kOutAcc32 ? 0.f : p.scale[row0 + 4 * (16 * j + ln.n)];
     rw.bit[j] = OUT == kOutAcc32 ? 0.f : p.bias[row0 + 4 * (16 * j + ln.n)];
   }
-  // Every channel group of this wavefront has landed.  (Waiting group by group, with the weights
-  // behind the activations, measured the same: 10.90 against 10.87 us on 64 x 512 -> 512 @14x14.)
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   // in place: 16 dwords (16 channels x 4 positions) per quad -> 4 cells
 #pragma unroll
   for (int u = 0; u < BPW; ++u) {
