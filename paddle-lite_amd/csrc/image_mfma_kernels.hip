@@ -235,32 +235,36 @@ __global__ void __launch_bounds__(512) ImageMfmaKernel(const ImageMfmaParams p) 
     rw.sct[j] = OUT == kOutAcc32 ? 0.f : p.scale[row0 + 4 * (16 * j + ln.n)];
     rw.bit[j] = OUT == kOutAcc32 ? 0.f : p.bias[row0 + 4 * (16 * j + ln.n)];
   }
-  // in place: 16 dwords (16 channels x 4 positions) per quad -> 4 cells
+  // in place: 16 dwords (16 channels x 4 positions) per quad -> 4 cells.  The dwords of all of the
+  // wavefront's channel groups are read first (one wait instead of one per group), then every group is
+  // transposed and written back; a group is touched by this wavefront only.
+  uint32_t r[BPW][16];
+  if (lane < qpi) {
 #pragma unroll
-  for (int u = 0; u < BPW; ++u) {
-    const int kg = wave * BPW + u;
-    uint32_t* blk = reinterpret_cast<uint32_t*>(lbase + kg * (kgs * 16));
-    uint32_t r[16];
-    if (lane < qpi) {
+    for (int u = 0; u < BPW; ++u) {
+      const uint32_t* blk = reinterpret_cast<const uint32_t*>(lbase + (wave * BPW + u) * (kgs * 16));
 #pragma unroll
-      for (int i = 0; i < 16; ++i) r[i] = blk[i * qpi + lane];
+      for (int i = 0; i < 16; ++i) r[u][i] = blk[i * qpi + lane];
     }
-    // every lane has read before any lane overwrites
-    __builtin_amdgcn_s_waitcnt(0xc07f);
-    __builtin_amdgcn_sched_barrier(0);
-    if (lane < qpi) {
+  }
+  // every lane has read before any lane overwrites
+  __builtin_amdgcn_s_waitcnt(0xc07f);
+  __builtin_amdgcn_sched_barrier(0);
+  if (lane < qpi) {
+#pragma unroll
+    for (int u = 0; u < BPW; ++u) {
       // Two stages of byte permutes.  The second stage is done cell by cell so
       // that the four dwords of a cell (one per block of four channels) are
       // produced next to each other, where the 16-byte store wants them.
       uint32_t lo[4][2], hi[4][2];
 #pragma unroll
       for (int b4 = 0; b4 < 4; ++b4) {
-        lo[b4][0] = __builtin_amdgcn_perm(r[4 * b4 + 1], r[4 * b4], 0x05010400u);      // positions 0, 1 of channels 4 b4, 4 b4 + 1
-        hi[b4][0] = __builtin_amdgcn_perm(r[4 * b4 + 1], r[4 * b4], 0x07030602u);      // positions 2, 3
-        lo[b4][1] = __builtin_amdgcn_perm(r[4 * b4 + 3], r[4 * b4 + 2], 0x05010400u);  // the same of channels 4 b4 + 2, 4 b4 + 3
-        hi[b4][1] = __builtin_amdgcn_perm(r[4 * b4 + 3], r[4 * b4 + 2], 0x07030602u);
+        lo[b4][0] = __builtin_amdgcn_perm(r[u][4 * b4 + 1], r[u][4 * b4], 0x05010400u);      // positions 0, 1 of channels 4 b4, 4 b4 + 1
+        hi[b4][0] = __builtin_amdgcn_perm(r[u][4 * b4 + 1], r[u][4 * b4], 0x07030602u);      // positions 2, 3
+        lo[b4][1] = __builtin_amdgcn_perm(r[u][4 * b4 + 3], r[u][4 * b4 + 2], 0x05010400u);  // the same of channels 4 b4 + 2, 4 b4 + 3
+        hi[b4][1] = __builtin_amdgcn_perm(r[u][4 * b4 + 3], r[u][4 * b4 + 2], 0x07030602u);
       }
-      uint4* cells = reinterpret_cast<uint4*>(blk) + lane;
+      uint4* cells = reinterpret_cast<uint4*>(lbase + (wave * BPW + u) * (kgs * 16)) + lane;
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
