@@ -144,6 +144,8 @@ struct pl_sparse_conv_handle {
   // fp32 tile walk (whole tile and lists in LDS)
   DevBuf tw_stream, tw_first, tw_desc;
   int tw_built = 0;  // list streams of the tile walk uploaded
+  int64_t tw_stream_work = 0;  // work units (entry batches + 2 per row group) of the fullest of the sixteen unsplit streams
+  int walk_split = -1;          // sixteenths of the row groups' work dealt to the CUs without a tile: -1 by rule, 0 never, 1 .. 8 forced
   int walk_tiled = 1;            // 0 never, 1 when the problem suits it, 2 whenever the shape allows
   int cw_groups = 8;  // row groups per wavefront of the fp32 walk over channel chunks: 8, or 4 on request
   int walk_chunked = 1;  // 0 never, 1 when the problem is large enough, 2 whenever the shape allows
@@ -361,6 +363,9 @@ int BuildChunkWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h, bool ha
 // kTileWalkWaves list streams (longest list first, each to the stream with the
 // least work so far); a stream is the concatenation of its groups' batches of
 // four entries as records of byte offsets and weights.
+// Main / spare divisions of the tile walk's row groups that are prepared: spare shares of 1/16 .. 8/16.
+constexpr int kTileWalkSplits = 8;
+
 int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_handle* h) {
   h->tw_built = 0;
   if (pl::TileWalkLdsBytes(L.ic) > static_cast<size_t>(pl::kMaxLdsBytes)) return PL_OK;  // too many channels for one tile: other walks
@@ -370,57 +375,83 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
   std::vector<int> order(n_groups);
   for (int g = 0; g < n_groups; ++g) order[g] = g;
   std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return L.groups[a].count > L.groups[b].count; });
-  std::vector<std::vector<int>> members(streams);
-  std::vector<int64_t> load(streams, 0);
-  for (int g : order) {
-    int best = 0;
-    for (int s2 = 1; s2 < streams; ++s2)
-      if (load[s2] < load[best]) best = s2;
-    members[best].push_back(g);
-    load[best] += (L.groups[g].count + 3) / 4 + 2;  // batches, plus the group's epilogue
-  }
+  auto work = [&](int g) { return static_cast<int64_t>((L.groups[g].count + 3) / 4 + 2); };  // batches, plus the group's epilogue
   const uint32_t rec_words = 4 + 4 * nr;
   const uint32_t chunk_words = pl::kTileWalkChunkBytes / 4;
   const uint32_t recs_per_chunk = chunk_words / rec_words;
   const uint32_t zero_row = static_cast<uint32_t>(L.ic) * pl::kTileWalkTile * 4;
-  std::vector<uint32_t> stream, first(streams, 0), counts(streams, 0);
-  for (int s2 = 0; s2 < streams; ++s2) {
-    first[s2] = static_cast<uint32_t>(stream.size() / chunk_words);
-    counts[s2] = static_cast<uint32_t>(members[s2].size());
-    uint32_t recs = 0;
-    auto pad_chunk = [&]() {
-      while (stream.size() % chunk_words != 0) stream.push_back(0u);
-    };
-    auto put = [&](const uint32_t* rec) {
-      if (recs == recs_per_chunk) {  // records do not straddle chunks
-        pad_chunk();
-        recs = 0;
-      }
-      stream.insert(stream.end(), rec, rec + rec_words);
-      ++recs;
-    };
-    for (int g : members[s2]) {
-      const pl::RowGroup& rg = L.groups[g];
-      uint32_t rec[12] = {0};
-      rec[0] = static_cast<uint32_t>(rg.row0) | (static_cast<uint32_t>(rg.nrows) << 24);
-      rec[1] = rg.count;
-      if (bias) {
-        std::memcpy(&rec[2], &bias[rg.row0], 4);
-        if (rg.nrows == 2) std::memcpy(&rec[3], &bias[rg.row0 + 1], 4);
-      }
-      put(rec);
-      for (uint32_t e0 = 0; e0 < rg.count; e0 += 4) {
-        for (uint32_t e = 0; e < 4; ++e) {
-          const bool real = e0 + e < rg.count;
-          rec[e] = real ? L.ic_index[rg.first + e0 + e] * pl::kTileWalkTile * 4 : zero_row;
-          rec[4 + e * nr] = real ? L.w0[rg.first + e0 + e] : 0u;
-          if (nr == 2) rec[4 + e * nr + 1] = real ? L.w1[rg.first + e0 + e] : 0u;
+  std::vector<uint32_t> stream, first, counts;
+  // Sixteen streams for the given row groups (largest first): each group goes to the stream with the least work so far.
+  // Returns the work of the fullest stream.
+  auto emit = [&](const std::vector<int>& part) {
+    std::vector<std::vector<int>> members(streams);
+    std::vector<int64_t> load(streams, 0);
+    for (int g : part) {
+      int best = 0;
+      for (int s2 = 1; s2 < streams; ++s2)
+        if (load[s2] < load[best]) best = s2;
+      members[best].push_back(g);
+      load[best] += work(g);
+    }
+    for (int s2 = 0; s2 < streams; ++s2) {
+      first.push_back(static_cast<uint32_t>(stream.size() / chunk_words));
+      counts.push_back(static_cast<uint32_t>(members[s2].size()));
+      uint32_t recs = 0;
+      auto pad_chunk = [&]() {
+        while (stream.size() % chunk_words != 0) stream.push_back(0u);
+      };
+      auto put = [&](const uint32_t* rec) {
+        if (recs == recs_per_chunk) {  // records do not straddle chunks
+          pad_chunk();
+          recs = 0;
+        }
+        stream.insert(stream.end(), rec, rec + rec_words);
+        ++recs;
+      };
+      for (int g : members[s2]) {
+        const pl::RowGroup& rg = L.groups[g];
+        uint32_t rec[12] = {0};
+        rec[0] = static_cast<uint32_t>(rg.row0) | (static_cast<uint32_t>(rg.nrows) << 24);
+        rec[1] = rg.count;
+        if (bias) {
+          std::memcpy(&rec[2], &bias[rg.row0], 4);
+          if (rg.nrows == 2) std::memcpy(&rec[3], &bias[rg.row0 + 1], 4);
         }
         put(rec);
+        for (uint32_t e0 = 0; e0 < rg.count; e0 += 4) {
+          for (uint32_t e = 0; e < 4; ++e) {
+            const bool real = e0 + e < rg.count;
+            rec[e] = real ? L.ic_index[rg.first + e0 + e] * pl::kTileWalkTile * 4 : zero_row;
+            rec[4 + e * nr] = real ? L.w0[rg.first + e0 + e] : 0u;
+            if (nr == 2) rec[4 + e * nr + 1] = real ? L.w1[rg.first + e0 + e] : 0u;
+          }
+          put(rec);
+        }
+      }
+      pad_chunk();
+      stream.insert(stream.end(), chunk_words, 0u);  // the spare chunk the prefetch may touch
+    }
+    return *std::max_element(load.begin(), load.end());
+  };
+  // Set 0: all row groups in one part.  Sets 1 .. kTileWalkSplits: a spare part with about s / 16 of the work
+  // (a mix of sizes: going through the groups from the largest, a group joins the spare part whenever that
+  // keeps the part at or below its share), the rest in the main part.
+  h->tw_stream_work = emit(order);
+  for (int s16 = 1; s16 <= kTileWalkSplits; ++s16) {
+    std::vector<int> main_part, spare_part;
+    int64_t all_w = 0, spare_w = 0;
+    for (int g : order) {
+      const int64_t w = work(g);
+      all_w += w;
+      if ((spare_w + w) * 16 <= static_cast<int64_t>(s16) * all_w) {
+        spare_part.push_back(g);
+        spare_w += w;
+      } else {
+        main_part.push_back(g);
       }
     }
-    pad_chunk();
-    stream.insert(stream.end(), chunk_words, 0u);  // the spare chunk the prefetch may touch
+    emit(main_part);
+    emit(spare_part);
   }
   hipError_t e = h->tw_stream.Upload(stream.data(), stream.size() * sizeof(uint32_t));
   if (e == hipSuccess) e = h->tw_first.Upload(first.data(), first.size() * sizeof(uint32_t));
@@ -616,6 +647,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   h->wg_slots_default = h->wg_slots;
   if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_I8_WIDE")) h->mfma_i8_wide = std::atoi(e) != 0;
   if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_TILED")) h->walk_tiled = std::max(0, std::min(2, std::atoi(e)));
+  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_SPLIT")) h->walk_split = std::max(-1, std::min(kTileWalkSplits, std::atoi(e)));
   if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_CHUNKED")) h->walk_chunked = std::max(0, std::min(2, std::atoi(e)));
   if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_SUB_TILES")) h->mfma_sub_tiles = std::max(0, std::min(2, std::atoi(e)));
   if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_TILE_QUADS")) h->mfma_tile_quads = std::max(0, std::min(32, std::atoi(e)));
@@ -825,17 +857,42 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     if (h->mfma_tile_quads > 0) c.tile_quads = h->mfma_tile_quads;
     e = pl::LaunchBlockMfma(c, p, s);
   } else if (!h->int8 && !h->half && vec && h->tw_built != 0 && h->walk_tiled > 0 &&
-             (h->walk_tiled == 2 || 32 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kTileWalkTile)) >= 5 * h->wg_slots_default)) {
-    // fp32 with 128-position tiles for at least 5/16 of the CUs (a tile takes
-    // about 24 us whatever their number; measured crossover against the other
-    // walks between 49 and 98 tiles on 256 CUs): the walk with the tile and
-    // the lists in LDS
+             (h->walk_tiled == 2 || 64 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kTileWalkTile)) >= 5 * h->wg_slots_default)) {
+    // fp32 with 128-position tiles for at least 5/32 of the CUs (with the row
+    // groups of a tile shared between two CUs a launch takes about 14.5 us up
+    // to half as many tiles as CUs; measured crossover against the other walks
+    // between 24 and 49 tiles on 256 CUs): the walk with the tile and the
+    // lists in LDS
     pl::TileWalkParams p{};
     p.x = static_cast<const float*>(x_dev);
     p.out = static_cast<float*>(out_dev);
     p.stream = h->tw_stream.ptr;
-    p.stream_first = static_cast<const uint32_t*>(h->tw_first.ptr);
-    p.stream_groups = static_cast<const uint32_t*>(h->tw_desc.ptr);
+    // With fewer tiles than CUs, the CUs without a tile take a share of the row groups of several tiles each
+    // (one after the other, each staged anew).  The share that evens out the two kinds of workgroup: a main
+    // workgroup spends S + (1 - f) W, a spare one r (S + f W) for its r tiles, with S the staging time of a tile
+    // and W the walk of all row groups, so f = (1 - (r - 1) S / W) / (r + 1).  S and W in cycles, fitted to
+    // measurements (a tile of 256 channels costs a spare workgroup about 5.6 K cycles besides its walk; 355
+    // cycles per work unit of the fullest stream).  Rounded down: a share above the balance point costs r
+    // times what one below it costs.
+    const int tiles = CeilDiv(static_cast<int>(P), pl::kTileWalkTile);
+    const int cus = std::max(8, h->wg_slots_default / 2) / 8 * 8;
+    int s16 = 0;
+    if (tiles < cus && h->walk_split != 0) {
+      const int per_xcd = CeilDiv(tiles, 8), spare = cus / 8 - per_xcd;
+      if (spare >= 1) {
+        const int r = CeilDiv(per_xcd, spare);
+        const double sw = (2000.0 + 14.0 * h->ic) / (355.0 * static_cast<double>(std::max<int64_t>(1, h->tw_stream_work)));
+        const double f = (1.0 - (r - 1) * sw) / (r + 1);
+        s16 = h->walk_split > 0 ? h->walk_split : static_cast<int>(f * 16.0 + 0.3);
+        s16 = std::max(0, std::min(kTileWalkSplits, s16));
+      }
+    }
+    // stream tables: set 0 has one part, sets 1 .. 8 two
+    const size_t table = s16 == 0 ? 0 : static_cast<size_t>(pl::kTileWalkWaves) * (2 * s16 - 1);
+    p.stream_first = static_cast<const uint32_t*>(h->tw_first.ptr) + table;
+    p.stream_groups = static_cast<const uint32_t*>(h->tw_desc.ptr) + table;
+    p.split = s16 != 0;
+    p.split_slots = cus / 8;
     p.n_groups = h->n_groups;
     p.M = h->oc;
     p.K = h->ic;

@@ -115,14 +115,18 @@ struct TileWalkParams {
   // behind the last channel), then 4 x nrows float bit patterns (entry-major).
   // Records do not straddle chunks; every stream ends with one spare chunk.
   const void* stream;
-  const uint32_t* stream_first;   // [kTileWalkWaves] first chunk of every stream
-  const uint32_t* stream_groups;  // [kTileWalkWaves] row groups in every stream
+  const uint32_t* stream_first;   // [kTileWalkWaves] first chunk of every stream; with `split`, [2 * kTileWalkWaves]: main part, spare part
+  const uint32_t* stream_groups;  // row groups in every stream, same shape
   int n_groups;
   int M, K;
   int hw;
   uint32_t P;
   DevAct act;
   int tiles;                     // filled in by the launcher
+  // 1: the row groups are dealt into a main and a spare part; the grid then has
+  // split_slots workgroups per XCD (one per CU), more than any XCD has tiles.
+  int split;
+  int split_slots;
 };
 
 // LDS the kernel needs for K input channels.

@@ -17,6 +17,10 @@
 // spread over the whole walk.  The order of the fused multiply-adds of one
 // output is the index order and the accumulator starts at the bias, as in the
 // other walks (same bits).
+// With fewer tiles than CUs, the row groups can be dealt into a main and a
+// spare part (two sets of sixteen streams): the tile's own workgroup walks the
+// main part, and the workgroups on the CUs that have no tile of their own walk
+// the spare parts of several tiles, one tile after the other.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -42,29 +46,21 @@ constexpr int kTP = kTileWalkTile;      // positions per workgroup
 constexpr int kWaves = kTileWalkWaves;  // wavefronts per workgroup = list streams
 constexpr int kChunkBytes = kTileWalkChunkBytes;
 
-// Workgroup id -> tile: each XCD (linear id mod 8) owns a contiguous range of tiles.
-__device__ __forceinline__ int XcdTile(int tiles) {
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int first = (xcd * tiles) >> 3, last = ((xcd + 1) * tiles) >> 3;
-  const int t = first + slot;
-  return t < last ? t : -1;
-}
-
+// One tile: stage it, then walk the streams of one part (0 main, 1 spare).
 template <int NR, int ACT>
-__device__ __forceinline__ void TileWalkBody(const TileWalkParams& p, float* tile) {
+__device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile, int tile_id, int part) {
   constexpr int kRecBytes = NR == 2 ? 48 : 32;  // four byte offsets, then 4 * NR weights
   constexpr int kRecs = kChunkBytes / kRecBytes;
-  const int tile_id = XcdTile(p.tiles);
-  if (tile_id < 0) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int sidx = part * kWaves + wave;
   const uint32_t tile0 = (uint32_t)tile_id * (uint32_t)kTP;
   char* tile_bytes = reinterpret_cast<char*>(tile);
   char* lbuf = tile_bytes + (size_t)(p.K + 1) * kTP * 4 + wave * kChunkBytes;
 
   // the wavefront's list stream: chunks of kChunkBytes, lane i holds bytes
   // [16 i, 16 i + 16) and [1024 + 8 i, 1024 + 8 i + 8) of a chunk
-  const char* sp = reinterpret_cast<const char*>(p.stream) + (size_t)((ConstWords)p.stream_first)[wave] * kChunkBytes;
+  const char* sp = reinterpret_cast<const char*>(p.stream) + (size_t)((ConstWords)p.stream_first)[sidx] * kChunkBytes;
   u4 pa = *reinterpret_cast<const u4*>(sp + 16 * lane);
   u2 pb = *reinterpret_cast<const u2*>(sp + 1024 + 8 * lane);
 
@@ -117,7 +113,7 @@ __device__ __forceinline__ void TileWalkBody(const TileWalkParams& p, float* til
     }
     return lbuf + (rec++) * kRecBytes;
   };
-  const int n_groups = (int)((ConstWords)p.stream_groups)[wave];
+  const int n_groups = (int)((ConstWords)p.stream_groups)[sidx];
   for (int j = 0; j < n_groups; ++j) {
     // header record of the row group: first row | rows << 24, entries, bias bits of its rows
     const u4 hdr = *reinterpret_cast<const u4*>(next());
@@ -183,6 +179,26 @@ __device__ __forceinline__ void TileWalkBody(const TileWalkParams& p, float* til
   }
 }
 
+// Workgroup id -> tiles: each XCD (linear id mod 8) owns a contiguous range of
+// tiles.  Its first workgroups take one tile each (main part); with a spare
+// part, the workgroups behind them share the range's tiles among themselves.
+template <int NR, int ACT>
+__device__ __forceinline__ void TileWalkBody(const TileWalkParams& p, float* tile) {
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int first = (xcd * p.tiles) >> 3, last = ((xcd + 1) * p.tiles) >> 3;
+  const int count = last - first;
+  if (slot < count) {
+    WalkOneTile<NR, ACT>(p, tile, first + slot, 0);
+    return;
+  }
+  if (p.split == 0) return;
+  const int n_spare = (int)(gridDim.x >> 3) - count;
+  for (int t = first + (slot - count); t < last; t += n_spare) {
+    WalkOneTile<NR, ACT>(p, tile, t, 1);
+    __syncthreads();  // every wavefront has left the tile before the next one is staged
+  }
+}
+
 template <int NR>
 __global__ void __launch_bounds__(64 * kTileWalkWaves) TileWalkKernel(const TileWalkParams p) {
   extern __shared__ float tile_lds[];
@@ -203,7 +219,12 @@ hipError_t LaunchTileWalk(int nrows, const TileWalkParams& p, hipStream_t stream
   if (lds > (size_t)kMaxLdsBytes) return hipErrorInvalidValue;
   TileWalkParams q = p;
   q.tiles = (int)((p.P + kTP - 1) / kTP);
-  dim3 grid(8u * (((uint32_t)q.tiles + 7) / 8)), block(64 * kWaves);
+  uint32_t slots = ((uint32_t)q.tiles + 7) / 8;  // workgroups per XCD
+  if (q.split != 0) {
+    if (q.split_slots < (int)slots + 1) return hipErrorInvalidValue;  // every XCD needs a spare workgroup
+    slots = (uint32_t)q.split_slots;
+  }
+  dim3 grid(8u * slots), block(64 * kWaves);
   if (nrows == 2) return LaunchWithLds(TileWalkKernel<2>, grid, block, lds, stream, q);
   return LaunchWithLds(TileWalkKernel<1>, grid, block, lds, stream, q);
 }

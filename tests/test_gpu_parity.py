@@ -201,6 +201,13 @@ def test_fp32_tiled_walk(shape, paired, act, monkeypatch):
     monkeypatch.setenv("PL_SPARSE_CONV_WALK_TILED", "2")
     got = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired)
     assert_same(case, got, want, "fp32 tiled %s %s" % (act, shape))
+    # the row groups dealt differently between the tile's own workgroup and the
+    # workgroups of the CUs without a tile (none, 3/16, half of the work; the
+    # run above took the share the library computes): the same bits
+    for split in ("0", "3", "8"):
+        monkeypatch.setenv("PL_SPARSE_CONV_WALK_SPLIT", split)
+        assert np.array_equal(got, run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired)), "split %s" % split
+    monkeypatch.delenv("PL_SPARSE_CONV_WALK_SPLIT")
     # and the plain walk gives the same bits (same order of fused multiply-adds)
     monkeypatch.setenv("PL_SPARSE_CONV_WALK_TILED", "0")
     monkeypatch.setenv("PL_SPARSE_CONV_WALK_CHUNKED", "0")
