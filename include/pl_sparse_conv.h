@@ -75,7 +75,9 @@ enum {
  *   PL_ALGO_IMAGE_MFMA int8 only, oc a multiple of 128, ic = 128 / 256 / 512,
  *                     H*W a multiple of 4 in [16, 256]: one workgroup per
  *                     (image, 128 output rows) keeps the whole image in LDS
- *                     and multiplies it with dense 16x64 weight tiles
+ *                     and multiplies it with dense 16x64 weight tiles; also
+ *                     7 x 7 maps with ic = 256 / 512 / 1024 (two images per
+ *                     workgroup)
  * With PL_ALGO_AUTO an int8 handle may hold more than one form and choose per
  * call by batch and H*W: see pl_sparse_conv_algo_for(). */
 enum { PL_ALGO_AUTO = 0, PL_ALGO_ROW_WALK = 1, PL_ALGO_BLOCK_MFMA = 2, PL_ALGO_IMAGE_MFMA = 3 };

@@ -44,6 +44,9 @@ using epilogue::TruncPackI8x4;
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+// the same with the alignment of its elements only: rows of 49 outputs start anywhere
+typedef uint32_t u4a __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t u1a __attribute__((aligned(1)));
 
 // 4 dwords holding 4 channels x 4 positions -> 4 positions x 4 channels.
 __device__ __forceinline__ void Transpose4x4(uint32_t& r0, uint32_t& r1, uint32_t& r2, uint32_t& r3) {
@@ -302,6 +305,185 @@ __global__ void __launch_bounds__(512) ImageMfmaKernel(const ImageMfmaParams p) 
   }
 }
 
+// ---------------------------------------------------------------------------
+// 7 x 7 maps.  A channel row is 49 bytes, so rows are not dword aligned and an
+// image is small: a workgroup takes two images (98 positions) and 128 output
+// rows.  A unit is one channel group of one image (16 x 49 = 784 bytes,
+// contiguous in NCHW, a multiple of 16): it is moved into LDS by 49 lanes of
+// one direct load, into a slot of 1 KB, and regrouped in place there into 13
+// quads x 4 cells (the last quad holds position 48 and three bytes that are
+// never used).  Lanes regroup four units at a time (13 quads each); a
+// channel's dword of a quad is put together from the two aligned dwords it
+// straddles (v_alignbyte_b32, shift = channel mod 4).
+// The 26 quads of the two images form two windows of 16 quad columns, one per
+// wavefront of a pair; a lane's column is (image, quad) = (g / 13, g % 13).
+constexpr int kSmallHw = 49, kSmallQuads = 13, kSmallSlotCells = 64;
+
+template <int KS, int OUT>
+__global__ void __launch_bounds__(512) SmallMapMfmaKernel(const ImageMfmaParams p) {
+  extern __shared__ uint4 lds_raw[];
+  uint4* xt = lds_raw + 16;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int item = (int)(blockIdx.x & 7u) * p.per_xcd + (int)(blockIdx.x >> 3);
+  if (item >= p.items) return;
+  const int pair = item / p.row_groups, rg = item - pair * p.row_groups;
+  const int n0 = 2 * pair;
+  const int n_img = min(2, p.batch - n0);  // the last pair of an odd batch holds one image
+  const int rho = wave & 3, half = wave >> 2;
+  constexpr int NKG = 4 * KS, UNITS = 2 * NKG, UPW = UNITS / 8;
+  static_assert(UPW % 4 == 0, "units are regrouped four at a time");
+  constexpr int kSlotBytes = kSmallSlotCells * 16;
+
+  // activations: one direct load per unit, 49 lanes x 16 bytes
+  char* lbase = reinterpret_cast<char*>(xt);
+#pragma unroll
+  for (int t = 0; t < UPW; ++t) {
+    const int u = wave * UPW + t;
+    const int m = u / NKG, kg = u % NKG;
+    const int img = n0 + min(m, n_img - 1);  // a missing second image repeats the first; its results are not stored
+    const int8_t* src = p.x + ((size_t)img * p.K + 16 * kg) * kSmallHw + lane * 16;
+    if (lane < kSmallHw) __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src, (__attribute__((address_space(3))) void*)(lbase + u * kSlotBytes), 16, 0, 0);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the builtin, so that the compiler knows no direct load is in flight
+  // weights of the wavefront's two row tiles (all channels), scales and biases: they arrive during the regrouping
+  v4i a[2][KS];
+  const v4i* wt = static_cast<const v4i*>(p.wtiles) + ((size_t)(rg * 4 + rho) * 2 * KS) * 64 + lane;
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) a[j][ks] = wt[(j * KS + ks) * 64];
+  Lane ln;
+  ln.n = lane & 15;
+  ln.kq = lane >> 4;
+  const int row0 = rg * 128 + rho;  // the wavefront's rows: row0 + 4 m, m = 0 .. 31
+  Rows rw;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      rw.sc[j][i] = OUT == kOutAcc32 ? 0.f : p.scale[row0 + 4 * (16 * j + 4 * ln.kq + i)];
+      rw.bi[j][i] = OUT == kOutAcc32 ? 0.f : p.bias[row0 + 4 * (16 * j + 4 * ln.kq + i)];
+    }
+    rw.sct[j] = rw.bit[j] = 0.f;
+  }
+
+  // regrouping in place, four units per pass: lane = 13 * (unit of the pass) + quad
+  {
+    const int uj = (lane * 20) >> 8;  // lane / 13 for lane < 64
+    const int q = lane - kSmallQuads * uj;
+#pragma unroll
+    for (int pass = 0; pass < UPW / 4; ++pass) {
+      char* slot = lbase + (wave * UPW + 4 * pass + uj) * kSlotBytes;
+      const uint32_t* words = reinterpret_cast<const uint32_t*>(slot) + q;
+      uint32_t r[16];
+      if (lane < 4 * kSmallQuads) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          // bytes 49 i + 4 q .. + 3 of the unit: dword (49 i >> 2) + q, shifted by i mod 4 bytes
+          const uint32_t d0 = words[(kSmallHw * i) >> 2];
+          if ((i & 3) == 0) {
+            r[i] = d0;
+          } else {
+            const uint32_t d1 = words[((kSmallHw * i) >> 2) + 1];
+            r[i] = __builtin_amdgcn_alignbyte(d1, d0, i & 3);
+          }
+        }
+      }
+      // every lane has read before any lane overwrites
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+      __builtin_amdgcn_sched_barrier(0);
+      if (lane < 4 * kSmallQuads) {
+        uint32_t lo[4][2], hi[4][2];
+#pragma unroll
+        for (int b4 = 0; b4 < 4; ++b4) {
+          lo[b4][0] = __builtin_amdgcn_perm(r[4 * b4 + 1], r[4 * b4], 0x05010400u);
+          hi[b4][0] = __builtin_amdgcn_perm(r[4 * b4 + 1], r[4 * b4], 0x07030602u);
+          lo[b4][1] = __builtin_amdgcn_perm(r[4 * b4 + 3], r[4 * b4 + 2], 0x05010400u);
+          hi[b4][1] = __builtin_amdgcn_perm(r[4 * b4 + 3], r[4 * b4 + 2], 0x07030602u);
+        }
+        uint4* cells = reinterpret_cast<uint4*>(slot) + q;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+          uint4 cell;
+          cell.x = __builtin_amdgcn_perm((c & 2) ? hi[0][1] : lo[0][1], (c & 2) ? hi[0][0] : lo[0][0], sel);
+          cell.y = __builtin_amdgcn_perm((c & 2) ? hi[1][1] : lo[1][1], (c & 2) ? hi[1][0] : lo[1][0], sel);
+          cell.z = __builtin_amdgcn_perm((c & 2) ? hi[2][1] : lo[2][1], (c & 2) ? hi[2][0] : lo[2][0], sel);
+          cell.w = __builtin_amdgcn_perm((c & 2) ? hi[3][1] : lo[3][1], (c & 2) ? hi[3][0] : lo[3][0], sel);
+          cells[c * kSmallQuads] = cell;
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // the wavefront's window: quad columns 16 half .. 16 half + 15 of the 26
+  const int g = 16 * half + ln.n;
+  const bool live = g < 2 * kSmallQuads;
+  const int gc = live ? g : 2 * kSmallQuads - 1;
+  const int m = gc >= kSmallQuads ? 1 : 0, ql = gc - kSmallQuads * m;
+  const uint4* bbase = xt + (m * NKG + ln.kq) * kSmallSlotCells + ql;  // + ks * 4 * kSmallSlotCells + c * kSmallQuads
+  v4i acc[2][4];
+#pragma unroll
+  for (int o = 0; o < 2; ++o)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[o][c] = v4i{0, 0, 0, 0};
+  uint4 bq[2][4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) bq[0][c] = bbase[c * kSmallQuads];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    if (ks + 1 < KS) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) bq[(ks + 1) & 1][c] = bbase[(ks + 1) * 4 * kSmallSlotCells + c * kSmallQuads];
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const uint4 u = bq[ks & 1][c];
+      const v4i bv = v4i{(int)u.x, (int)u.y, (int)u.z, (int)u.w};
+#pragma unroll
+      for (int o = 0; o < 2; ++o) acc[o][c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[o][ks], bv, acc[o][c], 0, 0, 0);
+    }
+  }
+  if (!live || m >= n_img) return;
+  constexpr int kElem = OUT == kOutI8 ? 1 : 4;
+  char* obase = static_cast<char*>(p.out) + (((size_t)(n0 + m) * p.M + row0) * kSmallHw + 4 * ql) * kElem;
+  const bool last = ql == kSmallQuads - 1;  // position 48 only
+  DispatchAct(OUT == kOutAcc32 ? 0 : p.act.type, [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
+#pragma unroll
+    for (int o = 0; o < 2; ++o) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const u4 v = Finish4<OUT, ACT>(acc[o][0][i], acc[o][1][i], acc[o][2][i], acc[o][3][i], rw.sc[o][i], rw.bi[o][i], p.act);
+        char* ptr = obase + (size_t)(4 * (16 * o + 4 * ln.kq + i)) * kSmallHw * kElem;
+        if (OUT == kOutI8) {
+          if (last) *reinterpret_cast<uint8_t*>(ptr) = (uint8_t)(v.x & 0xffu);
+          else *reinterpret_cast<u1a*>(ptr) = v.x;
+        } else {
+          if (last) *reinterpret_cast<uint32_t*>(ptr) = v.x;
+          else *reinterpret_cast<u4a*>(ptr) = v;
+        }
+      }
+    }
+  });
+}
+
+template <int OUT>
+hipError_t SmallByKs(const ImageMfmaParams& q, dim3 grid, size_t lds, hipStream_t s) {
+  const dim3 block(512);
+  switch (q.K / 64) {
+    case 4:
+      return LaunchWithLds(SmallMapMfmaKernel<4, OUT>, grid, block, lds, s, q);
+    case 8:
+      return LaunchWithLds(SmallMapMfmaKernel<8, OUT>, grid, block, lds, s, q);
+    case 16:
+      return LaunchWithLds(SmallMapMfmaKernel<16, OUT>, grid, block, lds, s, q);
+    default:
+      return hipErrorInvalidValue;
+  }
+}
+
 template <int OUT>
 hipError_t ByKs(const ImageMfmaParams& q, dim3 grid, size_t lds, hipStream_t s) {
   const dim3 block(512);
@@ -333,6 +515,7 @@ hipError_t ByKs(const ImageMfmaParams& q, dim3 grid, size_t lds, hipStream_t s) 
 
 bool ImageMfmaFits(int M, int K, int hw) {
   if (M <= 0 || M % 128 != 0) return false;
+  if (hw == kSmallHw) return (K == 256 || K == 512 || K == 1024) && 256 + (size_t)2 * (K / 16) * kSmallSlotCells * 16 <= (size_t)kMaxLdsBytes;
   if (K != 128 && K != 256 && K != 512) return false;
   if (hw < 16 || hw > 256 || hw % 4 != 0) return false;
   const int qpi = hw / 4, kgs = (4 * qpi + 15) / 16 * 16;
@@ -344,6 +527,25 @@ hipError_t LaunchImageMfma(int out_kind, const ImageMfmaParams& p, hipStream_t s
   if (!ImageMfmaFits(p.M, p.K, p.hw)) return hipErrorInvalidValue;
   if (reinterpret_cast<uintptr_t>(p.x) % 16 != 0 || reinterpret_cast<uintptr_t>(p.out) % 16 != 0) return hipErrorInvalidValue;
   ImageMfmaParams q = p;
+  if (p.hw == kSmallHw) {
+    q.row_groups = p.M / 128;
+    const int64_t small_items = (int64_t)((p.batch + 1) / 2) * q.row_groups;
+    if (small_items > (1 << 28)) return hipErrorInvalidValue;
+    q.items = (int)small_items;
+    q.per_xcd = (q.items + 7) / 8;
+    const size_t small_lds = 256 + (size_t)2 * (p.K / 16) * kSmallSlotCells * 16;
+    const dim3 small_grid(8u * (uint32_t)q.per_xcd);
+    switch (out_kind) {
+      case kOutF32:
+        return SmallByKs<kOutF32>(q, small_grid, small_lds, stream);
+      case kOutI8:
+        return SmallByKs<kOutI8>(q, small_grid, small_lds, stream);
+      case kOutAcc32:
+        return SmallByKs<kOutAcc32>(q, small_grid, small_lds, stream);
+      default:
+        return hipErrorInvalidValue;
+    }
+  }
   q.qpi = p.hw / 4;
   q.kgs = (4 * q.qpi + 15) / 16 * 16;  // a channel group's cells start on a 256-byte boundary: conflict-free operand reads
   q.row_groups = p.M / 128;

@@ -579,7 +579,9 @@ pl::WalkConfig ChooseWalk(const pl_sparse_conv_handle* h, uint32_t P) {
 // occupy the chip, and the block kernel otherwise.
 int AlgoForCall(const pl_sparse_conv_handle* h, int batch, int im_size, bool aligned16) {
   if (!h->auto_int8) return h->algo;
-  if (h->wtiles.ptr && aligned16 && pl::ImageMfmaFits(h->oc, h->ic, im_size) && static_cast<int64_t>(batch) * (h->oc / 128) >= h->image_min_items) return PL_ALGO_IMAGE_MFMA;
+  // work items: (image, row group), for 7 x 7 maps (pair of images, row group)
+  const int64_t image_items = static_cast<int64_t>(im_size == 49 ? (batch + 1) / 2 : batch) * (h->oc / 128);
+  if (h->wtiles.ptr && aligned16 && pl::ImageMfmaFits(h->oc, h->ic, im_size) && image_items >= h->image_min_items) return PL_ALGO_IMAGE_MFMA;
   return h->algo;
 }
 
@@ -617,8 +619,8 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   const bool int8 = desc->kind != PL_KIND_FP32 && !half;
   if (int8 && desc->kind != PL_KIND_INT8_ACC32 && !desc->scale) return Fail(PL_ERR_BAD_ARG, "int8 kinds need per-channel scales");
   if ((desc->algo == PL_ALGO_BLOCK_MFMA || desc->algo == PL_ALGO_IMAGE_MFMA) && !int8) return Fail(PL_ERR_UNSUPPORTED, "the MFMA algorithms exist for int8 only");
-  if (desc->algo == PL_ALGO_IMAGE_MFMA && !pl::ImageMfmaFits(desc->oc, desc->ic, 16))
-    return Fail(PL_ERR_UNSUPPORTED, "the image MFMA algorithm needs oc %% 128 == 0 and ic = 128, 256 or 512 (oc = %d, ic = %d)", desc->oc, desc->ic);
+  if (desc->algo == PL_ALGO_IMAGE_MFMA && !pl::ImageMfmaFits(desc->oc, desc->ic, 16) && !pl::ImageMfmaFits(desc->oc, desc->ic, 49))
+    return Fail(PL_ERR_UNSUPPORTED, "the image MFMA algorithm needs oc %% 128 == 0 and ic = 128, 256, 512 or (7 x 7 maps) 1024 (oc = %d, ic = %d)", desc->oc, desc->ic);
 
   int ndev = 0;
   if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
@@ -711,7 +713,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   int rc = PL_OK;
   if (algo == PL_ALGO_ROW_WALK) rc = BuildRowWalk(L, h);
   if (rc == PL_OK && algo == PL_ALGO_BLOCK_MFMA) rc = BuildBlockMfma(L, h);
-  if (rc == PL_OK && (algo == PL_ALGO_IMAGE_MFMA || (h->auto_int8 && pl::ImageMfmaFits(desc->oc, desc->ic, 16)))) rc = BuildImageMfma(L, h);
+  if (rc == PL_OK && (algo == PL_ALGO_IMAGE_MFMA || (h->auto_int8 && (pl::ImageMfmaFits(desc->oc, desc->ic, 16) || pl::ImageMfmaFits(desc->oc, desc->ic, 49))))) rc = BuildImageMfma(L, h);
   if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8) rc = BuildChunkWalk(L, h);
   if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8 && !half) rc = BuildTileWalk(L, desc->bias, h);
   if (rc == PL_OK) {
@@ -804,7 +806,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.slices = CeilDiv(h->n_groups, p.groups_per_slice);
     e = pl::LaunchHalfWalk(h->semi ? 2 : 1, tp, threads, p, s);
   } else if (AlgoForCall(h, batch, im_size, aligned16) == PL_ALGO_IMAGE_MFMA) {
-    if (!pl::ImageMfmaFits(h->oc, h->ic, im_size)) return Fail(PL_ERR_UNSUPPORTED, "the image MFMA algorithm needs H*W a multiple of 4 in [16, 256] that fits LDS with %d channels (H*W = %d)", h->ic, im_size);
+    if (!pl::ImageMfmaFits(h->oc, h->ic, im_size)) return Fail(PL_ERR_UNSUPPORTED, "the image MFMA algorithm needs H*W = 49 or a multiple of 4 in [16, 256] that fits LDS with %d channels (H*W = %d)", h->ic, im_size);
     if (reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(out_dev) % 16 != 0) return Fail(PL_ERR_UNSUPPORTED, "the image MFMA algorithm needs 16-byte aligned tensors");
     pl::ImageMfmaParams p{};
     p.x = static_cast<const int8_t*>(x_dev);

@@ -256,7 +256,8 @@ struct ImageMfmaParams {
 };
 
 // M a multiple of 128, K = 128, 256 or 512, hw a multiple of 4 in [16, 256]
-// and the image's cells within the LDS of a CU.
+// and the image's cells within the LDS of a CU; or 7 x 7 maps (hw = 49) with
+// K = 256, 512 or 1024 (two images per workgroup).
 bool ImageMfmaFits(int M, int K, int hw);
 // Needs ImageMfmaFits and 16-byte aligned x / out.
 hipError_t LaunchImageMfma(int out_kind, const ImageMfmaParams& p, hipStream_t stream);

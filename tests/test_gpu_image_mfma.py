@@ -2,7 +2,8 @@
 image in LDS) against the CPU oracle through the C ABI: bit-exact for every
 int8 kind.  Shapes cover every class of row alignment (H*W / 4 mod 4 = 0..3),
 one to sixteen window quads left over at the end of a row, images smaller
-than one window, every supported channel count and several row groups."""
+than one window, every supported channel count and several row groups; and
+the kernel for 7 x 7 maps (two images per workgroup)."""
 import copy
 import sys
 
@@ -58,6 +59,29 @@ def test_image_mfma_bit_exact(shape, kind):
         assert np.array_equal(got.astype(np.int64), ref)
 
 
+# 7 x 7 maps (49-byte channel rows, two images per workgroup): every supported
+# channel count, one and several row groups, odd batches (a last pair with one
+# image) and a single image.
+SMALL_MAP_SHAPES = [(2, 256, 128, 7, 7), (5, 512, 256, 7, 7), (1, 1024, 128, 7, 7), (4, 1024, 256, 7, 7), (3, 512, 128, 7, 7)]
+
+
+@pytest.mark.parametrize("kind", sorted(KINDS))
+@pytest.mark.parametrize("shape", SMALL_MAP_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_small_map_mfma_bit_exact(shape, kind):
+    announce("small map", shape, kind)
+    batch, ic, oc, h, w = shape
+    k = KINDS[kind]
+    for act in (("none",) if kind == "acc32" else ("relu", "hswish")):
+        case = case_for(k, batch, ic, oc, h, w, 0.9, False, ACTS[act], seed=ic + 5 * oc + batch)
+        got = run_hip(case, capi.ALGO_IMAGE_MFMA)
+        want = run_oracle(case, oracle_pack(case))
+        assert_same(case, got, want, "small map %s %s %s" % (kind, act, shape))
+        assert np.array_equal(got, run_hip(case, capi.ALGO_BLOCK_MFMA))
+    if kind == "acc32":
+        ref = np.einsum("mk,bkp->bmp", case.dense.astype(np.int64), case.x.reshape(batch, ic, -1).astype(np.int64)).reshape(got.shape)
+        assert np.array_equal(got.astype(np.int64), ref)
+
+
 @pytest.mark.parametrize("act", sorted(ACTS))
 @pytest.mark.parametrize("out_int8", [False, True], ids=["fp32out", "int8out"])
 @pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
@@ -100,7 +124,9 @@ def test_auto_picks_the_image_kernel_only_where_it_applies():
     kernel, _ = make_kernel(case, capi.ALGO_AUTO)
     assert L.pl_sparse_conv_algo_for(kernel._handle, 64, 196) == capi.ALGO_IMAGE_MFMA
     assert L.pl_sparse_conv_algo_for(kernel._handle, 2, 196) == capi.ALGO_BLOCK_MFMA      # too few work items
-    assert L.pl_sparse_conv_algo_for(kernel._handle, 64, 49) == capi.ALGO_BLOCK_MFMA      # 7x7 is not a multiple of 4
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 64, 49) == capi.ALGO_IMAGE_MFMA      # 7x7 maps: pairs of images, 32 x 4 work items
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 32, 49) == capi.ALGO_BLOCK_MFMA      # too few of them
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 64, 50) == capi.ALGO_BLOCK_MFMA      # not a multiple of 4
     assert L.pl_sparse_conv_algo_for(kernel._handle, 64, 28 * 28) == capi.ALGO_BLOCK_MFMA  # does not fit LDS
     # the same handle serves all of them
     import torch
