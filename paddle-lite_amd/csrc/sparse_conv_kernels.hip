@@ -1192,15 +1192,16 @@ hipError_t LaunchBlockMfma(const MfmaConfig& cfg, const MfmaParams& p, hipStream
   uint32_t tiles = (q.total_quads + cfg.tile_quads - 1) / cfg.tile_quads;
   q.row_groups = (p.row_blocks + 3) / 4;
   // Streaming variant: large maps with 128 or 256 channels, whole row groups,
-  // 16-byte row pieces, tiles cut per image with at most 5 % of the quads of
-  // the per-image tiling empty, and several tiles for every resident workgroup.
+  // 16-byte row pieces, tiles cut per image with at most 15 % of the quads of
+  // the per-image tiling empty (28 x 28 maps: 12.5 %), and at least one tile
+  // for every resident workgroup.
   if (cfg.stream && (cfg.out_kind == kOutI8 || cfg.out_kind == kOutF32) && (p.ksteps == 4 || p.ksteps == 8) && p.K == 32 * p.ksteps && cfg.ks_max == p.ksteps &&
       p.hw % 16 == 0 && p.small && p.row_blocks % 4 == 0 && p.M == 32 * p.row_blocks && cfg.tile_quads == 32 && reinterpret_cast<uintptr_t>(p.out) % 16 == 0) {
     const int tpi = (q.qpi + 31) / 32;
     const int64_t stream_tiles = (int64_t)(p.P / (uint32_t)p.hw) * tpi;
     const int per_cu = p.ksteps == 4 ? 3 : 2;  // resident workgroups per CU, by registers
     int lanes = std::max(1, cfg.cus * per_cu / 8 / q.row_groups);
-    if (stream_tiles < (1ll << 30) && (cfg.stream == 2 || (tpi * 32 * 100 <= q.qpi * 105 && stream_tiles >= (int64_t)8 * lanes * 4))) {
+    if (stream_tiles < (1ll << 30) && (cfg.stream == 2 || (tpi * 32 * 100 <= q.qpi * 115 && stream_tiles >= (int64_t)8 * lanes))) {
       lanes = (int)std::min<int64_t>(lanes, (stream_tiles + 7) / 8);
       q.stream_tpi = tpi;
       q.stream_tiles = (int)stream_tiles;
