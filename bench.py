@@ -481,7 +481,9 @@ def run_mobilenet(args):
         want = O.dwconv3x3_int8(x[:2].cpu().numpy(), dwc.filter[:, 0], dw.w_scale_, dw.bias_, a, out="int8", stride=dwc.stride, pad=1)
         assert np.array_equal(t[:2].cpu().numpy(), want), "depthwise layer %d differs from the oracle" % (i + 1)
         dw_bytes = dwc.algorithmic_bytes(batch)
-        steps_list.append(("depthwise", dwc.name, (lambda k=dw, xi=x, ti=t: k.Run(xi, ti)), dw_bytes))
+        # the C entry point itself: the kernel class's argument checks cost more host time per launch than the small layers run
+        steps_list.append(("depthwise", dwc.name, (lambda h=dw._handle, xp=C.c_void_p(x.data_ptr()), tp=C.c_void_p(t.data_ptr()), size=dwc.in_size: capi.check(
+            L.pl_dwconv3x3_run(h, xp, tp, batch, size, size, C.c_void_p(stream)))), dw_bytes))
         case = wl.config5_layer(i)
         kernel, weights = helpers.make_kernel(case)
         ic, oc, hw = wl.MOBILENET_V1_POINTWISE[i]

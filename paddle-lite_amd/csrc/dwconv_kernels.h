@@ -24,6 +24,7 @@ struct DwConvParams {
   int item_rows;           // output rows per thread: 1, 2 or 4, 0 = chosen by the launcher
   int item_cols;           // groups of 4 output columns per thread: 1, 2 or 4, 0 = chosen by the launcher
   int share_lanes;         // 1: lanes load only their own dwords and exchange the rest; 0: every lane loads all; -1 = chosen by the launcher
+  int row_items;           // planes with w + 2 * pad <= 16: 1 = one whole output row per thread, 0 = the item shapes above, -1 = chosen by the launcher
   // filled in by the launcher
   int groups_w;            // column groups per output row
   int items;               // ceil(oh / rows) * groups_w per plane
@@ -34,6 +35,7 @@ struct DwConvParams {
   uint32_t magic_groups;   // likewise for groups_w
   uint32_t magic_blocks;   // likewise for blocks_per_group
   uint32_t magic_channels; // likewise for channels
+  int row_lds_in;          // row items: bytes of LDS for the staged input
 };
 
 // stride 1 or 2; out_kind kOutF32 or kOutI8.

@@ -14,6 +14,7 @@
 
 #include "dwconv_kernels.h"
 #include "epilogue.h"
+#include "launch_lds.h"
 
 namespace pl {
 namespace {
@@ -275,6 +276,180 @@ __global__ void __launch_bounds__(256) DwConv3x3Kernel(const DwConvParams p) {
   });
 }
 
+// ---------------------------------------------------------------------------
+// Narrow planes (w + 2 * pad <= 16: the 14 x 14 and 7 x 7 maps).  Their rows
+// start at any byte address, and global memory is slow with that: the general
+// kernel spends 8.5 us on 64 x 512 planes of 14 x 14 whatever its instruction
+// count.  Here an item is one whole output row of a plane (up to 14 outputs at
+// stride 1, 7 at stride 2), items are numbered through all planes, 256 per
+// workgroup, one per thread, and global memory is touched in aligned 16-byte
+// pieces only:
+//   * the input bytes the workgroup's rows need are one contiguous range; it
+//     is copied to LDS as whole 16-byte pieces (tensors are 16-byte aligned);
+//   * per input row a thread reads the five aligned dwords around the 16 bytes
+//     that start at column -pad from LDS, shifts them into place
+//     (v_alignbyte_b32), masks the bytes outside the row once and slides the
+//     byte windows of its outputs out of them;
+//   * int8 outputs go to LDS byte by byte (the workgroup's output rows are
+//     one contiguous range too) and leave as aligned 16-byte pieces; fp32
+//     outputs are stored directly (dword aligned).
+struct DwRowStage {
+  char* lds_in;      // holds the input bytes from `in_base` on, preceded by 16 bytes of slack
+  int64_t in_base;   // offset of the first staged byte in the tensor (a multiple of 16)
+  char* lds_out;     // int8 output rows of the workgroup, item-major
+};
+
+template <int STRIDE, int NOUT, int OUT, int ACT>
+__device__ __forceinline__ void DwRowItem(const DwConvParams& p, const DwRowStage& st, uint32_t plane, int c, int oy, bool live) {
+  // byte b of a window is column b - pad
+  uint32_t mask[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    uint32_t m = 0xffffffffu;
+    const int below = p.pad - 4 * k;          // bytes of the dword in front of column 0
+    const int inside = p.pad + p.w - 4 * k;   // bytes of the dword, from its first, up to the end of the row
+    if (below > 0) m &= 0xffffffffu << (8 * below);
+    m = inside <= 0 ? 0u : (inside < 4 ? m & (0xffffffffu >> (8 * (4 - inside))) : m);
+    mask[k] = m;
+  }
+  int acc[NOUT];
+#pragma unroll
+  for (int j = 0; j < NOUT; ++j) acc[j] = 0;
+  float s = 0.f, b = 0.f;
+  if (live) {
+    const uint32_t wrow[3] = {p.wpack[4 * c], p.wpack[4 * c + 1], p.wpack[4 * c + 2]};
+    s = p.scale[c];
+    b = p.bias[c];
+    const int iy0 = STRIDE * oy - p.pad;
+    const int64_t plane_at = (int64_t)plane * (uint32_t)(p.h * p.w) - st.in_base + 16;  // LDS offset of the plane's first byte
+    uint32_t D[3][4];
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+      // a row outside [0, h) is zero padding: it reads its neighbour and meets a zero filter row below
+      const uint32_t at = (uint32_t)(plane_at + (uint32_t)(min(max(iy0 + r, 0), p.h - 1) * p.w) - p.pad);
+      const uint32_t* words = reinterpret_cast<const uint32_t*>(st.lds_in + (at & ~3u));
+      uint32_t e[5];
+#pragma unroll
+      for (int k = 0; k < 5; ++k) e[k] = words[k];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) D[r][k] = __builtin_amdgcn_alignbyte(e[k + 1], e[k], at & 3u);
+    }
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+      const int iy = iy0 + r;
+      const int wr = (int)(wrow[r] & ((iy >= 0 && iy < p.h) ? 0xffffffffu : 0u));
+      uint32_t d[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) d[k] = D[r][k] & mask[k];
+#pragma unroll
+      for (int j = 0; j < NOUT; ++j) {
+        const int first = STRIDE * j, k = first / 4, sh = first % 4;
+        const int win = sh == 0 ? (int)d[k] : (int)__builtin_amdgcn_alignbyte(k + 1 < 4 ? d[k + 1] : 0u, d[k], sh);
+        acc[j] = __builtin_amdgcn_sdot4(win, wr, acc[j], false);
+      }
+    }
+  }
+  if (OUT == kOutI8) {
+    // the low byte of the truncated value is the int8 output
+    char* dst = st.lds_out + (uint32_t)threadIdx.x * (uint32_t)p.ow;
+#pragma unroll
+    for (int j = 0; j < NOUT; ++j)
+      if (j < p.ow) dst[j] = (char)static_cast<int>(ActQuantF<ACT>(__builtin_fmaf((float)acc[j], s, b), p.act));
+  } else if (live) {
+    float* dst = static_cast<float*>(p.out) + ((size_t)plane * (uint32_t)p.oh + (uint32_t)oy) * (uint32_t)p.ow;
+    constexpr int NG = (NOUT + 3) / 4;
+#pragma unroll
+    for (int q4 = 0; q4 < NG; ++q4) {
+      const int n_out = min(4, p.ow - 4 * q4);
+      if (n_out <= 0) break;
+      float v[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) v[k] = 4 * q4 + k < NOUT ? ActivateT<ACT>(__builtin_fmaf((float)acc[4 * q4 + k < NOUT ? 4 * q4 + k : 0], s, b), p.act) : 0.0f;
+      if (n_out == 4) {  // a four-dword store needs dword alignment only
+        *reinterpret_cast<v4f*>(dst + 4 * q4) = v4f{v[0], v[1], v[2], v[3]};
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (k < n_out) dst[4 * q4 + k] = v[k];
+      }
+    }
+  }
+}
+
+template <int STRIDE, int NOUT, int OUT>
+__global__ void __launch_bounds__(256) DwRowKernel(const DwConvParams p) {
+  extern __shared__ uint4 dw_lds[];
+  const int tid = (int)threadIdx.x;
+  const uint32_t total = p.planes * (uint32_t)p.oh;  // items
+  const uint32_t first = 256u * blockIdx.x, last = min(first + 255u, total - 1u);
+  const uint32_t plane_a = DivMagic(first, (uint32_t)p.oh, p.magic_items), plane_b = DivMagic(last, (uint32_t)p.oh, p.magic_items);
+  const int oy_a = (int)(first - plane_a * (uint32_t)p.oh), oy_b = (int)(last - plane_b * (uint32_t)p.oh);
+  const int64_t hw = (int64_t)p.h * p.w;
+  // the input bytes the workgroup's rows need, widened to whole 16-byte pieces
+  const int64_t need_lo = (int64_t)plane_a * hw + (int64_t)max(0, STRIDE * oy_a - p.pad) * p.w;
+  const int64_t need_hi = (int64_t)plane_b * hw + (int64_t)min(p.h, STRIDE * oy_b - p.pad + 3) * p.w;
+  DwRowStage st;
+  st.in_base = need_lo & ~(int64_t)15;
+  st.lds_in = reinterpret_cast<char*>(dw_lds);
+  st.lds_out = st.lds_in + p.row_lds_in;
+  const int pieces = (int)((need_hi - st.in_base + 15) >> 4);
+  uint4 piece[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int j = tid + 256 * u;
+    const int64_t at = st.in_base + 16 * (int64_t)j;
+    piece[u] = make_uint4(0, 0, 0, 0);
+    if (j < pieces) {
+      if (at + 16 <= p.in_bytes) {
+        piece[u] = *reinterpret_cast<const uint4*>(p.x + at);
+      } else {  // the tensor's last, partial piece
+        uint32_t w4[4] = {0, 0, 0, 0};
+        for (int t = 0; t < 16; ++t)
+          if (at + t < p.in_bytes) w4[t >> 2] |= (uint32_t)(uint8_t)p.x[at + t] << (8 * (t & 3));
+        piece[u] = make_uint4(w4[0], w4[1], w4[2], w4[3]);
+      }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int j = tid + 256 * u;
+    if (j < pieces) *reinterpret_cast<uint4*>(st.lds_in + 16 + 16 * j) = piece[u];
+  }
+  __syncthreads();
+  const uint32_t item = first + (uint32_t)tid;
+  const bool live = item < total;
+  const uint32_t plane = live ? DivMagic(item, (uint32_t)p.oh, p.magic_items) : plane_b;
+  const int oy = live ? (int)(item - plane * (uint32_t)p.oh) : oy_b;
+  const int c = (int)(plane - DivMagic(plane, (uint32_t)p.channels, p.magic_channels) * (uint32_t)p.channels);
+  DispatchAct(p.act.type, [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
+    DwRowItem<STRIDE, NOUT, OUT, ACT>(p, st, plane, c, oy, live);
+  });
+  if (OUT == kOutI8) {
+    __syncthreads();
+    // the workgroup's output rows: 256 * ow bytes from item `first` on, a multiple of 16 at a multiple of 16
+    const int64_t out_at = (int64_t)first * p.ow + 16 * (int64_t)tid;
+    const int64_t out_end = (int64_t)total * p.ow;
+    if (tid < 16 * p.ow) {
+      int8_t* dst = static_cast<int8_t*>(p.out) + out_at;
+      const uint4 v = *reinterpret_cast<const uint4*>(st.lds_out + 16 * tid);
+      if (out_at + 16 <= out_end) {
+        *reinterpret_cast<uint4*>(dst) = v;
+      } else {  // the tensor's last, partial piece
+        const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+        for (int t = 0; t < 16; ++t)
+          if (out_at + t < out_end) dst[t] = (int8_t)(w4[t >> 2] >> (8 * (t & 3)));
+      }
+    }
+  }
+}
+
+template <int STRIDE, int NOUT>
+hipError_t LaunchRows(int out_kind, dim3 grid, size_t lds, hipStream_t stream, const DwConvParams& q) {
+  if (out_kind == kOutI8) return LaunchWithLds(DwRowKernel<STRIDE, NOUT, kOutI8>, grid, dim3(256), lds, stream, q);
+  return LaunchWithLds(DwRowKernel<STRIDE, NOUT, kOutF32>, grid, dim3(256), lds, stream, q);
+}
+
 template <int STRIDE, int R, int CG>
 void LaunchShape(int out_kind, dim3 grid, hipStream_t stream, const DwConvParams& q) {
   if (out_kind == kOutI8) {
@@ -303,6 +478,25 @@ hipError_t LaunchDwConv3x3(int stride, int out_kind, const DwConvParams& p, hipS
   // 28x28 11.2 / - / 10.2 / 11.8 / 12.0.
   int rows = p.item_rows, cg = p.item_cols;
   const bool rows_given = rows == 1 || rows == 2 || rows == 4, cols_given = cg == 1 || cg == 2 || cg == 4;
+  // Narrow planes of 16-byte aligned tensors: one output row per thread, global memory touched in aligned
+  // 16-byte pieces only, unless an item shape is asked for.  The input range of a workgroup (the planes
+  // its 256 rows touch) must fit 16 KB of LDS.
+  {
+    const int64_t planes_per_wg = (256 + p.oh - 1) / p.oh + 1;
+    const int64_t lds_in = ((planes_per_wg * p.h * p.w + 15) / 16 + 6) * 16;  // 16 bytes in front, alignment of the first piece, windows that reach past the last row
+    const bool aligned = reinterpret_cast<uintptr_t>(p.x) % 16 == 0 && reinterpret_cast<uintptr_t>(p.out) % 16 == 0;
+    if (p.w + 2 * p.pad <= 16 && lds_in <= 16384 && aligned && (p.row_items > 0 || (p.row_items < 0 && !rows_given && !cols_given))) {
+      const uint64_t items64 = (uint64_t)p.planes * (uint64_t)p.oh;
+      if (items64 >= (1ull << 31)) return hipErrorInvalidValue;
+      q.magic_items = Magic(p.oh);
+      q.magic_channels = Magic(p.channels);
+      q.row_lds_in = (int)lds_in;
+      const size_t lds = (size_t)lds_in + (out_kind == kOutI8 ? (size_t)256 * p.ow : 0);
+      dim3 row_grid((uint32_t)((items64 + 255) / 256));
+      if (stride == 1) return p.ow <= 7 ? LaunchRows<1, 7>(out_kind, row_grid, lds, stream, q) : LaunchRows<1, 14>(out_kind, row_grid, lds, stream, q);
+      return LaunchRows<2, 7>(out_kind, row_grid, lds, stream, q);
+    }
+  }
   if (!cols_given) cg = stride == 1 ? ((p.oh >= 24 && p.ow >= 24) ? 2 : 1) : (p.ow >= 14 ? 2 : 1);
   if (!rows_given) rows = stride == 1 ? 2 : (cg == 2 ? 1 : 2);
   if (stride == 2 && rows == 4) rows = 2;

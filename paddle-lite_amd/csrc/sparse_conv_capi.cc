@@ -1122,6 +1122,7 @@ struct pl_dwconv_handle {
   int item_rows = 0;     // 0 = chosen per shape; PL_DWCONV_ROWS overrides
   int item_cols = 0;     // 0 = chosen per shape; PL_DWCONV_COLS overrides
   int share_lanes = -1;  // -1 = chosen per shape; PL_DWCONV_SHARE_LANES overrides
+  int row_items = -1;    // -1 = chosen per shape; PL_DWCONV_ROW_ITEMS overrides
 };
 
 int pl_dwconv3x3_prepare(const pl_dwconv_desc* desc, pl_dwconv_handle** out_handle) {
@@ -1163,6 +1164,7 @@ int pl_dwconv3x3_prepare(const pl_dwconv_desc* desc, pl_dwconv_handle** out_hand
   if (const char* e2 = std::getenv("PL_DWCONV_ROWS")) h->item_rows = std::atoi(e2);
   if (const char* e2 = std::getenv("PL_DWCONV_COLS")) h->item_cols = std::atoi(e2);
   if (const char* e2 = std::getenv("PL_DWCONV_SHARE_LANES")) h->share_lanes = std::atoi(e2) != 0 ? 1 : 0;
+  if (const char* e2 = std::getenv("PL_DWCONV_ROW_ITEMS")) h->row_items = std::atoi(e2) != 0 ? 1 : 0;
   // filter rows as the dot-product operand (w0, w1, w2, 0)
   std::vector<uint32_t> wpack(static_cast<size_t>(desc->channels) * 4, 0u);
   for (int c = 0; c < desc->channels; ++c)
@@ -1209,6 +1211,7 @@ int pl_dwconv3x3_run(pl_dwconv_handle* h, const int8_t* x_dev, void* out_dev, in
   p.item_rows = h->item_rows;
   p.item_cols = h->item_cols;
   p.share_lanes = h->share_lanes;
+  p.row_items = h->row_items;
   const hipError_t e = pl::LaunchDwConv3x3(h->stride, h->kind == PL_KIND_INT8_INT8 ? pl::kOutI8 : pl::kOutF32, p, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? PL_OK : FailHip(e, "depthwise convolution launch");
 }

@@ -115,6 +115,21 @@ def test_item_shapes(monkeypatch, stride, rows, cols, out):
             run_case(n, c, h, w, stride, pad, out, ACTS["relu6"](), True, seed=1000 * rows + 100 * cols + 10 * i + pad + stride)
 
 
+# narrow planes (w + 2 * pad <= 16) take one whole output row per thread by
+# default; both that kernel and the general one, on every width it covers
+@pytest.mark.parametrize("row_items", ["0", "1"])
+@pytest.mark.parametrize("stride", [1, 2])
+@pytest.mark.parametrize("out", ["int8", "fp32"])
+def test_narrow_planes(monkeypatch, row_items, stride, out):
+    monkeypatch.setenv("PL_DWCONV_ROW_ITEMS", row_items)
+    for pad in (0, 1):
+        for w in range(3 - 2 * pad if 3 - 2 * pad > 0 else 1, 17 - 2 * pad):
+            h = 1 + (5 * w) % 9 if pad else 3 + (5 * w) % 7
+            run_case(2, 3, h, w, stride, pad, out, ACTS["hswish"](), True, seed=100 * w + 10 * pad + stride)
+    run_case(3, 70, 14, 14, stride, 1, out, ACTS["relu"](), False, seed=5 + stride)  # several workgroups, the first and the last at the tensor's ends
+    run_case(5, 33, 7, 7, stride, 1, out, ACTS["relu6"](), True, seed=6 + stride)
+
+
 @pytest.mark.parametrize("stride", [1, 2])
 def test_large_planes(stride):
     # more than 2^16 items per plane, and a plane whose item count is odd
