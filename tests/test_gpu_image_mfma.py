@@ -85,6 +85,51 @@ def test_small_map_mfma_bit_exact(shape, kind):
 @pytest.mark.parametrize("act", sorted(ACTS))
 @pytest.mark.parametrize("out_int8", [False, True], ids=["fp32out", "int8out"])
 @pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
+def test_small_map_mfma_activations_and_structures(paired, out_int8, act):
+    announce("small map acts", paired, out_int8, act)
+    kind = capi.KIND_INT8_INT8 if out_int8 else capi.KIND_INT8_FP32
+    case = case_for(kind, 3, 256, 128, 7, 7, 0.8, paired, ACTS[act], seed=78)
+    if act == "none":
+        case.bias = None
+    got = run_hip(case, capi.ALGO_IMAGE_MFMA, force_semi=paired)
+    want = run_oracle(case, oracle_pack(case, force_semi=paired))
+    assert_same(case, got, want, "small map %s" % act)
+
+
+def test_small_map_mfma_extremes_and_surroundings():
+    """Largest magnitudes (accumulators of 1024 x 127 x 127), an empty output
+    row, and the bytes around the output tensor stay untouched (rows of 49
+    outputs are stored as dwords and single bytes at odd addresses)."""
+    import torch
+
+    announce("small map extremes")
+    case = case_for(capi.KIND_INT8_ACC32, 3, 1024, 128, 7, 7, 0.5, False, AP(), seed=11)
+    case.dense[7] = 0
+    case.dense[64:66] = 127
+    case.x[1] = -127
+    got = run_hip(case, capi.ALGO_IMAGE_MFMA)
+    ref = np.einsum("mk,bkp->bmp", case.dense.astype(np.int64), case.x.reshape(3, 1024, -1).astype(np.int64)).reshape(got.shape)
+    assert np.array_equal(got.astype(np.int64), ref)
+    assert np.all(got[:, 7] == 0)
+    case8 = case_for(capi.KIND_INT8_INT8, 3, 512, 128, 7, 7, 0.9, False, ACTS["relu"], seed=12)
+    kernel, _ = make_kernel(case8, capi.ALGO_IMAGE_MFMA)
+    numel = 3 * 128 * 49
+    guard = 64
+    buf = torch.full((numel + 2 * guard,), 77, dtype=torch.int8, device="cuda")
+    x = torch.from_numpy(case8.x).cuda()
+    L = capi.lib()
+    import ctypes as C
+
+    capi.check(L.pl_sparse_conv_run(kernel._handle, x.data_ptr(), buf.data_ptr() + guard, 3, 49, C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    host = buf.cpu().numpy()
+    assert (host[:guard] == 77).all() and (host[guard + numel:] == 77).all()
+    assert np.array_equal(host[guard:guard + numel].reshape(3, 128, 7, 7), run_oracle(case8, oracle_pack(case8)))
+
+
+@pytest.mark.parametrize("act", sorted(ACTS))
+@pytest.mark.parametrize("out_int8", [False, True], ids=["fp32out", "int8out"])
+@pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
 def test_image_mfma_activations_and_structures(paired, out_int8, act):
     announce("image acts", paired, out_int8, act)
     kind = capi.KIND_INT8_INT8 if out_int8 else capi.KIND_INT8_FP32
