@@ -365,6 +365,8 @@ int BuildChunkWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h, bool ha
 // four entries as records of byte offsets and weights.
 // Main / spare divisions of the tile walk's row groups that are prepared: spare shares of 1/16 .. 8/16.
 constexpr int kTileWalkSplits = 8;
+// Equal divisions that are prepared (two equal parts are the 8/16 division above).
+constexpr int kTileWalkEqualParts[] = {3, 4, 5, 6, 8, 10};
 
 int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_handle* h) {
   h->tw_built = 0;
@@ -381,19 +383,19 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
   const uint32_t recs_per_chunk = chunk_words / rec_words;
   const uint32_t zero_row = static_cast<uint32_t>(L.ic) * pl::kTileWalkTile * 4;
   std::vector<uint32_t> stream, first, counts;
-  // Sixteen streams for the given row groups (largest first): each group goes to the stream with the least work so far.
-  // Returns the work of the fullest stream.
-  auto emit = [&](const std::vector<int>& part) {
-    std::vector<std::vector<int>> members(streams);
-    std::vector<int64_t> load(streams, 0);
+  // Streams for the given row groups (largest first): each group goes to the stream with the least work so far.
+  // Sixteen streams make one part.  Returns the work of the fullest stream.
+  auto emit = [&](const std::vector<int>& part, int n_streams) {
+    std::vector<std::vector<int>> members(n_streams);
+    std::vector<int64_t> load(n_streams, 0);
     for (int g : part) {
       int best = 0;
-      for (int s2 = 1; s2 < streams; ++s2)
+      for (int s2 = 1; s2 < n_streams; ++s2)
         if (load[s2] < load[best]) best = s2;
       members[best].push_back(g);
       load[best] += work(g);
     }
-    for (int s2 = 0; s2 < streams; ++s2) {
+    for (int s2 = 0; s2 < n_streams; ++s2) {
       first.push_back(static_cast<uint32_t>(stream.size() / chunk_words));
       counts.push_back(static_cast<uint32_t>(members[s2].size()));
       uint32_t recs = 0;
@@ -436,7 +438,7 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
   // Set 0: all row groups in one part.  Sets 1 .. kTileWalkSplits: a spare part with about s / 16 of the work
   // (a mix of sizes: going through the groups from the largest, a group joins the spare part whenever that
   // keeps the part at or below its share), the rest in the main part.
-  h->tw_stream_work = emit(order);
+  h->tw_stream_work = emit(order, streams);
   for (int s16 = 1; s16 <= kTileWalkSplits; ++s16) {
     std::vector<int> main_part, spare_part;
     int64_t all_w = 0, spare_w = 0;
@@ -450,9 +452,12 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
         main_part.push_back(g);
       }
     }
-    emit(main_part);
-    emit(spare_part);
+    emit(main_part, streams);
+    emit(spare_part, streams);
   }
+  // Equal parts for problems with at most half as many tiles as CUs: n workgroups per tile, each with a
+  // sixteenth-of-n share of the row groups.
+  for (int n : kTileWalkEqualParts) emit(order, streams * n);
   hipError_t e = h->tw_stream.Upload(stream.data(), stream.size() * sizeof(uint32_t));
   if (e == hipSuccess) e = h->tw_first.Upload(first.data(), first.size() * sizeof(uint32_t));
   if (e == hipSuccess) e = h->tw_desc.Upload(counts.data(), counts.size() * sizeof(uint32_t));
@@ -859,12 +864,11 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     if (h->mfma_tile_quads > 0) c.tile_quads = h->mfma_tile_quads;
     e = pl::LaunchBlockMfma(c, p, s);
   } else if (!h->int8 && !h->half && vec && h->tw_built != 0 && h->walk_tiled > 0 &&
-             (h->walk_tiled == 2 || 64 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kTileWalkTile)) >= 5 * h->wg_slots_default)) {
-    // fp32 with 128-position tiles for at least 5/32 of the CUs (with the row
-    // groups of a tile shared between two CUs a launch takes about 14.5 us up
-    // to half as many tiles as CUs; measured crossover against the other walks
-    // between 24 and 49 tiles on 256 CUs): the walk with the tile and the
-    // lists in LDS
+             (h->walk_tiled == 2 || 32 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kTileWalkTile)) >= h->wg_slots_default)) {
+    // fp32 with 128-position tiles for at least a sixteenth of the CUs (the
+    // row groups of a tile are shared between up to ten CUs; measured
+    // crossover against the other walks between 13 and 25 tiles on 256 CUs):
+    // the walk with the tile and the lists in LDS
     pl::TileWalkParams p{};
     p.x = static_cast<const float*>(x_dev);
     p.out = static_cast<float*>(out_dev);
@@ -878,10 +882,15 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     // times what one below it costs.
     const int tiles = CeilDiv(static_cast<int>(P), pl::kTileWalkTile);
     const int cus = std::max(8, h->wg_slots_default / 2) / 8 * 8;
-    int s16 = 0;
+    int s16 = 0, equal_parts = 0;
     if (tiles < cus && h->walk_split != 0) {
       const int per_xcd = CeilDiv(tiles, 8), spare = cus / 8 - per_xcd;
-      if (spare >= 1) {
+      if (h->walk_split < 0 && per_xcd * 3 <= cus / 8) {
+        // at most a third as many tiles as CUs: n workgroups per tile, equal shares
+        const int room = (cus / 8) / per_xcd;
+        for (int n : kTileWalkEqualParts)
+          if (n <= room) equal_parts = n;
+      } else if (spare >= 1) {
         const int r = CeilDiv(per_xcd, spare);
         const double sw = (2000.0 + 14.0 * h->ic) / (355.0 * static_cast<double>(std::max<int64_t>(1, h->tw_stream_work)));
         const double f = (1.0 - (r - 1) * sw) / (r + 1);
@@ -889,11 +898,19 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
         s16 = std::max(0, std::min(kTileWalkSplits, s16));
       }
     }
-    // stream tables: set 0 has one part, sets 1 .. 8 two
-    const size_t table = s16 == 0 ? 0 : static_cast<size_t>(pl::kTileWalkWaves) * (2 * s16 - 1);
+    // stream tables: set 0 has one part, sets 1 .. 8 two, then the equal divisions
+    size_t table = s16 == 0 ? 0 : static_cast<size_t>(pl::kTileWalkWaves) * (2 * s16 - 1);
+    if (equal_parts != 0) {
+      table = static_cast<size_t>(pl::kTileWalkWaves) * (1 + 2 * kTileWalkSplits);
+      for (int n : kTileWalkEqualParts) {
+        if (n == equal_parts) break;
+        table += static_cast<size_t>(pl::kTileWalkWaves) * n;
+      }
+    }
     p.stream_first = static_cast<const uint32_t*>(h->tw_first.ptr) + table;
     p.stream_groups = static_cast<const uint32_t*>(h->tw_desc.ptr) + table;
-    p.split = s16 != 0;
+    p.split = equal_parts != 0 ? 2 : (s16 != 0 ? 1 : 0);
+    p.parts = equal_parts;
     p.split_slots = cus / 8;
     p.n_groups = h->n_groups;
     p.M = h->oc;

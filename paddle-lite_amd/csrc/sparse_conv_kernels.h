@@ -125,8 +125,12 @@ struct TileWalkParams {
   int tiles;                     // filled in by the launcher
   // 1: the row groups are dealt into a main and a spare part; the grid then has
   // split_slots workgroups per XCD (one per CU), more than any XCD has tiles.
+  // 2: `parts` equal parts, as many workgroups per tile (parts x the tiles of
+  // an XCD must not exceed split_slots); the stream tables then hold
+  // parts x kTileWalkWaves entries.
   int split;
   int split_slots;
+  int parts;
 };
 
 // LDS the kernel needs for K input channels.

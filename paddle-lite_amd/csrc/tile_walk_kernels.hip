@@ -20,7 +20,8 @@
 // With fewer tiles than CUs, the row groups can be dealt into a main and a
 // spare part (two sets of sixteen streams): the tile's own workgroup walks the
 // main part, and the workgroups on the CUs that have no tile of their own walk
-// the spare parts of several tiles, one tile after the other.
+// the spare parts of several tiles, one tile after the other.  With at most a
+// third as many tiles as CUs, n workgroups share a tile with equal parts.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -187,6 +188,12 @@ __device__ __forceinline__ void TileWalkBody(const TileWalkParams& p, float* til
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int first = (xcd * p.tiles) >> 3, last = ((xcd + 1) * p.tiles) >> 3;
   const int count = last - first;
+  if (p.split == 2) {
+    // equal parts: part = slot / count of tile slot % count
+    const int part = count > 0 ? slot / count : p.parts;
+    if (part < p.parts) WalkOneTile<NR, ACT>(p, tile, first + (slot - part * count), part);
+    return;
+  }
   if (slot < count) {
     WalkOneTile<NR, ACT>(p, tile, first + slot, 0);
     return;
@@ -220,7 +227,10 @@ hipError_t LaunchTileWalk(int nrows, const TileWalkParams& p, hipStream_t stream
   TileWalkParams q = p;
   q.tiles = (int)((p.P + kTP - 1) / kTP);
   uint32_t slots = ((uint32_t)q.tiles + 7) / 8;  // workgroups per XCD
-  if (q.split != 0) {
+  if (q.split == 2) {
+    if (q.parts < 2 || (int64_t)q.parts * slots > q.split_slots) return hipErrorInvalidValue;
+    slots *= (uint32_t)q.parts;
+  } else if (q.split != 0) {
     if (q.split_slots < (int)slots + 1) return hipErrorInvalidValue;  // every XCD needs a spare workgroup
     slots = (uint32_t)q.split_slots;
   }
