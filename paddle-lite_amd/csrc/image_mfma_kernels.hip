@@ -20,6 +20,7 @@
 //     the first window instead of after the whole tile.
 //   * The quads that the shifted windows leave over at the end of a row are
 //     computed with the operands swapped (positions as matrix rows).
+// A second kernel below takes 7 x 7 maps, two images per workgroup.
 //
 // Reference semantics: out = act(fmaf(float(acc), scale, bias)) per output,
 // int32 accumulation over all channels (sparse_conv_impl.cc:1661-1685 computes
@@ -47,18 +48,6 @@ typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 // the same with the alignment of its elements only: rows of 49 outputs start anywhere
 typedef uint32_t u4a __attribute__((ext_vector_type(4), aligned(4)));
 typedef uint32_t u1a __attribute__((aligned(1)));
-
-// 4 dwords holding 4 channels x 4 positions -> 4 positions x 4 channels.
-__device__ __forceinline__ void Transpose4x4(uint32_t& r0, uint32_t& r1, uint32_t& r2, uint32_t& r3) {
-  const uint32_t a = __builtin_amdgcn_perm(r1, r0, 0x05010400u);
-  const uint32_t b = __builtin_amdgcn_perm(r1, r0, 0x07030602u);
-  const uint32_t c = __builtin_amdgcn_perm(r3, r2, 0x05010400u);
-  const uint32_t d = __builtin_amdgcn_perm(r3, r2, 0x07030602u);
-  r0 = __builtin_amdgcn_perm(c, a, 0x05040100u);
-  r1 = __builtin_amdgcn_perm(c, a, 0x07060302u);
-  r2 = __builtin_amdgcn_perm(d, b, 0x05040100u);
-  r3 = __builtin_amdgcn_perm(d, b, 0x07060302u);
-}
 
 // 16 bytes written through to memory as streaming data (sc1 nt).  Measured on
 // 64 x 512 -> 512 @14x14, fp32 output, whole sectors: plain 13.8 us, sc1 12.3,
