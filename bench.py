@@ -40,6 +40,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib", "mobilenet", "density-sweep", "floors"])
     ap.add_argument("--algo", default="auto", choices=["auto", "walk", "mfma", "image"])
+    ap.add_argument("--image-kernel", default="rule", choices=["rule", "regroup", "transpose"], help="which image MFMA kernel a handle uses where both apply (pl_sparse_conv_tuning.image_kernel)")
     ap.add_argument("--fp16", action="store_true", help="run an fp32 configuration (c1, c2) through the half-precision kernel")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cache-resident", action="store_true", help="reuse one buffer set (reported, never the headline)")
@@ -584,7 +585,8 @@ def main():
         case.name += "_fp16"
         args.no_cpu_baseline = True  # the CPU baselines are fp32 / int8 paths
     algo = {"auto": capi.ALGO_AUTO, "walk": capi.ALGO_ROW_WALK, "mfma": capi.ALGO_BLOCK_MFMA, "image": capi.ALGO_IMAGE_MFMA}[args.algo]
-    kernel, weights = helpers.make_kernel(case, algo=algo)
+    tune = capi.tuning(image_kernel={"rule": 0, "regroup": capi.IMAGE_KERNEL_REGROUP, "transpose": capi.IMAGE_KERNEL_TRANSPOSE}[args.image_kernel])
+    kernel, weights = helpers.make_kernel(case, algo=algo, tuning=tune)
     info = kernel.info()
     ops = case.algorithmic_ops()
     nbytes = case.algorithmic_bytes(weights)
@@ -662,11 +664,14 @@ def main():
     per_algo = None
     if case.kind in (capi.KIND_INT8_FP32, capi.KIND_INT8_INT8):
         per_algo = {algo_name: round(kernel_ms * 1e3, 3)}
-        for a, name in sorted(algo_names.items()):
+        others = sorted(algo_names.items())
+        if algo_name == "image_mfma":
+            others.append((capi.ALGO_IMAGE_MFMA, "image_mfma_regroup"))  # the image kernel that regroups in LDS
+        for a, name in others:
             if name in per_algo:
                 continue
             try:
-                other, _ = helpers.make_kernel(case, algo=a)
+                other, _ = helpers.make_kernel(case, algo=a, tuning=capi.tuning(image_kernel=capi.IMAGE_KERNEL_REGROUP) if name == "image_mfma_regroup" else None)
             except capi.SparseConvError:
                 continue  # this shape is outside the algorithm's range
             if L.pl_sparse_conv_run_sequence(other._handle, xp, op, n_sets, case.batch, case.im_size, 50, C.c_void_p(stream), None) < 0:

@@ -95,6 +95,36 @@ typedef struct pl_activation {
   float hs_threshold;  /* hard_swish_threshold                              */
 } pl_activation;
 
+/* Tuning overrides of one handle; every field 0 = the library's own rule.
+ * The reference configures its kernels through setters and a config struct,
+ * never through process state (lite/api/paddle_api.h:542-547); this struct is
+ * the counterpart for the choices this library makes per handle.  Fields
+ * marked (switch) take PL_TUNE_RULE / PL_TUNE_NEVER / PL_TUNE_ALWAYS, where
+ * ALWAYS means "whenever the shape allows it". */
+enum { PL_TUNE_RULE = 0, PL_TUNE_NEVER = 1, PL_TUNE_ALWAYS = 2 };
+typedef struct pl_sparse_conv_tuning {
+  int32_t image_kernel;      /* PL_ALGO_IMAGE_MFMA: 1 (and the rule) = the kernel
+                                that regroups the image in LDS, 2 = the kernel
+                                with transposing LDS reads (H*W = 4 mod 8 only;
+                                slightly slower where measured)                */
+  int32_t image_min_items;   /* fewest (image, 128 rows) work items for which
+                                PL_ALGO_AUTO takes the image kernel            */
+  int32_t mfma_stream;       /* (switch) streaming form of the block kernel    */
+  int32_t mfma_sub_tiles;    /* (switch) several tiles per workgroup, ic <= 64 */
+  int32_t mfma_tile_quads;   /* block kernel: position quads per tile, 8 .. 32 */
+  int32_t mfma_narrow_i8_stores; /* 1 = 4-byte int8 stores in the block kernel */
+  int32_t wg_slots;          /* workgroups taken as resident at once           */
+  int32_t walk_tiled;        /* (switch) fp32 walk with tile and lists in LDS  */
+  int32_t walk_split;        /* that walk: 1 = row groups not divided between
+                                CUs, 1 + k = k sixteenths to the spare CUs     */
+  int32_t walk_chunked;      /* (switch) fp32 / fp16 walk over channel chunks  */
+  int32_t chunk_walk_groups; /* that walk: row groups per wavefront, 4 or 8    */
+  int32_t walk_tile;         /* plain walk: positions per tile (power of two)  */
+  int32_t walk_threads;      /* plain walk: threads per workgroup              */
+  int32_t walk_slices;       /* plain walk: row slices                         */
+  int32_t reserved[2];       /* must be 0                                      */
+} pl_sparse_conv_tuning;
+
 /* Everything PrepareForRun() knows.  All pointers are HOST pointers and are
  * only read during pl_sparse_conv_prepare(). Replaces the argument list of
  * sparse_conv_*_pipelined (lite/backends/arm/math/sparse_conv_impl.h:38-73,
@@ -116,6 +146,8 @@ typedef struct pl_sparse_conv_desc {
   const float* scale;            /* oc merged scales; int8 kinds only       */
   const float* bias;             /* oc merged biases or NULL                */
   pl_activation act;
+  pl_sparse_conv_tuning tuning;  /* struct_size may also be the offset of this
+                                    field: then every rule applies            */
 } pl_sparse_conv_desc;
 
 typedef struct pl_sparse_conv_info {
@@ -262,6 +294,13 @@ typedef struct pl_dwconv_desc {
   const float* scale;       /* [channels]                                    */
   const float* bias;        /* [channels] or NULL                            */
   pl_activation act;
+  /* tuning, 0 = the library's rule (struct_size may also be the offset of
+   * item_rows: then every rule applies) */
+  int32_t item_rows;        /* output rows per thread: 1, 2 or 4             */
+  int32_t item_cols;        /* groups of four output columns per thread      */
+  int32_t share_lanes;      /* PL_TUNE_*: neighbouring lanes exchange dwords  */
+  int32_t row_items;        /* PL_TUNE_*: one output row per thread through
+                               LDS (narrow planes)                           */
 } pl_dwconv_desc;
 
 typedef struct pl_dwconv_handle pl_dwconv_handle;

@@ -11,6 +11,8 @@ PL_OK, PL_ERR_BAD_ARG, PL_ERR_BAD_LAYOUT, PL_ERR_UNSUPPORTED, PL_ERR_HIP, PL_ERR
 KIND_FP32, KIND_INT8_FP32, KIND_INT8_INT8, KIND_INT8_ACC32, KIND_FP16 = 0, 1, 2, 3, 4
 ACT_NONE, ACT_RELU, ACT_RELU6, ACT_LEAKY_RELU, ACT_HARD_SWISH = 0, 1, 2, 4, 10
 ALGO_AUTO, ALGO_ROW_WALK, ALGO_BLOCK_MFMA, ALGO_IMAGE_MFMA = 0, 1, 2, 3
+TUNE_RULE, TUNE_NEVER, TUNE_ALWAYS = 0, 1, 2
+IMAGE_KERNEL_REGROUP, IMAGE_KERNEL_TRANSPOSE = 1, 2
 
 EXPORTS = [
     "pl_sparse_conv_abi_version",
@@ -46,6 +48,37 @@ class Activation(C.Structure):
     ]
 
 
+class Tuning(C.Structure):
+    """pl_sparse_conv_tuning: every field 0 = the library's rule."""
+    _fields_ = [
+        ("image_kernel", C.c_int32),
+        ("image_min_items", C.c_int32),
+        ("mfma_stream", C.c_int32),
+        ("mfma_sub_tiles", C.c_int32),
+        ("mfma_tile_quads", C.c_int32),
+        ("mfma_narrow_i8_stores", C.c_int32),
+        ("wg_slots", C.c_int32),
+        ("walk_tiled", C.c_int32),
+        ("walk_split", C.c_int32),
+        ("walk_chunked", C.c_int32),
+        ("chunk_walk_groups", C.c_int32),
+        ("walk_tile", C.c_int32),
+        ("walk_threads", C.c_int32),
+        ("walk_slices", C.c_int32),
+        ("reserved", C.c_int32 * 2),
+    ]
+
+
+def tuning(**fields):
+    """A Tuning with the named fields set (the rest stay 0 = by rule)."""
+    t = Tuning()
+    for name, value in fields.items():
+        if name not in dict(Tuning._fields_) or name == "reserved":
+            raise ValueError("no tuning field %r" % name)
+        setattr(t, name, int(value))
+    return t
+
+
 class DwConvDesc(C.Structure):
     _fields_ = [
         ("struct_size", C.c_uint32),
@@ -57,6 +90,10 @@ class DwConvDesc(C.Structure):
         ("scale", C.c_void_p),
         ("bias", C.c_void_p),
         ("act", Activation),
+        ("item_rows", C.c_int32),
+        ("item_cols", C.c_int32),
+        ("share_lanes", C.c_int32),
+        ("row_items", C.c_int32),
     ]
 
 
@@ -78,6 +115,7 @@ class Desc(C.Structure):
         ("scale", C.c_void_p),
         ("bias", C.c_void_p),
         ("act", Activation),
+        ("tuning", Tuning),
     ]
 
 

@@ -142,6 +142,7 @@ template <int KS, int OUT>
 __device__ __forceinline__ void Tail(const uint4* __restrict__ xt, int kgs, int qpi, int q0, const v4i (&a)[2][KS], const Rows& rw, const DevAct& act, char* __restrict__ orow, int hw, Lane ln) {
   int tq = q0 + (ln.n >> 2);
   if (tq > qpi - 1) tq = qpi - 1;  // rows past the end of the image row: any valid cell, results unused
+  if (tq < 0) tq = 0;              // likewise in front of it (rows shorter than a window, shifted left)
   const uint4* tb = xt + ln.kq * kgs + (ln.n & 3) * qpi + tq;
   v4i acc[2] = {v4i{0, 0, 0, 0}, v4i{0, 0, 0, 0}};
 #pragma unroll
@@ -153,7 +154,8 @@ __device__ __forceinline__ void Tail(const uint4* __restrict__ xt, int kgs, int 
   }
   constexpr int kElem = OUT == kOutI8 ? 1 : 4;
   const int q = q0 + ln.kq;
-  if (q >= qpi) return;
+  // quads in front of the row belong to the previous row's last sector and are written by its wavefront
+  if (q < 0 || q >= qpi) return;
   DispatchAct(OUT == kOutAcc32 ? 0 : act.type, [&](auto act_c) {
     constexpr int ACT = decltype(act_c)::value;
 #pragma unroll

@@ -6,13 +6,16 @@
 
 #include <algorithm>
 #include <cstdarg>
+#include <cstddef>
 #include <cstdio>
 #include <cstdlib>
 #include <cmath>
 #include <cstring>
+#include <initializer_list>
 #include <memory>
 #include <new>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "../../include/pl_sparse_conv.h"
@@ -144,6 +147,10 @@ struct pl_sparse_conv_handle {
   // fp32 tile walk (whole tile and lists in LDS)
   DevBuf tw_stream, tw_first, tw_desc;
   int tw_built = 0;  // list streams of the tile walk uploaded
+  // host copy of the streams and, per header record, (word index of its bias, first row | rows << 24):
+  // the headers carry the bias, so a new bias is patched in here and the streams are uploaded again
+  std::vector<uint32_t> tw_host_stream;
+  std::vector<std::pair<uint32_t, uint32_t>> tw_bias_slots;
   int64_t tw_stream_work = 0;  // work units (entry batches + 2 per row group) of the fullest of the sixteen unsplit streams
   int walk_split = -1;          // sixteenths of the row groups' work dealt to the CUs without a tile: -1 by rule, 0 never, 1 .. 8 forced
   int walk_tiled = 1;            // 0 never, 1 when the problem suits it, 2 whenever the shape allows
@@ -166,6 +173,8 @@ struct pl_sparse_conv_handle {
   int mfma_sub_tiles = 1;   // several tiles per workgroup for <= 64 input channels: 0 never, 1 when enough workgroups remain, 2 always
   // image MFMA (dense 16x64 tiles, rows of a tile four apart)
   DevBuf wtiles;
+  DevBuf wtiles_tr;      // the same tiles in the channel order of the kernel with transposing LDS reads
+  int image_kernel = 0;  // 0 by rule, 1 regrouping kernel, 2 transposing-read kernel
   // int8 handles prepared with PL_ALGO_AUTO hold several forms and choose per call
   bool auto_int8 = false;
   int image_min_items = 128;  // fewest (image, 128-row group) work items for which the image kernel is chosen
@@ -176,7 +185,7 @@ struct pl_sparse_conv_handle {
   int padded_rows = 0;
 
   int64_t DeviceBytes() const {
-    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + cw_desc.bytes + cw_idx.bytes + cw_wts.bytes + hw_kidx.bytes + hw_wts.bytes + hw_bias.bytes + wblocks.bytes + kmask.bytes + wtiles.bytes + scale.bytes + bias.bytes);
+    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + cw_desc.bytes + cw_idx.bytes + cw_wts.bytes + hw_kidx.bytes + hw_wts.bytes + hw_bias.bytes + wblocks.bytes + kmask.bytes + wtiles.bytes + wtiles_tr.bytes + tw_stream.bytes + tw_first.bytes + tw_desc.bytes + scale.bytes + bias.bytes);
   }
 };
 
@@ -382,7 +391,10 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
   const uint32_t chunk_words = pl::kTileWalkChunkBytes / 4;
   const uint32_t recs_per_chunk = chunk_words / rec_words;
   const uint32_t zero_row = static_cast<uint32_t>(L.ic) * pl::kTileWalkTile * 4;
-  std::vector<uint32_t> stream, first, counts;
+  std::vector<uint32_t>& stream = h->tw_host_stream;
+  stream.clear();
+  h->tw_bias_slots.clear();
+  std::vector<uint32_t> first, counts;
   // Streams for the given row groups (largest first): each group goes to the stream with the least work so far.
   // Sixteen streams make one part.  Returns the work of the fullest stream.
   auto emit = [&](const std::vector<int>& part, int n_streams) {
@@ -420,6 +432,7 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
           if (rg.nrows == 2) std::memcpy(&rec[3], &bias[rg.row0 + 1], 4);
         }
         put(rec);
+        h->tw_bias_slots.emplace_back(static_cast<uint32_t>(stream.size() - rec_words + 2), rec[0]);
         for (uint32_t e0 = 0; e0 < rg.count; e0 += 4) {
           for (uint32_t e = 0; e < 4; ++e) {
             const bool real = e0 + e < rg.count;
@@ -528,6 +541,40 @@ int BuildImageMfma(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
   return PL_OK;
 }
 
+// The same tiles for the image kernel with transposing LDS reads.  That kernel
+// takes the channels of a k-step in the order its reads deliver them: a step
+// holds the 64 channels of one parity out of 128, and byte b of lane group g
+// is channel 64 (b / 8) + 4 (8 (g % 2) + b % 8) + 2 (g / 2) + parity of them
+// (image_tr_kernels.hip).  Any order is right as long as weights and
+// activations agree: the dot product is an exact integer sum.
+int BuildImageTrMfma(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
+  const int steps = L.ic / 64;
+  std::vector<int8_t> tiles(static_cast<size_t>(L.oc) * L.ic, 0);
+  auto put = [&](int row, uint32_t c, uint32_t wbits) {
+    const int8_t w = static_cast<int8_t>(wbits & 0xffu);
+    if (w == 0) return;
+    const int rg = row / 128, rl = row % 128;
+    const int rho = rl & 3, m32 = rl >> 2;  // row = rg * 128 + rho + 4 * (16 j + m)
+    const int j = m32 >> 4, m = m32 & 15;
+    const int cc = static_cast<int>(c & 127u);
+    const int step = 2 * static_cast<int>(c >> 7) + (cc & 1);
+    const int u = cc >> 1;            // 32 r + 2 t + (g / 2)
+    const int r = u >> 5, t = (u & 31) >> 1, ghi = u & 1;
+    const int g = 2 * ghi + (t >> 3), b = 8 * r + (t & 7);
+    const int lane = m + 16 * g;
+    tiles[((((static_cast<size_t>(rg) * 4 + rho) * 2 + j) * steps + step) * 64 + lane) * 16 + b] = w;
+  };
+  for (const pl::RowGroup& g : L.groups) {
+    for (uint32_t j = 0; j < g.count; ++j) {
+      put(g.row0, L.ic_index[g.first + j], L.w0[g.first + j]);
+      if (g.nrows == 2) put(g.row0 + 1, L.ic_index[g.first + j], L.w1[g.first + j]);
+    }
+  }
+  const hipError_t e = h->wtiles_tr.Upload(tiles.data(), tiles.size());
+  if (e != hipSuccess) return FailHip(e, "uploading the weight tiles");
+  return PL_OK;
+}
+
 int UploadEpilogue(pl_sparse_conv_handle* h, const float* scale, const float* bias) {
   const size_t n = static_cast<size_t>(h->padded_rows);
   if (scale) {
@@ -615,7 +662,14 @@ int pl_device_count(void) {
 int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handle** out_handle) {
   if (!desc || !out_handle) return Fail(PL_ERR_BAD_ARG, "null argument");
   *out_handle = nullptr;
-  if (desc->struct_size != sizeof(pl_sparse_conv_desc)) return Fail(PL_ERR_BAD_ARG, "pl_sparse_conv_desc size mismatch (%u vs %zu)", desc->struct_size, sizeof(pl_sparse_conv_desc));
+  if (desc->struct_size != sizeof(pl_sparse_conv_desc) && desc->struct_size != offsetof(pl_sparse_conv_desc, tuning))
+    return Fail(PL_ERR_BAD_ARG, "pl_sparse_conv_desc size mismatch (%u vs %zu)", desc->struct_size, sizeof(pl_sparse_conv_desc));
+  pl_sparse_conv_tuning tune{};
+  if (desc->struct_size == sizeof(pl_sparse_conv_desc)) tune = desc->tuning;
+  if (tune.reserved[0] != 0 || tune.reserved[1] != 0) return Fail(PL_ERR_BAD_ARG, "pl_sparse_conv_tuning.reserved must be 0");
+  for (int32_t sw : {tune.mfma_stream, tune.mfma_sub_tiles, tune.walk_tiled, tune.walk_chunked})
+    if (sw < PL_TUNE_RULE || sw > PL_TUNE_ALWAYS) return Fail(PL_ERR_BAD_ARG, "a tuning switch is not PL_TUNE_RULE, PL_TUNE_NEVER or PL_TUNE_ALWAYS");
+  if (tune.image_kernel < 0 || tune.image_kernel > 2) return Fail(PL_ERR_BAD_ARG, "tuning.image_kernel must be 0, 1 or 2");
   if (desc->kind < PL_KIND_FP32 || desc->kind > PL_KIND_FP16) return Fail(PL_ERR_BAD_ARG, "unknown kind %d", desc->kind);
   if (desc->algo < PL_ALGO_AUTO || desc->algo > PL_ALGO_IMAGE_MFMA) return Fail(PL_ERR_BAD_ARG, "unknown algo %d", desc->algo);
   if (desc->oc <= 0 || desc->ic <= 0 || desc->im_size <= 0) return Fail(PL_ERR_BAD_ARG, "oc, ic and im_size must be positive");
@@ -652,20 +706,22 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   h->device = dev;
   h->wg_slots = 2 * std::max(1, prop.multiProcessorCount);
   h->wg_slots_default = h->wg_slots;
-  if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_I8_WIDE")) h->mfma_i8_wide = std::atoi(e) != 0;
-  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_TILED")) h->walk_tiled = std::max(0, std::min(2, std::atoi(e)));
-  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_SPLIT")) h->walk_split = std::max(-1, std::min(kTileWalkSplits, std::atoi(e)));
-  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_CHUNKED")) h->walk_chunked = std::max(0, std::min(2, std::atoi(e)));
-  if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_SUB_TILES")) h->mfma_sub_tiles = std::max(0, std::min(2, std::atoi(e)));
-  if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_TILE_QUADS")) h->mfma_tile_quads = std::max(0, std::min(32, std::atoi(e)));
-  // tuning switches for experiments; the defaults are what measured best
-  if (const char* e = std::getenv("PL_SPARSE_CONV_WG_SLOTS")) h->wg_slots = std::max(1, std::atoi(e));
-  if (const char* e = std::getenv("PL_SPARSE_CONV_MFMA_STREAM")) h->mfma_stream = std::max(0, std::min(2, std::atoi(e)));
-  if (const char* e = std::getenv("PL_SPARSE_CONV_IMAGE_MIN_ITEMS")) h->image_min_items = std::max(1, std::atoi(e));
-  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_TILE")) h->walk_tile = std::atoi(e);
-  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_THREADS")) h->walk_threads = std::atoi(e);
-  if (const char* e = std::getenv("PL_SPARSE_CONV_WALK_SLICES")) h->walk_slices = std::atoi(e);
-  if (const char* e = std::getenv("PL_SPARSE_CONV_CHUNK_WALK_GROUPS")) h->cw_groups = std::atoi(e) == 4 ? 4 : 8;
+  // tuning overrides (0 = the rule); the switches are kept as 0 never, 1 by rule, 2 whenever possible
+  auto sw = [](int32_t t) { return t == PL_TUNE_NEVER ? 0 : (t == PL_TUNE_ALWAYS ? 2 : 1); };
+  h->mfma_stream = sw(tune.mfma_stream);
+  h->mfma_sub_tiles = sw(tune.mfma_sub_tiles);
+  h->walk_tiled = sw(tune.walk_tiled);
+  h->walk_chunked = sw(tune.walk_chunked);
+  h->mfma_i8_wide = tune.mfma_narrow_i8_stores == 0;
+  if (tune.walk_split > 0) h->walk_split = std::min(kTileWalkSplits, tune.walk_split - 1);
+  if (tune.mfma_tile_quads > 0) h->mfma_tile_quads = std::max(8, std::min(32, tune.mfma_tile_quads));
+  if (tune.wg_slots > 0) h->wg_slots = tune.wg_slots;
+  if (tune.image_min_items > 0) h->image_min_items = tune.image_min_items;
+  h->image_kernel = tune.image_kernel;
+  h->walk_tile = tune.walk_tile;
+  h->walk_threads = tune.walk_threads;
+  h->walk_slices = tune.walk_slices;
+  h->cw_groups = tune.chunk_walk_groups == 4 ? 4 : 8;
   h->kind = desc->kind;
   h->oc = desc->oc;
   h->ic = desc->ic;
@@ -719,6 +775,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   if (algo == PL_ALGO_ROW_WALK) rc = BuildRowWalk(L, h);
   if (rc == PL_OK && algo == PL_ALGO_BLOCK_MFMA) rc = BuildBlockMfma(L, h);
   if (rc == PL_OK && (algo == PL_ALGO_IMAGE_MFMA || (h->auto_int8 && (pl::ImageMfmaFits(desc->oc, desc->ic, 16) || pl::ImageMfmaFits(desc->oc, desc->ic, 49))))) rc = BuildImageMfma(L, h);
+  if (rc == PL_OK && h->wtiles.ptr && pl::ImageTrMfmaFits(desc->oc, desc->ic, 20)) rc = BuildImageTrMfma(L, h);
   if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8) rc = BuildChunkWalk(L, h);
   if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8 && !half) rc = BuildTileWalk(L, desc->bias, h);
   if (rc == PL_OK) {
@@ -816,7 +873,6 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     pl::ImageMfmaParams p{};
     p.x = static_cast<const int8_t*>(x_dev);
     p.out = out_dev;
-    p.wtiles = h->wtiles.ptr;
     p.scale = static_cast<const float*>(h->scale.ptr);
     p.bias = static_cast<const float*>(h->bias.ptr);
     p.M = h->oc;
@@ -824,7 +880,17 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.hw = im_size;
     p.batch = batch;
     p.act = h->act;
-    e = pl::LaunchImageMfma(OutKind(h->kind), p, s);
+    // The kernel with transposing LDS reads runs on request only: on 64 x 512 -> 512 @14x14 it is about 4 %
+    // slower than the kernel that regroups the image (9.9 against 9.7 us).
+    const bool tr_fits = h->wtiles_tr.ptr != nullptr && pl::ImageTrMfmaFits(h->oc, h->ic, im_size);
+    if (h->image_kernel == 2 && !tr_fits) return Fail(PL_ERR_UNSUPPORTED, "the image kernel with transposing LDS reads needs H*W = 4 (mod 8) from 20 on, ic = 128, 256 or 512 and an image that leaves 41 KB of LDS free (H*W = %d, ic = %d)", im_size, h->ic);
+    if (tr_fits && h->image_kernel == 2) {
+      p.wtiles = h->wtiles_tr.ptr;
+      e = pl::LaunchImageTrMfma(OutKind(h->kind), p, s);
+    } else {
+      p.wtiles = h->wtiles.ptr;
+      e = pl::LaunchImageMfma(OutKind(h->kind), p, s);
+    }
   } else if (h->algo == PL_ALGO_BLOCK_MFMA) {
     pl::MfmaParams p{};
     p.x = static_cast<const int8_t*>(x_dev);
@@ -1022,6 +1088,16 @@ int pl_sparse_conv_set_epilogue(pl_sparse_conv_handle* h, const float* scale, co
   if (scale && !h->int8) return Fail(PL_ERR_BAD_ARG, "floating-point kernels take no scales");
   int rc = h->half ? UploadHalfBias(h, bias) : UploadEpilogue(h, scale, bias);
   if (rc != PL_OK) return rc;
+  if (bias && h->tw_built) {
+    // the tile walk starts its accumulators from the bias in its header records
+    for (const auto& slot : h->tw_bias_slots) {
+      const uint32_t row0 = slot.second & 0xffffffu, nrows = slot.second >> 24;
+      std::memcpy(&h->tw_host_stream[slot.first], &bias[row0], 4);
+      if (nrows == 2) std::memcpy(&h->tw_host_stream[slot.first + 1], &bias[row0 + 1], 4);
+    }
+    const hipError_t e = h->tw_stream.Upload(h->tw_host_stream.data(), h->tw_host_stream.size() * sizeof(uint32_t));
+    if (e != hipSuccess) return FailHip(e, "uploading the tile-walk list streams");
+  }
   if (act) {
     h->act = ToDevAct(*act);
     h->act_h = ToDevActH(*act);
@@ -1136,16 +1212,20 @@ struct pl_dwconv_handle {
   int kind = 0, channels = 0, stride = 1, pad = 0;
   DevBuf wpack, scale, bias;
   pl::DevAct act{};
-  int item_rows = 0;     // 0 = chosen per shape; PL_DWCONV_ROWS overrides
-  int item_cols = 0;     // 0 = chosen per shape; PL_DWCONV_COLS overrides
-  int share_lanes = -1;  // -1 = chosen per shape; PL_DWCONV_SHARE_LANES overrides
-  int row_items = -1;    // -1 = chosen per shape; PL_DWCONV_ROW_ITEMS overrides
+  int item_rows = 0;     // 0 = chosen per shape
+  int item_cols = 0;     // 0 = chosen per shape
+  int share_lanes = -1;  // -1 = chosen per shape, 0 / 1 forced
+  int row_items = -1;    // -1 = chosen per shape, 0 / 1 forced
 };
 
 int pl_dwconv3x3_prepare(const pl_dwconv_desc* desc, pl_dwconv_handle** out_handle) {
   if (!desc || !out_handle) return Fail(PL_ERR_BAD_ARG, "null argument");
   *out_handle = nullptr;
-  if (desc->struct_size != sizeof(pl_dwconv_desc)) return Fail(PL_ERR_BAD_ARG, "pl_dwconv_desc size mismatch (%u vs %zu)", desc->struct_size, sizeof(pl_dwconv_desc));
+  if (desc->struct_size != sizeof(pl_dwconv_desc) && desc->struct_size != offsetof(pl_dwconv_desc, item_rows))
+    return Fail(PL_ERR_BAD_ARG, "pl_dwconv_desc size mismatch (%u vs %zu)", desc->struct_size, sizeof(pl_dwconv_desc));
+  const bool tuned = desc->struct_size == sizeof(pl_dwconv_desc);
+  if (tuned && (desc->share_lanes < PL_TUNE_RULE || desc->share_lanes > PL_TUNE_ALWAYS || desc->row_items < PL_TUNE_RULE || desc->row_items > PL_TUNE_ALWAYS))
+    return Fail(PL_ERR_BAD_ARG, "a tuning switch is not PL_TUNE_RULE, PL_TUNE_NEVER or PL_TUNE_ALWAYS");
   if (desc->kind != PL_KIND_INT8_FP32 && desc->kind != PL_KIND_INT8_INT8) return Fail(PL_ERR_BAD_ARG, "kind must be int8 -> fp32 or int8 -> int8");
   if (desc->channels <= 0) return Fail(PL_ERR_BAD_ARG, "channels must be positive");
   if (desc->stride != 1 && desc->stride != 2) return Fail(PL_ERR_UNSUPPORTED, "stride %d: only 1 and 2 exist", desc->stride);
@@ -1178,10 +1258,12 @@ int pl_dwconv3x3_prepare(const pl_dwconv_desc* desc, pl_dwconv_handle** out_hand
   h->pad = desc->pad;
   h->act = ToDevAct(desc->act);
   h->act.hs_inv_scale = desc->act.hs_scale;  // this op multiplies by the scale itself
-  if (const char* e2 = std::getenv("PL_DWCONV_ROWS")) h->item_rows = std::atoi(e2);
-  if (const char* e2 = std::getenv("PL_DWCONV_COLS")) h->item_cols = std::atoi(e2);
-  if (const char* e2 = std::getenv("PL_DWCONV_SHARE_LANES")) h->share_lanes = std::atoi(e2) != 0 ? 1 : 0;
-  if (const char* e2 = std::getenv("PL_DWCONV_ROW_ITEMS")) h->row_items = std::atoi(e2) != 0 ? 1 : 0;
+  if (tuned) {
+    h->item_rows = desc->item_rows;
+    h->item_cols = desc->item_cols;
+    h->share_lanes = desc->share_lanes == PL_TUNE_RULE ? -1 : (desc->share_lanes == PL_TUNE_ALWAYS ? 1 : 0);
+    h->row_items = desc->row_items == PL_TUNE_RULE ? -1 : (desc->row_items == PL_TUNE_ALWAYS ? 1 : 0);
+  }
   // filter rows as the dot-product operand (w0, w1, w2, 0)
   std::vector<uint32_t> wpack(static_cast<size_t>(desc->channels) * 4, 0u);
   for (int c = 0; c < desc->channels; ++c)

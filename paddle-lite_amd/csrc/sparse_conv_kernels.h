@@ -266,6 +266,18 @@ bool ImageMfmaFits(int M, int K, int hw);
 // Needs ImageMfmaFits and 16-byte aligned x / out.
 hipError_t LaunchImageMfma(int out_kind, const ImageMfmaParams& p, hipStream_t stream);
 
+// The same work item with the image kept in LDS as it lies in memory and the
+// operands read with transposing LDS reads (image_tr_kernels.hip).  wtiles
+// then holds the tiles in that kernel's channel order:
+// [row group][rho][j][step = 2 (c / 128) + c % 2][64 lanes][16 bytes], lane l
+// byte b of a step holding row rho + 4 (16 j + l % 16) and channel
+// 128 (step / 2) + step % 2 + 64 (b / 8) + 4 (8 (g % 2) + b % 8) + 2 (g / 2), g = l / 16.
+// M a multiple of 128, K = 128, 256 or 512, hw = 4 (mod 8) from 20 on and
+// the image plus 41 KB of staging buffers within the LDS of a CU.
+bool ImageTrMfmaFits(int M, int K, int hw);
+// Needs ImageTrMfmaFits and 16-byte aligned x / out.
+hipError_t LaunchImageTrMfma(int out_kind, const ImageMfmaParams& p, hipStream_t stream);
+
 // Largest dynamic LDS size a kernel of this library may be given.
 constexpr int kMaxLdsBytes = 160 * 1024;
 constexpr int kMfmaTilePos = 128;

@@ -45,7 +45,9 @@ class DepthwiseConv(object):
     :257-322 (int8 output: / output_scale, bias / output_scale, relu6
     coefficient and hard_swish offset and threshold / output_scale)."""
 
-    def __init__(self, param, out_precision="int8"):
+    def __init__(self, param, out_precision="int8", item_rows=0, item_cols=0, share_lanes=capi.TUNE_RULE, row_items=capi.TUNE_RULE):
+        # the four tuning arguments are the fields of pl_dwconv_desc of the same names (0 = by rule)
+        self.tuning = (int(item_rows), int(item_cols), int(share_lanes), int(row_items))
         out = str(np.dtype(out_precision))
         if out not in ("int8", "float32"):
             raise ValueError("no depthwise kernel with %s output" % out)
@@ -112,6 +114,7 @@ class DepthwiseConv(object):
         d.scale = self.w_scale_.ctypes.data
         d.bias = bias.ctypes.data if bias is not None else None
         d.act = a
+        d.item_rows, d.item_cols, d.share_lanes, d.row_items = self.tuning
         h = C.c_void_p()
         capi.check(capi.lib().pl_dwconv3x3_prepare(C.byref(d), C.byref(h)))
         self._release()

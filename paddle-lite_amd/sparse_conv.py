@@ -151,13 +151,14 @@ class SparseConvKernel(object):
     output scale once and leaves the slope alone.
     """
 
-    def __init__(self, param, precision="float32", out_precision="float32", algo=capi.ALGO_AUTO, reference_quirks=True):
+    def __init__(self, param, precision="float32", out_precision="float32", algo=capi.ALGO_AUTO, reference_quirks=True, tuning=None):
         key = (str(np.dtype(precision)), str(np.dtype(out_precision)))
         if key not in _KINDS:
             raise ValueError("no sparse_conv2d kernel for %s -> %s" % key)
         self.kind = _KINDS[key]
         self.param = param
         self.algo = algo
+        self.tuning = tuning  # capi.Tuning or None (every rule of the library applies)
         self.reference_quirks = reference_quirks
         self._handle = None
         self._first_epoch = True
@@ -227,6 +228,8 @@ class SparseConvKernel(object):
         d.scale = scale.ctypes.data if scale is not None else None
         d.bias = bias.ctypes.data if bias is not None else None
         d.act = a
+        if self.tuning is not None:
+            d.tuning = self.tuning
         h = C.c_void_p()
         capi.check(capi.lib().pl_sparse_conv_prepare(C.byref(d), C.byref(h)))
         self._release()

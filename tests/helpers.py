@@ -73,20 +73,20 @@ def run_oracle(case, packed=None, quirks=False, x=None):
 _PREC = {capi.KIND_FP32: ("float32", "float32"), capi.KIND_INT8_FP32: ("int8", "float32"), capi.KIND_INT8_INT8: ("int8", "int8"), capi.KIND_INT8_ACC32: ("int8", "int32"), capi.KIND_FP16: ("float16", "float16")}
 
 
-def make_kernel(case, algo=capi.ALGO_AUTO, force_semi=None, quirks=False, im_size=None):
+def make_kernel(case, algo=capi.ALGO_AUTO, force_semi=None, quirks=False, im_size=None, tuning=None):
     weights = pla.detect_and_pack(case.dense, im_size or case.im_size, force_semi=force_semi)
     param = pla.SparseConvParam(weights, bias=case.bias, activation_param=case.act, enable_int8=case.kind not in (capi.KIND_FP32, capi.KIND_FP16), input_scale=case.input_scale,
                                 weight_scale=case.weight_scale if case.weight_scale is not None else (), output_scale=case.output_scale)
     prec = _PREC[case.kind]
-    k = pla.SparseConvKernel(param, prec[0], prec[1], algo=algo, reference_quirks=quirks)
+    k = pla.SparseConvKernel(param, prec[0], prec[1], algo=algo, reference_quirks=quirks, tuning=tuning)
     k.PrepareForRun()
     return k, weights
 
 
-def run_hip(case, algo=capi.ALGO_AUTO, force_semi=None, quirks=False, x=None, kernel=None):
+def run_hip(case, algo=capi.ALGO_AUTO, force_semi=None, quirks=False, x=None, kernel=None, tuning=None):
     import torch
 
-    k = kernel or make_kernel(case, algo, force_semi, quirks)[0]
+    k = kernel or make_kernel(case, algo, force_semi, quirks, tuning=tuning)[0]
     xd = torch.from_numpy(case.x if x is None else x).cuda()
     out = k.Run(xd)
     torch.cuda.synchronize()

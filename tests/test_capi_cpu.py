@@ -31,11 +31,37 @@ def test_library_exports_every_declared_symbol():
     assert L.pl_sparse_conv_abi_version() == capi.ABI_VERSION
 
 
-def test_struct_layout_matches_header():
-    # pl_sparse_conv_desc: 8 x int32, then pointers / int64, then the 24-byte activation
+def test_struct_layout_matches_header(tmp_path):
+    """sizeof and offsetof of every field of the header's structs, printed by a
+    C program compiled against the header, equal the ctypes mirror's."""
+    import shutil
+    import subprocess
+
+    structs = {"pl_activation": capi.Activation, "pl_sparse_conv_tuning": capi.Tuning, "pl_sparse_conv_desc": capi.Desc, "pl_sparse_conv_info": capi.Info, "pl_dwconv_desc": capi.DwConvDesc}
     assert C.sizeof(capi.Activation) == 24
-    assert C.sizeof(capi.Desc) == 8 * 4 + 7 * 8 + 24
-    assert C.sizeof(capi.Info) == 4 * 4 + 6 * 8 or C.sizeof(capi.Info) == 3 * 4 + 4 + 6 * 8
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler")
+    lines = ["#include <stdio.h>", "#include <stddef.h>", '#include "pl_sparse_conv.h"', "int main(void) {"]
+    for cname, cls in sorted(structs.items()):
+        lines.append('  printf("%s %%zu\\n", sizeof(%s));' % (cname, cname))
+        for fname, _ in cls._fields_:
+            lines.append('  printf("%s.%s %%zu\\n", offsetof(%s, %s));' % (cname, fname, cname, fname))
+    lines += ["  return 0;", "}"]
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.check_call([gcc, "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
+    want = dict(l.split() for l in subprocess.check_output([str(exe)], text=True).splitlines())
+    for cname, cls in structs.items():
+        assert C.sizeof(cls) == int(want[cname]), cname
+        for fname, _ in cls._fields_:
+            assert getattr(cls, fname).offset == int(want["%s.%s" % (cname, fname)]), (cname, fname)
+    # every field of the header's structs is mirrored (declarators inside the typedef's braces)
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "pl_sparse_conv.h")).read(), flags=re.S)
+    for cname, cls in structs.items():
+        body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (cname, cname), text, flags=re.S).group(1)
+        assert body.count(";") + body.count(",") == len(cls._fields_), cname
 
 
 def _rand(rng, oc, ic, density, dtype, paired):

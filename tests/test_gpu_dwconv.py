@@ -27,7 +27,7 @@ def oracle_act(ap):
     return a
 
 
-def run_case(n, c, h, w, stride, pad, out, act, bias, seed, guard=64):
+def run_case(n, c, h, w, stride, pad, out, act, bias, seed, guard=64, **tuning):
     import torch
 
     rng = np.random.RandomState(seed)
@@ -37,7 +37,7 @@ def run_case(n, c, h, w, stride, pad, out, act, bias, seed, guard=64):
     b = (rng.standard_normal(c) * 0.5).astype(np.float32) if bias else None
     param = pla.ConvParam(filt, b, strides=(stride, stride), paddings=(pad, pad, pad, pad), activation_param=act, input_scale=0.02, weight_scale=ws,
                           output_scale=0.11 if out == "int8" else 1.0)
-    k = pla.DepthwiseConv(param, out_precision="int8" if out == "int8" else "float32")
+    k = pla.DepthwiseConv(param, out_precision="int8" if out == "int8" else "float32", **tuning)
     k.PrepareForRun()
     # the tensor sits inside a larger buffer whose surroundings must stay
     # untouched (output) and must not matter (input)
@@ -107,27 +107,24 @@ ITEM_SHAPES = {1: [(2, 1), (4, 1), (1, 2), (2, 2), (4, 2), (1, 4), (2, 4)], 2: [
 
 @pytest.mark.parametrize("stride,rows,cols", [(s, r, c) for s in (1, 2) for (r, c) in ITEM_SHAPES[s]])
 @pytest.mark.parametrize("out", ["int8", "fp32"])
-def test_item_shapes(monkeypatch, stride, rows, cols, out):
-    monkeypatch.setenv("PL_DWCONV_ROWS", str(rows))
-    monkeypatch.setenv("PL_DWCONV_COLS", str(cols))
+def test_item_shapes(stride, rows, cols, out):
     for i, (n, c, h, w) in enumerate([(2, 3, 7, 7), (1, 5, 14, 14), (2, 2, 33, 17), (1, 4, 30, 61), (2, 40, 28, 28), (1, 2, 3, 70)]):
         for pad in (0, 1):
-            run_case(n, c, h, w, stride, pad, out, ACTS["relu6"](), True, seed=1000 * rows + 100 * cols + 10 * i + pad + stride)
+            run_case(n, c, h, w, stride, pad, out, ACTS["relu6"](), True, seed=1000 * rows + 100 * cols + 10 * i + pad + stride, item_rows=rows, item_cols=cols)
 
 
 # narrow planes (w + 2 * pad <= 16) take one whole output row per thread by
 # default; both that kernel and the general one, on every width it covers
-@pytest.mark.parametrize("row_items", ["0", "1"])
+@pytest.mark.parametrize("row_items", [capi.TUNE_NEVER, capi.TUNE_ALWAYS], ids=["general", "row-items"])
 @pytest.mark.parametrize("stride", [1, 2])
 @pytest.mark.parametrize("out", ["int8", "fp32"])
-def test_narrow_planes(monkeypatch, row_items, stride, out):
-    monkeypatch.setenv("PL_DWCONV_ROW_ITEMS", row_items)
+def test_narrow_planes(row_items, stride, out):
     for pad in (0, 1):
         for w in range(3 - 2 * pad if 3 - 2 * pad > 0 else 1, 17 - 2 * pad):
             h = 1 + (5 * w) % 9 if pad else 3 + (5 * w) % 7
-            run_case(2, 3, h, w, stride, pad, out, ACTS["hswish"](), True, seed=100 * w + 10 * pad + stride)
-    run_case(3, 70, 14, 14, stride, 1, out, ACTS["relu"](), False, seed=5 + stride)  # several workgroups, the first and the last at the tensor's ends
-    run_case(5, 33, 7, 7, stride, 1, out, ACTS["relu6"](), True, seed=6 + stride)
+            run_case(2, 3, h, w, stride, pad, out, ACTS["hswish"](), True, seed=100 * w + 10 * pad + stride, row_items=row_items)
+    run_case(3, 70, 14, 14, stride, 1, out, ACTS["relu"](), False, seed=5 + stride, row_items=row_items)  # several workgroups, the first and the last at the tensor's ends
+    run_case(5, 33, 7, 7, stride, 1, out, ACTS["relu6"](), True, seed=6 + stride, row_items=row_items)
 
 
 @pytest.mark.parametrize("stride", [1, 2])

@@ -59,14 +59,12 @@ CHUNKED_SHAPES = [(2, 64, 64, 4, 4), (1, 96, 48, 8, 6), (3, 130, 67, 4, 5), (1, 
 @pytest.mark.parametrize("act", ["none", "relu6", "hswish"])
 @pytest.mark.parametrize("shape", CHUNKED_SHAPES, ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
-def test_fp16_chunked_walk(shape, paired, act, monkeypatch):
+def test_fp16_chunked_walk(shape, paired, act):
     batch, ic, oc, h, w = shape
     case = half_case(batch, ic, oc, h, w, 0.75, paired, ACTS[act], seed=ic + 3 * oc)
     want = run_oracle(case, oracle_pack(case, force_semi=paired))
-    monkeypatch.setenv("PL_SPARSE_CONV_WALK_CHUNKED", "2")
-    got = run_hip(case, capi.ALGO_AUTO, force_semi=paired)
+    got = run_hip(case, capi.ALGO_AUTO, force_semi=paired, tuning=capi.tuning(walk_chunked=capi.TUNE_ALWAYS))
     assert_same(case, got, want, "fp16 chunked %s %s" % (act, shape))
     # the plain half-precision walk gives the same bits (same order of operations)
-    monkeypatch.setenv("PL_SPARSE_CONV_WALK_CHUNKED", "0")
-    plain = run_hip(case, capi.ALGO_AUTO, force_semi=paired)
+    plain = run_hip(case, capi.ALGO_AUTO, force_semi=paired, tuning=capi.tuning(walk_chunked=capi.TUNE_NEVER))
     assert np.array_equal(got.view(np.uint16), plain.view(np.uint16))

@@ -37,21 +37,34 @@ def case_for(kind, batch, ic, oc, h, w, sparsity, paired, act, seed):
 
 # (batch, ic, oc, h, w).  H*W/4 mod 4: 14x14 -> 1, 6x10 -> 3, 8x8 -> 0, 6x9 -> ... (54 is not a multiple of 4, excluded),
 # 10x10 -> 1, 12x14 -> 2, 16x16 -> 0 (largest image), 4x4 -> 0 (smaller than a window), 5x8 -> 2, 4x7 -> 3
+# Maps with H*W = 4 (mod 8) can also be taken by the kernel with transposing LDS reads when it is
+# asked for; both run here on every such shape (4x59 is the largest with 512 channels, 12x21 the largest at all,
+# 2x10 the smallest, 6x6 / 4x11 / 4x13 have two to four windows per row).
 SHAPES = [
     (3, 512, 128, 14, 14), (2, 256, 256, 6, 10), (2, 128, 128, 8, 8), (1, 512, 384, 10, 10), (2, 256, 128, 12, 14),
     (1, 512, 128, 16, 16), (3, 128, 256, 4, 4), (2, 256, 128, 5, 8), (2, 128, 128, 4, 7), (1, 512, 128, 9, 12), (9, 256, 128, 2, 10),
+    (2, 512, 128, 4, 59), (1, 256, 128, 12, 21), (1, 128, 256, 6, 6), (2, 256, 128, 4, 11), (3, 128, 128, 4, 13),
 ]
+IMAGE_KERNELS = {"regroup": capi.IMAGE_KERNEL_REGROUP, "transpose": capi.IMAGE_KERNEL_TRANSPOSE}
 
 
+@pytest.mark.parametrize("image_kernel", sorted(IMAGE_KERNELS))
 @pytest.mark.parametrize("kind", sorted(KINDS))
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
-def test_image_mfma_bit_exact(shape, kind):
-    announce("image", shape, kind)
+def test_image_mfma_bit_exact(shape, kind, image_kernel):
+    announce("image", shape, kind, image_kernel)
     batch, ic, oc, h, w = shape
     k = KINDS[kind]
+    if image_kernel == "transpose" and (h * w) % 8 != 4:
+        # refused, not rerouted
+        case = case_for(k, batch, ic, oc, h, w, 0.85, False, ACTS["none"], seed=1)
+        with pytest.raises(capi.SparseConvError) as e:
+            run_hip(case, capi.ALGO_IMAGE_MFMA, tuning=capi.tuning(image_kernel=capi.IMAGE_KERNEL_TRANSPOSE))
+        assert e.value.code == capi.PL_ERR_UNSUPPORTED
+        return
     for act in (("none",) if kind == "acc32" else ("leaky", "hswish")):
         case = case_for(k, batch, ic, oc, h, w, 0.85, False, ACTS[act], seed=ic + 3 * oc + h * w)
-        got = run_hip(case, capi.ALGO_IMAGE_MFMA)
+        got = run_hip(case, capi.ALGO_IMAGE_MFMA, tuning=capi.tuning(image_kernel=IMAGE_KERNELS[image_kernel]))
         want = run_oracle(case, oracle_pack(case))
         assert_same(case, got, want, "image %s %s %s" % (kind, act, shape))
     if kind == "acc32":
@@ -134,9 +147,48 @@ def test_image_mfma_activations_and_structures(paired, out_int8, act):
     announce("image acts", paired, out_int8, act)
     kind = capi.KIND_INT8_INT8 if out_int8 else capi.KIND_INT8_FP32
     case = case_for(kind, 2, 128, 128, 14, 14, 0.8, paired, ACTS[act], seed=77)
-    got = run_hip(case, capi.ALGO_IMAGE_MFMA, force_semi=paired)
     want = run_oracle(case, oracle_pack(case, force_semi=paired))
-    assert_same(case, got, want, "image %s" % act)
+    for name, which in sorted(IMAGE_KERNELS.items()):
+        got = run_hip(case, capi.ALGO_IMAGE_MFMA, force_semi=paired, tuning=capi.tuning(image_kernel=which))
+        assert_same(case, got, want, "image %s %s" % (name, act))
+
+
+def test_image_mfma_transposing_kernel_extremes_and_surroundings():
+    """Largest magnitudes (accumulators of 512 x 127 x 127 of either sign), an
+    empty output row, channels of one parity only, and the bytes around the
+    output tensor stay untouched (the windows of a row class reach in front of
+    and behind the row; those lanes must not store)."""
+    import ctypes as C
+
+    import torch
+
+    announce("image transpose extremes")
+    tr = capi.tuning(image_kernel=capi.IMAGE_KERNEL_TRANSPOSE)
+    case = case_for(capi.KIND_INT8_ACC32, 3, 512, 128, 14, 14, 0.5, False, AP(), seed=21)
+    case.dense[7] = 0
+    case.dense[64:66] = 127
+    case.dense[66:68] = -127
+    case.dense[80, 0::2] = 0   # odd channels only
+    case.dense[81, 1::2] = 0   # even channels only
+    case.x[1] = -127
+    got = run_hip(case, capi.ALGO_IMAGE_MFMA, tuning=tr)
+    ref = np.einsum("mk,bkp->bmp", case.dense.astype(np.int64), case.x.reshape(3, 512, -1).astype(np.int64)).reshape(got.shape)
+    assert np.array_equal(got.astype(np.int64), ref)
+    assert np.all(got[:, 7] == 0)
+    for kind, dt in ((capi.KIND_INT8_FP32, torch.float32), (capi.KIND_INT8_INT8, torch.int8)):
+        c2 = case_for(kind, 3, 256, 256, 10, 10, 0.9, False, ACTS["relu"], seed=12)
+        kernel, _ = make_kernel(c2, capi.ALGO_IMAGE_MFMA, tuning=tr)
+        numel = 3 * 256 * 100
+        guard = 64
+        fill = 77
+        buf = torch.full((numel + 2 * guard,), fill, dtype=dt, device="cuda")
+        x = torch.from_numpy(c2.x).cuda()
+        esz = buf.element_size()
+        capi.check(capi.lib().pl_sparse_conv_run(kernel._handle, x.data_ptr(), buf.data_ptr() + guard * esz, 3, 100, C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        torch.cuda.synchronize()
+        host = buf.cpu().numpy()
+        assert (host[:guard] == fill).all() and (host[guard + numel:] == fill).all()
+        assert np.array_equal(host[guard:guard + numel].reshape(3, 256, 10, 10), run_oracle(c2, oracle_pack(c2)))
 
 
 def test_image_mfma_agrees_with_the_other_algorithms_and_no_bias():

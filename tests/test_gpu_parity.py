@@ -84,14 +84,13 @@ FEW_CHANNEL_SHAPES = [(3, 32, 64, 16, 16), (2, 64, 128, 12, 12), (2, 20, 32, 16,
 
 @pytest.mark.parametrize("kind", ["acc32", "fp32out", "int8out"])
 @pytest.mark.parametrize("shape", FEW_CHANNEL_SHAPES, ids=lambda s: "x".join(map(str, s)))
-def test_few_channel_tiles_bit_exact(shape, kind, monkeypatch):
+def test_few_channel_tiles_bit_exact(shape, kind):
     announce("few-channel", shape, kind)
-    monkeypatch.setenv("PL_SPARSE_CONV_MFMA_SUB_TILES", "2")
     k = {"acc32": capi.KIND_INT8_ACC32, "fp32out": capi.KIND_INT8_FP32, "int8out": capi.KIND_INT8_INT8}[kind]
     batch, ic, oc, h, w = shape
     for act in ("relu", "hswish"):
         case = small_case(k, batch, ic, oc, h, w, 0.6, False, AP() if kind == "acc32" else ACTS[act], seed=3 * ic + oc, output_scale=0.05 if kind == "int8out" else 1.0)
-        got = run_hip(case, capi.ALGO_BLOCK_MFMA)
+        got = run_hip(case, capi.ALGO_BLOCK_MFMA, tuning=capi.tuning(mfma_sub_tiles=capi.TUNE_ALWAYS))
         want = run_oracle(case, oracle_pack(case))
         assert_same(case, got, want, "few-channel %s %s %s" % (kind, act, shape))
 
@@ -102,13 +101,12 @@ def test_few_channel_tiles_bit_exact(shape, kind, monkeypatch):
 @pytest.mark.parametrize("kind", ["acc32", "fp32out", "int8out"])
 @pytest.mark.parametrize("tq", [32, 25, 13, 8])
 @pytest.mark.parametrize("shape", [(3, 512, 96, 14, 14), (2, 512, 160, 16, 16), (5, 512, 33, 7, 7)], ids=lambda s: "x".join(map(str, s)))
-def test_tile_widths_bit_exact(shape, tq, kind, monkeypatch):
+def test_tile_widths_bit_exact(shape, tq, kind):
     announce("tile-width", shape, tq, kind)
-    monkeypatch.setenv("PL_SPARSE_CONV_MFMA_TILE_QUADS", str(tq))
     k = {"acc32": capi.KIND_INT8_ACC32, "fp32out": capi.KIND_INT8_FP32, "int8out": capi.KIND_INT8_INT8}[kind]
     batch, ic, oc, h, w = shape
     case = small_case(k, batch, ic, oc, h, w, 0.85, False, AP() if kind == "acc32" else ACTS["relu"], seed=oc + tq, output_scale=0.1 if kind == "int8out" else 1.0)
-    got = run_hip(case, capi.ALGO_BLOCK_MFMA)
+    got = run_hip(case, capi.ALGO_BLOCK_MFMA, tuning=capi.tuning(mfma_tile_quads=tq))
     want = run_oracle(case, oracle_pack(case))
     assert_same(case, got, want, "tile-width %s %s tq=%d" % (kind, shape, tq))
 
@@ -162,21 +160,17 @@ CHUNKED_SHAPES = [(2, 64, 64, 4, 4), (1, 96, 48, 8, 6), (3, 130, 67, 4, 5), (1, 
 @pytest.mark.parametrize("act", ["none", "relu6", "hswish"])
 @pytest.mark.parametrize("shape", CHUNKED_SHAPES, ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
-def test_fp32_chunked_walk(shape, paired, act, monkeypatch):
+def test_fp32_chunked_walk(shape, paired, act):
     announce("fp32 chunked", shape, paired, act)
     batch, ic, oc, h, w = shape
     case = small_case(capi.KIND_FP32, batch, ic, oc, h, w, 0.75, paired, ACTS[act], seed=ic + 3 * oc)
     want = run_oracle(case, oracle_pack(case, force_semi=paired))
-    monkeypatch.setenv("PL_SPARSE_CONV_WALK_CHUNKED", "2")
-    got = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired)
+    got = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired, tuning=capi.tuning(walk_chunked=capi.TUNE_ALWAYS))
     assert_same(case, got, want, "fp32 chunked %s %s" % (act, shape))
     # four row groups per wavefront instead of eight: the same bits
-    monkeypatch.setenv("PL_SPARSE_CONV_CHUNK_WALK_GROUPS", "4")
-    assert np.array_equal(got, run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired))
-    monkeypatch.delenv("PL_SPARSE_CONV_CHUNK_WALK_GROUPS")
+    assert np.array_equal(got, run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired, tuning=capi.tuning(walk_chunked=capi.TUNE_ALWAYS, chunk_walk_groups=4)))
     # and the plain walk gives the same bits (same order of fused multiply-adds)
-    monkeypatch.setenv("PL_SPARSE_CONV_WALK_CHUNKED", "0")
-    plain = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired)
+    plain = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired, tuning=capi.tuning(walk_chunked=capi.TUNE_NEVER, walk_tiled=capi.TUNE_NEVER))
     assert np.array_equal(got, plain)
 
 
@@ -192,26 +186,21 @@ TILED_SHAPES = [(2, 64, 8, 4, 4), (1, 96, 48, 8, 6), (3, 130, 67, 4, 5), (1, 264
 @pytest.mark.parametrize("act", ["none", "relu6", "hswish"])
 @pytest.mark.parametrize("shape", TILED_SHAPES, ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
-def test_fp32_tiled_walk(shape, paired, act, monkeypatch):
+def test_fp32_tiled_walk(shape, paired, act):
     announce("fp32 tiled", shape, paired, act)
     batch, ic, oc, h, w = shape
     sparsity = 0.3 if ic == 256 else 0.75  # the dense case: lists of ~180 entries, several LDS pieces per stream
     case = small_case(capi.KIND_FP32, batch, ic, oc, h, w, sparsity, paired, ACTS[act], seed=ic + 3 * oc)
     want = run_oracle(case, oracle_pack(case, force_semi=paired))
-    monkeypatch.setenv("PL_SPARSE_CONV_WALK_TILED", "2")
-    got = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired)
+    got = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired, tuning=capi.tuning(walk_tiled=capi.TUNE_ALWAYS))
     assert_same(case, got, want, "fp32 tiled %s %s" % (act, shape))
     # the row groups dealt differently between the tile's own workgroup and the
     # workgroups of the CUs without a tile (none, 3/16, half of the work; the
     # run above took the share the library computes): the same bits
-    for split in ("0", "3", "8"):
-        monkeypatch.setenv("PL_SPARSE_CONV_WALK_SPLIT", split)
-        assert np.array_equal(got, run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired)), "split %s" % split
-    monkeypatch.delenv("PL_SPARSE_CONV_WALK_SPLIT")
+    for split in (0, 3, 8):  # the field holds 1 + sixteenths
+        assert np.array_equal(got, run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired, tuning=capi.tuning(walk_tiled=capi.TUNE_ALWAYS, walk_split=1 + split))), "split %s" % split
     # and the plain walk gives the same bits (same order of fused multiply-adds)
-    monkeypatch.setenv("PL_SPARSE_CONV_WALK_TILED", "0")
-    monkeypatch.setenv("PL_SPARSE_CONV_WALK_CHUNKED", "0")
-    plain = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired)
+    plain = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired, tuning=capi.tuning(walk_tiled=capi.TUNE_NEVER, walk_chunked=capi.TUNE_NEVER))
     assert np.array_equal(got, plain)
 
 
@@ -271,6 +260,28 @@ def test_set_epilogue_replaces_scales():
     case.weight_scale = new_ws
     assert_same(case, run_hip(case, kernel=kernel), run_oracle(case), "after set_epilogue")
     del C
+
+
+@pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
+def test_set_epilogue_replaces_the_bias_of_every_fp32_walk(paired):
+    """The walk with the tile and the lists in LDS starts its accumulators from
+    the bias carried in its list headers: a new bias must reach those too, and
+    a handle prepared without a bias must take one."""
+    announce("set_epilogue bias", paired)
+    for had_bias in (True, False):
+        case = small_case(capi.KIND_FP32, 3, 130, 67, 4, 5, 0.75, paired, ACTS["relu6"], seed=31)
+        new_bias = np.linspace(-0.7, 0.9, 67).astype(np.float32)
+        if not had_bias:
+            case.bias = None
+        outs = []
+        for tune in (capi.tuning(walk_tiled=capi.TUNE_ALWAYS), capi.tuning(walk_tiled=capi.TUNE_NEVER, walk_chunked=capi.TUNE_NEVER), capi.tuning(walk_tiled=capi.TUNE_NEVER, walk_chunked=capi.TUNE_ALWAYS)):
+            kernel, _ = make_kernel(case, capi.ALGO_ROW_WALK, force_semi=paired, tuning=tune)
+            capi.check(capi.lib().pl_sparse_conv_set_epilogue(kernel._handle, None, new_bias.ctypes.data, None))
+            outs.append(run_hip(case, kernel=kernel))
+        case.bias = new_bias
+        want = run_oracle(case, oracle_pack(case, force_semi=paired))
+        assert_same(case, outs[0], want, "tile walk after set_epilogue(bias)")
+        assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
 
 
 @pytest.mark.parametrize("quirks", [True, False], ids=["reference_quirks", "scaled_once"])

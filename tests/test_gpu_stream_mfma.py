@@ -14,6 +14,9 @@ from helpers import capi, workloads, pla, make_kernel, run_hip, run_oracle, orac
 
 pytestmark = pytest.mark.gpu
 
+STREAM_ALWAYS = capi.tuning(mfma_stream=capi.TUNE_ALWAYS)
+STREAM_NEVER = capi.tuning(mfma_stream=capi.TUNE_NEVER)
+
 AP = pla.ActivationParam
 ACTS = {
     "none": AP(),
@@ -41,39 +44,35 @@ SHAPES = [
 
 @pytest.mark.parametrize("out_int8", [False, True], ids=["fp32out", "int8out"])
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
-def test_stream_mfma_bit_exact(shape, out_int8, monkeypatch):
+def test_stream_mfma_bit_exact(shape, out_int8):
     announce("stream", shape, out_int8)
     batch, ic, oc, h, w = shape
     for act in ("leaky", "hswish"):
         case = case_for(out_int8, batch, ic, oc, h, w, 0.8, False, ACTS[act], seed=ic + oc + h)
         want = run_oracle(case, oracle_pack(case))
-        monkeypatch.setenv("PL_SPARSE_CONV_MFMA_STREAM", "2")
-        got = run_hip(case, capi.ALGO_BLOCK_MFMA)
+        got = run_hip(case, capi.ALGO_BLOCK_MFMA, tuning=STREAM_ALWAYS)
         assert_same(case, got, want, "stream %s %s" % (act, shape))
-        monkeypatch.setenv("PL_SPARSE_CONV_MFMA_STREAM", "0")
-        assert np.array_equal(got, run_hip(case, capi.ALGO_BLOCK_MFMA))
+        assert np.array_equal(got, run_hip(case, capi.ALGO_BLOCK_MFMA, tuning=STREAM_NEVER))
 
 
 @pytest.mark.parametrize("act", sorted(ACTS))
 @pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
-def test_stream_mfma_activations_and_structures(paired, act, monkeypatch):
+def test_stream_mfma_activations_and_structures(paired, act):
     announce("stream acts", paired, act)
-    monkeypatch.setenv("PL_SPARSE_CONV_MFMA_STREAM", "2")
     for out_int8 in (False, True):
         case = case_for(out_int8, 2, 128, 128, 16, 12, 0.75, paired, ACTS[act], seed=11)
-        got = run_hip(case, capi.ALGO_BLOCK_MFMA, force_semi=paired)
+        got = run_hip(case, capi.ALGO_BLOCK_MFMA, force_semi=paired, tuning=STREAM_ALWAYS)
         assert_same(case, got, run_oracle(case, oracle_pack(case, force_semi=paired)), "stream %s" % act)
 
 
-def test_stream_mfma_absent_blocks_and_no_bias(monkeypatch):
+def test_stream_mfma_absent_blocks_and_no_bias():
     announce("stream blocks")
-    monkeypatch.setenv("PL_SPARSE_CONV_MFMA_STREAM", "2")
     case = case_for(True, 3, 256, 256, 16, 16, 0.5, False, ACTS["relu6"], seed=3)
     case.dense[32:64, :] = 0        # a row block without weights
     case.dense[:, 64:128] = 0       # two k-steps no row uses
     case.dense[128:160, 0:224] = 0  # a row block with one k-step
     case.bias = None
-    got = run_hip(case, capi.ALGO_BLOCK_MFMA)
+    got = run_hip(case, capi.ALGO_BLOCK_MFMA, tuning=STREAM_ALWAYS)
     assert_same(case, got, run_oracle(case, oracle_pack(case)), "absent blocks")
     kernel, _ = make_kernel(case, capi.ALGO_BLOCK_MFMA)
     info = kernel.info()
@@ -85,14 +84,8 @@ def test_auto_takes_the_streaming_kernel_on_the_large_semi_structured_config_and
     kernel with streaming switched off (the full-size parity run is in
     test_gpu_full_size.py)."""
     announce("stream c4-like")
-    import os
-
     case = workloads.config4(batch=16)
     got = run_hip(case, capi.ALGO_AUTO)
-    os.environ["PL_SPARSE_CONV_MFMA_STREAM"] = "0"
-    try:
-        ref = run_hip(case, capi.ALGO_AUTO)
-    finally:
-        del os.environ["PL_SPARSE_CONV_MFMA_STREAM"]
+    ref = run_hip(case, capi.ALGO_AUTO, tuning=STREAM_NEVER)
     assert np.array_equal(got, ref)
     assert_same(case, got[:2], run_oracle(case, oracle_pack(case), x=case.x[:2]), "c4-like")
