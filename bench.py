@@ -38,9 +38,10 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib", "mobilenet", "density-sweep", "floors"])
+    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib", "mobilenet", "density-sweep", "floors", "store-shapes"])
     ap.add_argument("--algo", default="auto", choices=["auto", "walk", "mfma", "image"])
     ap.add_argument("--image-kernel", default="rule", choices=["rule", "regroup", "transpose"], help="which image MFMA kernel a handle uses where both apply (pl_sparse_conv_tuning.image_kernel)")
+    ap.add_argument("--image-regroup", default="rule", choices=["rule", "valu"], help="regrouping image kernel: by transposing LDS reads where that exists (rule) or by the vector ALU everywhere (pl_sparse_conv_tuning.image_tr_regroup)")
     ap.add_argument("--fp16", action="store_true", help="run an fp32 configuration (c1, c2) through the half-precision kernel")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cache-resident", action="store_true", help="reuse one buffer set (reported, never the headline)")
@@ -274,10 +275,72 @@ def run_density_sweep(args):
     return 0
 
 
+def load_probes():
+    """bench_probes/libpl_probe.so, built on first use (hipcc) when the tree does not hold it yet."""
+    import importlib
+
+    here = os.path.dirname(os.path.abspath(__file__))
+    if here not in sys.path:
+        sys.path.insert(0, here)
+    bp = importlib.import_module("bench_probes.build_probes")
+    if not os.path.exists(bp.LIB_PATH):
+        bp.build()
+    return C.CDLL(bp.LIB_PATH)
+
+
+def run_store_shapes(args):
+    """How the shape of a store instruction decides the write rate of the metric shape's fp32 output
+    (64 x 512 x 14 x 14 floats, 25.7 MB; rows of 784 bytes start 16 bytes further into a 64-byte sector
+    each): store-only kernels on the image kernels' grid and row assignment, rotating buffers."""
+    import torch
+
+    P = load_probes()
+    P.pl_probe_store_shape.restype = C.c_int
+    P.pl_probe_store_shape.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_float)]
+    out_bytes = 64 * 512 * 196 * 4
+    n_sets = int(LLC_BYTES * 1.25 // out_bytes) + 1
+    outs = [torch.empty(out_bytes // 4, dtype=torch.float32, device="cuda") for _ in range(n_sets)]
+    op = (C.c_void_p * n_sets)(*[t.data_ptr() for t in outs])
+    stream = torch.cuda.current_stream().cuda_stream
+    steps = max(200, args.steps)
+
+    def run(mode, pol, n):
+        ms = C.c_float(0.0)
+        rc = P.pl_probe_store_shape(mode, pol, op, n_sets, n, C.c_void_p(stream), C.byref(ms))
+        if rc != 0:
+            raise RuntimeError("pl_probe_store_shape(%d, %d) failed with HIP error %d" % (mode, pol, rc))
+        return ms.value * 1e3 / n
+
+    settle(lambda: run(1, 0, 200))
+    shapes = ["16 rows x 64 B", "4 rows x 256 B on sector boundaries", "8 rows x 128 B lines"]
+    policies = ["sc1 nt", "nt", "plain"]
+    rows = {}
+    for rep_i in range(3):
+        for m, shape in enumerate(shapes):
+            for pol, pname in enumerate(policies):
+                run(m, pol, 100)
+                key = "%s, %s" % (shape, pname)
+                rows[key] = round(min(run(m, pol, steps), rows.get(key, 1e9)), 2)
+    # every pattern writes every float of a workgroup's rows exactly once
+    for m in range(3):
+        outs[0].fill_(float("nan"))
+        run(m, 2, 1)
+        torch.cuda.synchronize()
+        assert not bool(torch.isnan(outs[0]).any()), "store pattern %d leaves floats unwritten" % m
+    print(json.dumps({
+        "metric": "store-only kernels over the metric shape's fp32 output: us per launch",
+        "unit": "us", "n_gpus": 1, "steps": steps, "data": "synthetic",
+        "config": {"workload": "store_shapes_c3_output", "output_MB": out_bytes / 1e6, "buffer_sets": n_sets, "grid": "256 workgroups x 512 threads"},
+        "us_per_launch": rows,
+        "TBs": {k: round(out_bytes / (v * 1e-6) / 1e12, 2) for k, v in rows.items()},
+    }))
+    return 0
+
+
 def run_floors(args):
     """What the device needs for the launch and the memory traffic of the
     metric shape (64 x 512 -> 512 @14x14, int8 -> fp32) without the
-    arithmetic: the probes of paddle-lite_amd/csrc/probe_kernels.hip on the
+    arithmetic: the probes of bench_probes/floor_probes.hip on the
     image kernel's grid and rotating buffers, next to the image kernel itself.
     Not the headline metric: printed as its own JSON line."""
     import torch
@@ -285,12 +348,7 @@ def run_floors(args):
     import helpers
 
     capi, wl = helpers.capi, helpers.workloads
-    here = os.path.dirname(os.path.abspath(__file__))
-    path = os.path.join(here, "paddle-lite_amd", "lib", "libpl_probe.so")
-    if not os.path.exists(path):
-        sys.stderr.write("the floor probes are not built: run __graft_entry__.build()\n")
-        return 2
-    P = C.CDLL(path)
+    P = load_probes()
     P.pl_probe_floor.restype = C.c_int
     P.pl_probe_floor.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_float)]
     case = wl.CONFIGS["c3"]()
@@ -320,7 +378,7 @@ def run_floors(args):
         return ms.value * 1e3 / n
 
     settle(lambda: image(200))
-    names = ["empty", "write", "stream", "load", "load_write", "load_transpose_write"]
+    names = ["empty", "write", "stream", "load", "load_write", "load_transpose_write", "load_transposing_reads_write"]
     rows = {}
     for rep_i in range(3):  # three rounds, the best of each
         for k, name in enumerate(names):
@@ -569,6 +627,8 @@ def main():
         return run_density_sweep(args)
     if args.config == "floors":
         return run_floors(args)
+    if args.config == "store-shapes":
+        return run_store_shapes(args)
     if args.config == "c5":
         return run_c5(args)
     if args.config == "calib":
@@ -585,7 +645,8 @@ def main():
         case.name += "_fp16"
         args.no_cpu_baseline = True  # the CPU baselines are fp32 / int8 paths
     algo = {"auto": capi.ALGO_AUTO, "walk": capi.ALGO_ROW_WALK, "mfma": capi.ALGO_BLOCK_MFMA, "image": capi.ALGO_IMAGE_MFMA}[args.algo]
-    tune = capi.tuning(image_kernel={"rule": 0, "regroup": capi.IMAGE_KERNEL_REGROUP, "transpose": capi.IMAGE_KERNEL_TRANSPOSE}[args.image_kernel])
+    tune = capi.tuning(image_kernel={"rule": 0, "regroup": capi.IMAGE_KERNEL_REGROUP, "transpose": capi.IMAGE_KERNEL_TRANSPOSE}[args.image_kernel],
+                       image_tr_regroup=capi.TUNE_NEVER if args.image_regroup == "valu" else capi.TUNE_RULE)
     kernel, weights = helpers.make_kernel(case, algo=algo, tuning=tune)
     info = kernel.info()
     ops = case.algorithmic_ops()
@@ -666,12 +727,15 @@ def main():
         per_algo = {algo_name: round(kernel_ms * 1e3, 3)}
         others = sorted(algo_names.items())
         if algo_name == "image_mfma":
-            others.append((capi.ALGO_IMAGE_MFMA, "image_mfma_regroup"))  # the image kernel that regroups in LDS
+            others.append((capi.ALGO_IMAGE_MFMA, "image_mfma_valu_regroup"))  # the image kernel with the regrouping done by the vector ALU
+            others.append((capi.ALGO_IMAGE_MFMA, "image_mfma_transposing_reads"))  # the image kernel that never regroups
         for a, name in others:
             if name in per_algo:
                 continue
             try:
-                other, _ = helpers.make_kernel(case, algo=a, tuning=capi.tuning(image_kernel=capi.IMAGE_KERNEL_REGROUP) if name == "image_mfma_regroup" else None)
+                other_tune = {"image_mfma_valu_regroup": capi.tuning(image_kernel=capi.IMAGE_KERNEL_REGROUP, image_tr_regroup=capi.TUNE_NEVER),
+                              "image_mfma_transposing_reads": capi.tuning(image_kernel=capi.IMAGE_KERNEL_TRANSPOSE)}.get(name)
+                other, _ = helpers.make_kernel(case, algo=a, tuning=other_tune)
             except capi.SparseConvError:
                 continue  # this shape is outside the algorithm's range
             if L.pl_sparse_conv_run_sequence(other._handle, xp, op, n_sets, case.batch, case.im_size, 50, C.c_void_p(stream), None) < 0:

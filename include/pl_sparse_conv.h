@@ -122,7 +122,11 @@ typedef struct pl_sparse_conv_tuning {
   int32_t walk_tile;         /* plain walk: positions per tile (power of two)  */
   int32_t walk_threads;      /* plain walk: threads per workgroup              */
   int32_t walk_slices;       /* plain walk: row slices                         */
-  int32_t reserved[2];       /* must be 0                                      */
+  int32_t image_tr_regroup;  /* (switch) regrouping image kernel: the regrouping
+                                done by transposing LDS reads where that exists
+                                (ic = 512, 14 x 14 maps); NEVER = by the vector
+                                ALU everywhere                                 */
+  int32_t reserved;          /* must be 0                                      */
 } pl_sparse_conv_tuning;
 
 /* Everything PrepareForRun() knows.  All pointers are HOST pointers and are

@@ -86,22 +86,6 @@ def build_library(verbose=False):
     return LIB_PATH
 
 
-PROBE_LIB_PATH = os.path.join(LIB_DIR, "libpl_probe.so")
-
-
-def build_probe(verbose=False):
-    """The floor probes of bench.py --config floors (launch and memory floors
-    of the metric shape): a library of their own, nothing of the operator."""
-    os.makedirs(LIB_DIR, exist_ok=True)
-    cmd = [hipcc()] + HIPCC_FLAGS + ["-x", "hip", "-shared", os.path.join(CSRC, "probe_kernels.hip"), "-o", PROBE_LIB_PATH]
-    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    if res.returncode != 0:
-        raise RuntimeError("hipcc failed: %s\n%s" % (" ".join(cmd), res.stdout))
-    return PROBE_LIB_PATH
-
-
 LITE_DIR = os.path.join(PKG, "lite")
 LITE_LIB_PATH = os.path.join(LIB_DIR, "libpl_lite_hip.so")
 ROOT = os.path.dirname(PKG)

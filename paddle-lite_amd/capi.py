@@ -65,7 +65,8 @@ class Tuning(C.Structure):
         ("walk_tile", C.c_int32),
         ("walk_threads", C.c_int32),
         ("walk_slices", C.c_int32),
-        ("reserved", C.c_int32 * 2),
+        ("image_tr_regroup", C.c_int32),
+        ("reserved", C.c_int32),
     ]
 
 

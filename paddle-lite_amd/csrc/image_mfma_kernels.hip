@@ -172,7 +172,18 @@ __device__ __forceinline__ void Tail(const uint4* __restrict__ xt, int kgs, int 
 // reads become immediates (64 x 512 -> 512 @14x14: 10.8 -> 10.4 us); the image
 // size in bytes stays a run-time value on purpose (as a constant it changed the
 // schedule of the direct loads and the stores and cost more than it saved).
-template <int KS, int OUT, int QPI>
+//
+// TRG (512 channels, 14 x 14 maps): the regrouping is done by the LDS itself.  ds_read_b64_tr_b8 hands
+// lane j of a group of 16 lanes byte j % 8 of the eight bytes that lane 2 b + j / 8 of the group addressed, as
+// its byte b: eight channels of one position per lane when the 16 lanes address eight channel rows (two
+// runs of eight positions each).  Two such reads are one operand cell, which is then written where the
+// windows expect it; no vector ALU transposes (64 x 512 -> 512 @14x14: 9.7 -> see the measurements).  The
+// read ignores the low three address bits and rows of 196 bytes start 8-byte aligned only for even
+// channels, so a cell holds channels of one parity (for odd channels the aligned runs cover positions
+// 8 u + 4 .. 8 u + 11), and channels of a cell are four apart so that the 16 rows of a half wavefront fall
+// into different banks: channel 64 ks + 4 (8 (g % 2) + b % 8) + 2 (b / 8) + g / 2 is byte b of cell group g
+// of k-step ks.  The weight tiles come in the same order (the order inside an integer dot product is free).
+template <int KS, int OUT, int QPI, bool TRG = false>
 __global__ void __launch_bounds__(512) ImageMfmaKernel(const ImageMfmaParams p) {
   extern __shared__ uint4 lds_raw[];
   // shifted windows read up to three cells in front of a row of cells
@@ -191,15 +202,27 @@ __global__ void __launch_bounds__(512) ImageMfmaKernel(const ImageMfmaParams p) 
   const int8_t* ximg = p.x + (size_t)n * p.K * hw;
   char* lbase = reinterpret_cast<char*>(xt);
   const int blk_bytes = 16 * hw;
-#pragma unroll
-  for (int u = 0; u < BPW; ++u) {
-    const int kg = wave * BPW + u;
-    const int8_t* src = ximg + (size_t)kg * blk_bytes + lane * 16;
-    char* dst = lbase + kg * (kgs * 16);
-    for (int t = 0; t < p.dma_full; ++t)
+  if (TRG) {
+    // the wavefront's 64 channel rows as they lie in memory, at the start of the region of its four cell groups
+    const int bytes = BPW * blk_bytes;
+    const int8_t* src = ximg + (size_t)wave * bytes + lane * 16;
+    char* dst = lbase + wave * BPW * (kgs * 16);
+    const int full = bytes >> 10, rem_lanes = (bytes & 1023) >> 4;
+    for (int t = 0; t < full; ++t)
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + t * 1024), (__attribute__((address_space(3))) void*)(dst + t * 1024), 16, 0, 0);
-    if (lane < p.dma_rem_lanes)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + p.dma_full * 1024), (__attribute__((address_space(3))) void*)(dst + p.dma_full * 1024), 16, 0, 0);
+    if (lane < rem_lanes)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + full * 1024), (__attribute__((address_space(3))) void*)(dst + full * 1024), 16, 0, 0);
+  } else {
+#pragma unroll
+    for (int u = 0; u < BPW; ++u) {
+      const int kg = wave * BPW + u;
+      const int8_t* src = ximg + (size_t)kg * blk_bytes + lane * 16;
+      char* dst = lbase + kg * (kgs * 16);
+      for (int t = 0; t < p.dma_full; ++t)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + t * 1024), (__attribute__((address_space(3))) void*)(dst + t * 1024), 16, 0, 0);
+      if (lane < p.dma_rem_lanes)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + p.dma_full * 1024), (__attribute__((address_space(3))) void*)(dst + p.dma_full * 1024), 16, 0, 0);
+    }
   }
   // Every channel group of this wavefront has landed.  (The builtin, not an assembly statement: the
   // compiler then knows that no direct load is in flight any more and puts no wait of its own in front
@@ -229,6 +252,29 @@ __global__ void __launch_bounds__(512) ImageMfmaKernel(const ImageMfmaParams p) 
     rw.sct[j] = OUT == kOutAcc32 ? 0.f : p.scale[row0 + 4 * (16 * j + ln.n)];
     rw.bit[j] = OUT == kOutAcc32 ? 0.f : p.bias[row0 + 4 * (16 * j + ln.n)];
   }
+  if (TRG) {
+    static_assert(!TRG || (KS == 8 && QPI > 0 && (QPI & 1)), "regrouping by transposing reads: 512 channels, rows of 4 (mod 8) bytes");
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    auto reg = (__attribute__((address_space(3))) char*)lbase + wave * BPW * (kgs * 16);
+    const int g = lane >> 4, s16 = lane & 15, par = g >> 1;
+    // the lane addresses channel row 4 (8 (g % 2) + s16 / 2) + g / 2 (+ 2 for the second read), run s16 % 2
+    const int rbase = (4 * (8 * (g & 1) + (s16 >> 1)) + par) * hw + 8 * (s16 & 1) - 4 * par;
+    constexpr int NWIN = (4 * QPI + 3) / 16 + 1;  // windows of 16 positions; those of odd channels start at -4
+    v2i rr[NWIN][2];
+#pragma unroll
+    for (int i = 0; i < NWIN; ++i)
+#pragma unroll
+      for (int r2 = 0; r2 < 2; ++r2) rr[i][r2] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<__attribute__((address_space(3))) v2i*>(reg + rbase + 16 * i + 2 * r2 * hw));
+    // every lane has read before any lane overwrites
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_sched_barrier(0);
+    auto cells = reinterpret_cast<__attribute__((address_space(3))) v4i*>(reg + g * (kgs * 16));
+#pragma unroll
+    for (int i = 0; i < NWIN; ++i) {
+      const int pos = 16 * i - 4 * par + s16;
+      if (pos >= 0 && pos < 4 * QPI) cells[(pos & 3) * QPI + (pos >> 2)] = v4i{rr[i][0].x, rr[i][0].y, rr[i][1].x, rr[i][1].y};
+    }
+  } else {
   // in place: 16 dwords (16 channels x 4 positions) per quad -> 4 cells.  The dwords of all of the
   // wavefront's channel groups are read first (one wait instead of one per group), then every group is
   // transposed and written back; a group is touched by this wavefront only.
@@ -270,6 +316,7 @@ __global__ void __launch_bounds__(512) ImageMfmaKernel(const ImageMfmaParams p) 
         cells[c * qpi] = cell;
       }
     }
+  }
   }
   __syncthreads();
 
@@ -485,6 +532,7 @@ hipError_t ByKs(const ImageMfmaParams& q, dim3 grid, size_t lds, hipStream_t s) 
       case 4:
         return LaunchWithLds(ImageMfmaKernel<4, OUT, 49>, grid, block, lds, s, q);
       case 8:
+        if (q.tr_regroup) return LaunchWithLds(ImageMfmaKernel<8, OUT, 49, true>, grid, block, lds, s, q);
         return LaunchWithLds(ImageMfmaKernel<8, OUT, 49>, grid, block, lds, s, q);
       default:
         return hipErrorInvalidValue;
@@ -513,8 +561,11 @@ bool ImageMfmaFits(int M, int K, int hw) {
   return 256 + (size_t)(K / 16) * kgs * 16 <= (size_t)kMaxLdsBytes;
 }
 
+bool ImageMfmaRegroupsByTransposingReads(int K, int hw) { return K == 512 && hw == 196; }
+
 hipError_t LaunchImageMfma(int out_kind, const ImageMfmaParams& p, hipStream_t stream) {
   if (p.batch <= 0) return hipSuccess;
+  if (p.tr_regroup && !ImageMfmaRegroupsByTransposingReads(p.K, p.hw)) return hipErrorInvalidValue;
   if (!ImageMfmaFits(p.M, p.K, p.hw)) return hipErrorInvalidValue;
   if (reinterpret_cast<uintptr_t>(p.x) % 16 != 0 || reinterpret_cast<uintptr_t>(p.out) % 16 != 0) return hipErrorInvalidValue;
   ImageMfmaParams q = p;

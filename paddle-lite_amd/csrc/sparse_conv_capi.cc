@@ -173,6 +173,8 @@ struct pl_sparse_conv_handle {
   int mfma_sub_tiles = 1;   // several tiles per workgroup for <= 64 input channels: 0 never, 1 when enough workgroups remain, 2 always
   // image MFMA (dense 16x64 tiles, rows of a tile four apart)
   DevBuf wtiles;
+  DevBuf wtiles_rg;      // the same tiles in the channel order of the regrouping by transposing LDS reads (ic = 512)
+  bool image_tr_regroup = true;
   DevBuf wtiles_tr;      // the same tiles in the channel order of the kernel with transposing LDS reads
   int image_kernel = 0;  // 0 by rule, 1 regrouping kernel, 2 transposing-read kernel
   // int8 handles prepared with PL_ALGO_AUTO hold several forms and choose per call
@@ -185,7 +187,7 @@ struct pl_sparse_conv_handle {
   int padded_rows = 0;
 
   int64_t DeviceBytes() const {
-    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + cw_desc.bytes + cw_idx.bytes + cw_wts.bytes + hw_kidx.bytes + hw_wts.bytes + hw_bias.bytes + wblocks.bytes + kmask.bytes + wtiles.bytes + wtiles_tr.bytes + tw_stream.bytes + tw_first.bytes + tw_desc.bytes + scale.bytes + bias.bytes);
+    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + cw_desc.bytes + cw_idx.bytes + cw_wts.bytes + hw_kidx.bytes + hw_wts.bytes + hw_bias.bytes + wblocks.bytes + kmask.bytes + wtiles.bytes + wtiles_rg.bytes + wtiles_tr.bytes + tw_stream.bytes + tw_first.bytes + tw_desc.bytes + scale.bytes + bias.bytes);
   }
 };
 
@@ -541,6 +543,34 @@ int BuildImageMfma(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
   return PL_OK;
 }
 
+// The same tiles for the regrouping image kernel where it regroups by transposing LDS reads: byte b of
+// lane group g of k-step ks is channel 64 ks + 4 (8 (g % 2) + b % 8) + 2 (b / 8) + g / 2 (image_mfma_kernels.hip).
+int BuildImageMfmaTrRegroup(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
+  const int kss = L.ic / 64;
+  std::vector<int8_t> tiles(static_cast<size_t>(L.oc) * L.ic, 0);
+  auto put = [&](int row, uint32_t c, uint32_t wbits) {
+    const int8_t w = static_cast<int8_t>(wbits & 0xffu);
+    if (w == 0) return;
+    const int rg = row / 128, rl = row % 128;
+    const int rho = rl & 3, m32 = rl >> 2;  // row = rg * 128 + rho + 4 * (16 j + m)
+    const int j = m32 >> 4, m = m32 & 15;
+    const int ks = static_cast<int>(c >> 6), cc = static_cast<int>(c & 63u);
+    const int par = cc & 1, r = (cc >> 1) & 1, t = cc >> 2;
+    const int g = 2 * par + (t >> 3), b = 8 * r + (t & 7);
+    const int lane = m + 16 * g;
+    tiles[((((static_cast<size_t>(rg) * 4 + rho) * 2 + j) * kss + ks) * 64 + lane) * 16 + b] = w;
+  };
+  for (const pl::RowGroup& g : L.groups) {
+    for (uint32_t j = 0; j < g.count; ++j) {
+      put(g.row0, L.ic_index[g.first + j], L.w0[g.first + j]);
+      if (g.nrows == 2) put(g.row0 + 1, L.ic_index[g.first + j], L.w1[g.first + j]);
+    }
+  }
+  const hipError_t e = h->wtiles_rg.Upload(tiles.data(), tiles.size());
+  if (e != hipSuccess) return FailHip(e, "uploading the weight tiles");
+  return PL_OK;
+}
+
 // The same tiles for the image kernel with transposing LDS reads.  That kernel
 // takes the channels of a k-step in the order its reads deliver them: a step
 // holds the 64 channels of one parity out of 128, and byte b of lane group g
@@ -666,8 +696,8 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
     return Fail(PL_ERR_BAD_ARG, "pl_sparse_conv_desc size mismatch (%u vs %zu)", desc->struct_size, sizeof(pl_sparse_conv_desc));
   pl_sparse_conv_tuning tune{};
   if (desc->struct_size == sizeof(pl_sparse_conv_desc)) tune = desc->tuning;
-  if (tune.reserved[0] != 0 || tune.reserved[1] != 0) return Fail(PL_ERR_BAD_ARG, "pl_sparse_conv_tuning.reserved must be 0");
-  for (int32_t sw : {tune.mfma_stream, tune.mfma_sub_tiles, tune.walk_tiled, tune.walk_chunked})
+  if (tune.reserved != 0) return Fail(PL_ERR_BAD_ARG, "pl_sparse_conv_tuning.reserved must be 0");
+  for (int32_t sw : {tune.mfma_stream, tune.mfma_sub_tiles, tune.walk_tiled, tune.walk_chunked, tune.image_tr_regroup})
     if (sw < PL_TUNE_RULE || sw > PL_TUNE_ALWAYS) return Fail(PL_ERR_BAD_ARG, "a tuning switch is not PL_TUNE_RULE, PL_TUNE_NEVER or PL_TUNE_ALWAYS");
   if (tune.image_kernel < 0 || tune.image_kernel > 2) return Fail(PL_ERR_BAD_ARG, "tuning.image_kernel must be 0, 1 or 2");
   if (desc->kind < PL_KIND_FP32 || desc->kind > PL_KIND_FP16) return Fail(PL_ERR_BAD_ARG, "unknown kind %d", desc->kind);
@@ -718,6 +748,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   if (tune.wg_slots > 0) h->wg_slots = tune.wg_slots;
   if (tune.image_min_items > 0) h->image_min_items = tune.image_min_items;
   h->image_kernel = tune.image_kernel;
+  h->image_tr_regroup = tune.image_tr_regroup != PL_TUNE_NEVER;
   h->walk_tile = tune.walk_tile;
   h->walk_threads = tune.walk_threads;
   h->walk_slices = tune.walk_slices;
@@ -776,6 +807,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   if (rc == PL_OK && algo == PL_ALGO_BLOCK_MFMA) rc = BuildBlockMfma(L, h);
   if (rc == PL_OK && (algo == PL_ALGO_IMAGE_MFMA || (h->auto_int8 && (pl::ImageMfmaFits(desc->oc, desc->ic, 16) || pl::ImageMfmaFits(desc->oc, desc->ic, 49))))) rc = BuildImageMfma(L, h);
   if (rc == PL_OK && h->wtiles.ptr && pl::ImageTrMfmaFits(desc->oc, desc->ic, 20)) rc = BuildImageTrMfma(L, h);
+  if (rc == PL_OK && h->wtiles.ptr && pl::ImageMfmaRegroupsByTransposingReads(desc->ic, 196)) rc = BuildImageMfmaTrRegroup(L, h);
   if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8) rc = BuildChunkWalk(L, h);
   if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8 && !half) rc = BuildTileWalk(L, desc->bias, h);
   if (rc == PL_OK) {
@@ -888,7 +920,8 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
       p.wtiles = h->wtiles_tr.ptr;
       e = pl::LaunchImageTrMfma(OutKind(h->kind), p, s);
     } else {
-      p.wtiles = h->wtiles.ptr;
+      p.tr_regroup = h->image_tr_regroup && h->wtiles_rg.ptr != nullptr && pl::ImageMfmaRegroupsByTransposingReads(h->ic, im_size);
+      p.wtiles = p.tr_regroup ? h->wtiles_rg.ptr : h->wtiles.ptr;
       e = pl::LaunchImageMfma(OutKind(h->kind), p, s);
     }
   } else if (h->algo == PL_ALGO_BLOCK_MFMA) {

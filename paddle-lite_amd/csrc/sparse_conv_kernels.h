@@ -257,12 +257,17 @@ struct ImageMfmaParams {
   int items, per_xcd;  // work items (image, row group) in all and per XCD
   int dma_full, dma_rem_lanes;  // 1 KB pieces of a channel group and the lanes of the last, partial piece
   int align;           // fp32 / int32 output: windows shifted onto 64-byte sector boundaries
+  // set by the caller of LaunchImageMfma: wtiles holds the tiles in the channel order of the regrouping by
+  // transposing LDS reads (byte b of lane group g of k-step ks = channel 64 ks + 4 (8 (g % 2) + b % 8) + 2 (b / 8) + g / 2);
+  // only where ImageMfmaRegroupsByTransposingReads(K, hw)
+  int tr_regroup;
 };
 
 // M a multiple of 128, K = 128, 256 or 512, hw a multiple of 4 in [16, 256]
 // and the image's cells within the LDS of a CU; or 7 x 7 maps (hw = 49) with
 // K = 256, 512 or 1024 (two images per workgroup).
 bool ImageMfmaFits(int M, int K, int hw);
+bool ImageMfmaRegroupsByTransposingReads(int K, int hw);
 // Needs ImageMfmaFits and 16-byte aligned x / out.
 hipError_t LaunchImageMfma(int out_kind, const ImageMfmaParams& p, hipStream_t stream);
 

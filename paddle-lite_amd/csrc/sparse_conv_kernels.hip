@@ -44,11 +44,6 @@
 #endif
 #define PL_PART_MFMA_ANY (PL_PART_MFMA_F32 || PL_PART_MFMA_I8 || PL_PART_MFMA_ACC32)
 
-// Phase marks for tuning builds; compiled out of the library.
-#ifndef PL_PHASE_MARK
-#define PL_PHASE_MARK(i)
-#endif
-
 namespace pl {
 namespace {
 
@@ -296,12 +291,8 @@ __device__ __forceinline__ void RowWalkBody(const WalkParams& p, uint32_t* tile)
   const int slice = (blockIdx.x >> 3) % p.slices;
   if (tile_id < 0) return;
   const uint32_t tile0 = (uint32_t)tile_id * (uint32_t)TP;
-
-  PL_PHASE_MARK(0);
   StageTile<INT8, TP>(tile, p, tile0);
-  PL_PHASE_MARK(1);
   __syncthreads();
-  PL_PHASE_MARK(2);
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -366,7 +357,6 @@ __device__ __forceinline__ void RowWalkBody(const WalkParams& p, uint32_t* tile)
       StoreRow<OUT, PPL>(p, row, gpos, v, acc);
     }
   }
-  PL_PHASE_MARK(3);
 }
 
 template <bool INT8, int OUT, int NR, int TP>
@@ -746,7 +736,6 @@ __device__ __forceinline__ void MfmaTile(const MfmaParams& p, uint4* xt, uint32_
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
           CommitX<kFast>(r[u], xt, p, qs, kFast ? true : live, kFast ? (quad_on && live) : quad_on, 2 * ks_first + 8 * (pass0 + u), kg0, jc, 2 * ks_first);
-          PL_PHASE_MARK(2);
           __syncthreads();
           if (wave_on) multiply(4 * (pass0 + u), 4 * (pass0 + u) + 4);
         }
@@ -774,7 +763,6 @@ __device__ __forceinline__ void MfmaTile(const MfmaParams& p, uint4* xt, uint32_
     do_chunk(0);
   }
   if (!wave_on) return;
-  PL_PHASE_MARK(4);
   if (!kEarlyConsts) LoadRowConsts<OUT>(rc, p, rbc, lane);
   MfmaFinish<OUT, ACT, VEC>(p, reinterpret_cast<uint32_t*>(xt + (size_t)2 * (kLoopK ? KC : p.ksteps) * kMfmaTilePos), acc, rc, rb, lane, quad0, J);
 }
@@ -862,9 +850,7 @@ __device__ __forceinline__ void MfmaBody(const MfmaParams& p, uint4* xt) {
   const bool wave_on = rb < p.row_blocks;
   const int rbc = wave_on ? rb : p.row_blocks - 1;
   const uint32_t kmask = wave_on ? p.kmask[(size_t)rbc * p.kmask_words] : 0u;  // first 32 k-steps; chunked kernels read their own words
-  PL_PHASE_MARK(0);
   MfmaTile<KSMAX, OUT, ACT, VEC>(p, xt, kmask, rb, rbc, wave_on, tile);
-  PL_PHASE_MARK(6);
 }
 
 // ------------------------------------------------------ streaming block MFMA

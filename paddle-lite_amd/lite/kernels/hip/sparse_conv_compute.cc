@@ -166,9 +166,16 @@ void SparseConvCompute<P, O>::Run() {
                                         : static_cast<void*>(param.output->template mutable_data<int8_t>(TargetType::kHIP));
   const int rc = pl_sparse_conv_run(handle_, param.x->raw_data(), out, batch, im_size, ctx.stream());
   if (rc != PL_OK) LOG(FATAL) << "pl_sparse_conv_run failed (" << rc << "): " << pl_last_error();
+  last_batch_ = batch;
+  last_im_size_ = im_size;
+}
+
+template <PrecisionType P, PrecisionType O>
+std::string SparseConvCompute<P, O>::kernel_func_name() const {
+  if (handle_ == nullptr || last_batch_ < 0) return "NotImplForSparseConv";
   static const char* const kAlgo[] = {"auto", "row_walk", "block_mfma", "image_mfma"};
-  const int algo = pl_sparse_conv_algo_for(handle_, batch, im_size);
-  kernel_func_name_ = std::string("pl_sparse_conv_run/") + (algo >= 0 && algo <= 3 ? kAlgo[algo] : "unknown");
+  const int algo = pl_sparse_conv_algo_for(handle_, last_batch_, last_im_size_);
+  return std::string("pl_sparse_conv_run/") + (algo >= 0 && algo <= 3 ? kAlgo[algo] : "unknown");
 }
 
 template class SparseConvCompute<PRECISION(kFloat), PRECISION(kFloat)>;

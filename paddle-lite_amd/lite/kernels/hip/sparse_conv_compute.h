@@ -33,9 +33,12 @@ class SparseConvCompute : public KernelLite<TARGET(kHIP), Ptype> {
 
   // The math entry point and algorithm of the last Run(), for the profiler
   // (the ARM class reports "sparse_conv_fp32_pipelined" etc. through
-  // KERNEL_FUNC_NAME, lite/kernels/arm/sparse_conv_compute.h:34-43).
-  void SetProfileRuntimeKernelInfo(paddle::lite::profile::OpCharacter* ch) const { ch->kernel_func_name = kernel_func_name_; }
-  const std::string& kernel_func_name() const { return kernel_func_name_; }
+  // KERNEL_FUNC_NAME, lite/kernels/arm/sparse_conv_compute.h:34-43, compiled
+  // in under LITE_WITH_PROFILE only).  Run() only remembers the call's shape;
+  // the name is put together here, when a profiler asks
+  // (lite/core/program.cc:789-816 asks after the kernel has run).
+  void SetProfileRuntimeKernelInfo(paddle::lite::profile::OpCharacter* ch) const { ch->kernel_func_name = kernel_func_name(); }
+  std::string kernel_func_name() const;
 
  private:
   void Upload(int kind);
@@ -45,7 +48,7 @@ class SparseConvCompute : public KernelLite<TARGET(kHIP), Ptype> {
   std::vector<float> w_scale_;
   pl_sparse_conv_handle* handle_{nullptr};
   int64_t ic_{0};  // input channels the weights were prepared for
-  std::string kernel_func_name_{"NotImplForSparseConv"};
+  int last_batch_{-1}, last_im_size_{-1};  // shape of the last Run(); -1 before the first
 };
 
 // The reference divides the int8-output leaky_relu slope by the output scale

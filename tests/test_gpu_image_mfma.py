@@ -46,6 +46,8 @@ SHAPES = [
     (2, 512, 128, 4, 59), (1, 256, 128, 12, 21), (1, 128, 256, 6, 6), (2, 256, 128, 4, 11), (3, 128, 128, 4, 13),
 ]
 IMAGE_KERNELS = {"regroup": capi.IMAGE_KERNEL_REGROUP, "transpose": capi.IMAGE_KERNEL_TRANSPOSE}
+# the regrouping kernel regroups 512-channel 14 x 14 images by transposing LDS reads unless told otherwise
+VALU_REGROUP = capi.tuning(image_kernel=capi.IMAGE_KERNEL_REGROUP, image_tr_regroup=capi.TUNE_NEVER)
 
 
 @pytest.mark.parametrize("image_kernel", sorted(IMAGE_KERNELS))
@@ -67,9 +69,30 @@ def test_image_mfma_bit_exact(shape, kind, image_kernel):
         got = run_hip(case, capi.ALGO_IMAGE_MFMA, tuning=capi.tuning(image_kernel=IMAGE_KERNELS[image_kernel]))
         want = run_oracle(case, oracle_pack(case))
         assert_same(case, got, want, "image %s %s %s" % (kind, act, shape))
+        if image_kernel == "regroup" and (ic, h * w) == (512, 196):
+            assert np.array_equal(got, run_hip(case, capi.ALGO_IMAGE_MFMA, tuning=VALU_REGROUP)), "regrouping by the vector ALU"
     if kind == "acc32":
         ref = np.einsum("mk,bkp->bmp", case.dense.astype(np.int64), case.x.reshape(batch, ic, -1).astype(np.int64)).reshape(got.shape)
         assert np.array_equal(got.astype(np.int64), ref)
+
+
+@pytest.mark.parametrize("act", sorted(ACTS))
+@pytest.mark.parametrize("kind", sorted(KINDS))
+def test_image_mfma_regroup_by_transposing_reads(kind, act):
+    """512 channels, 14 x 14: the regrouping image kernel lets the LDS transpose (its own order of the
+    channels inside a k-step); several row groups, an odd batch, every activation, channels of one parity
+    only in some rows, and the same bits as with the vector-ALU regrouping."""
+    announce("image tr regroup", kind, act)
+    k = KINDS[kind]
+    if kind == "acc32" and act != "none":
+        pytest.skip("accumulators have no activation")
+    case = case_for(k, 5, 512, 256, 14, 14, 0.85, False, ACTS[act], seed=len(act) + 31)
+    case.dense[3, 0::2] = 0
+    case.dense[4, 1::2] = 0
+    case.dense[9] = 0
+    got = run_hip(case, capi.ALGO_IMAGE_MFMA)
+    assert_same(case, got, run_oracle(case, oracle_pack(case)), "tr regroup %s %s" % (kind, act))
+    assert np.array_equal(got, run_hip(case, capi.ALGO_IMAGE_MFMA, tuning=VALU_REGROUP))
 
 
 # 7 x 7 maps (49-byte channel rows, two images per workgroup): every supported
