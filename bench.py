@@ -504,6 +504,21 @@ def run_c5(args):
     return 0
 
 
+def run_lite_program_bench(batch):
+    """The same body through the C++ operator surface (op descriptions -> detect pass -> chain pass ->
+    mir::HipProgram), measured by bench_probes/lite_program_bench in a process of its own: host time per
+    step, the eager sequence and its replay as a HIP graph.  None when the program is not built."""
+    import subprocess
+
+    exe = os.path.join(ROOT, "bench_probes", "lite_program_bench")
+    if not os.path.exists(exe):
+        return None
+    res = subprocess.run([exe, "--batch", str(batch), "--sequences", "40"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    if res.returncode != 0:
+        raise RuntimeError("lite_program_bench failed (%d): %s" % (res.returncode, res.stderr[-2000:]))
+    return json.loads(res.stdout.strip().splitlines()[-1])
+
+
 def run_mobilenet(args):
     """The convolutional body of MobileNetV1-1.0 at batch 64 in int8: thirteen
     times (depthwise 3x3, relu) then (pointwise 1x1 through sparse_conv2d, 90 %
@@ -591,6 +606,8 @@ def run_mobilenet(args):
     dw_us = sum(p["kernel_us"] for p in per_layer if p["kind"] == "depthwise")
     pw_us = sum(p["kernel_us"] for p in per_layer if p["kind"] == "pointwise")
     print(json.dumps({
+        "lite_program": run_lite_program_bench(batch),
+        "lite_program_batch_1": run_lite_program_bench(1),
         "metric": "MobileNetV1-1.0 convolutional body, int8, batch 64: images/s of the 26-launch sequence",
         "value": batch * steps / wall,
         "unit": "images/s",

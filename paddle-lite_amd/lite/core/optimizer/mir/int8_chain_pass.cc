@@ -162,13 +162,22 @@ HipProgram::HipProgram(const std::vector<ProgramStep>& steps, Scope* scope) {
   }
 }
 
-void HipProgram::Run() {
-  for (size_t i = 0; i < kernels_.size(); ++i) {
+void HipProgram::Enqueue(size_t first, size_t last) {
+  CHECK(first <= last && last <= kernels_.size()) << "steps " << first << " .. " << last << " of " << kernels_.size();
+  for (size_t i = first; i < last; ++i) {
     CHECK(ops_[i]->CheckShape()) << "shape check failed at step " << i;
     CHECK(ops_[i]->InferShape()) << "shape inference failed at step " << i;
     kernels_[i]->Launch();
   }
+}
+
+void HipProgram::Sync() {
   if (!kernels_.empty()) kernels_.back()->mutable_context_as<HIPContext>()->Sync();
+}
+
+void HipProgram::Run() {
+  Enqueue(0, kernels_.size());
+  Sync();
 }
 
 }  // namespace mir

@@ -53,6 +53,11 @@ class HipProgram {
  public:
   HipProgram(const std::vector<ProgramStep>& steps, Scope* scope);
   void Run();   // enqueue every step and wait for the stream
+  // Enqueues steps [first, last) and returns without waiting: shape check, shape inference and
+  // Launch of each, nothing else, so that a caller can time the host side of a step or record
+  // the steps into a stream capture.
+  void Enqueue(size_t first, size_t last);
+  void Sync();  // waits for the stream of the last step
   size_t size() const { return kernels_.size(); }
   const KernelBase& kernel(size_t i) const { return *kernels_[i]; }
 
