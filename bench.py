@@ -30,7 +30,36 @@ METRICS = {
     "c2": "sparse 1x1 conv nnz-GOP/s + % HBM roofline (fp32 semi-structured, N=32, 256->512@28x28, 90%)",
     "c3": "sparse 1x1 conv nnz-GOP/s + % HBM roofline (int8, N=64, 512->512@14x14, 85%)",
     "c4": "sparse 1x1 conv nnz-GOP/s + % HBM roofline (int8->int8 semi-structured, N=128, 128->256@56x56, 75%)",
+    "custom": "sparse 1x1 conv nnz-GOP/s + % HBM roofline (shape from the command line)",
 }
+
+
+def custom_case(args):
+    """The case --config custom describes; sizes are bounded so that a typing mistake cannot ask for a
+    tensor the box does not hold."""
+    import helpers
+
+    wl = helpers.workloads
+    h, w = (1, args.N) if args.N > 0 else (args.hw, args.hw)
+    if not (1 <= args.M <= 8192 and 1 <= args.K <= 8192 and 1 <= h * w <= 1 << 16 and 1 <= args.batch <= 1024 and 0.0 <= args.sparsity < 1.0):
+        raise SystemExit("custom: M, K in 1..8192, positions in 1..65536, batch in 1..1024, sparsity in [0, 1)")
+    if float(args.batch) * h * w * (args.M * 4 + args.K * 4) > 8e9:
+        raise SystemExit("custom: more than 8 GB of input and output per launch")
+    act = wl.ActivationParam() if args.act == "none" else wl.ActivationParam(args.act, Leaky_relu_alpha=0.1)
+    name = "custom_%s_N%d_%dx%d_%dx%d_%s%d" % (args.kind, args.batch, args.K, args.M, h, w, "semi" if args.semi else "s", int(round(args.sparsity * 100)))
+    if args.kind in ("fp32", "fp16"):
+        return wl.make_fp32(name, args.batch, args.K, args.M, h, w, args.sparsity, args.semi, act, seed=args.seed)
+    case = wl.make_int8(name, args.batch, args.K, args.M, h, w, args.sparsity, args.semi, act, out_int8=args.kind == "int8_int8", seed=args.seed)
+    if args.kind == "int8_int8":  # three sigma of the accumulator on 127, as the MobileNet layers choose it
+        sigma_acc = np_sqrt(args.K * (1.0 - args.sparsity)) * 73.3 * 73.3
+        case.output_scale = float(3.0 * sigma_acc * float(case.weight_scale.mean()) * case.input_scale / 127.0)
+    return case
+
+
+def np_sqrt(v):
+    import numpy as np
+
+    return float(np.sqrt(v))
 
 
 def parse():
@@ -38,10 +67,21 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib", "mobilenet", "density-sweep", "floors", "store-shapes"])
+    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib", "mobilenet", "density-sweep", "floors", "store-shapes", "custom", "small-batch"])
     ap.add_argument("--algo", default="auto", choices=["auto", "walk", "mfma", "image"])
     ap.add_argument("--image-kernel", default="rule", choices=["rule", "regroup", "transpose"], help="which image MFMA kernel a handle uses where both apply (pl_sparse_conv_tuning.image_kernel)")
     ap.add_argument("--image-regroup", default="rule", choices=["rule", "valu"], help="regrouping image kernel: by transposing LDS reads where that exists (rule) or by the vector ALU everywhere (pl_sparse_conv_tuning.image_tr_regroup)")
+    # --config custom: any shape through the same measurement (parity-checked against the oracle on two images)
+    ap.add_argument("--M", type=int, default=512, help="custom: output channels")
+    ap.add_argument("--K", type=int, default=512, help="custom: input channels")
+    ap.add_argument("--hw", type=int, default=14, help="custom: side of the square map (H = W)")
+    ap.add_argument("--N", type=int, default=0, help="custom: positions per image as a 1 x N map instead of --hw")
+    ap.add_argument("--batch", type=int, default=64, help="custom: images per launch")
+    ap.add_argument("--semi", action="store_true", help="custom: semi-structured mask (pairs of output channels share their nonzero columns)")
+    ap.add_argument("--sparsity", type=float, default=0.85, help="custom: fraction of zero weights")
+    ap.add_argument("--act", default="relu", choices=["none", "relu", "relu6", "leaky_relu", "hard_swish"], help="custom: fused activation")
+    ap.add_argument("--kind", default="int8_fp32", choices=["fp32", "fp16", "int8_fp32", "int8_int8"], help="custom: input -> output precision")
+    ap.add_argument("--seed", type=int, default=0, help="custom: seed of the synthetic tensors")
     ap.add_argument("--fp16", action="store_true", help="run an fp32 configuration (c1, c2) through the half-precision kernel")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cache-resident", action="store_true", help="reuse one buffer set (reported, never the headline)")
@@ -504,6 +544,33 @@ def run_c5(args):
     return 0
 
 
+SMALL_BATCH_SHAPES = [(32, 64, 112), (64, 128, 56), (128, 128, 56), (128, 256, 28), (256, 256, 28), (256, 512, 14), (512, 512, 14), (512, 1024, 7), (1024, 1024, 7)]
+SMALL_BATCHES = (1, 4, 16, 64)
+
+
+def run_small_batch(args):
+    """The nine distinct pointwise shapes of MobileNetV1-1.0 (int8 -> int8, relu, 90 % zeros) at 1, 4, 16 and
+    64 images per launch: the algorithm a PL_ALGO_AUTO handle picks and its time next to every algorithm forced
+    (helpers.algo_times: every handle parity-checked against the oracle, buffer sets rotated, the best of three
+    timed runs).  One JSON line; `auto_over_best` is what the selection rule costs where it picks wrong."""
+    import helpers
+
+    wl = helpers.workloads
+    rows = []
+    worst = 0.0
+    for ic, oc, hw in SMALL_BATCH_SHAPES:
+        for batch in SMALL_BATCHES:
+            case = wl.config5_layer(wl.MOBILENET_V1_POINTWISE.index((ic, oc, hw)), batch=batch)
+            times, picked = helpers.algo_times(case, warm=100, steps=500)
+            best = min(v for k, v in times.items() if k != "auto")
+            worst = max(worst, times["auto"] / best)
+            rows.append({"shape": "%d->%d @%dx%d" % (ic, oc, hw, hw), "batch": batch, "auto_picks": picked, "us": {k: round(v, 2) for k, v in times.items()}, "auto_over_best": round(times["auto"] / best, 3),
+                         "frac_of_8TBs": round(case.algorithmic_bytes(helpers.pla.detect_and_pack(case.dense, case.im_size)) / (times["auto"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 3)})
+    print(json.dumps({"metric": "int8 pointwise layers of MobileNetV1 at small batch: us per launch by algorithm", "unit": "us", "n_gpus": 1, "data": "synthetic", "dtype": "int8",
+                      "config": {"workload": "small_batch_int8", "sparsity": 0.9, "parity_checked": True}, "worst_auto_over_best": round(worst, 3), "rows": rows}))
+    return 0
+
+
 def run_lite_program_bench(batch):
     """The same body through the C++ operator surface (op descriptions -> detect pass -> chain pass ->
     mir::HipProgram), measured by bench_probes/lite_program_bench in a process of its own: host time per
@@ -652,7 +719,13 @@ def main():
         return run_calib(args)
     if args.config == "mobilenet":
         return run_mobilenet(args)
-    case = wl.CONFIGS[args.config]()
+    if args.config == "small-batch":
+        return run_small_batch(args)
+    if args.config == "custom":
+        case = custom_case(args)
+        args.fp16 = args.fp16 or args.kind == "fp16"
+    else:
+        case = wl.CONFIGS[args.config]()
     if args.fp16:
         if case.kind != capi.KIND_FP32:
             sys.stderr.write("--fp16 applies to the fp32 configurations\n")
@@ -738,7 +811,7 @@ def main():
     algo_names = {capi.ALGO_ROW_WALK: "row_walk", capi.ALGO_BLOCK_MFMA: "block_mfma", capi.ALGO_IMAGE_MFMA: "image_mfma"}
     algo_name = algo_names[capi.check(L.pl_sparse_conv_algo_for(kernel._handle, case.batch, case.im_size))]
     traffic, traffic_detail = measured_traffic(case.name, algo_name)
-    # int8: the same launch through every algorithm the shape allows (same rotating buffers, 300 launches each)
+    # int8: the same launch through every algorithm the shape allows (same rotating buffers, 200 untimed then 1000 timed launches each)
     per_algo = None
     if case.kind in (capi.KIND_INT8_FP32, capi.KIND_INT8_INT8):
         per_algo = {algo_name: round(kernel_ms * 1e3, 3)}
@@ -755,13 +828,13 @@ def main():
                 other, _ = helpers.make_kernel(case, algo=a, tuning=other_tune)
             except capi.SparseConvError:
                 continue  # this shape is outside the algorithm's range
-            if L.pl_sparse_conv_run_sequence(other._handle, xp, op, n_sets, case.batch, case.im_size, 50, C.c_void_p(stream), None) < 0:
+            if L.pl_sparse_conv_run_sequence(other._handle, xp, op, n_sets, case.batch, case.im_size, 200, C.c_void_p(stream), None) < 0:
                 continue
             torch.cuda.synchronize()
             assert np.array_equal(outs[0][:nchk].cpu().numpy(), want), "%s output differs from the oracle" % name
             ms_o = C.c_float(0.0)
-            capi.check(L.pl_sparse_conv_run_sequence(other._handle, xp, op, n_sets, case.batch, case.im_size, 300, C.c_void_p(stream), C.byref(ms_o)))
-            per_algo[name] = round(ms_o.value * 1e3 / 300, 3)
+            capi.check(L.pl_sparse_conv_run_sequence(other._handle, xp, op, n_sets, case.batch, case.im_size, 1000, C.c_void_p(stream), C.byref(ms_o)))
+            per_algo[name] = round(ms_o.value * 1e3 / 1000, 3)
     line = {
         "metric": METRICS[args.config] + (" (half-precision kernel)" if args.fp16 else ""),
         "value": ops * args.steps / wall / 1e9,

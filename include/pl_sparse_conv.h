@@ -78,8 +78,10 @@ enum {
  *                     and multiplies it with dense 16x64 weight tiles; also
  *                     7 x 7 maps with ic = 256 / 512 / 1024 (two images per
  *                     workgroup)
- * With PL_ALGO_AUTO an int8 handle may hold more than one form and choose per
- * call by batch and H*W: see pl_sparse_conv_algo_for(). */
+ * With PL_ALGO_AUTO an int8 handle holds every form its shape allows and
+ * chooses per call by batch and H*W (the image kernel where it applies, the
+ * row walk for at most 256 positions in all on maps other than 7 x 7, the
+ * block kernel otherwise): see pl_sparse_conv_algo_for(). */
 enum { PL_ALGO_AUTO = 0, PL_ALGO_ROW_WALK = 1, PL_ALGO_BLOCK_MFMA = 2, PL_ALGO_IMAGE_MFMA = 3 };
 
 /* Activation constants, used as given (replaces the fields of
@@ -108,7 +110,7 @@ typedef struct pl_sparse_conv_tuning {
                                 with transposing LDS reads (H*W = 4 mod 8 only;
                                 slightly slower where measured)                */
   int32_t image_min_items;   /* fewest (image, 128 rows) work items for which
-                                PL_ALGO_AUTO takes the image kernel            */
+                                PL_ALGO_AUTO takes the image kernel (rule: 1)  */
   int32_t mfma_stream;       /* (switch) streaming form of the block kernel    */
   int32_t mfma_sub_tiles;    /* (switch) several tiles per workgroup, ic <= 64 */
   int32_t mfma_tile_quads;   /* block kernel: position quads per tile, 8 .. 32 */

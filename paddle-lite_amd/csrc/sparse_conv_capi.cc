@@ -179,7 +179,8 @@ struct pl_sparse_conv_handle {
   int image_kernel = 0;  // 0 by rule, 1 regrouping kernel, 2 transposing-read kernel
   // int8 handles prepared with PL_ALGO_AUTO hold several forms and choose per call
   bool auto_int8 = false;
-  int image_min_items = 128;  // fewest (image, 128-row group) work items for which the image kernel is chosen
+  int image_min_items = 1;  // fewest (image, 128-row group) work items for which the image kernel is chosen
+  bool auto_walk = false;   // an automatic int8 handle that also holds the row walk's lists
   // row-walk tuning read once at prepare (0 = chosen per problem)
   int walk_tile = 0, walk_threads = 0, walk_slices = 0;
   // epilogue
@@ -655,12 +656,20 @@ pl::WalkConfig ChooseWalk(const pl_sparse_conv_handle* h, uint32_t P) {
   return c;
 }
 
-// The algorithm one call uses.  Handles prepared for one algorithm use it;
-// int8 handles prepared with PL_ALGO_AUTO take the image kernel where its
-// shape conditions hold and there are enough (image, row group) work items to
-// occupy the chip, and the block kernel otherwise.
+// The algorithm one call uses.  Handles prepared for one algorithm use it.  An int8 handle prepared with
+// PL_ALGO_AUTO holds the forms of every algorithm its shape allows and picks per call, by what was measured on
+// the pointwise shapes of MobileNetV1 at 1 to 64 images per launch:
+//  * the image kernel wherever its shape conditions hold (it ties with or beats the block kernel from 4 work
+//    items on, by 2x on 7 x 7 maps at any batch) - except
+//  * the row walk for at most 256 positions in all on maps other than 7 x 7 (one 14 x 14 image: a handful of
+//    image-kernel workgroups each walk a long dependent chain, the walk spreads the rows over the chip;
+//    5.97 against 7.2 us with 512 channels), and
+//  * the block kernel otherwise.
+// tuning.image_min_items raises the number of (image, 128-row group) work items the image kernel asks for.
 int AlgoForCall(const pl_sparse_conv_handle* h, int batch, int im_size, bool aligned16) {
   if (!h->auto_int8) return h->algo;
+  const int64_t positions = static_cast<int64_t>(batch) * im_size;
+  if (h->auto_walk && im_size != 49 && positions <= 256) return PL_ALGO_ROW_WALK;
   // work items: (image, row group), for 7 x 7 maps (pair of images, row group)
   const int64_t image_items = static_cast<int64_t>(im_size == 49 ? (batch + 1) / 2 : batch) * (h->oc / 128);
   if (h->wtiles.ptr && aligned16 && pl::ImageMfmaFits(h->oc, h->ic, im_size) && image_items >= h->image_min_items) return PL_ALGO_IMAGE_MFMA;
@@ -804,6 +813,10 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   const bool mfma_forms = algo == PL_ALGO_BLOCK_MFMA || algo == PL_ALGO_IMAGE_MFMA;
   int rc = PL_OK;
   if (algo == PL_ALGO_ROW_WALK) rc = BuildRowWalk(L, h);
+  if (h->auto_int8 && static_cast<size_t>(CeilDiv(desc->ic, 4)) * 4 * 16 <= static_cast<size_t>(pl::kMaxLdsBytes)) {
+    rc = BuildRowWalk(L, h);  // for calls of a few hundred positions
+    h->auto_walk = rc == PL_OK;
+  }
   if (rc == PL_OK && algo == PL_ALGO_BLOCK_MFMA) rc = BuildBlockMfma(L, h);
   if (rc == PL_OK && (algo == PL_ALGO_IMAGE_MFMA || (h->auto_int8 && (pl::ImageMfmaFits(desc->oc, desc->ic, 16) || pl::ImageMfmaFits(desc->oc, desc->ic, 49))))) rc = BuildImageMfma(L, h);
   if (rc == PL_OK && h->wtiles.ptr && pl::ImageTrMfmaFits(desc->oc, desc->ic, 20)) rc = BuildImageTrMfma(L, h);
@@ -849,6 +862,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
   const bool aligned16 = reinterpret_cast<uintptr_t>(x_dev) % 16 == 0 && reinterpret_cast<uintptr_t>(out_dev) % 16 == 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipError_t e;
+  const int call_algo = AlgoForCall(h, batch, im_size, aligned16);
   if (h->half && (im_size % 4 == 0) && (reinterpret_cast<uintptr_t>(x_dev) % 8 == 0) && (reinterpret_cast<uintptr_t>(out_dev) % 8 == 0) && h->walk_chunked > 0 && h->cw_chunks > 0 &&
       (h->walk_chunked == 2 || (h->ic > 128 && static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kChunkWalkTile)) * h->cw_slices >= 256))) {
     // many channels and enough work for every CU: walk over channel chunks
@@ -899,7 +913,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.groups_per_slice = CeilDiv(h->n_groups, slices);
     p.slices = CeilDiv(h->n_groups, p.groups_per_slice);
     e = pl::LaunchHalfWalk(h->semi ? 2 : 1, tp, threads, p, s);
-  } else if (AlgoForCall(h, batch, im_size, aligned16) == PL_ALGO_IMAGE_MFMA) {
+  } else if (call_algo == PL_ALGO_IMAGE_MFMA) {
     if (!pl::ImageMfmaFits(h->oc, h->ic, im_size)) return Fail(PL_ERR_UNSUPPORTED, "the image MFMA algorithm needs H*W = 49 or a multiple of 4 in [16, 256] that fits LDS with %d channels (H*W = %d)", h->ic, im_size);
     if (reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(out_dev) % 16 != 0) return Fail(PL_ERR_UNSUPPORTED, "the image MFMA algorithm needs 16-byte aligned tensors");
     pl::ImageMfmaParams p{};
@@ -924,7 +938,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
       p.wtiles = p.tr_regroup ? h->wtiles_rg.ptr : h->wtiles.ptr;
       e = pl::LaunchImageMfma(OutKind(h->kind), p, s);
     }
-  } else if (h->algo == PL_ALGO_BLOCK_MFMA) {
+  } else if (call_algo == PL_ALGO_BLOCK_MFMA) {
     pl::MfmaParams p{};
     p.x = static_cast<const int8_t*>(x_dev);
     p.out = out_dev;

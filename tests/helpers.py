@@ -109,3 +109,54 @@ def assert_same(case, got, want, what=""):
         if not np.array_equal(got, want):
             bad = np.argwhere(got != want)
             raise AssertionError("%s: %d of %d elements differ, first at %s: got %r want %r" % (what, len(bad), got.size, tuple(bad[0]), got[tuple(bad[0])], want[tuple(bad[0])]))
+
+
+ALGO_NAMES = {capi.ALGO_ROW_WALK: "row_walk", capi.ALGO_BLOCK_MFMA: "block_mfma", capi.ALGO_IMAGE_MFMA: "image_mfma"}
+
+
+def algo_times(case, warm=100, steps=500, repeats=3, max_sets=24, rotation_bytes=320 << 20):
+    """Device time per launch (us, events inside pl_sparse_conv_run_sequence) of an int8 case with the
+    algorithm left to the handle ("auto") and with each algorithm forced; an algorithm the shape is outside of
+    is left out.  Every handle's output on the first two images is compared with the oracle before it is
+    timed.  Buffer sets rotate (up to `max_sets` of them, `rotation_bytes` in all); the runs of the handles are
+    interleaved `repeats` times and the smallest time of each is kept, so that a clock ramp or another
+    process's burst does not land on one algorithm.  Returns (times, name of the algorithm auto picked)."""
+    import ctypes as C
+
+    import torch
+
+    L = capi.lib()
+    oc = case.dense.shape[0]
+    out_dtype = {capi.KIND_INT8_FP32: torch.float32, capi.KIND_INT8_INT8: torch.int8}[case.kind]
+    set_bytes = case.x.nbytes + case.batch * oc * case.im_size * (1 if out_dtype == torch.int8 else 4)
+    n_sets = max(1, min(max_sets, int(rotation_bytes // set_bytes) + 1))
+    x0 = torch.from_numpy(case.x).cuda()
+    xs = [x0] + [x0.clone() for _ in range(n_sets - 1)]
+    outs = [torch.empty((case.batch, oc) + tuple(case.x.shape[2:]), dtype=out_dtype, device="cuda") for _ in range(n_sets)]
+    xp = (C.c_void_p * n_sets)(*[t.data_ptr() for t in xs])
+    op = (C.c_void_p * n_sets)(*[t.data_ptr() for t in outs])
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    nchk = min(case.batch, 2)
+    want = run_oracle(case, x=case.x[:nchk])
+    handles = {}
+    for name, algo in [("auto", capi.ALGO_AUTO)] + [(n, a) for a, n in sorted(ALGO_NAMES.items())]:
+        try:
+            k, _ = make_kernel(case, algo=algo)
+        except capi.SparseConvError:
+            continue
+        outs[0].zero_()
+        if L.pl_sparse_conv_run_sequence(k._handle, xp, op, n_sets, case.batch, case.im_size, 1, stream, None) < 0:
+            continue  # outside this algorithm's range at this batch or map size
+        torch.cuda.synchronize()
+        assert np.array_equal(outs[0][:nchk].cpu().numpy(), want), "%s: %s differs from the oracle" % (case.name, name)
+        handles[name] = k
+    picked = ALGO_NAMES[capi.check(L.pl_sparse_conv_algo_for(handles["auto"]._handle, case.batch, case.im_size))]
+    times = {}
+    for _ in range(repeats):
+        for name, k in handles.items():
+            capi.check(L.pl_sparse_conv_run_sequence(k._handle, xp, op, n_sets, case.batch, case.im_size, warm, stream, None))
+            ms = C.c_float(0.0)
+            capi.check(L.pl_sparse_conv_run_sequence(k._handle, xp, op, n_sets, case.batch, case.im_size, steps, stream, C.byref(ms)))
+            us = ms.value * 1e3 / steps
+            times[name] = min(times.get(name, us), us)
+    return times, picked

@@ -243,15 +243,22 @@ def test_auto_picks_the_image_kernel_only_where_it_applies():
     case = case_for(capi.KIND_INT8_FP32, 64, 512, 512, 14, 14, 0.85, False, ACTS["leaky"], seed=0)
     kernel, _ = make_kernel(case, capi.ALGO_AUTO)
     assert L.pl_sparse_conv_algo_for(kernel._handle, 64, 196) == capi.ALGO_IMAGE_MFMA
-    assert L.pl_sparse_conv_algo_for(kernel._handle, 2, 196) == capi.ALGO_BLOCK_MFMA      # too few work items
-    assert L.pl_sparse_conv_algo_for(kernel._handle, 64, 49) == capi.ALGO_IMAGE_MFMA      # 7x7 maps: pairs of images, 32 x 4 work items
-    assert L.pl_sparse_conv_algo_for(kernel._handle, 32, 49) == capi.ALGO_BLOCK_MFMA      # too few of them
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 2, 196) == capi.ALGO_IMAGE_MFMA      # from two images on
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 1, 196) == capi.ALGO_ROW_WALK        # at most 256 positions in all: the walk
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 64, 49) == capi.ALGO_IMAGE_MFMA      # 7x7 maps: pairs of images
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 1, 49) == capi.ALGO_IMAGE_MFMA       # at any batch
     assert L.pl_sparse_conv_algo_for(kernel._handle, 64, 50) == capi.ALGO_BLOCK_MFMA      # not a multiple of 4
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 4, 50) == capi.ALGO_ROW_WALK         # 200 positions
     assert L.pl_sparse_conv_algo_for(kernel._handle, 64, 28 * 28) == capi.ALGO_BLOCK_MFMA  # does not fit LDS
+    # tuning.image_min_items asks for more (image, 128-row group) work items before the image kernel is taken
+    picky, _ = make_kernel(case, capi.ALGO_AUTO, tuning=capi.tuning(image_min_items=128))
+    assert L.pl_sparse_conv_algo_for(picky._handle, 64, 196) == capi.ALGO_IMAGE_MFMA
+    assert L.pl_sparse_conv_algo_for(picky._handle, 2, 196) == capi.ALGO_BLOCK_MFMA
+    assert L.pl_sparse_conv_algo_for(picky._handle, 32, 49) == capi.ALGO_BLOCK_MFMA
     # the same handle serves all of them
     import torch
 
-    for batch, h, w in ((2, 14, 14), (3, 7, 7)):
+    for batch, h, w in ((2, 14, 14), (1, 14, 14), (3, 7, 7), (1, 7, 7)):
         sub = copy.copy(case)  # same weights, another input size (the oracle's offsets are baked per H*W)
         sub.x = np.ascontiguousarray(case.x[:batch, :, :h, :w])
         got = kernel.Run(torch.from_numpy(sub.x).cuda()).cpu().numpy()
