@@ -138,6 +138,46 @@ def build_host_mirror(verbose=False):
     return LITE_LIB_PATH, HOST_TEST_BIN
 
 
+SANITIZE_FLAGS = ["-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-static-libasan", "-static-libubsan", "-fno-omit-frame-pointer", "-O1", "-g"]
+
+
+def _compile_host_object(job):
+    cmd, obj = job
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    return obj, res.returncode, res.stdout, " ".join(cmd)
+
+
+def build_sanitized(out_dir):
+    """The host side once more with AddressSanitizer and UndefinedBehaviorSanitizer (host code only): every
+    file of the C++ mirror, the layout decoder of the library and the CPU oracle compiled into
+    out_dir/sparse_conv_hip_test and out_dir/model_file_tool.  The device library stays as it is: the test
+    program's --cpu mode and the model-file tool never call into it.  Returns the two paths; raises
+    RuntimeError when the compiler has no sanitizer runtime."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    os.makedirs(out_dir, exist_ok=True)
+    oracle_dir = os.path.join(ROOT, "oracle")
+    inc = ["-I" + PKG, "-I" + os.path.join(ROOT, "include"), "-I" + oracle_dir, "-I/opt/rocm/include"]
+    cxx = ["g++", "-std=c++17", "-Wall", "-D__HIP_PLATFORM_AMD__"] + SANITIZE_FLAGS + inc
+    cc = ["gcc", "-std=c11"] + SANITIZE_FLAGS + inc
+    shared = [os.path.join(LITE_DIR, s) for s in LITE_SOURCES] + [os.path.join(CSRC, "sparse_layout.cc")]
+    jobs, objs = [], {}
+    for src in shared + [HOST_TEST_SRC, MODEL_TOOL_SRC, os.path.join(oracle_dir, "sparse_conv_oracle.c")]:
+        obj = os.path.join(out_dir, os.path.relpath(src, ROOT).replace(os.sep, "_") + ".o")
+        objs[src] = obj
+        jobs.append(((cc if src.endswith(".c") else cxx) + ["-c", src, "-o", obj], obj))
+    with ThreadPoolExecutor(max_workers=min(6, os.cpu_count() or 1)) as pool:
+        for obj, rc, out, cmd in pool.map(_compile_host_object, jobs):
+            if rc != 0:
+                raise RuntimeError("sanitizer build failed: %s\n%s" % (cmd, out))
+    link = ["-L" + LIB_DIR, "-lpl_sparse_conv", "-L/opt/rocm/lib", "-lamdhip64", "-lm", "-Wl,-rpath," + LIB_DIR + ":/opt/rocm/lib"]
+    test_bin, tool_bin = os.path.join(out_dir, "sparse_conv_hip_test"), os.path.join(out_dir, "model_file_tool")
+    common = [objs[s] for s in shared]
+    _run(["g++"] + SANITIZE_FLAGS + ["-o", test_bin, objs[HOST_TEST_SRC], objs[os.path.join(oracle_dir, "sparse_conv_oracle.c")]] + common + link, False)
+    _run(["g++"] + SANITIZE_FLAGS + ["-o", tool_bin, objs[MODEL_TOOL_SRC]] + common + link, False)
+    return test_bin, tool_bin
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
     print(build_host_mirror(verbose=True))
