@@ -69,7 +69,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib", "mobilenet", "density-sweep", "floors", "store-shapes", "custom", "small-batch"])
     ap.add_argument("--algo", default="auto", choices=["auto", "walk", "mfma", "image"])
-    ap.add_argument("--image-kernel", default="rule", choices=["rule", "regroup", "transpose"], help="which image MFMA kernel a handle uses where both apply (pl_sparse_conv_tuning.image_kernel)")
+    ap.add_argument("--image-kernel", default="rule", choices=["rule", "regroup", "transpose", "rows"], help="which image MFMA kernel a handle uses where both apply (pl_sparse_conv_tuning.image_kernel)")
     ap.add_argument("--image-regroup", default="rule", choices=["rule", "valu"], help="regrouping image kernel: by transposing LDS reads where that exists (rule) or by the vector ALU everywhere (pl_sparse_conv_tuning.image_tr_regroup)")
     # --config custom: any shape through the same measurement (parity-checked against the oracle on two images)
     ap.add_argument("--M", type=int, default=512, help="custom: output channels")
@@ -735,7 +735,7 @@ def main():
         case.name += "_fp16"
         args.no_cpu_baseline = True  # the CPU baselines are fp32 / int8 paths
     algo = {"auto": capi.ALGO_AUTO, "walk": capi.ALGO_ROW_WALK, "mfma": capi.ALGO_BLOCK_MFMA, "image": capi.ALGO_IMAGE_MFMA}[args.algo]
-    tune = capi.tuning(image_kernel={"rule": 0, "regroup": capi.IMAGE_KERNEL_REGROUP, "transpose": capi.IMAGE_KERNEL_TRANSPOSE}[args.image_kernel],
+    tune = capi.tuning(image_kernel={"rule": 0, "regroup": capi.IMAGE_KERNEL_REGROUP, "transpose": capi.IMAGE_KERNEL_TRANSPOSE, "rows": capi.IMAGE_KERNEL_ROWS}[args.image_kernel],
                        image_tr_regroup=capi.TUNE_NEVER if args.image_regroup == "valu" else capi.TUNE_RULE)
     kernel, weights = helpers.make_kernel(case, algo=algo, tuning=tune)
     info = kernel.info()
@@ -817,13 +817,15 @@ def main():
         per_algo = {algo_name: round(kernel_ms * 1e3, 3)}
         others = sorted(algo_names.items())
         if algo_name == "image_mfma":
-            others.append((capi.ALGO_IMAGE_MFMA, "image_mfma_valu_regroup"))  # the image kernel with the regrouping done by the vector ALU
+            others.append((capi.ALGO_IMAGE_MFMA, "image_mfma_regroup_in_lds"))  # a pair of wavefronts per two row tiles, image landed in LDS and regrouped there
+            others.append((capi.ALGO_IMAGE_MFMA, "image_mfma_valu_regroup"))  # the same with the regrouping done by the vector ALU
             others.append((capi.ALGO_IMAGE_MFMA, "image_mfma_transposing_reads"))  # the image kernel that never regroups
         for a, name in others:
             if name in per_algo:
                 continue
             try:
-                other_tune = {"image_mfma_valu_regroup": capi.tuning(image_kernel=capi.IMAGE_KERNEL_REGROUP, image_tr_regroup=capi.TUNE_NEVER),
+                other_tune = {"image_mfma_regroup_in_lds": capi.tuning(image_kernel=capi.IMAGE_KERNEL_REGROUP),
+                              "image_mfma_valu_regroup": capi.tuning(image_kernel=capi.IMAGE_KERNEL_REGROUP, image_tr_regroup=capi.TUNE_NEVER),
                               "image_mfma_transposing_reads": capi.tuning(image_kernel=capi.IMAGE_KERNEL_TRANSPOSE)}.get(name)
                 other, _ = helpers.make_kernel(case, algo=a, tuning=other_tune)
             except capi.SparseConvError:

@@ -105,10 +105,13 @@ typedef struct pl_activation {
  * ALWAYS means "whenever the shape allows it". */
 enum { PL_TUNE_RULE = 0, PL_TUNE_NEVER = 1, PL_TUNE_ALWAYS = 2 };
 typedef struct pl_sparse_conv_tuning {
-  int32_t image_kernel;      /* PL_ALGO_IMAGE_MFMA: 1 (and the rule) = the kernel
-                                that regroups the image in LDS, 2 = the kernel
-                                with transposing LDS reads (H*W = 4 mod 8 only;
-                                slightly slower where measured)                */
+  int32_t image_kernel;      /* PL_ALGO_IMAGE_MFMA: 3 (and the rule wherever it
+                                applies) = one row tile per wavefront, image
+                                through registers; 1 = a pair of wavefronts per
+                                two row tiles, image regrouped in LDS (the rule
+                                for 7 x 7 maps); 2 = the kernel with transposing
+                                LDS reads (H*W = 4 mod 8 only); a kernel asked
+                                for outside its shapes is PL_ERR_UNSUPPORTED   */
   int32_t image_min_items;   /* fewest (image, 128 rows) work items for which
                                 PL_ALGO_AUTO takes the image kernel (rule: 1)  */
   int32_t mfma_stream;       /* (switch) streaming form of the block kernel    */

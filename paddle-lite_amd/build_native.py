@@ -37,6 +37,7 @@ SOURCES = [
     ("dwconv_kernels.hip", "dwconv_kernels.o", []),
     ("image_mfma_kernels.hip", "image_mfma_kernels.o", []),
     ("image_tr_kernels.hip", "image_tr_kernels.o", []),
+    ("image_rows_kernels.hip", "image_rows_kernels.o", []),
     ("sparse_conv_kernels.hip", "sparse_conv_kernels_walk.o", ["-DPL_KERNEL_PART=0"]),
     ("sparse_conv_kernels.hip", "sparse_conv_kernels_mfma_f32.o", ["-DPL_KERNEL_PART=1"]),
     ("sparse_conv_kernels.hip", "sparse_conv_kernels_mfma_i8.o", ["-DPL_KERNEL_PART=2"]),

@@ -12,7 +12,7 @@ KIND_FP32, KIND_INT8_FP32, KIND_INT8_INT8, KIND_INT8_ACC32, KIND_FP16 = 0, 1, 2,
 ACT_NONE, ACT_RELU, ACT_RELU6, ACT_LEAKY_RELU, ACT_HARD_SWISH = 0, 1, 2, 4, 10
 ALGO_AUTO, ALGO_ROW_WALK, ALGO_BLOCK_MFMA, ALGO_IMAGE_MFMA = 0, 1, 2, 3
 TUNE_RULE, TUNE_NEVER, TUNE_ALWAYS = 0, 1, 2
-IMAGE_KERNEL_REGROUP, IMAGE_KERNEL_TRANSPOSE = 1, 2
+IMAGE_KERNEL_REGROUP, IMAGE_KERNEL_TRANSPOSE, IMAGE_KERNEL_ROWS = 1, 2, 3
 
 EXPORTS = [
     "pl_sparse_conv_abi_version",

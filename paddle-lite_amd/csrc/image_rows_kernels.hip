@@ -1,0 +1,332 @@
+// Image MFMA, one row tile per wavefront: int8 sparse 1x1 convolution for feature maps of which one image
+// ([K x H*W] int8) fits the LDS of a CU.  Same work split over the chip as image_mfma_kernels.hip (one workgroup
+// of eight wavefronts per image and 128 output rows, the image held in LDS as 16-byte cells of 16 channels of
+// one position), with three differences that were each measured on 64 x 512 -> 512 @14x14, fp32 output:
+//
+//   * The image goes through registers, not through an LDS landing area.  A lane loads the dword (four
+//     positions) of one position quad for each of 16 consecutive channels, transposes the 16 x 4 bytes with
+//     two stages of v_perm_b32 and writes four cells.  LDS then takes the image once (writes run at about
+//     72 bytes per clock per CU, half the read rate); landing it by direct loads and regrouping it in place
+//     writes it twice and was 0.3 us slower.  The weight tiles of two k-steps are requested behind every
+//     regrouped channel group, so that they queue up behind the image and arrive in the order the
+//     multiplication uses them.
+//   * A wavefront owns ONE tile of 16 output rows and all positions (the other kernel gives a pair of
+//     wavefronts two tiles and splits the positions).  Every wavefront then loads only its own 8 KB of
+//     weights - half the weight traffic of the workgroup - and every unit of work is small: a window of 64
+//     positions is 32 matrix instructions, after which its 16 x 64 outputs are finished (scale, bias,
+//     activation) and stored between the k-steps of the next window, where the vector ALU would idle.
+//   * The rows of a tile are 8 apart (row = w + 8 m for wavefront w).  A row of 196 fp32 outputs is 784
+//     bytes = 6 1/8 lines of 128 bytes, so rows 8 apart start at the same offset inside a line; the
+//     wavefront shifts its windows left by that offset and every 256-byte piece it stores is two whole
+//     lines.  With rows 4 apart pieces start on 64-byte boundaries only and half of them straddle lines;
+//     partially written lines cost the memory system a second access (9.24 -> 9.09 us).
+//
+// Wavefronts 4 .. 7 take their windows in descending order, so that at any time both ends of the rows are
+// being written rather than one column of the output (another 0.05 us).
+//
+// Reference semantics: out = act(fmaf(float(acc), scale, bias)) per output, int32 accumulation over all
+// channels (sparse_conv_impl.cc:1661-1685 computes the same sum over the nonzeros only; zeros add nothing to
+// an integer sum).
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <type_traits>
+
+#include "epilogue.h"
+#include "launch_lds.h"
+#include "sparse_conv_kernels.h"
+
+namespace pl {
+namespace {
+
+using epilogue::ActivateT;
+using epilogue::ActQuantF;
+using epilogue::DispatchAct;
+using epilogue::TruncPackI8x4;
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+
+constexpr int kRowStride = 8;  // rows of a tile: w + 8 m
+
+// 16 bytes written through to memory as streaming data (sc1 nt).  The wait state after the store keeps the data
+// registers intact until the store has read them (the compiler does not see a store inside the assembly
+// statement).
+__device__ __forceinline__ void StoreThrough(u4 v, void* p) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n s_nop 1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void StorePlain(u4 v, void* p) { *reinterpret_cast<u4*>(p) = v; }
+
+struct Lane {
+  int n;   // column of a 16x16 tile
+  int kq;  // quarter of the wavefront: channel group of an operand, rows 4 kq .. 4 kq + 3 of a result
+};
+
+template <int OUT, int ACT>
+__device__ __forceinline__ u4 Finish4(int a0, int a1, int a2, int a3, float s, float b, const DevAct& act) {
+  if (OUT == kOutAcc32) return u4{(uint32_t)a0, (uint32_t)a1, (uint32_t)a2, (uint32_t)a3};
+  const float v0 = __builtin_fmaf((float)a0, s, b), v1 = __builtin_fmaf((float)a1, s, b), v2 = __builtin_fmaf((float)a2, s, b), v3 = __builtin_fmaf((float)a3, s, b);
+  if (OUT == kOutI8) return u4{TruncPackI8x4(ActQuantF<ACT>(v0, act), ActQuantF<ACT>(v1, act), ActQuantF<ACT>(v2, act), ActQuantF<ACT>(v3, act)), 0u, 0u, 0u};
+  return u4{__float_as_uint(ActivateT<ACT>(v0, act)), __float_as_uint(ActivateT<ACT>(v1, act)), __float_as_uint(ActivateT<ACT>(v2, act)), __float_as_uint(ActivateT<ACT>(v3, act))};
+}
+
+// Row 4 kq + i of a window's results (positions 4 q .. 4 q + 3 per lane): epilogue and store.  `partial`: the
+// lane's line is shared with the end of the previous output row and merges in L2 (plain store).
+template <int OUT, int ACT>
+__device__ __forceinline__ void StoreRow(const v4i (&acc)[4], int i, float sc, float bi, const DevAct& act, char* __restrict__ orow, int hw, int q, bool partial, Lane ln) {
+  constexpr int kElem = OUT == kOutI8 ? 1 : 4;
+  const u4 v = Finish4<OUT, ACT>(acc[0][i], acc[1][i], acc[2][i], acc[3][i], sc, bi, act);
+  char* ptr = orow + ((size_t)(kRowStride * (4 * ln.kq + i)) * hw + 4 * q) * kElem;
+  if (OUT == kOutI8) {
+    if (q >= 0) *reinterpret_cast<uint32_t*>(ptr) = v.x;
+  } else if (partial) {
+    if (q >= 0) StorePlain(v, ptr);
+  } else {
+    StoreThrough(v, ptr);
+  }
+}
+
+// One window of 16 position quads times the wavefront's row tile.  When EPI, the four rows of the previous
+// window (accumulators accp, first quad qp) are finished and stored between the k-steps, one row per KS / 4
+// k-steps (all of them behind the last k-step when KS < 4).  The operand cells of two k-steps are in flight.
+template <int KS, int OUT, int ACT, bool EPI>
+__device__ __forceinline__ void Window(const uint4* __restrict__ xt, int kgs, int cps, int q0, const v4i (&a)[KS], v4i (&acc)[4], const v4i (&accp)[4], int qp, bool partialp, const float (&sc)[4],
+                                       const float (&bi)[4], const DevAct& act, char* __restrict__ orow, int hw, Lane ln) {
+  const uint4* bbase = xt + ln.kq * kgs + (q0 + ln.n);  // + ks * 4 * kgs + c * cps
+#pragma unroll
+  for (int c = 0; c < 4; ++c) acc[c] = v4i{0, 0, 0, 0};
+  constexpr int PF = 2;
+  constexpr int kStepsPerRow = KS >= 4 ? KS / 4 : 1;
+  uint4 bq[PF + 1][4];
+#pragma unroll
+  for (int d = 0; d < PF; ++d)
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      if (d < KS) bq[d][c] = bbase[d * 4 * kgs + c * cps];
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    if (ks + PF < KS) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) bq[(ks + PF) % (PF + 1)][c] = bbase[(ks + PF) * 4 * kgs + c * cps];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const uint4 u = bq[ks % (PF + 1)][c];
+      acc[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[ks], v4i{(int)u.x, (int)u.y, (int)u.z, (int)u.w}, acc[c], 0, 0, 0);
+    }
+    if (EPI && ks % kStepsPerRow == 0 && ks / kStepsPerRow < 4) {
+      const int i = ks / kStepsPerRow;
+      StoreRow<OUT, ACT>(accp, i, sc[i], bi[i], act, orow, hw, qp + ln.n, partialp && ln.n < kRowStride, ln);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (EPI && KS < 4) {
+#pragma unroll
+    for (int i = KS; i < 4; ++i) StoreRow<OUT, ACT>(accp, i, sc[i], bi[i], act, orow, hw, qp + ln.n, partialp && ln.n < kRowStride, ln);
+  }
+}
+
+// QPI: quads per image when known at compile time (49 = 14 x 14 maps), else 0: the LDS offsets of the cells
+// then become immediates.
+template <int KS, int OUT, int QPI>
+__global__ void __launch_bounds__(512) ImageRowsMfmaKernel(const ImageMfmaParams p) {
+  extern __shared__ uint4 lds_raw[];
+  // shifted windows read up to seven cells in front of a row of cells
+  uint4* xt = lds_raw + 16;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // a contiguous range of work items per XCD, the row groups of one image next to each other
+  const int item = (int)(blockIdx.x & 7u) * p.per_xcd + (int)(blockIdx.x >> 3);
+  if (item >= p.items) return;
+  const int n = item / p.row_groups, rg = item - n * p.row_groups;
+  const int qpi = QPI ? QPI : p.qpi, kgs = QPI ? (4 * QPI + 15) / 16 * 16 : p.kgs, hw = p.hw;
+  const int cps = qpi;  // cells of position c of every quad lie qpi cells apart
+  constexpr int NKG = 4 * KS, BPW = NKG / 8;
+  static_assert(NKG % 8 == 0, "channel groups are dealt evenly to the eight wavefronts");
+
+  // the image: dword (channel, quad) of the wavefront's channel groups, lane = quad
+  uint32_t r[BPW][16];
+  {
+    const uint32_t* x32 = reinterpret_cast<const uint32_t*>(p.x + (size_t)n * p.K * hw) + lane;
+    if (lane < qpi) {
+#pragma unroll
+      for (int u = 0; u < BPW; ++u)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) r[u][i] = x32[((wave * BPW + u) * 16 + i) * qpi];
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  // every channel group becomes four cells per quad; the weights of KS / BPW k-steps are requested behind it
+  char* lbase = reinterpret_cast<char*>(xt);
+  v4i a[KS];
+  const v4i* wt = static_cast<const v4i*>(p.wtiles) + ((size_t)(rg * 8 + wave) * KS) * 64 + lane;
+#pragma unroll
+  for (int u = 0; u < BPW; ++u) {
+    if (lane < qpi) {
+      // Two stages of byte permutes.  The second stage is done cell by cell so that the four dwords of a
+      // cell (one per block of four channels) are produced next to each other, where the 16-byte write
+      // wants them.
+      uint32_t lo[4][2], hi[4][2];
+#pragma unroll
+      for (int b4 = 0; b4 < 4; ++b4) {
+        lo[b4][0] = __builtin_amdgcn_perm(r[u][4 * b4 + 1], r[u][4 * b4], 0x05010400u);      // positions 0, 1 of channels 4 b4, 4 b4 + 1
+        hi[b4][0] = __builtin_amdgcn_perm(r[u][4 * b4 + 1], r[u][4 * b4], 0x07030602u);      // positions 2, 3
+        lo[b4][1] = __builtin_amdgcn_perm(r[u][4 * b4 + 3], r[u][4 * b4 + 2], 0x05010400u);  // the same of channels 4 b4 + 2, 4 b4 + 3
+        hi[b4][1] = __builtin_amdgcn_perm(r[u][4 * b4 + 3], r[u][4 * b4 + 2], 0x07030602u);
+      }
+      uint4* cells = reinterpret_cast<uint4*>(lbase + (wave * BPW + u) * (kgs * 16)) + lane;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+        uint4 cell;
+        cell.x = __builtin_amdgcn_perm((c & 2) ? hi[0][1] : lo[0][1], (c & 2) ? hi[0][0] : lo[0][0], sel);
+        cell.y = __builtin_amdgcn_perm((c & 2) ? hi[1][1] : lo[1][1], (c & 2) ? hi[1][0] : lo[1][0], sel);
+        cell.z = __builtin_amdgcn_perm((c & 2) ? hi[2][1] : lo[2][1], (c & 2) ? hi[2][0] : lo[2][0], sel);
+        cell.w = __builtin_amdgcn_perm((c & 2) ? hi[3][1] : lo[3][1], (c & 2) ? hi[3][0] : lo[3][0], sel);
+        cells[c * qpi] = cell;
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = u * (KS / BPW); ks < (u + 1) * (KS / BPW); ++ks) a[ks] = wt[ks * 64];
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  Lane ln;
+  ln.n = lane & 15;
+  ln.kq = lane >> 4;
+  const int row0 = rg * 128 + wave;  // the wavefront's rows: row0 + 8 m, m = 0 .. 15
+  float sc[4], bi[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    sc[i] = OUT == kOutAcc32 ? 0.f : p.scale[row0 + kRowStride * (4 * ln.kq + i)];
+    bi[i] = OUT == kOutAcc32 ? 0.f : p.bias[row0 + kRowStride * (4 * ln.kq + i)];
+  }
+  // row n of the tile (results of the swapped product)
+  const float sct = OUT == kOutAcc32 ? 0.f : p.scale[row0 + kRowStride * ln.n];
+  const float bit = OUT == kOutAcc32 ? 0.f : p.bias[row0 + kRowStride * ln.n];
+  __syncthreads();
+
+  // windows shifted left by sh quads so that fp32 / int32 row pieces start on 128-byte boundaries: output row
+  // r starts r * qpi quads into the tensor
+  const int sh = p.align ? ((row0 * qpi) & (kRowStride - 1)) : 0;
+  const int nqt = (qpi + sh) >> 4;       // full windows
+  const int left = qpi + sh - 16 * nqt;  // quads after the last window
+  const int ntail = (left + 3) >> 2;
+  constexpr int kElem = OUT == kOutI8 ? 1 : 4;
+  char* orow = static_cast<char*>(p.out) + ((size_t)n * p.M + row0) * hw * kElem;
+  DispatchAct(OUT == kOutAcc32 ? 0 : p.act.type, [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
+    if (nqt > 0) {
+      const bool descending = wave >= 4;
+      auto win = [&](int t) { return descending ? nqt - 1 - t : t; };
+      // the first line of window 0 holds the end of the previous output row when the window is shifted
+      auto partial = [&](int t) { return win(t) == 0 && sh > 0; };
+      v4i acc_a[4], acc_b[4];
+      Window<KS, OUT, ACT, false>(xt, kgs, cps, 16 * win(0) - sh, a, acc_a, acc_a, 0, false, sc, bi, p.act, orow, hw, ln);
+      int t = 1;
+      // two windows per round so that the accumulator sets alternate without copies
+      for (; t + 1 < nqt; t += 2) {
+        Window<KS, OUT, ACT, true>(xt, kgs, cps, 16 * win(t) - sh, a, acc_b, acc_a, 16 * win(t - 1) - sh, partial(t - 1), sc, bi, p.act, orow, hw, ln);
+        Window<KS, OUT, ACT, true>(xt, kgs, cps, 16 * win(t + 1) - sh, a, acc_a, acc_b, 16 * win(t) - sh, partial(t), sc, bi, p.act, orow, hw, ln);
+      }
+      if (t < nqt) {
+        Window<KS, OUT, ACT, true>(xt, kgs, cps, 16 * win(t) - sh, a, acc_b, acc_a, 16 * win(t - 1) - sh, partial(t - 1), sc, bi, p.act, orow, hw, ln);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) StoreRow<OUT, ACT>(acc_b, i, sc[i], bi[i], p.act, orow, hw, 16 * win(t) - sh + ln.n, partial(t) && ln.n < kRowStride, ln);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) StoreRow<OUT, ACT>(acc_a, i, sc[i], bi[i], p.act, orow, hw, 16 * win(t - 1) - sh + ln.n, partial(t - 1) && ln.n < kRowStride, ln);
+      }
+    }
+    // The quads the windows leave over, four at a time, operands swapped: rows of the product are positions
+    // (quad q0 + m / 4, position m % 4), columns are output rows; a lane ends with the four positions of quad
+    // q0 + kq of row n.  Their lines are shared with the start of the next output row: plain stores.
+    for (int t = 0; t < ntail; ++t) {
+      const int q0 = 16 * nqt - sh + 4 * t;
+      int tq = q0 + (ln.n >> 2);
+      if (tq > qpi - 1) tq = qpi - 1;  // rows past the end of the image row: any valid cell, results unused
+      if (tq < 0) tq = 0;              // likewise in front of it (rows shorter than a window, shifted left)
+      const uint4* tb = xt + ln.kq * kgs + (ln.n & 3) * cps + tq;
+      v4i acc = v4i{0, 0, 0, 0};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const uint4 u = tb[ks * 4 * kgs];
+        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)u.x, (int)u.y, (int)u.z, (int)u.w}, a[ks], acc, 0, 0, 0);
+      }
+      const int q = q0 + ln.kq;
+      if (q >= 0 && q < qpi) {
+        const u4 v = Finish4<OUT, ACT>(acc[0], acc[1], acc[2], acc[3], sct, bit, p.act);
+        char* ptr = orow + ((size_t)(kRowStride * ln.n) * hw + 4 * q) * kElem;
+        if (OUT == kOutI8) *reinterpret_cast<uint32_t*>(ptr) = v.x; else StorePlain(v, ptr);
+      }
+    }
+  });
+}
+
+template <int OUT>
+hipError_t ByKs(const ImageMfmaParams& q, dim3 grid, size_t lds, hipStream_t s) {
+  const dim3 block(512);
+  if (q.qpi == 49) {
+    switch (q.K / 64) {
+      case 2:
+        return LaunchWithLds(ImageRowsMfmaKernel<2, OUT, 49>, grid, block, lds, s, q);
+      case 4:
+        return LaunchWithLds(ImageRowsMfmaKernel<4, OUT, 49>, grid, block, lds, s, q);
+      case 8:
+        return LaunchWithLds(ImageRowsMfmaKernel<8, OUT, 49>, grid, block, lds, s, q);
+      default:
+        return hipErrorInvalidValue;
+    }
+  }
+  switch (q.K / 64) {
+    case 2:
+      return LaunchWithLds(ImageRowsMfmaKernel<2, OUT, 0>, grid, block, lds, s, q);
+    case 4:
+      return LaunchWithLds(ImageRowsMfmaKernel<4, OUT, 0>, grid, block, lds, s, q);
+    case 8:
+      return LaunchWithLds(ImageRowsMfmaKernel<8, OUT, 0>, grid, block, lds, s, q);
+    default:
+      return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace
+
+bool ImageRowsMfmaFits(int M, int K, int hw) {
+  if (M <= 0 || M % 128 != 0) return false;
+  if (K != 128 && K != 256 && K != 512) return false;
+  if (hw < 16 || hw > 256 || hw % 4 != 0) return false;
+  const int qpi = hw / 4, kgs = (4 * qpi + 15) / 16 * 16;
+  return 256 + (size_t)(K / 16) * kgs * 16 <= (size_t)kMaxLdsBytes;
+}
+
+hipError_t LaunchImageRowsMfma(int out_kind, const ImageMfmaParams& p, hipStream_t stream) {
+  if (p.batch <= 0) return hipSuccess;
+  if (!ImageRowsMfmaFits(p.M, p.K, p.hw)) return hipErrorInvalidValue;
+  // the image is read as dwords, the output written as 16-byte pieces
+  if (reinterpret_cast<uintptr_t>(p.x) % 4 != 0 || reinterpret_cast<uintptr_t>(p.out) % 16 != 0) return hipErrorInvalidValue;
+  ImageMfmaParams q = p;
+  q.qpi = p.hw / 4;
+  q.kgs = (4 * q.qpi + 15) / 16 * 16;  // a channel group's cells start on a 256-byte boundary: conflict-free operand reads
+  q.row_groups = p.M / 128;
+  const int64_t items = (int64_t)p.batch * q.row_groups;
+  if (items > (1 << 28)) return hipErrorInvalidValue;
+  q.items = (int)items;
+  q.per_xcd = (q.items + 7) / 8;
+  q.align = out_kind != kOutI8;
+  const size_t lds = 256 + (size_t)(p.K / 16) * q.kgs * 16;
+  const dim3 grid(8u * (uint32_t)q.per_xcd);
+  switch (out_kind) {
+    case kOutF32:
+      return ByKs<kOutF32>(q, grid, lds, stream);
+    case kOutI8:
+      return ByKs<kOutI8>(q, grid, lds, stream);
+    case kOutAcc32:
+      return ByKs<kOutAcc32>(q, grid, lds, stream);
+    default:
+      return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace pl

@@ -176,6 +176,7 @@ struct pl_sparse_conv_handle {
   DevBuf wtiles_rg;      // the same tiles in the channel order of the regrouping by transposing LDS reads (ic = 512)
   bool image_tr_regroup = true;
   DevBuf wtiles_tr;      // the same tiles in the channel order of the kernel with transposing LDS reads
+  DevBuf wtiles_rows;    // tiles of rows 8 apart, for the image kernel with one row tile per wavefront
   int image_kernel = 0;  // 0 by rule, 1 regrouping kernel, 2 transposing-read kernel
   // int8 handles prepared with PL_ALGO_AUTO hold several forms and choose per call
   bool auto_int8 = false;
@@ -188,7 +189,7 @@ struct pl_sparse_conv_handle {
   int padded_rows = 0;
 
   int64_t DeviceBytes() const {
-    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + cw_desc.bytes + cw_idx.bytes + cw_wts.bytes + hw_kidx.bytes + hw_wts.bytes + hw_bias.bytes + wblocks.bytes + kmask.bytes + wtiles.bytes + wtiles_rg.bytes + wtiles_tr.bytes + tw_stream.bytes + tw_first.bytes + tw_desc.bytes + scale.bytes + bias.bytes);
+    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + cw_desc.bytes + cw_idx.bytes + cw_wts.bytes + hw_kidx.bytes + hw_wts.bytes + hw_bias.bytes + wblocks.bytes + kmask.bytes + wtiles.bytes + wtiles_rg.bytes + wtiles_tr.bytes + wtiles_rows.bytes + tw_stream.bytes + tw_first.bytes + tw_desc.bytes + scale.bytes + bias.bytes);
   }
 };
 
@@ -544,6 +545,32 @@ int BuildImageMfma(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
   return PL_OK;
 }
 
+// The tiles of the image kernel with one row tile per wavefront: tile w (0 .. 7) of a row group holds rows
+// w + 8 m, m = 0 .. 15; [row group][w][k-step][64 lanes][16 bytes], lane l = row m = l % 16, channels
+// 64 ks + 16 (l / 16) .. + 15 (image_rows_kernels.hip).
+int BuildImageRowsMfma(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
+  const int kss = L.ic / 64;
+  std::vector<int8_t> tiles(static_cast<size_t>(L.oc) * L.ic, 0);
+  auto put = [&](int row, uint32_t c, uint32_t wbits) {
+    const int8_t w = static_cast<int8_t>(wbits & 0xffu);
+    if (w == 0) return;
+    const int rg = row / 128, rl = row % 128;
+    const int tile = rl & 7, m = rl >> 3;
+    const int ks = c >> 6, kk = c & 63;
+    const int lane = m + 16 * (kk >> 4), t = kk & 15;
+    tiles[(((static_cast<size_t>(rg) * 8 + tile) * kss + ks) * 64 + lane) * 16 + t] = w;
+  };
+  for (const pl::RowGroup& g : L.groups) {
+    for (uint32_t j = 0; j < g.count; ++j) {
+      put(g.row0, L.ic_index[g.first + j], L.w0[g.first + j]);
+      if (g.nrows == 2) put(g.row0 + 1, L.ic_index[g.first + j], L.w1[g.first + j]);
+    }
+  }
+  const hipError_t e = h->wtiles_rows.Upload(tiles.data(), tiles.size());
+  if (e != hipSuccess) return FailHip(e, "uploading the weight tiles");
+  return PL_OK;
+}
+
 // The same tiles for the regrouping image kernel where it regroups by transposing LDS reads: byte b of
 // lane group g of k-step ks is channel 64 ks + 4 (8 (g % 2) + b % 8) + 2 (b / 8) + g / 2 (image_mfma_kernels.hip).
 int BuildImageMfmaTrRegroup(const pl::DecodedLayout& L, pl_sparse_conv_handle* h) {
@@ -708,7 +735,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   if (tune.reserved != 0) return Fail(PL_ERR_BAD_ARG, "pl_sparse_conv_tuning.reserved must be 0");
   for (int32_t sw : {tune.mfma_stream, tune.mfma_sub_tiles, tune.walk_tiled, tune.walk_chunked, tune.image_tr_regroup})
     if (sw < PL_TUNE_RULE || sw > PL_TUNE_ALWAYS) return Fail(PL_ERR_BAD_ARG, "a tuning switch is not PL_TUNE_RULE, PL_TUNE_NEVER or PL_TUNE_ALWAYS");
-  if (tune.image_kernel < 0 || tune.image_kernel > 2) return Fail(PL_ERR_BAD_ARG, "tuning.image_kernel must be 0, 1 or 2");
+  if (tune.image_kernel < 0 || tune.image_kernel > 3) return Fail(PL_ERR_BAD_ARG, "tuning.image_kernel must be 0, 1, 2 or 3");
   if (desc->kind < PL_KIND_FP32 || desc->kind > PL_KIND_FP16) return Fail(PL_ERR_BAD_ARG, "unknown kind %d", desc->kind);
   if (desc->algo < PL_ALGO_AUTO || desc->algo > PL_ALGO_IMAGE_MFMA) return Fail(PL_ERR_BAD_ARG, "unknown algo %d", desc->algo);
   if (desc->oc <= 0 || desc->ic <= 0 || desc->im_size <= 0) return Fail(PL_ERR_BAD_ARG, "oc, ic and im_size must be positive");
@@ -821,6 +848,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   if (rc == PL_OK && (algo == PL_ALGO_IMAGE_MFMA || (h->auto_int8 && (pl::ImageMfmaFits(desc->oc, desc->ic, 16) || pl::ImageMfmaFits(desc->oc, desc->ic, 49))))) rc = BuildImageMfma(L, h);
   if (rc == PL_OK && h->wtiles.ptr && pl::ImageTrMfmaFits(desc->oc, desc->ic, 20)) rc = BuildImageTrMfma(L, h);
   if (rc == PL_OK && h->wtiles.ptr && pl::ImageMfmaRegroupsByTransposingReads(desc->ic, 196)) rc = BuildImageMfmaTrRegroup(L, h);
+  if (rc == PL_OK && h->wtiles.ptr && pl::ImageRowsMfmaFits(desc->oc, desc->ic, 16)) rc = BuildImageRowsMfma(L, h);
   if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8) rc = BuildChunkWalk(L, h);
   if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8 && !half) rc = BuildTileWalk(L, desc->bias, h);
   if (rc == PL_OK) {
@@ -929,10 +957,17 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     // The kernel with transposing LDS reads runs on request only: on 64 x 512 -> 512 @14x14 it is about 4 %
     // slower than the kernel that regroups the image (9.9 against 9.7 us).
     const bool tr_fits = h->wtiles_tr.ptr != nullptr && pl::ImageTrMfmaFits(h->oc, h->ic, im_size);
+    // One row tile per wavefront and the image through registers: the rule wherever it applies (every shape of
+    // the image algorithm but the 7 x 7 maps).
+    const bool rows_fits = h->wtiles_rows.ptr != nullptr && pl::ImageRowsMfmaFits(h->oc, h->ic, im_size);
+    if (h->image_kernel == 3 && !rows_fits) return Fail(PL_ERR_UNSUPPORTED, "the image kernel with one row tile per wavefront takes no 7 x 7 maps (H*W = %d, ic = %d)", im_size, h->ic);
     if (h->image_kernel == 2 && !tr_fits) return Fail(PL_ERR_UNSUPPORTED, "the image kernel with transposing LDS reads needs H*W = 4 (mod 8) from 20 on, ic = 128, 256 or 512 and an image that leaves 41 KB of LDS free (H*W = %d, ic = %d)", im_size, h->ic);
     if (tr_fits && h->image_kernel == 2) {
       p.wtiles = h->wtiles_tr.ptr;
       e = pl::LaunchImageTrMfma(OutKind(h->kind), p, s);
+    } else if (rows_fits && (h->image_kernel == 0 || h->image_kernel == 3)) {
+      p.wtiles = h->wtiles_rows.ptr;
+      e = pl::LaunchImageRowsMfma(OutKind(h->kind), p, s);
     } else {
       p.tr_regroup = h->image_tr_regroup && h->wtiles_rg.ptr != nullptr && pl::ImageMfmaRegroupsByTransposingReads(h->ic, im_size);
       p.wtiles = p.tr_regroup ? h->wtiles_rg.ptr : h->wtiles.ptr;

@@ -279,6 +279,13 @@ hipError_t LaunchImageMfma(int out_kind, const ImageMfmaParams& p, hipStream_t s
 // 128 (step / 2) + step % 2 + 64 (b / 8) + 4 (8 (g % 2) + b % 8) + 2 (g / 2), g = l / 16.
 // M a multiple of 128, K = 128, 256 or 512, hw = 4 (mod 8) from 20 on and
 // the image plus 41 KB of staging buffers within the LDS of a CU.
+// The image kernel with one row tile (rows 8 apart) per wavefront and the image brought in through registers
+// (image_rows_kernels.hip): wtiles = [row group][tile w = 0 .. 7][k-step][64 lanes][16 bytes], lane l of tile w
+// holds row w + 8 (l % 16), channels 64 ks + 16 (l / 16) .. + 15.  M a multiple of 128, K = 128, 256 or 512, hw a
+// multiple of 4 in [16, 256] and the image's cells within the LDS of a CU; x 4-byte and out 16-byte aligned.
+bool ImageRowsMfmaFits(int M, int K, int hw);
+hipError_t LaunchImageRowsMfma(int out_kind, const ImageMfmaParams& p, hipStream_t stream);
+
 bool ImageTrMfmaFits(int M, int K, int hw);
 // Needs ImageTrMfmaFits and 16-byte aligned x / out.
 hipError_t LaunchImageTrMfma(int out_kind, const ImageMfmaParams& p, hipStream_t stream);

@@ -45,7 +45,8 @@ SHAPES = [
     (1, 512, 128, 16, 16), (3, 128, 256, 4, 4), (2, 256, 128, 5, 8), (2, 128, 128, 4, 7), (1, 512, 128, 9, 12), (9, 256, 128, 2, 10),
     (2, 512, 128, 4, 59), (1, 256, 128, 12, 21), (1, 128, 256, 6, 6), (2, 256, 128, 4, 11), (3, 128, 128, 4, 13),
 ]
-IMAGE_KERNELS = {"regroup": capi.IMAGE_KERNEL_REGROUP, "transpose": capi.IMAGE_KERNEL_TRANSPOSE}
+IMAGE_KERNELS = {"regroup": capi.IMAGE_KERNEL_REGROUP, "transpose": capi.IMAGE_KERNEL_TRANSPOSE, "rows": capi.IMAGE_KERNEL_ROWS}
+REGROUP = capi.tuning(image_kernel=capi.IMAGE_KERNEL_REGROUP)
 # the regrouping kernel regroups 512-channel 14 x 14 images by transposing LDS reads unless told otherwise
 VALU_REGROUP = capi.tuning(image_kernel=capi.IMAGE_KERNEL_REGROUP, image_tr_regroup=capi.TUNE_NEVER)
 
@@ -90,7 +91,7 @@ def test_image_mfma_regroup_by_transposing_reads(kind, act):
     case.dense[3, 0::2] = 0
     case.dense[4, 1::2] = 0
     case.dense[9] = 0
-    got = run_hip(case, capi.ALGO_IMAGE_MFMA)
+    got = run_hip(case, capi.ALGO_IMAGE_MFMA, tuning=REGROUP)
     assert_same(case, got, run_oracle(case, oracle_pack(case)), "tr regroup %s %s" % (kind, act))
     assert np.array_equal(got, run_hip(case, capi.ALGO_IMAGE_MFMA, tuning=VALU_REGROUP))
 
@@ -176,7 +177,8 @@ def test_image_mfma_activations_and_structures(paired, out_int8, act):
         assert_same(case, got, want, "image %s %s" % (name, act))
 
 
-def test_image_mfma_transposing_kernel_extremes_and_surroundings():
+@pytest.mark.parametrize("image_kernel", ["transpose", "rows"])
+def test_image_mfma_shifted_window_kernels_extremes_and_surroundings(image_kernel):
     """Largest magnitudes (accumulators of 512 x 127 x 127 of either sign), an
     empty output row, channels of one parity only, and the bytes around the
     output tensor stay untouched (the windows of a row class reach in front of
@@ -185,8 +187,8 @@ def test_image_mfma_transposing_kernel_extremes_and_surroundings():
 
     import torch
 
-    announce("image transpose extremes")
-    tr = capi.tuning(image_kernel=capi.IMAGE_KERNEL_TRANSPOSE)
+    announce("image extremes", image_kernel)
+    tr = capi.tuning(image_kernel=IMAGE_KERNELS[image_kernel])
     case = case_for(capi.KIND_INT8_ACC32, 3, 512, 128, 14, 14, 0.5, False, AP(), seed=21)
     case.dense[7] = 0
     case.dense[64:66] = 127
