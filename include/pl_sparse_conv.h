@@ -79,9 +79,9 @@ enum {
  *                     7 x 7 maps with ic = 256 / 512 / 1024 (two images per
  *                     workgroup)
  * With PL_ALGO_AUTO an int8 handle holds every form its shape allows and
- * chooses per call by batch and H*W (the image kernel where it applies, the
- * row walk for at most 256 positions in all on maps other than 7 x 7, the
- * block kernel otherwise): see pl_sparse_conv_algo_for(). */
+ * chooses per call by batch and H*W (the image kernels where they apply, else
+ * the row walk for at most 256 positions in all, else the block kernel): see
+ * pl_sparse_conv_algo_for(). */
 enum { PL_ALGO_AUTO = 0, PL_ALGO_ROW_WALK = 1, PL_ALGO_BLOCK_MFMA = 2, PL_ALGO_IMAGE_MFMA = 3 };
 
 /* Activation constants, used as given (replaces the fields of

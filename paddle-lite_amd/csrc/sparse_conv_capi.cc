@@ -686,20 +686,19 @@ pl::WalkConfig ChooseWalk(const pl_sparse_conv_handle* h, uint32_t P) {
 // The algorithm one call uses.  Handles prepared for one algorithm use it.  An int8 handle prepared with
 // PL_ALGO_AUTO holds the forms of every algorithm its shape allows and picks per call, by what was measured on
 // the pointwise shapes of MobileNetV1 at 1 to 64 images per launch:
-//  * the image kernel wherever its shape conditions hold (it ties with or beats the block kernel from 4 work
-//    items on, by 2x on 7 x 7 maps at any batch) - except
-//  * the row walk for at most 256 positions in all on maps other than 7 x 7 (one 14 x 14 image: a handful of
-//    image-kernel workgroups each walk a long dependent chain, the walk spreads the rows over the chip;
-//    5.97 against 7.2 us with 512 channels), and
-//  * the block kernel otherwise.
-// tuning.image_min_items raises the number of (image, 128-row group) work items the image kernel asks for.
+//  * the image kernels wherever their shape conditions hold: they tie with or beat the block kernel at every
+//    batch (by 2x on 7 x 7 maps, where the block kernel has too few tiles for the chip), and stay within 10 % of
+//    the row walk on a single 14 x 14 image of 512 channels, the one case where the walk is ahead;
+//  * else the row walk for at most 256 positions in all (it spreads the output rows over the chip where the
+//    block kernel would have one or two tiles);
+//  * else the block kernel.
+// tuning.image_min_items raises the number of (image, 128-row group) work items the image kernels ask for.
 int AlgoForCall(const pl_sparse_conv_handle* h, int batch, int im_size, bool aligned16) {
   if (!h->auto_int8) return h->algo;
-  const int64_t positions = static_cast<int64_t>(batch) * im_size;
-  if (h->auto_walk && im_size != 49 && positions <= 256) return PL_ALGO_ROW_WALK;
   // work items: (image, row group), for 7 x 7 maps (pair of images, row group)
   const int64_t image_items = static_cast<int64_t>(im_size == 49 ? (batch + 1) / 2 : batch) * (h->oc / 128);
   if (h->wtiles.ptr && aligned16 && pl::ImageMfmaFits(h->oc, h->ic, im_size) && image_items >= h->image_min_items) return PL_ALGO_IMAGE_MFMA;
+  if (h->auto_walk && static_cast<int64_t>(batch) * im_size <= 256) return PL_ALGO_ROW_WALK;
   return h->algo;
 }
 

@@ -246,7 +246,7 @@ def test_auto_picks_the_image_kernel_only_where_it_applies():
     kernel, _ = make_kernel(case, capi.ALGO_AUTO)
     assert L.pl_sparse_conv_algo_for(kernel._handle, 64, 196) == capi.ALGO_IMAGE_MFMA
     assert L.pl_sparse_conv_algo_for(kernel._handle, 2, 196) == capi.ALGO_IMAGE_MFMA      # from two images on
-    assert L.pl_sparse_conv_algo_for(kernel._handle, 1, 196) == capi.ALGO_ROW_WALK        # at most 256 positions in all: the walk
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 1, 196) == capi.ALGO_IMAGE_MFMA      # and for a single one
     assert L.pl_sparse_conv_algo_for(kernel._handle, 64, 49) == capi.ALGO_IMAGE_MFMA      # 7x7 maps: pairs of images
     assert L.pl_sparse_conv_algo_for(kernel._handle, 1, 49) == capi.ALGO_IMAGE_MFMA       # at any batch
     assert L.pl_sparse_conv_algo_for(kernel._handle, 64, 50) == capi.ALGO_BLOCK_MFMA      # not a multiple of 4
@@ -256,6 +256,7 @@ def test_auto_picks_the_image_kernel_only_where_it_applies():
     picky, _ = make_kernel(case, capi.ALGO_AUTO, tuning=capi.tuning(image_min_items=128))
     assert L.pl_sparse_conv_algo_for(picky._handle, 64, 196) == capi.ALGO_IMAGE_MFMA
     assert L.pl_sparse_conv_algo_for(picky._handle, 2, 196) == capi.ALGO_BLOCK_MFMA
+    assert L.pl_sparse_conv_algo_for(picky._handle, 1, 196) == capi.ALGO_ROW_WALK         # 196 positions in all
     assert L.pl_sparse_conv_algo_for(picky._handle, 32, 49) == capi.ALGO_BLOCK_MFMA
     # the same handle serves all of them
     import torch
