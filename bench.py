@@ -84,6 +84,7 @@ def parse():
     ap.add_argument("--seed", type=int, default=0, help="custom: seed of the synthetic tensors")
     ap.add_argument("--fp16", action="store_true", help="run an fp32 configuration (c1, c2) through the half-precision kernel")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-lite-program", action="store_true", help="mobilenet: skip the measurement of the C++ operator surface (a child process; left out under a profiler)")
     ap.add_argument("--cache-resident", action="store_true", help="reuse one buffer set (reported, never the headline)")
     ap.add_argument("--copy-calibration", action="store_true", help="also launch a plain 64 MiB device copy 20 times, the known-size kernel that counter runs scale FETCH_SIZE / WRITE_SIZE by")
     return ap.parse_args()
@@ -673,8 +674,8 @@ def run_mobilenet(args):
     dw_us = sum(p["kernel_us"] for p in per_layer if p["kind"] == "depthwise")
     pw_us = sum(p["kernel_us"] for p in per_layer if p["kind"] == "pointwise")
     print(json.dumps({
-        "lite_program": run_lite_program_bench(batch),
-        "lite_program_batch_1": run_lite_program_bench(1),
+        "lite_program": None if args.no_lite_program else run_lite_program_bench(batch),
+        "lite_program_batch_1": None if args.no_lite_program else run_lite_program_bench(1),
         "metric": "MobileNetV1-1.0 convolutional body, int8, batch 64: images/s of the 26-launch sequence",
         "value": batch * steps / wall,
         "unit": "images/s",
