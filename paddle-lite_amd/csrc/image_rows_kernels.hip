@@ -21,8 +21,9 @@
 //     lines.  With rows 4 apart pieces start on 64-byte boundaries only and half of them straddle lines;
 //     partially written lines cost the memory system a second access (9.24 -> 9.09 us).
 //
-// Wavefronts 4 .. 7 take their windows in descending order, so that at any time both ends of the rows are
-// being written rather than one column of the output (another 0.05 us).
+// Wavefront w starts with window w mod (windows per row) and goes round from there, so that at any time all
+// parts of the rows are being written rather than one column of the output (all wavefronts ascending 9.9 - 10.4 us,
+// the upper four descending 9.23, going round 9.09 in one run).
 //
 // Reference semantics: out = act(fmaf(float(acc), scale, bias)) per output, int32 accumulation over all
 // channels (sparse_conv_impl.cc:1661-1685 computes the same sum over the nonzeros only; zeros add nothing to
@@ -49,11 +50,12 @@ typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 
 constexpr int kRowStride = 8;  // rows of a tile: w + 8 m
 
-// 16 bytes written through to memory as streaming data (sc1 nt).  The wait state after the store keeps the data
+// 16 bytes stored as streaming data (nt).  Measured on the metric shape with this kernel's whole-line pieces: nt
+// 8.93 us, sc1 nt 9.05, sc0 sc1 nt 9.06, sc1 10.9, no policy 11.9.  The wait state after the store keeps the data
 // registers intact until the store has read them (the compiler does not see a store inside the assembly
 // statement).
 __device__ __forceinline__ void StoreThrough(u4 v, void* p) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n s_nop 1" ::"v"(p), "v"(v) : "memory");
+  asm volatile("global_store_dwordx4 %0, %1, off nt\n s_nop 1" ::"v"(p), "v"(v) : "memory");
 }
 __device__ __forceinline__ void StorePlain(u4 v, void* p) { *reinterpret_cast<u4*>(p) = v; }
 
@@ -218,8 +220,8 @@ __global__ void __launch_bounds__(512) ImageRowsMfmaKernel(const ImageMfmaParams
   DispatchAct(OUT == kOutAcc32 ? 0 : p.act.type, [&](auto act_c) {
     constexpr int ACT = decltype(act_c)::value;
     if (nqt > 0) {
-      const bool descending = wave >= 4;
-      auto win = [&](int t) { return descending ? nqt - 1 - t : t; };
+      // wavefront w starts with window w mod nqt and goes round from there
+      auto win = [&](int t) { return (t + wave) % nqt; };
       // the first line of window 0 holds the end of the previous output row when the window is shifted
       auto partial = [&](int t) { return win(t) == 0 && sh > 0; };
       v4i acc_a[4], acc_b[4];
