@@ -50,14 +50,21 @@ typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 
 constexpr int kRowStride = 8;  // rows of a tile: w + 8 m
 
-// 16 bytes stored as streaming data (nt).  Measured on the metric shape with this kernel's whole-line pieces: nt
-// 8.93 us, sc1 nt 9.05, sc0 sc1 nt 9.06, sc1 10.9, no policy 11.9.  The wait state after the store keeps the data
-// registers intact until the store has read them (the compiler does not see a store inside the assembly
-// statement).
-__device__ __forceinline__ void StoreThrough(u4 v, void* p) {
-  asm volatile("global_store_dwordx4 %0, %1, off nt\n s_nop 1" ::"v"(p), "v"(v) : "memory");
+// 16 bytes stored as streaming data (nt) at a wave-uniform base plus an unsigned 32-bit lane offset (no 64-bit
+// address arithmetic per store).  Measured on the metric shape with this kernel's whole-line pieces: nt 8.93 us,
+// sc1 nt 9.05, sc0 sc1 nt 9.06, sc1 10.9, no policy 11.9.  The wait state after the store keeps the data registers
+// intact until the store has read them (the compiler does not see a store inside the assembly statement).
+__device__ __forceinline__ void StoreStreaming(u4 v, char* base, uint32_t off) {
+  asm volatile("global_store_dwordx4 %0, %1, %2 nt\n s_nop 1" ::"v"(off), "v"(v), "s"(base) : "memory");
 }
 __device__ __forceinline__ void StorePlain(u4 v, void* p) { *reinterpret_cast<u4*>(p) = v; }
+// A pointer that is the same in every lane, as a scalar register pair (the halves are taken as unsigned: a low
+// half with its top bit set must not be sign-extended into the high half).
+__device__ __forceinline__ char* Uniform(char* p) {
+  const uint64_t a = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a), hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32));
+  return reinterpret_cast<char*>(((uint64_t)hi << 32) | (uint64_t)lo);
+}
 
 struct Lane {
   int n;   // column of a 16x16 tile
@@ -78,13 +85,15 @@ template <int OUT, int ACT>
 __device__ __forceinline__ void StoreRow(const v4i (&acc)[4], int i, float sc, float bi, const DevAct& act, char* __restrict__ orow, int hw, int q, bool partial, Lane ln) {
   constexpr int kElem = OUT == kOutI8 ? 1 : 4;
   const u4 v = Finish4<OUT, ACT>(acc[0][i], acc[1][i], acc[2][i], acc[3][i], sc, bi, act);
-  char* ptr = orow + ((size_t)(kRowStride * (4 * ln.kq + i)) * hw + 4 * q) * kElem;
+  // at most 128 rows of at most 256 four-byte positions behind orow: the offset fits 32 bits; it is negative only
+  // for the quads in front of a row, which are not stored
+  const int off = ((kRowStride * (4 * ln.kq + i)) * hw + 4 * q) * kElem;
   if (OUT == kOutI8) {
-    if (q >= 0) *reinterpret_cast<uint32_t*>(ptr) = v.x;
+    if (q >= 0) *reinterpret_cast<uint32_t*>(orow + off) = v.x;
   } else if (partial) {
-    if (q >= 0) StorePlain(v, ptr);
+    if (q >= 0) StorePlain(v, orow + off);
   } else {
-    StoreThrough(v, ptr);
+    StoreStreaming(v, orow, (uint32_t)off);
   }
 }
 
@@ -150,12 +159,16 @@ __global__ void __launch_bounds__(512) ImageRowsMfmaKernel(const ImageMfmaParams
   // the image: dword (channel, quad) of the wavefront's channel groups, lane = quad
   uint32_t r[BPW][16];
   {
-    const uint32_t* x32 = reinterpret_cast<const uint32_t*>(p.x + (size_t)n * p.K * hw) + lane;
+    // one address per channel group, the channel's offset in the instruction (16 rows of at most 256 bytes)
+    const char* ximg = reinterpret_cast<const char*>(p.x) + (size_t)n * p.K * hw + lane * 4;
+    const int row_bytes = QPI ? 4 * QPI : hw;
     if (lane < qpi) {
 #pragma unroll
-      for (int u = 0; u < BPW; ++u)
+      for (int u = 0; u < BPW; ++u) {
+        const char* group = ximg + (size_t)((wave * BPW + u) * 16) * row_bytes;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) r[u][i] = x32[((wave * BPW + u) * 16 + i) * qpi];
+        for (int i = 0; i < 16; ++i) r[u][i] = *reinterpret_cast<const uint32_t*>(group + i * row_bytes);
+      }
     }
   }
   __builtin_amdgcn_sched_barrier(0);
@@ -216,8 +229,8 @@ __global__ void __launch_bounds__(512) ImageRowsMfmaKernel(const ImageMfmaParams
   const int left = qpi + sh - 16 * nqt;  // quads after the last window
   const int ntail = (left + 3) >> 2;
   constexpr int kElem = OUT == kOutI8 ? 1 : 4;
-  char* orow = static_cast<char*>(p.out) + ((size_t)n * p.M + row0) * hw * kElem;
-  DispatchAct(OUT == kOutAcc32 ? 0 : p.act.type, [&](auto act_c) {
+  char* orow = Uniform(static_cast<char*>(p.out) + ((size_t)n * p.M + row0) * hw * kElem);
+  DispatchAct(OUT == kOutAcc32 ? 0 : epilogue::LeakyAsMax(p.act), [&](auto act_c) {
     constexpr int ACT = decltype(act_c)::value;
     if (nqt > 0) {
       // wavefront w starts with window w mod nqt and goes round from there
