@@ -67,7 +67,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib", "mobilenet", "density-sweep", "floors", "store-shapes", "custom", "small-batch"])
+    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib", "mobilenet", "density-sweep", "floors", "store-shapes", "device-rates", "custom", "small-batch"])
     ap.add_argument("--algo", default="auto", choices=["auto", "walk", "mfma", "image"])
     ap.add_argument("--image-kernel", default="rule", choices=["rule", "regroup", "transpose", "rows"], help="which image MFMA kernel a handle uses where both apply (pl_sparse_conv_tuning.image_kernel)")
     ap.add_argument("--image-regroup", default="rule", choices=["rule", "valu"], help="regrouping image kernel: by transposing LDS reads where that exists (rule) or by the vector ALU everywhere (pl_sparse_conv_tuning.image_tr_regroup)")
@@ -327,6 +327,70 @@ def load_probes():
     if not os.path.exists(bp.LIB_PATH):
         bp.build()
     return C.CDLL(bp.LIB_PATH)
+
+
+def run_device_rates(args):
+    """Instruction rates of a CU measured with the probes of bench_probes/rate_probes.hip: LDS reads and writes by
+    width and access pattern (bytes per clock and CU), the int8 matrix instruction and the fp32 multiply-add (clocks
+    per instruction and SIMD), and the launch-to-launch time of an empty grid.  One workgroup per CU; medians over
+    the wavefronts of the third launch."""
+    import numpy as np
+    import torch
+
+    P = load_probes()
+    P.pl_probe_lds_rate.restype = C.c_int
+    P.pl_probe_lds_rate.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_longlong)]
+    P.pl_probe_alu_rate.restype = C.c_int
+    P.pl_probe_alu_rate.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_longlong)]
+    out = torch.zeros(256 * 8 * 2, dtype=torch.int64, device="cuda")
+    sink = torch.zeros(16, dtype=torch.int32, device="cuda")
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    lds_names = ["ds_read_b128, 1 KB contiguous per instruction", "ds_read_b64", "ds_read_b32", "ds_read_b64_tr_b8", "ds_write_b128", "ds_write_b64",
+                 "ds_read_b128, operand cells: 16 cells per quarter wavefront, quarters 3328 B apart", "ds_read_b128, the same with quarters 3392 B apart"]
+    lds = {}
+    for mode, name in enumerate(lds_names):
+        n = C.c_longlong(0)
+        for _ in range(3):
+            rc = P.pl_probe_lds_rate(mode, out.data_ptr(), sink.data_ptr(), stream, C.byref(n))
+            if rc != 0:
+                raise RuntimeError("pl_probe_lds_rate(%d) failed with HIP error %d" % (mode, rc))
+        torch.cuda.synchronize()
+        counts = out.cpu().numpy().reshape(256, 8, 2)
+        wg = np.median(counts[:, :, 1].max(axis=1))  # a workgroup is through when its slowest wavefront is
+        lds[name] = round(8.0 * n.value / wg, 1)
+    alu_names = ["v_mfma_i32_16x16x64_i8, independent", "v_mfma_i32_16x16x64_i8, dependent chain", "v_fma_f32, independent", "4 x (v_mfma + 2 v_fma_f32): per matrix instruction"]
+    alu = {}
+    ticks = []
+    for mode, name in enumerate(alu_names):
+        for waves in (4, 8):
+            n = C.c_longlong(0)
+            for _ in range(3):
+                rc = P.pl_probe_alu_rate(mode, waves, out.data_ptr(), sink.data_ptr(), stream, C.byref(n))
+                if rc != 0:
+                    raise RuntimeError("pl_probe_alu_rate(%d) failed with HIP error %d" % (mode, rc))
+            torch.cuda.synchronize()
+            counts = out.cpu().numpy()[:256 * waves * 2].reshape(256 * waves, 2)
+            clk, ns = float(np.median(counts[:, 0])), float(np.median(counts[:, 1])) * 10.0
+            per_simd = waves // 4
+            alu["%s, %d wavefront%s per SIMD" % (name, per_simd, "s" if per_simd > 1 else "")] = {"clocks_per_instruction_and_SIMD": round(clk / (n.value * per_simd), 2),
+                                                                                           "ns_per_instruction_and_SIMD": round(ns / (n.value * per_simd), 2)}
+            ticks.append(clk / ns)
+    # empty grid, launch to launch
+    P.pl_probe_floor.restype = C.c_int
+    P.pl_probe_floor.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_float)]
+    x = torch.zeros(64 * 512 * 196, dtype=torch.int8, device="cuda")
+    o = torch.zeros(64 * 512 * 196, dtype=torch.float32, device="cuda")
+    xp, op = (C.c_void_p * 1)(x.data_ptr()), (C.c_void_p * 1)(o.data_ptr())
+    ms = C.c_float(0.0)
+    for n in (2000, 4000):
+        rc = P.pl_probe_floor(0, xp, op, 1, 64, 512, 512, 196, n, stream, C.byref(ms))
+        if rc != 0:
+            raise RuntimeError("pl_probe_floor failed with HIP error %d" % rc)
+    print(json.dumps({"metric": "instruction rates of one CU (one workgroup of eight wavefronts per CU)", "n_gpus": 1, "data": "synthetic",
+                      "config": {"workload": "device_rates", "grid": "256 workgroups"},
+                      "lds_bytes_per_clock_and_CU": lds, "alu": alu, "s_memtime_counts_per_ns": round(float(np.median(ticks)), 2),
+                      "empty_grid_256x512_us_launch_to_launch": round(ms.value * 1e3 / 4000, 2)}))
+    return 0
 
 
 def run_store_shapes(args):
@@ -714,6 +778,8 @@ def main():
         return run_floors(args)
     if args.config == "store-shapes":
         return run_store_shapes(args)
+    if args.config == "device-rates":
+        return run_device_rates(args)
     if args.config == "c5":
         return run_c5(args)
     if args.config == "calib":

@@ -1,5 +1,5 @@
-"""Builds bench_probes/libpl_probe.so from floor_probes.hip (hipcc, gfx950): the probes measure launch,
-memory and store-pattern floors for bench.py; nothing of the operator links them.  build_programs() builds
+"""Builds bench_probes/libpl_probe.so from floor_probes.hip and rate_probes.hip (hipcc, gfx950): the probes measure
+launch, memory and store-pattern floors and instruction rates for bench.py; nothing of the operator links them.  build_programs() builds
 bench_probes/lite_program_bench, the host-cost and graph-replay measurement of the C++ operator surface
 (it links the package's two libraries, so they are built first)."""
 import os
@@ -13,7 +13,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
 
 def build(verbose=False):
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    cmd = [exe] + FLAGS + ["-x", "hip", "-shared", os.path.join(HERE, "floor_probes.hip"), "-o", LIB_PATH]
+    cmd = [exe] + FLAGS + ["-x", "hip", "-shared", os.path.join(HERE, "floor_probes.hip"), os.path.join(HERE, "rate_probes.hip"), "-o", LIB_PATH]
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if verbose:
         print(" ".join(cmd), flush=True)
