@@ -141,17 +141,22 @@ __device__ __forceinline__ void Window(const uint4* __restrict__ xt, int kgs, in
 
 // QPI: quads per image when known at compile time (49 = 14 x 14 maps), else 0: the LDS offsets of the cells
 // then become immediates.
+//
+// The arguments in front of the parameter block repeat the fields that the first loads of a wavefront need.
+// Leading scalar arguments reach a wavefront in registers (kernel-argument preload, switched on for this file
+// by the build); the block behind them is fetched from memory, which the image loads would otherwise wait for.
 template <int KS, int OUT, int QPI>
-__global__ void __launch_bounds__(512) ImageRowsMfmaKernel(const ImageMfmaParams p) {
+__global__ void __launch_bounds__(512) ImageRowsMfmaKernel(const int8_t* x, const void* wtiles, void* out, int per_xcd, int items,
+                                                           int row_groups, int K, int hw_arg, int M, const ImageMfmaParams p) {
   extern __shared__ uint4 lds_raw[];
   // shifted windows read up to seven cells in front of a row of cells
   uint4* xt = lds_raw + 16;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // a contiguous range of work items per XCD, the row groups of one image next to each other
-  const int item = (int)(blockIdx.x & 7u) * p.per_xcd + (int)(blockIdx.x >> 3);
-  if (item >= p.items) return;
-  const int n = item / p.row_groups, rg = item - n * p.row_groups;
-  const int qpi = QPI ? QPI : p.qpi, kgs = QPI ? (4 * QPI + 15) / 16 * 16 : p.kgs, hw = p.hw;
+  const int item = (int)(blockIdx.x & 7u) * per_xcd + (int)(blockIdx.x >> 3);
+  if (item >= items) return;
+  const int n = item / row_groups, rg = item - n * row_groups;
+  const int qpi = QPI ? QPI : p.qpi, kgs = QPI ? (4 * QPI + 15) / 16 * 16 : p.kgs, hw = hw_arg;
   const int cps = qpi;  // cells of position c of every quad lie qpi cells apart
   constexpr int NKG = 4 * KS, BPW = NKG / 8;
   static_assert(NKG % 8 == 0, "channel groups are dealt evenly to the eight wavefronts");
@@ -160,7 +165,7 @@ __global__ void __launch_bounds__(512) ImageRowsMfmaKernel(const ImageMfmaParams
   uint32_t r[BPW][16];
   {
     // one address per channel group, the channel's offset in the instruction (16 rows of at most 256 bytes)
-    const char* ximg = reinterpret_cast<const char*>(p.x) + (size_t)n * p.K * hw + lane * 4;
+    const char* ximg = reinterpret_cast<const char*>(x) + (size_t)n * K * hw + lane * 4;
     const int row_bytes = QPI ? 4 * QPI : hw;
     if (lane < qpi) {
 #pragma unroll
@@ -175,7 +180,7 @@ __global__ void __launch_bounds__(512) ImageRowsMfmaKernel(const ImageMfmaParams
   // every channel group becomes four cells per quad; the weights of KS / BPW k-steps are requested behind it
   char* lbase = reinterpret_cast<char*>(xt);
   v4i a[KS];
-  const v4i* wt = static_cast<const v4i*>(p.wtiles) + ((size_t)(rg * 8 + wave) * KS) * 64 + lane;
+  const v4i* wt = static_cast<const v4i*>(wtiles) + ((size_t)(rg * 8 + wave) * KS) * 64 + lane;
 #pragma unroll
   for (int u = 0; u < BPW; ++u) {
     if (lane < qpi) {
@@ -229,7 +234,7 @@ __global__ void __launch_bounds__(512) ImageRowsMfmaKernel(const ImageMfmaParams
   const int left = qpi + sh - 16 * nqt;  // quads after the last window
   const int ntail = (left + 3) >> 2;
   constexpr int kElem = OUT == kOutI8 ? 1 : 4;
-  char* orow = Uniform(static_cast<char*>(p.out) + ((size_t)n * p.M + row0) * hw * kElem);
+  char* orow = Uniform(static_cast<char*>(out) + ((size_t)n * M + row0) * hw * kElem);
   DispatchAct(OUT == kOutAcc32 ? 0 : epilogue::LeakyAsMax(p.act), [&](auto act_c) {
     constexpr int ACT = decltype(act_c)::value;
     if (nqt > 0) {
@@ -285,22 +290,22 @@ hipError_t ByKs(const ImageMfmaParams& q, dim3 grid, size_t lds, hipStream_t s) 
   if (q.qpi == 49) {
     switch (q.K / 64) {
       case 2:
-        return LaunchWithLds(ImageRowsMfmaKernel<2, OUT, 49>, grid, block, lds, s, q);
+        return LaunchWithLds(ImageRowsMfmaKernel<2, OUT, 49>, grid, block, lds, s, q.x, q.wtiles, q.out, q.per_xcd, q.items, q.row_groups, q.K, q.hw, q.M, q);
       case 4:
-        return LaunchWithLds(ImageRowsMfmaKernel<4, OUT, 49>, grid, block, lds, s, q);
+        return LaunchWithLds(ImageRowsMfmaKernel<4, OUT, 49>, grid, block, lds, s, q.x, q.wtiles, q.out, q.per_xcd, q.items, q.row_groups, q.K, q.hw, q.M, q);
       case 8:
-        return LaunchWithLds(ImageRowsMfmaKernel<8, OUT, 49>, grid, block, lds, s, q);
+        return LaunchWithLds(ImageRowsMfmaKernel<8, OUT, 49>, grid, block, lds, s, q.x, q.wtiles, q.out, q.per_xcd, q.items, q.row_groups, q.K, q.hw, q.M, q);
       default:
         return hipErrorInvalidValue;
     }
   }
   switch (q.K / 64) {
     case 2:
-      return LaunchWithLds(ImageRowsMfmaKernel<2, OUT, 0>, grid, block, lds, s, q);
+      return LaunchWithLds(ImageRowsMfmaKernel<2, OUT, 0>, grid, block, lds, s, q.x, q.wtiles, q.out, q.per_xcd, q.items, q.row_groups, q.K, q.hw, q.M, q);
     case 4:
-      return LaunchWithLds(ImageRowsMfmaKernel<4, OUT, 0>, grid, block, lds, s, q);
+      return LaunchWithLds(ImageRowsMfmaKernel<4, OUT, 0>, grid, block, lds, s, q.x, q.wtiles, q.out, q.per_xcd, q.items, q.row_groups, q.K, q.hw, q.M, q);
     case 8:
-      return LaunchWithLds(ImageRowsMfmaKernel<8, OUT, 0>, grid, block, lds, s, q);
+      return LaunchWithLds(ImageRowsMfmaKernel<8, OUT, 0>, grid, block, lds, s, q.x, q.wtiles, q.out, q.per_xcd, q.items, q.row_groups, q.K, q.hw, q.M, q);
     default:
       return hipErrorInvalidValue;
   }

@@ -29,11 +29,11 @@ inline hipError_t EnableDynamicLds(const void* kernel, size_t lds) {
   return e;
 }
 
-template <typename Kernel, typename Params>
-hipError_t LaunchWithLds(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const Params& p) {
+template <typename Kernel, typename... Args>
+hipError_t LaunchWithLds(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const Args&... args) {
   const hipError_t e = EnableDynamicLds(reinterpret_cast<const void*>(kernel), lds);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);
+  hipLaunchKernelGGL(kernel, grid, block, lds, stream, args...);
   return hipGetLastError();
 }
 
