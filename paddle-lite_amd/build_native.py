@@ -21,14 +21,12 @@ HIPCC_FLAGS = [
     "-fno-gpu-rdc",
     # no packed fp32 VALU instructions in device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # leading scalar kernel arguments reach the wavefronts in registers instead of being loaded from the
+    # kernel-argument segment (as many as the user SGPRs hold; csrc/kernarg_head.h)
+    "-mllvm", "-amdgpu-kernarg-preload-count=14",
     "-Wall",
     "-Wno-unused-function",
 ]
-
-# Leading scalar kernel arguments are handed to the wavefronts in registers instead of being loaded from the
-# kernel-argument segment (up to what the user SGPRs hold).  Only arguments in front of the first by-value
-# struct qualify, so the flag changes nothing for kernels that take one parameter block.
-KERNARG_PRELOAD = ["-mllvm", "-amdgpu-kernarg-preload-count=14"]
 
 # (source, object name, extra flags); the kernel file is built as four
 # translation units so that they compile in parallel
@@ -42,7 +40,7 @@ SOURCES = [
     ("dwconv_kernels.hip", "dwconv_kernels.o", []),
     ("image_mfma_kernels.hip", "image_mfma_kernels.o", []),
     ("image_tr_kernels.hip", "image_tr_kernels.o", []),
-    ("image_rows_kernels.hip", "image_rows_kernels.o", KERNARG_PRELOAD),
+    ("image_rows_kernels.hip", "image_rows_kernels.o", []),
     ("sparse_conv_kernels.hip", "sparse_conv_kernels_walk.o", ["-DPL_KERNEL_PART=0"]),
     ("sparse_conv_kernels.hip", "sparse_conv_kernels_mfma_f32.o", ["-DPL_KERNEL_PART=1"]),
     ("sparse_conv_kernels.hip", "sparse_conv_kernels_mfma_i8.o", ["-DPL_KERNEL_PART=2"]),

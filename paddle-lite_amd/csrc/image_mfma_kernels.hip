@@ -31,6 +31,7 @@
 #include <type_traits>
 
 #include "epilogue.h"
+#include "kernarg_head.h"
 #include "launch_lds.h"
 #include "sparse_conv_kernels.h"
 
@@ -184,7 +185,8 @@ __device__ __forceinline__ void Tail(const uint4* __restrict__ xt, int kgs, int 
 // into different banks: channel 64 ks + 4 (8 (g % 2) + b % 8) + 2 (b / 8) + g / 2 is byte b of cell group g
 // of k-step ks.  The weight tiles come in the same order (the order inside an integer dot product is free).
 template <int KS, int OUT, int QPI, bool TRG = false>
-__global__ void __launch_bounds__(512) ImageMfmaKernel(const ImageMfmaParams p) {
+__global__ void __launch_bounds__(512) ImageMfmaKernel(PL_HEAD_PARAMS, const ImageMfmaParams block) {
+  const ImageMfmaParams p = WithHead(block, PL_HEAD_ARGS);
   extern __shared__ uint4 lds_raw[];
   // shifted windows read up to three cells in front of a row of cells
   uint4* xt = lds_raw + 16;
@@ -358,7 +360,8 @@ __global__ void __launch_bounds__(512) ImageMfmaKernel(const ImageMfmaParams p) 
 constexpr int kSmallHw = 49, kSmallQuads = 13, kSmallSlotCells = 64;
 
 template <int KS, int OUT>
-__global__ void __launch_bounds__(512) SmallMapMfmaKernel(const ImageMfmaParams p) {
+__global__ void __launch_bounds__(512) SmallMapMfmaKernel(PL_HEAD_PARAMS, const ImageMfmaParams block) {
+  const ImageMfmaParams p = WithHead(block, PL_HEAD_ARGS);
   extern __shared__ uint4 lds_raw[];
   uint4* xt = lds_raw + 16;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -512,11 +515,11 @@ hipError_t SmallByKs(const ImageMfmaParams& q, dim3 grid, size_t lds, hipStream_
   const dim3 block(512);
   switch (q.K / 64) {
     case 4:
-      return LaunchWithLds(SmallMapMfmaKernel<4, OUT>, grid, block, lds, s, q);
+      return LaunchWithHead(SmallMapMfmaKernel<4, OUT>, grid, block, lds, s, q);
     case 8:
-      return LaunchWithLds(SmallMapMfmaKernel<8, OUT>, grid, block, lds, s, q);
+      return LaunchWithHead(SmallMapMfmaKernel<8, OUT>, grid, block, lds, s, q);
     case 16:
-      return LaunchWithLds(SmallMapMfmaKernel<16, OUT>, grid, block, lds, s, q);
+      return LaunchWithHead(SmallMapMfmaKernel<16, OUT>, grid, block, lds, s, q);
     default:
       return hipErrorInvalidValue;
   }
@@ -528,23 +531,23 @@ hipError_t ByKs(const ImageMfmaParams& q, dim3 grid, size_t lds, hipStream_t s) 
   if (q.qpi == 49) {
     switch (q.K / 64) {
       case 2:
-        return LaunchWithLds(ImageMfmaKernel<2, OUT, 49>, grid, block, lds, s, q);
+        return LaunchWithHead(ImageMfmaKernel<2, OUT, 49>, grid, block, lds, s, q);
       case 4:
-        return LaunchWithLds(ImageMfmaKernel<4, OUT, 49>, grid, block, lds, s, q);
+        return LaunchWithHead(ImageMfmaKernel<4, OUT, 49>, grid, block, lds, s, q);
       case 8:
-        if (q.tr_regroup) return LaunchWithLds(ImageMfmaKernel<8, OUT, 49, true>, grid, block, lds, s, q);
-        return LaunchWithLds(ImageMfmaKernel<8, OUT, 49>, grid, block, lds, s, q);
+        if (q.tr_regroup) return LaunchWithHead(ImageMfmaKernel<8, OUT, 49, true>, grid, block, lds, s, q);
+        return LaunchWithHead(ImageMfmaKernel<8, OUT, 49>, grid, block, lds, s, q);
       default:
         return hipErrorInvalidValue;
     }
   }
   switch (q.K / 64) {
     case 2:
-      return LaunchWithLds(ImageMfmaKernel<2, OUT, 0>, grid, block, lds, s, q);
+      return LaunchWithHead(ImageMfmaKernel<2, OUT, 0>, grid, block, lds, s, q);
     case 4:
-      return LaunchWithLds(ImageMfmaKernel<4, OUT, 0>, grid, block, lds, s, q);
+      return LaunchWithHead(ImageMfmaKernel<4, OUT, 0>, grid, block, lds, s, q);
     case 8:
-      return LaunchWithLds(ImageMfmaKernel<8, OUT, 0>, grid, block, lds, s, q);
+      return LaunchWithHead(ImageMfmaKernel<8, OUT, 0>, grid, block, lds, s, q);
     default:
       return hipErrorInvalidValue;
   }

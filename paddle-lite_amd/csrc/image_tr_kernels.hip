@@ -47,6 +47,7 @@
 #include <type_traits>
 
 #include "epilogue.h"
+#include "kernarg_head.h"
 #include "launch_lds.h"
 #include "sparse_conv_kernels.h"
 
@@ -77,7 +78,8 @@ __device__ __forceinline__ void StoreThrough128(u4 v, char* base, uint32_t off) 
 // KS2 = K / 128: k-steps per channel parity.  HW: H*W when known at compile
 // time (LDS offsets become immediates), else 0.
 template <int KS2, int OUT, int HW>
-__global__ void __launch_bounds__(512) ImageTrKernel(const ImageMfmaParams p) {
+__global__ void __launch_bounds__(512) ImageTrKernel(PL_HEAD_PARAMS, const ImageMfmaParams block) {
+  const ImageMfmaParams p = WithHead(block, PL_HEAD_ARGS);
   extern __shared__ uint4 lds_raw[];
   PL_LDS char* img = (PL_LDS char*)lds_raw + kFrontPad;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -278,22 +280,22 @@ hipError_t ByKs(const ImageMfmaParams& q, dim3 grid, size_t lds, hipStream_t s) 
   if (q.hw == 196) {
     switch (q.K / 128) {
       case 1:
-        return LaunchWithLds(ImageTrKernel<1, OUT, 196>, grid, block, lds, s, q);
+        return LaunchWithHead(ImageTrKernel<1, OUT, 196>, grid, block, lds, s, q);
       case 2:
-        return LaunchWithLds(ImageTrKernel<2, OUT, 196>, grid, block, lds, s, q);
+        return LaunchWithHead(ImageTrKernel<2, OUT, 196>, grid, block, lds, s, q);
       case 4:
-        return LaunchWithLds(ImageTrKernel<4, OUT, 196>, grid, block, lds, s, q);
+        return LaunchWithHead(ImageTrKernel<4, OUT, 196>, grid, block, lds, s, q);
       default:
         return hipErrorInvalidValue;
     }
   }
   switch (q.K / 128) {
     case 1:
-      return LaunchWithLds(ImageTrKernel<1, OUT, 0>, grid, block, lds, s, q);
+      return LaunchWithHead(ImageTrKernel<1, OUT, 0>, grid, block, lds, s, q);
     case 2:
-      return LaunchWithLds(ImageTrKernel<2, OUT, 0>, grid, block, lds, s, q);
+      return LaunchWithHead(ImageTrKernel<2, OUT, 0>, grid, block, lds, s, q);
     case 4:
-      return LaunchWithLds(ImageTrKernel<4, OUT, 0>, grid, block, lds, s, q);
+      return LaunchWithHead(ImageTrKernel<4, OUT, 0>, grid, block, lds, s, q);
     default:
       return hipErrorInvalidValue;
   }

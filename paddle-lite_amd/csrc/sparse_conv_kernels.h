@@ -116,21 +116,24 @@ struct TileWalkParams {
   // Records do not straddle chunks; every stream ends with one spare chunk.
   const void* stream;
   const uint32_t* stream_first;   // [kTileWalkWaves] first chunk of every stream; with `split`, [2 * kTileWalkWaves]: main part, spare part
-  const uint32_t* stream_groups;  // row groups in every stream, same shape
-  int n_groups;
-  int M, K;
+  int K;
   int hw;
   uint32_t P;
-  DevAct act;
   int tiles;                     // filled in by the launcher
   // 1: the row groups are dealt into a main and a spare part; the grid then has
   // split_slots workgroups per XCD (one per CU), more than any XCD has tiles.
   // 2: `parts` equal parts, as many workgroups per tile (parts x the tiles of
   // an XCD must not exceed split_slots); the stream tables then hold
   // parts x kTileWalkWaves entries.
-  int split;
+  int16_t split;
+  int16_t parts;
+  // The first 56 bytes (kernarg_head.h) end behind act.type: what selects the tile, picks the activation and
+  // addresses the first loads.
+  DevAct act;
+  const uint32_t* stream_groups;  // row groups in every stream, same shape as stream_first
+  int n_groups;
+  int M;
   int split_slots;
-  int parts;
 };
 
 // LDS the kernel needs for K input channels.
@@ -238,23 +241,26 @@ hipError_t LaunchBlockMfma(const MfmaConfig& cfg, const MfmaParams& p, hipStream
 // Image MFMA SpMM (int8, image_mfma_kernels.hip): one workgroup per (image,
 // 128 output rows) with the whole image's activations in LDS.
 struct ImageMfmaParams {
+  // the first 56 bytes: what the first loads of a kernel need (kernarg_head.h)
   const int8_t* x;
   void* out;
   // dense 16x64 weight tiles in matrix-core operand order:
   // [row group of 128][class rho = 0..3][tile j = 0..1][k-step][64 lanes][16 bytes];
   // lane l of tile (rho, j) holds row rho + 4 (16 j + l % 16), channels 64 ks + 16 (l / 16) .. + 15
   const void* wtiles;
-  const float* scale;  // output-row order, at least M entries
-  const float* bias;   // likewise (zeros when the op has no bias)
   int M, K;
   int hw;
   int batch;
+  // filled in by the launcher
+  int items, per_xcd;  // work items (image, row group) in all and per XCD
+  int row_groups;      // M / 128
+  int qpi;             // position quads per image = hw / 4
+  // behind the head
+  const float* scale;  // output-row order, at least M entries
+  const float* bias;   // likewise (zeros when the op has no bias)
   DevAct act;
   // filled in by the launcher
-  int qpi;             // position quads per image = hw / 4
   int kgs;             // 16-byte cells per channel group in LDS (a multiple of 16)
-  int row_groups;      // M / 128
-  int items, per_xcd;  // work items (image, row group) in all and per XCD
   int dma_full, dma_rem_lanes;  // 1 KB pieces of a channel group and the lanes of the last, partial piece
   int align;           // fp32 / int32 output: windows shifted onto 64-byte sector boundaries
   // set by the caller of LaunchImageMfma: wtiles holds the tiles in the channel order of the regrouping by

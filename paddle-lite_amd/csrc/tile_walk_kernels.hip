@@ -28,6 +28,7 @@
 #include <type_traits>
 
 #include "epilogue.h"
+#include "kernarg_head.h"
 #include "launch_lds.h"
 #include "sparse_conv_kernels.h"
 
@@ -207,7 +208,8 @@ __device__ __forceinline__ void TileWalkBody(const TileWalkParams& p, float* til
 }
 
 template <int NR>
-__global__ void __launch_bounds__(64 * kTileWalkWaves) TileWalkKernel(const TileWalkParams p) {
+__global__ void __launch_bounds__(64 * kTileWalkWaves) TileWalkKernel(PL_HEAD_PARAMS, const TileWalkParams block) {
+  const TileWalkParams p = WithHead(block, PL_HEAD_ARGS);
   extern __shared__ float tile_lds[];
   DispatchAct(p.act.type, [&](auto act_c) {
     constexpr int ACT = decltype(act_c)::value;
@@ -235,8 +237,8 @@ hipError_t LaunchTileWalk(int nrows, const TileWalkParams& p, hipStream_t stream
     slots = (uint32_t)q.split_slots;
   }
   dim3 grid(8u * slots), block(64 * kWaves);
-  if (nrows == 2) return LaunchWithLds(TileWalkKernel<2>, grid, block, lds, stream, q);
-  return LaunchWithLds(TileWalkKernel<1>, grid, block, lds, stream, q);
+  if (nrows == 2) return LaunchWithHead(TileWalkKernel<2>, grid, block, lds, stream, q);
+  return LaunchWithHead(TileWalkKernel<1>, grid, block, lds, stream, q);
 }
 
 }  // namespace pl
