@@ -49,6 +49,18 @@ using epilogue::TruncPackI8x4;
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 
+// what the image and weight loads need arrives in registers
+PL_IN_HEAD(ImageMfmaParams, x);
+PL_IN_HEAD(ImageMfmaParams, out);
+PL_IN_HEAD(ImageMfmaParams, wtiles);
+PL_IN_HEAD(ImageMfmaParams, M);
+PL_IN_HEAD(ImageMfmaParams, K);
+PL_IN_HEAD(ImageMfmaParams, hw);
+PL_IN_HEAD(ImageMfmaParams, items);
+PL_IN_HEAD(ImageMfmaParams, per_xcd);
+PL_IN_HEAD(ImageMfmaParams, row_groups);
+PL_IN_HEAD(ImageMfmaParams, qpi);
+
 constexpr int kRowStride = 8;  // rows of a tile: w + 8 m
 
 // 16 bytes stored as streaming data (nt) at a wave-uniform base plus an unsigned 32-bit lane offset (no 64-bit

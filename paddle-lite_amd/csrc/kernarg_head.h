@@ -10,6 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstddef>
 #include <cstring>
 #include <type_traits>
 
@@ -33,6 +34,10 @@ __device__ __forceinline__ P WithHead(const P& block, PL_HEAD_PARAMS) {
   __builtin_memcpy(&p, h, sizeof(h));
   return p;
 }
+
+// Compile-time check that a field lies inside the head: PL_IN_HEAD(ImageMfmaParams, qpi).
+#define PL_IN_HEAD(Block, field) \
+  static_assert(offsetof(Block, field) + sizeof(Block::field) <= ::pl::kHeadWords * 8, #field " must lie in the first 56 bytes of " #Block)
 
 // Launches kernel(head words..., block).
 template <typename Kernel, typename P>

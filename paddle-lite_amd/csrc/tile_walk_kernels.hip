@@ -41,6 +41,18 @@ typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 typedef const __attribute__((address_space(4))) uint32_t* ConstWords;
 typedef const __attribute__((address_space(4))) float* ConstFloats;
 
+// what selects the tile, picks the activation and addresses the first loads arrives in registers
+PL_IN_HEAD(TileWalkParams, x);
+PL_IN_HEAD(TileWalkParams, stream);
+PL_IN_HEAD(TileWalkParams, stream_first);
+PL_IN_HEAD(TileWalkParams, K);
+PL_IN_HEAD(TileWalkParams, hw);
+PL_IN_HEAD(TileWalkParams, P);
+PL_IN_HEAD(TileWalkParams, tiles);
+PL_IN_HEAD(TileWalkParams, split);
+PL_IN_HEAD(TileWalkParams, parts);
+static_assert(offsetof(TileWalkParams, act) + sizeof(int) <= kHeadWords * 8, "act.type must lie in the first 56 bytes of TileWalkParams");
+
 using epilogue::ActivateT;
 using epilogue::DispatchAct;
 
