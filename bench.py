@@ -670,6 +670,7 @@ def run_mobilenet(args):
     batch = 64
     rng = np.random.RandomState(5)
     x = torch.from_numpy(rng.randint(-127, 128, size=(batch, 32, 112, 112)).astype(np.int8)).cuda()
+    keep_input = x  # the launches below hold device addresses, not tensors: the tensors must stay alive
     steps_list = []  # (kind, name, launch, bytes)
     keep = []
     total_bytes = 0.0
@@ -708,6 +709,37 @@ def run_mobilenet(args):
         for _, _, launch, _ in steps_list:
             launch()
 
+    # The same body with every pointwise layer that can do so running the depthwise layer behind it in its own
+    # launch (pl_sparse_conv_dwconv3x3_run: 14 x 14 maps; the tensor between the two is not written).
+    fused_list, fused_pairs = [], []
+    i = 0
+    while i < len(steps_list):
+        if steps_list[i][0] == "pointwise" and i + 1 < len(steps_list):
+            li = i // 2  # pointwise layer li, followed by the depthwise layer in front of pointwise layer li + 1
+            kernel, (dw_next, _, t_next, _) = keep[li][1], keep[li + 1]
+            size = wl.MOBILENET_V1_POINTWISE[li][2]
+            if L.pl_sparse_conv_dwconv3x3_pays(kernel._handle, dw_next._handle, batch, size, size):
+                t_in = keep[li][2]
+                fused_list.append(lambda hc=kernel._handle, hd=dw_next._handle, xi=t_in, oi=t_next, n=size: capi.check(
+                    L.pl_sparse_conv_dwconv3x3_run(hc, hd, C.c_void_p(xi.data_ptr()), C.c_void_p(oi.data_ptr()), batch, n, n, C.c_void_p(stream))))
+                fused_pairs.append("%s + %s" % (steps_list[i][1], steps_list[i + 1][1]))
+                i += 2
+                continue
+        fused_list.append(steps_list[i][2])
+        i += 1
+
+    def fused_sequence():
+        for launch in fused_list:
+            launch()
+
+    sequence()
+    torch.cuda.synchronize()
+    final_two_launches = keep[-1][3].clone()
+    keep[-1][3].zero_()
+    fused_sequence()
+    torch.cuda.synchronize()
+    fused_equal = bool(torch.equal(final_two_launches, keep[-1][3]))
+
     settle(sequence)
     per_layer = []
     for kind, name, launch, nbytes in steps_list:
@@ -735,6 +767,15 @@ def run_mobilenet(args):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     seq_us = e0.elapsed_time(e1) * 1e3 / steps
+    for _ in range(max(1, args.warmup // 26)):
+        fused_sequence()
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(steps):
+        fused_sequence()
+    e1.record()
+    torch.cuda.synchronize()
+    fused_seq_us = e0.elapsed_time(e1) * 1e3 / steps
     dw_us = sum(p["kernel_us"] for p in per_layer if p["kind"] == "depthwise")
     pw_us = sum(p["kernel_us"] for p in per_layer if p["kind"] == "pointwise")
     print(json.dumps({
@@ -751,6 +792,7 @@ def run_mobilenet(args):
         "config": {"workload": "mobilenet_v1_body_int8", "batch": batch, "launches": 26, "pointwise_sparsity": 0.9, "parity_checked": True},
         "roofline": {"bound": "hbm", "achieved": total_bytes / (seq_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": total_bytes / (seq_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_sequence": total_bytes, "sequence_us": seq_us, "host_enqueue_us_per_sequence": round(host_us, 1), "sum_depthwise_kernel_us": round(dw_us, 1), "sum_pointwise_kernel_us": round(pw_us, 1)},
+        "pairs_in_one_launch": {"pairs": fused_pairs, "launches": len(fused_list), "sequence_us": fused_seq_us, "output_equals_two_launches": fused_equal},
         "per_layer": per_layer,
         "nonzero_fraction_of_pointwise_outputs": nonzero,
     }))

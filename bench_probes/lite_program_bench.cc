@@ -10,6 +10,8 @@
 //   eager_sequence_us   the 26 convolution steps enqueued one by one, device time between two events
 //   graph_sequence_us   the same 26 steps captured once (kernel nodes only) and replayed
 //   graph_matches_eager the fetched fp32 output after graph replays equals the eager one byte for byte
+//   pairs_joined, pair_launch_sequence_us, pair_launch_matches_eager
+//                       the eager sequence with HipProgram's pair launches switched on
 // Parity of this path against the CPU oracle is the business of tests/cpp/sparse_conv_hip_test.cc; this
 // program only measures.
 #include <hip/hip_runtime.h>
@@ -236,6 +238,22 @@ int main(int argc, char** argv) {
     HIP_OK(hipEventElapsedTime(&ms, e0, e1));
     const double graph_us = ms * 1e3 / sequences;
 
+    // pair launches: a pointwise step and the depthwise step behind it as one launch where the library says it pays
+    program.set_pair_launch(true);
+    program.Run();
+    const size_t pairs = program.pairs_joined_last_enqueue();
+    const bool pairs_ok = fetched->memory_size() == eager_out.size() && std::memcmp(fetched->raw_data(), eager_out.data(), eager_out.size()) == 0;
+    for (int s = 0; s < 5; ++s) program.Enqueue(first, last);
+    HIP_OK(hipEventRecord(e0, stream));
+    const double p0 = NowUs();
+    for (int s = 0; s < sequences; ++s) program.Enqueue(first, last);
+    const double pairs_host_us = (NowUs() - p0) / sequences;
+    HIP_OK(hipEventRecord(e1, stream));
+    HIP_OK(hipEventSynchronize(e1));
+    HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+    const double pairs_us = ms * 1e3 / sequences;
+    program.set_pair_launch(false);
+
     std::printf("{\"workload\": \"mobilenet_v1_body_int8 through mir::HipProgram\", \"batch\": %d, \"sequences\": %d, \"steps\": [", batch, sequences);
     double host_sum = 0;
     for (size_t i = first; i < last; ++i) {
@@ -243,13 +261,13 @@ int main(int argc, char** argv) {
       std::printf("%s{\"kernel\": \"%s\", \"host_enqueue_us\": %.2f}", i == first ? "" : ", ", steps[i].kernel.c_str(), host_us[i] / sequences);
     }
     std::printf("], \"host_enqueue_us_per_sequence\": %.1f, \"host_enqueue_us_per_sequence_back_to_back\": %.1f, \"eager_sequence_us\": %.1f, \"graph_nodes\": %zu, \"graph_sequence_us\": %.1f, "
-                "\"host_us_per_graph_launch\": %.1f, \"graph_matches_eager\": %s}\n",
-                host_sum, host_sequence_us, eager_us, nodes, graph_us, host_graph_us, graph_ok ? "true" : "false");
+                "\"host_us_per_graph_launch\": %.1f, \"graph_matches_eager\": %s, \"pairs_joined\": %zu, \"pair_launch_sequence_us\": %.1f, \"pair_launch_host_enqueue_us_per_sequence\": %.1f, \"pair_launch_matches_eager\": %s}\n",
+                host_sum, host_sequence_us, eager_us, nodes, graph_us, host_graph_us, graph_ok ? "true" : "false", pairs, pairs_us, pairs_host_us, pairs_ok ? "true" : "false");
     HIP_OK(hipGraphExecDestroy(exec));
     HIP_OK(hipGraphDestroy(graph));
     HIP_OK(hipEventDestroy(e0));
     HIP_OK(hipEventDestroy(e1));
-    return graph_ok ? 0 : 1;
+    return graph_ok && pairs_ok ? 0 : 1;
   } catch (const FatalError& e) {
     std::fprintf(stderr, "fatal: %s\n", e.what());
     return 1;

@@ -324,6 +324,35 @@ int pl_dwconv3x3_run(pl_dwconv_handle* handle, const int8_t* x_dev, void* out_de
 
 void pl_dwconv3x3_destroy(pl_dwconv_handle* handle);
 
+/* ---- sparse_conv2d followed by the depthwise 3x3 convolution, one launch ----
+ * No counterpart in the reference, where the two layers are two kernels
+ * (Instruction::Run per op, lite/core/program.cc:789-816) with the tensor
+ * between them in memory.  Here the pointwise kernel keeps the 16 output
+ * channels of a wavefront in LDS as int8 planes and runs the depthwise layer
+ * on them: the intermediate tensor is never written, one launch instead of
+ * two.  Results are those of pl_sparse_conv_run followed by pl_dwconv3x3_run,
+ * bit for bit.  Both handles int8 -> int8, 14 x 14 maps, depthwise padding 1
+ * and stride 1 or 2, depthwise channels = pointwise output channels, a
+ * pointwise handle that the image algorithm with one row tile per wavefront
+ * serves (oc % 128 == 0, ic = 128, 256 or 512, algo AUTO or IMAGE_MFMA).
+ * _fits returns 1 when a pair can run this way, else 0; _run returns
+ * PL_ERR_UNSUPPORTED with the reason for a pair that cannot (it does not
+ * consult _pays).
+ * x_dev: int8 NCHW [batch, ic, h, w]; out_dev: int8 NCHW [batch, oc, oh, ow]
+ * of the depthwise layer; both 4-byte aligned. */
+int pl_sparse_conv_dwconv3x3_fits(const pl_sparse_conv_handle* conv, const pl_dwconv_handle* dw,
+                                  int32_t h, int32_t w);
+/* 1 when the pair fits and the one launch is expected to be faster than the
+ * two at this batch: always for stride 2; for stride 1 when the launch has
+ * at least 7/8 as many workgroups (batch * oc / 128) as the device has CUs -
+ * the one launch keeps the depthwise work of a workgroup's 128 planes on its
+ * CU, which loses to the depthwise kernel's spread at small batches. */
+int pl_sparse_conv_dwconv3x3_pays(const pl_sparse_conv_handle* conv, const pl_dwconv_handle* dw,
+                                  int32_t batch, int32_t h, int32_t w);
+int pl_sparse_conv_dwconv3x3_run(pl_sparse_conv_handle* conv, pl_dwconv_handle* dw,
+                                 const void* x_dev, void* out_dev, int32_t batch,
+                                 int32_t h, int32_t w, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

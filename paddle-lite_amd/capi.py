@@ -34,6 +34,9 @@ EXPORTS = [
     "pl_dwconv3x3_prepare",
     "pl_dwconv3x3_run",
     "pl_dwconv3x3_destroy",
+    "pl_sparse_conv_dwconv3x3_fits",
+    "pl_sparse_conv_dwconv3x3_pays",
+    "pl_sparse_conv_dwconv3x3_run",
 ]
 
 
@@ -192,6 +195,12 @@ def lib():
     L.pl_dwconv3x3_run.restype = C.c_int
     L.pl_dwconv3x3_destroy.argtypes = [C.c_void_p]
     L.pl_dwconv3x3_destroy.restype = None
+    L.pl_sparse_conv_dwconv3x3_fits.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32]
+    L.pl_sparse_conv_dwconv3x3_fits.restype = C.c_int
+    L.pl_sparse_conv_dwconv3x3_pays.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32]
+    L.pl_sparse_conv_dwconv3x3_pays.restype = C.c_int
+    L.pl_sparse_conv_dwconv3x3_run.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]
+    L.pl_sparse_conv_dwconv3x3_run.restype = C.c_int
     if L.pl_sparse_conv_abi_version() != ABI_VERSION:
         raise LibraryMissing("libpl_sparse_conv.so has ABI %d, binding expects %d" % (L.pl_sparse_conv_abi_version(), ABI_VERSION))
     _lib = L

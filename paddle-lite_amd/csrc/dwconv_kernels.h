@@ -41,4 +41,11 @@ struct DwConvParams {
 // stride 1 or 2; out_kind kOutF32 or kOutI8.
 hipError_t LaunchDwConv3x3(int stride, int out_kind, const DwConvParams& p, hipStream_t stream);
 
+// The int8 -> int8 pointwise layer of image_rows_kernels.hip followed by the int8 -> int8 depthwise layer on its
+// output, in one launch: 14 x 14 maps, padding 1, stride 1 or 2.  p.out is not used; d.x is not used (the
+// depthwise input never leaves the CU); d.h, d.w, d.oh, d.ow, d.pad, d.channels, d.wpack, d.scale, d.bias, d.act
+// and d.out as for LaunchDwConv3x3.
+bool ImageRowsDwFits(int M, int K, int hw, int h, int w, int pad, int stride);
+hipError_t LaunchImageRowsDw(const ImageMfmaParams& p, const DwConvParams& d, int stride, hipStream_t stream);
+
 }  // namespace pl

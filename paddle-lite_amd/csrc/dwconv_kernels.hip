@@ -12,6 +12,7 @@
 #include <cstdint>
 #include <type_traits>
 
+#include "dw_row_item.h"
 #include "dwconv_kernels.h"
 #include "epilogue.h"
 #include "launch_lds.h"
@@ -293,88 +294,8 @@ __global__ void __launch_bounds__(256) DwConv3x3Kernel(const DwConvParams p) {
 //   * int8 outputs go to LDS byte by byte (the workgroup's output rows are
 //     one contiguous range too) and leave as aligned 16-byte pieces; fp32
 //     outputs are stored directly (dword aligned).
-struct DwRowStage {
-  char* lds_in;      // holds the input bytes from `in_base` on, preceded by 16 bytes of slack
-  int64_t in_base;   // offset of the first staged byte in the tensor (a multiple of 16)
-  char* lds_out;     // int8 output rows of the workgroup, item-major
-};
-
-template <int STRIDE, int NOUT, int OUT, int ACT>
-__device__ __forceinline__ void DwRowItem(const DwConvParams& p, const DwRowStage& st, uint32_t plane, int c, int oy, bool live) {
-  // byte b of a window is column b - pad
-  uint32_t mask[4];
-#pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    uint32_t m = 0xffffffffu;
-    const int below = p.pad - 4 * k;          // bytes of the dword in front of column 0
-    const int inside = p.pad + p.w - 4 * k;   // bytes of the dword, from its first, up to the end of the row
-    if (below > 0) m &= 0xffffffffu << (8 * below);
-    m = inside <= 0 ? 0u : (inside < 4 ? m & (0xffffffffu >> (8 * (4 - inside))) : m);
-    mask[k] = m;
-  }
-  int acc[NOUT];
-#pragma unroll
-  for (int j = 0; j < NOUT; ++j) acc[j] = 0;
-  float s = 0.f, b = 0.f;
-  if (live) {
-    const uint32_t wrow[3] = {p.wpack[4 * c], p.wpack[4 * c + 1], p.wpack[4 * c + 2]};
-    s = p.scale[c];
-    b = p.bias[c];
-    const int iy0 = STRIDE * oy - p.pad;
-    const int64_t plane_at = (int64_t)plane * (uint32_t)(p.h * p.w) - st.in_base + 16;  // LDS offset of the plane's first byte
-    uint32_t D[3][4];
-#pragma unroll
-    for (int r = 0; r < 3; ++r) {
-      // a row outside [0, h) is zero padding: it reads its neighbour and meets a zero filter row below
-      const uint32_t at = (uint32_t)(plane_at + (uint32_t)(min(max(iy0 + r, 0), p.h - 1) * p.w) - p.pad);
-      const uint32_t* words = reinterpret_cast<const uint32_t*>(st.lds_in + (at & ~3u));
-      uint32_t e[5];
-#pragma unroll
-      for (int k = 0; k < 5; ++k) e[k] = words[k];
-#pragma unroll
-      for (int k = 0; k < 4; ++k) D[r][k] = __builtin_amdgcn_alignbyte(e[k + 1], e[k], at & 3u);
-    }
-#pragma unroll
-    for (int r = 0; r < 3; ++r) {
-      const int iy = iy0 + r;
-      const int wr = (int)(wrow[r] & ((iy >= 0 && iy < p.h) ? 0xffffffffu : 0u));
-      uint32_t d[4];
-#pragma unroll
-      for (int k = 0; k < 4; ++k) d[k] = D[r][k] & mask[k];
-#pragma unroll
-      for (int j = 0; j < NOUT; ++j) {
-        const int first = STRIDE * j, k = first / 4, sh = first % 4;
-        const int win = sh == 0 ? (int)d[k] : (int)__builtin_amdgcn_alignbyte(k + 1 < 4 ? d[k + 1] : 0u, d[k], sh);
-        acc[j] = __builtin_amdgcn_sdot4(win, wr, acc[j], false);
-      }
-    }
-  }
-  if (OUT == kOutI8) {
-    // the low byte of the truncated value is the int8 output
-    char* dst = st.lds_out + (uint32_t)threadIdx.x * (uint32_t)p.ow;
-#pragma unroll
-    for (int j = 0; j < NOUT; ++j)
-      if (j < p.ow) dst[j] = (char)static_cast<int>(ActQuantF<ACT>(__builtin_fmaf((float)acc[j], s, b), p.act));
-  } else if (live) {
-    float* dst = static_cast<float*>(p.out) + ((size_t)plane * (uint32_t)p.oh + (uint32_t)oy) * (uint32_t)p.ow;
-    constexpr int NG = (NOUT + 3) / 4;
-#pragma unroll
-    for (int q4 = 0; q4 < NG; ++q4) {
-      const int n_out = min(4, p.ow - 4 * q4);
-      if (n_out <= 0) break;
-      float v[4];
-#pragma unroll
-      for (int k = 0; k < 4; ++k) v[k] = 4 * q4 + k < NOUT ? ActivateT<ACT>(__builtin_fmaf((float)acc[4 * q4 + k < NOUT ? 4 * q4 + k : 0], s, b), p.act) : 0.0f;
-      if (n_out == 4) {  // a four-dword store needs dword alignment only
-        *reinterpret_cast<v4f*>(dst + 4 * q4) = v4f{v[0], v[1], v[2], v[3]};
-      } else {
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-          if (k < n_out) dst[4 * q4 + k] = v[k];
-      }
-    }
-  }
-}
+using dwrow::DwRowItem;
+using dwrow::DwRowStage;
 
 template <int STRIDE, int NOUT, int OUT>
 __global__ void __launch_bounds__(256) DwRowKernel(const DwConvParams p) {
@@ -391,7 +312,7 @@ __global__ void __launch_bounds__(256) DwRowKernel(const DwConvParams p) {
   DwRowStage st;
   st.in_base = need_lo & ~(int64_t)15;
   st.lds_in = reinterpret_cast<char*>(dw_lds);
-  st.lds_out = st.lds_in + p.row_lds_in;
+  char* lds_out = st.lds_in + p.row_lds_in;  // int8 output rows of the workgroup, item-major
   const int pieces = (int)((need_hi - st.in_base + 15) >> 4);
   uint4 piece[4];
 #pragma unroll
@@ -423,7 +344,7 @@ __global__ void __launch_bounds__(256) DwRowKernel(const DwConvParams p) {
   const int c = (int)(plane - DivMagic(plane, (uint32_t)p.channels, p.magic_channels) * (uint32_t)p.channels);
   DispatchAct(p.act.type, [&](auto act_c) {
     constexpr int ACT = decltype(act_c)::value;
-    DwRowItem<STRIDE, NOUT, OUT, ACT>(p, st, plane, c, oy, live);
+    DwRowItem<STRIDE, NOUT, OUT, ACT>(p, st, plane, c, oy, live, lds_out + (uint32_t)tid * (uint32_t)p.ow);
   });
   if (OUT == kOutI8) {
     __syncthreads();
@@ -432,7 +353,7 @@ __global__ void __launch_bounds__(256) DwRowKernel(const DwConvParams p) {
     const int64_t out_end = (int64_t)total * p.ow;
     if (tid < 16 * p.ow) {
       int8_t* dst = static_cast<int8_t*>(p.out) + out_at;
-      const uint4 v = *reinterpret_cast<const uint4*>(st.lds_out + 16 * tid);
+      const uint4 v = *reinterpret_cast<const uint4*>(lds_out + 16 * tid);
       if (out_at + 16 <= out_end) {
         *reinterpret_cast<uint4*>(dst) = v;
       } else {  // the tensor's last, partial piece

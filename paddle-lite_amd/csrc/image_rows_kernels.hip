@@ -33,6 +33,7 @@
 #include <cstdint>
 #include <type_traits>
 
+#include "dw_row_item.h"
 #include "epilogue.h"
 #include "kernarg_head.h"
 #include "launch_lds.h"
@@ -62,6 +63,14 @@ PL_IN_HEAD(ImageMfmaParams, row_groups);
 PL_IN_HEAD(ImageMfmaParams, qpi);
 
 constexpr int kRowStride = 8;  // rows of a tile: w + 8 m
+// Output kind of the kernel that runs the following depthwise layer itself: int8 like kOutI8, written to the
+// wavefront's own planes in LDS (one plane of H x W bytes per row of its tile) instead of global memory.
+constexpr int kOutPlanes = 3;
+template <int OUT>
+constexpr int kPlaneStride = OUT == kOutPlanes ? 1 : kRowStride;  // rows of the tile are this many rows apart where they are stored
+__device__ __forceinline__ void StoreLds(uint32_t v, char* p) {
+  *reinterpret_cast<__attribute__((address_space(3))) uint32_t*>(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p))) = v;
+}
 
 // 16 bytes stored as streaming data (nt) at a wave-uniform base plus an unsigned 32-bit lane offset (no 64-bit
 // address arithmetic per store).  Measured on the metric shape with this kernel's whole-line pieces: nt 8.93 us,
@@ -92,7 +101,7 @@ template <int OUT, int ACT>
 __device__ __forceinline__ u4 Finish4(int a0, int a1, int a2, int a3, float s, float b, const DevAct& act) {
   if (OUT == kOutAcc32) return u4{(uint32_t)a0, (uint32_t)a1, (uint32_t)a2, (uint32_t)a3};
   const float v0 = __builtin_fmaf((float)a0, s, b), v1 = __builtin_fmaf((float)a1, s, b), v2 = __builtin_fmaf((float)a2, s, b), v3 = __builtin_fmaf((float)a3, s, b);
-  if (OUT == kOutI8) return u4{TruncPackI8x4(ActQuantF<ACT>(v0, act), ActQuantF<ACT>(v1, act), ActQuantF<ACT>(v2, act), ActQuantF<ACT>(v3, act)), 0u, 0u, 0u};
+  if (OUT == kOutI8 || OUT == kOutPlanes) return u4{TruncPackI8x4(ActQuantF<ACT>(v0, act), ActQuantF<ACT>(v1, act), ActQuantF<ACT>(v2, act), ActQuantF<ACT>(v3, act)), 0u, 0u, 0u};
   return u4{__float_as_uint(ActivateT<ACT>(v0, act)), __float_as_uint(ActivateT<ACT>(v1, act)), __float_as_uint(ActivateT<ACT>(v2, act)), __float_as_uint(ActivateT<ACT>(v3, act))};
 }
 
@@ -100,17 +109,74 @@ __device__ __forceinline__ u4 Finish4(int a0, int a1, int a2, int a3, float s, f
 // lane's line is shared with the end of the previous output row and merges in L2 (plain store).
 template <int OUT, int ACT>
 __device__ __forceinline__ void StoreRow(const v4i (&acc)[4], int i, float sc, float bi, const DevAct& act, char* __restrict__ orow, int hw, int q, bool partial, Lane ln) {
-  constexpr int kElem = OUT == kOutI8 ? 1 : 4;
+  constexpr int kElem = (OUT == kOutI8 || OUT == kOutPlanes) ? 1 : 4;
   const u4 v = Finish4<OUT, ACT>(acc[0][i], acc[1][i], acc[2][i], acc[3][i], sc, bi, act);
   // at most 128 rows of at most 256 four-byte positions behind orow: the offset fits 32 bits; it is negative only
   // for the quads in front of a row, which are not stored
-  const int off = ((kRowStride * (4 * ln.kq + i)) * hw + 4 * q) * kElem;
-  if (OUT == kOutI8) {
+  const int off = ((kPlaneStride<OUT> * (4 * ln.kq + i)) * hw + 4 * q) * kElem;
+  if (OUT == kOutPlanes) {
+    if (q >= 0) StoreLds(v.x, orow + off);
+  } else if (OUT == kOutI8) {
     if (q >= 0) StorePlain(v.x, orow + off);
   } else if (partial) {
     if (q >= 0) StorePlain(v, orow + off);
   } else {
     StoreStreaming(v, orow, (uint32_t)off);
+  }
+}
+
+// LDS of a wavefront behind the image's cells when the depthwise layer follows: its 16 planes of 14 x 14 int8
+// (16 bytes of slack in front, 48 behind: the rows are read as aligned dwords around them), then the planes of
+// the depthwise output.
+constexpr int kPlaneInBytes = 16 + 16 * 196 + 48, kPlaneBufBytes = kPlaneInBytes + 16 * 196;
+
+// The depthwise layer on the wavefront's planes: one output row of one plane per lane and pass (dw_row_item.h),
+// outputs collected plane-major in LDS, then stored: a plane of the tile's row m is channel row0 + 8 m.
+template <int STRIDE>
+__device__ __forceinline__ void DwStage(const DwConvParams& d, char* planes_in, char* planes_out, int n, int M, int row0, int lane) {
+  constexpr int NOUT = STRIDE == 1 ? 14 : 7;
+  constexpr int oh = NOUT, ow = NOUT;  // 14 x 14 planes, padding 1
+  constexpr int items = 16 * oh, passes = (items + 63) / 64;
+  dwrow::DwRowStage st;
+  st.lds_in = planes_in - 16;
+  st.in_base = 0;
+  // filter rows, scale and bias of every pass's channel first: one memory latency for all passes
+  uint32_t wrow[passes][3];
+  float sc[passes], bi[passes];
+#pragma unroll
+  for (int t = 0; t < passes; ++t) {
+    const int it = min(64 * t + lane, items - 1);
+    const int c = row0 + kRowStride * (it / oh);
+    wrow[t][0] = d.wpack[4 * c];
+    wrow[t][1] = d.wpack[4 * c + 1];
+    wrow[t][2] = d.wpack[4 * c + 2];
+    sc[t] = d.scale[c];
+    bi[t] = d.bias[c];
+  }
+  DispatchAct(d.act.type, [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
+#pragma unroll
+    for (int t = 0; t < passes; ++t) {
+      const int item = 64 * t + lane;
+      const bool live = item < items;
+      const int it = live ? item : items - 1;
+      const int m = it / oh, oy = it - m * oh;
+      dwrow::DwRowItemWith<STRIDE, NOUT, kOutI8, ACT>(d, st, (uint32_t)m, wrow[t], sc[t], bi[t], oy, live, planes_out + it * ow);
+    }
+  });
+  const int plane_bytes = oh * ow;
+  char* obase = static_cast<char*>(d.out) + ((size_t)n * M + row0) * plane_bytes;
+  if ((plane_bytes & 3) == 0) {
+    const int per = plane_bytes >> 2;
+    for (int k = lane; k < 16 * per; k += 64) {
+      const int m = k / per, j = k - m * per;
+      StorePlain(*reinterpret_cast<const uint32_t*>(planes_out + 4 * k), obase + (size_t)(kRowStride * m) * plane_bytes + 4 * j);
+    }
+  } else {
+    for (int k = lane; k < 16 * plane_bytes; k += 64) {
+      const int m = k / plane_bytes, j = k - m * plane_bytes;
+      *reinterpret_cast<__attribute__((address_space(1))) char*>(reinterpret_cast<uintptr_t>(obase + (size_t)(kRowStride * m) * plane_bytes + j)) = planes_out[k];
+    }
   }
 }
 
@@ -161,10 +227,11 @@ __device__ __forceinline__ void Window(const uint4* __restrict__ xt, int kgs, in
 //
 // The head of the parameter block arrives in registers (kernarg_head.h): the image loads do not wait for a
 // load of the kernel arguments from memory (8.36 -> 8.10 us on the metric shape).
-template <int KS, int OUT, int QPI>
-__global__ void __launch_bounds__(512) ImageRowsMfmaKernel(PL_HEAD_PARAMS, const ImageMfmaParams block) {
-  const ImageMfmaParams p = WithHead(block, PL_HEAD_ARGS);
-  extern __shared__ uint4 lds_raw[];
+//
+// dw (kOutPlanes only): the depthwise layer that follows; the wavefront then keeps its 16 output planes in LDS
+// and runs that layer on them (DwStage below).
+template <int KS, int OUT, int QPI, int DW_STRIDE = 0>
+__device__ __forceinline__ void RowsBody(const ImageMfmaParams& p, uint4* lds_raw, const DwConvParams* dw) {
   // shifted windows read up to seven cells in front of a row of cells
   uint4* xt = lds_raw + 16;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -249,8 +316,10 @@ __global__ void __launch_bounds__(512) ImageRowsMfmaKernel(PL_HEAD_PARAMS, const
   const int nqt = (qpi + sh) >> 4;       // full windows
   const int left = qpi + sh - 16 * nqt;  // quads after the last window
   const int ntail = (left + 3) >> 2;
-  constexpr int kElem = OUT == kOutI8 ? 1 : 4;
-  char* orow = Uniform(static_cast<char*>(p.out) + ((size_t)n * p.M + row0) * hw * kElem);
+  constexpr int kElem = (OUT == kOutI8 || OUT == kOutPlanes) ? 1 : 4;
+  // kOutPlanes: the wavefront's planes behind the image's cells, 16 bytes of slack in front of them
+  char* planes = reinterpret_cast<char*>(lds_raw) + 256 + (size_t)NKG * kgs * 16 + wave * kPlaneBufBytes;
+  char* orow = OUT == kOutPlanes ? planes + 16 : Uniform(static_cast<char*>(p.out) + ((size_t)n * p.M + row0) * hw * kElem);
   DispatchAct(OUT == kOutAcc32 ? 0 : epilogue::LeakyAsMax(p.act), [&](auto act_c) {
     constexpr int ACT = decltype(act_c)::value;
     if (nqt > 0) {
@@ -293,11 +362,28 @@ __global__ void __launch_bounds__(512) ImageRowsMfmaKernel(PL_HEAD_PARAMS, const
       const int q = q0 + ln.kq;
       if (q >= 0 && q < qpi) {
         const u4 v = Finish4<OUT, ACT>(acc[0], acc[1], acc[2], acc[3], sct, bit, p.act);
-        char* ptr = orow + ((size_t)(kRowStride * ln.n) * hw + 4 * q) * kElem;
-        if (OUT == kOutI8) StorePlain(v.x, ptr); else StorePlain(v, ptr);
+        char* ptr = orow + ((size_t)(kPlaneStride<OUT> * ln.n) * hw + 4 * q) * kElem;
+        if (OUT == kOutPlanes) StoreLds(v.x, ptr); else if (OUT == kOutI8) StorePlain(v.x, ptr); else StorePlain(v, ptr);
       }
     }
   });
+  if constexpr (OUT == kOutPlanes) DwStage<DW_STRIDE>(*dw, planes + 16, planes + kPlaneInBytes, n, p.M, row0, lane);
+}
+
+template <int KS, int OUT, int QPI>
+__global__ void __launch_bounds__(512) ImageRowsMfmaKernel(PL_HEAD_PARAMS, const ImageMfmaParams block) {
+  const ImageMfmaParams p = WithHead(block, PL_HEAD_ARGS);
+  extern __shared__ uint4 lds_raw[];
+  RowsBody<KS, OUT, QPI>(p, lds_raw, nullptr);
+}
+
+// The same followed by the depthwise 3 x 3 layer (14 x 14 planes, padding 1, stride DW_STRIDE, int8 output) on
+// the wavefront's own 16 planes: the pointwise output never leaves the CU.
+template <int KS, int DW_STRIDE>
+__global__ void __launch_bounds__(512) ImageRowsDwKernel(PL_HEAD_PARAMS, const ImageMfmaParams block, const DwConvParams dw) {
+  const ImageMfmaParams p = WithHead(block, PL_HEAD_ARGS);
+  extern __shared__ uint4 lds_raw[];
+  RowsBody<KS, kOutPlanes, 49, DW_STRIDE>(p, lds_raw, &dw);
 }
 
 template <int OUT>
@@ -360,6 +446,49 @@ hipError_t LaunchImageRowsMfma(int out_kind, const ImageMfmaParams& p, hipStream
       return ByKs<kOutI8>(q, grid, lds, stream);
     case kOutAcc32:
       return ByKs<kOutAcc32>(q, grid, lds, stream);
+    default:
+      return hipErrorInvalidValue;
+  }
+}
+
+// The pointwise layer followed by the depthwise 3 x 3 layer on its output, in one launch (14 x 14 maps).
+bool ImageRowsDwFits(int M, int K, int hw, int h, int w, int pad, int stride) {
+  if (!ImageRowsMfmaFits(M, K, hw) || hw != 196 || h != 14 || w != 14 || pad != 1 || (stride != 1 && stride != 2)) return false;
+  return 256 + (size_t)(K / 16) * 208 * 16 + (size_t)8 * kPlaneBufBytes <= (size_t)kMaxLdsBytes;
+}
+
+hipError_t LaunchImageRowsDw(const ImageMfmaParams& p, const DwConvParams& d, int stride, hipStream_t stream) {
+  if (p.batch <= 0) return hipSuccess;
+  if (!ImageRowsDwFits(p.M, p.K, p.hw, d.h, d.w, d.pad, stride) || d.channels != p.M) return hipErrorInvalidValue;
+  const int oh = (14 + 2 - 3) / stride + 1;
+  if (d.oh != oh || d.ow != oh) return hipErrorInvalidValue;
+  // the image is read as dwords; planes of 196 bytes are stored as dwords, planes of 49 bytes byte by byte
+  if (reinterpret_cast<uintptr_t>(p.x) % 4 != 0 || (stride == 1 && reinterpret_cast<uintptr_t>(d.out) % 4 != 0)) return hipErrorInvalidValue;
+  ImageMfmaParams q = p;
+  q.qpi = 49;
+  q.kgs = 208;
+  q.row_groups = p.M / 128;
+  const int64_t items = (int64_t)p.batch * q.row_groups;
+  if (items > (1 << 28)) return hipErrorInvalidValue;
+  q.items = (int)items;
+  q.per_xcd = (q.items + 7) / 8;
+  q.align = 0;
+  const size_t lds = 256 + (size_t)(p.K / 16) * q.kgs * 16 + (size_t)8 * kPlaneBufBytes;
+  const dim3 grid(8u * (uint32_t)q.per_xcd), block(512);
+  const int shape = 10 * (p.K / 64) + stride;
+  switch (shape) {
+    case 21:
+      return LaunchWithHead(ImageRowsDwKernel<2, 1>, grid, block, lds, stream, q, d);
+    case 22:
+      return LaunchWithHead(ImageRowsDwKernel<2, 2>, grid, block, lds, stream, q, d);
+    case 41:
+      return LaunchWithHead(ImageRowsDwKernel<4, 1>, grid, block, lds, stream, q, d);
+    case 42:
+      return LaunchWithHead(ImageRowsDwKernel<4, 2>, grid, block, lds, stream, q, d);
+    case 81:
+      return LaunchWithHead(ImageRowsDwKernel<8, 1>, grid, block, lds, stream, q, d);
+    case 82:
+      return LaunchWithHead(ImageRowsDwKernel<8, 2>, grid, block, lds, stream, q, d);
     default:
       return hipErrorInvalidValue;
   }

@@ -39,13 +39,13 @@ __device__ __forceinline__ P WithHead(const P& block, PL_HEAD_PARAMS) {
 #define PL_IN_HEAD(Block, field) \
   static_assert(offsetof(Block, field) + sizeof(Block::field) <= ::pl::kHeadWords * 8, #field " must lie in the first 56 bytes of " #Block)
 
-// Launches kernel(head words..., block).
-template <typename Kernel, typename P>
-hipError_t LaunchWithHead(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const P& p) {
+// Launches kernel(head words..., block, further arguments...).
+template <typename Kernel, typename P, typename... More>
+hipError_t LaunchWithHead(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const P& p, const More&... more) {
   static_assert(std::is_trivially_copyable<P>::value && sizeof(P) >= kHeadWords * 8 && alignof(P) == 8, "parameter block with an 8-byte aligned head");
   const void* h[kHeadWords];
   std::memcpy(h, &p, sizeof(h));
-  return LaunchWithLds(kernel, grid, block, lds, stream, h[0], h[1], h[2], h[3], h[4], h[5], h[6], p);
+  return LaunchWithLds(kernel, grid, block, lds, stream, h[0], h[1], h[2], h[3], h[4], h[5], h[6], p, more...);
 }
 
 }  // namespace pl

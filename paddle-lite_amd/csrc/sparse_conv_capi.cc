@@ -1398,4 +1398,75 @@ int pl_dwconv3x3_run(pl_dwconv_handle* h, const int8_t* x_dev, void* out_dev, in
 
 void pl_dwconv3x3_destroy(pl_dwconv_handle* h) { delete h; }
 
+// ---- pointwise + depthwise in one launch -----------------------------------
+namespace {
+// nullptr when the pair can run as one launch, else the reason
+const char* FusedPairProblem(const pl_sparse_conv_handle* c, const pl_dwconv_handle* d, int height, int width) {
+  if (c->kind != PL_KIND_INT8_INT8 || d->kind != PL_KIND_INT8_INT8) return "both layers must be int8 -> int8";
+  if (c->device != d->device) return "the handles belong to different devices";
+  if (c->wtiles_rows.ptr == nullptr) return "the pointwise handle holds no row tiles (oc % 128 == 0 and ic = 128, 256 or 512 are needed)";
+  if (!c->auto_int8 && c->algo != PL_ALGO_IMAGE_MFMA) return "the pointwise handle is tied to another algorithm";
+  if (c->image_kernel != 0 && c->image_kernel != 3) return "the pointwise handle is tied to another image kernel";
+  if (d->channels != c->oc) return "the depthwise layer must have as many channels as the pointwise layer has output channels";
+  if (!pl::ImageRowsDwFits(c->oc, c->ic, height * width, height, width, d->pad, d->stride)) return "needs 14 x 14 maps, depthwise padding 1 and stride 1 or 2";
+  return nullptr;
+}
+}  // namespace
+
+int pl_sparse_conv_dwconv3x3_fits(const pl_sparse_conv_handle* conv, const pl_dwconv_handle* dw, int32_t height, int32_t width) {
+  if (!conv || !dw || height <= 0 || width <= 0) return 0;
+  return FusedPairProblem(conv, dw, height, width) == nullptr ? 1 : 0;
+}
+
+int pl_sparse_conv_dwconv3x3_pays(const pl_sparse_conv_handle* conv, const pl_dwconv_handle* dw, int32_t batch, int32_t height, int32_t width) {
+  if (!pl_sparse_conv_dwconv3x3_fits(conv, dw, height, width) || batch <= 0) return 0;
+  // Measured on 512 -> 512 @14x14 (us, two launches against one): stride 2: 9.3 / 8.6 at one image, 11.6 / 9.0 at 64;
+  // stride 1: 9.5 / 11.4 at one image, 9.8 / 11.6 at 8, 13.5 / 12.4 at 64.  The one launch does the depthwise work of
+  // 128 planes on the CU that made them, whatever the batch; the depthwise kernel spreads a small batch over the chip.
+  if (dw->stride == 2) return 1;
+  const int64_t workgroups = static_cast<int64_t>(batch) * (conv->oc / 128);
+  const int cus = std::max(1, conv->wg_slots_default / 2);
+  return workgroups * 8 >= static_cast<int64_t>(cus) * 7 ? 1 : 0;
+}
+
+int pl_sparse_conv_dwconv3x3_run(pl_sparse_conv_handle* conv, pl_dwconv_handle* dw, const void* x_dev, void* out_dev, int32_t batch, int32_t height, int32_t width, void* stream) {
+  if (!conv || !dw) return Fail(PL_ERR_BAD_ARG, "null handle");
+  if (batch < 0 || height <= 0 || width <= 0) return Fail(PL_ERR_BAD_ARG, "bad batch or input size");
+  if (const char* why = FusedPairProblem(conv, dw, height, width)) return Fail(PL_ERR_UNSUPPORTED, "pointwise + depthwise in one launch: %s", why);
+  if (batch == 0) return PL_OK;
+  if (!x_dev || !out_dev) return Fail(PL_ERR_BAD_ARG, "null device pointer");
+  int cur_dev = -1;
+  if (hipGetDevice(&cur_dev) != hipSuccess || cur_dev != conv->device) return Fail(PL_ERR_BAD_ARG, "the handles belong to device %d, the current device is %d", conv->device, cur_dev);
+  if (static_cast<int64_t>(batch) * conv->oc > 0x7fffffffll) return Fail(PL_ERR_UNSUPPORTED, "tensor too large");
+  if (reinterpret_cast<uintptr_t>(x_dev) % 4 != 0 || reinterpret_cast<uintptr_t>(out_dev) % 4 != 0) return Fail(PL_ERR_UNSUPPORTED, "pointwise + depthwise in one launch needs 4-byte aligned tensors");
+  pl::ImageMfmaParams p{};
+  p.x = static_cast<const int8_t*>(x_dev);
+  p.out = nullptr;
+  p.wtiles = conv->wtiles_rows.ptr;
+  p.scale = static_cast<const float*>(conv->scale.ptr);
+  p.bias = static_cast<const float*>(conv->bias.ptr);
+  p.M = conv->oc;
+  p.K = conv->ic;
+  p.hw = height * width;
+  p.batch = batch;
+  p.act = conv->act;
+  pl::DwConvParams d{};
+  d.x = nullptr;
+  d.out = out_dev;
+  d.wpack = static_cast<const uint32_t*>(dw->wpack.ptr);
+  d.scale = static_cast<const float*>(dw->scale.ptr);
+  d.bias = static_cast<const float*>(dw->bias.ptr);
+  d.channels = dw->channels;
+  d.h = height;
+  d.w = width;
+  d.oh = (height + 2 * dw->pad - 3) / dw->stride + 1;
+  d.ow = (width + 2 * dw->pad - 3) / dw->stride + 1;
+  d.pad = dw->pad;
+  d.planes = static_cast<uint32_t>(static_cast<int64_t>(batch) * dw->channels);
+  d.in_bytes = static_cast<int64_t>(d.planes) * height * width;
+  d.act = dw->act;
+  const hipError_t e = pl::LaunchImageRowsDw(p, d, dw->stride, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? PL_OK : FailHip(e, "pointwise + depthwise launch");
+}
+
 }  // extern "C"

@@ -160,3 +160,32 @@ class DepthwiseConv(object):
             self._release()
         except Exception:
             pass
+
+
+def conv_dw_fits(conv, dw, h, w):
+    """True when `conv` (a prepared SparseConvKernel, int8 -> int8) followed by `dw` (a prepared DepthwiseConv,
+    int8 -> int8) can run as one launch on h x w maps (pl_sparse_conv_dwconv3x3_fits)."""
+    if conv._handle is None or dw._handle is None:
+        raise RuntimeError("PrepareForRun has not been called")
+    return bool(capi.lib().pl_sparse_conv_dwconv3x3_fits(conv._handle, dw._handle, int(h), int(w)))
+
+
+def run_conv_dw(conv, dw, x, out=None, stream=None):
+    """sparse_conv2d followed by depthwise_conv2d in one launch (pl_sparse_conv_dwconv3x3_run): the result of
+    dw.Run(conv.Run(x)), bit for bit, without the tensor between them.  Raises where conv_dw_fits is False."""
+    import torch
+
+    if conv._handle is None or dw._handle is None:
+        raise RuntimeError("PrepareForRun has not been called")
+    if not x.is_cuda or not x.is_contiguous() or x.dtype != torch.int8 or x.dim() != 4 or x.shape[1] != conv.param.weights.ic:
+        raise ValueError("x must be a contiguous int8 NCHW device tensor with %d channels" % conv.param.weights.ic)
+    n, _, h, w = x.shape
+    shape = dw.out_shape((n, conv.param.weights.oc, h, w))
+    if out is None:
+        out = torch.empty(shape, dtype=torch.int8, device=x.device)
+    elif tuple(out.shape) != shape or out.dtype != torch.int8 or not out.is_contiguous() or out.device != x.device:
+        raise ValueError("out must be a contiguous int8 tensor of shape %s on the device of x" % (shape,))
+    s = torch.cuda.current_stream(x.device).cuda_stream if stream is None else stream
+    with torch.cuda.device(x.device):
+        capi.check(capi.lib().pl_sparse_conv_dwconv3x3_run(conv._handle, dw._handle, C.c_void_p(x.data_ptr()), C.c_void_p(out.data_ptr()), n, h, w, C.c_void_p(s)))
+    return out

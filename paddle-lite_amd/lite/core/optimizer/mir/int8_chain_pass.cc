@@ -1,5 +1,8 @@
 #include "lite/core/optimizer/mir/int8_chain_pass.h"
 
+#include "lite/kernels/hip/pair_launch.h"
+#include "pl_sparse_conv.h"
+
 #include <algorithm>
 #include <map>
 
@@ -160,13 +163,48 @@ HipProgram::HipProgram(const std::vector<ProgramStep>& steps, Scope* scope) {
     ops_.emplace_back(std::move(op));
     kernels_.emplace_back(std::move(ks[0]));
   }
+  // which steps hand their output to the next step alone
+  only_reader_is_next_.assign(steps.size(), 0);
+  for (size_t i = 0; i + 1 < steps.size(); ++i) {
+    std::vector<std::string> outs;
+    for (const auto& kv : steps[i].op.outputs()) outs.insert(outs.end(), kv.second.begin(), kv.second.end());
+    if (outs.size() != 1) continue;
+    size_t readers = 0;
+    bool next_reads = false;
+    for (size_t j = 0; j < steps.size(); ++j)
+      for (const auto& kv : steps[j].op.inputs())
+        for (const std::string& name : kv.second)
+          if (name == outs[0]) {
+            ++readers;
+            if (j == i + 1) next_reads = true;
+          }
+    only_reader_is_next_[i] = readers == 1 && next_reads;
+  }
 }
 
 void HipProgram::Enqueue(size_t first, size_t last) {
   CHECK(first <= last && last <= kernels_.size()) << "steps " << first << " .. " << last << " of " << kernels_.size();
+  pairs_joined_ = 0;
   for (size_t i = first; i < last; ++i) {
     CHECK(ops_[i]->CheckShape()) << "shape check failed at step " << i;
     CHECK(ops_[i]->InferShape()) << "shape inference failed at step " << i;
+    if (pair_launch_ && i + 1 < last && only_reader_is_next_[i]) {
+      auto* a = dynamic_cast<kernels::hip::PairLaunch*>(kernels_[i].get());
+      auto* b = dynamic_cast<kernels::hip::PairLaunch*>(kernels_[i + 1].get());
+      if (a && b && a->pair_role() == kernels::hip::PairLaunch::kFirst && b->pair_role() == kernels::hip::PairLaunch::kSecond) {
+        CHECK(ops_[i + 1]->CheckShape()) << "shape check failed at step " << i + 1;
+        CHECK(ops_[i + 1]->InferShape()) << "shape inference failed at step " << i + 1;
+        kernels::hip::PairEndpoint ea, eb;
+        if (a->pair_endpoint(&ea) && b->pair_endpoint(&eb) && eb.x == ea.out && ea.stream == eb.stream &&
+            pl_sparse_conv_dwconv3x3_pays(static_cast<pl_sparse_conv_handle*>(ea.handle), static_cast<pl_dwconv_handle*>(eb.handle), ea.batch, ea.h, ea.w)) {
+          const int rc = pl_sparse_conv_dwconv3x3_run(static_cast<pl_sparse_conv_handle*>(ea.handle), static_cast<pl_dwconv_handle*>(eb.handle), ea.x, eb.out, ea.batch, ea.h, ea.w, ea.stream);
+          if (rc != PL_OK) LOG(FATAL) << "pl_sparse_conv_dwconv3x3_run failed (" << rc << "): " << pl_last_error();
+          ++pairs_joined_;
+          ++i;  // the depthwise step ran with this one
+          continue;
+        }
+      }
+    }
     kernels_[i]->Launch();
   }
 }

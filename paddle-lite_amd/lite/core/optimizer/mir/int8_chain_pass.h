@@ -58,12 +58,21 @@ class HipProgram {
   // the steps into a stream capture.
   void Enqueue(size_t first, size_t last);
   void Sync();  // waits for the stream of the last step
+  // Pair launches (lite/kernels/hip/pair_launch.h): an int8 -> int8 sparse_conv2d step followed by the int8 -> int8
+  // depthwise_conv2d step that is the only reader of its output runs as one launch where the library says that
+  // pays for the step's shapes (from the second Enqueue on: the first one prepares the kernels).  The tensor
+  // between the two steps is then not written.  Off by default.
+  void set_pair_launch(bool on) { pair_launch_ = on; }
+  size_t pairs_joined_last_enqueue() const { return pairs_joined_; }
   size_t size() const { return kernels_.size(); }
   const KernelBase& kernel(size_t i) const { return *kernels_[i]; }
 
  private:
   std::vector<std::shared_ptr<OpLite>> ops_;
   std::vector<std::unique_ptr<KernelBase>> kernels_;
+  std::vector<char> only_reader_is_next_;  // per step: its first output is read by step + 1 and by no other step
+  bool pair_launch_ = false;
+  size_t pairs_joined_ = 0;
 };
 
 }  // namespace mir

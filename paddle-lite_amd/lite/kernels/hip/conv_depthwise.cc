@@ -6,6 +6,7 @@
 // depthwise_conv2d int8 kernels (aliases int8_out / fp32_out,
 // conv_compute.cc:252-300).
 #include "lite/core/op_registry.h"
+#include "lite/kernels/hip/pair_launch.h"
 #include "lite/operators/op_params.h"
 #include "pl_sparse_conv.h"
 
@@ -15,7 +16,7 @@ namespace kernels {
 namespace hip {
 
 template <PrecisionType O>
-class DepthwiseConvInt8 : public KernelLite<TARGET(kHIP), PRECISION(kInt8)> {
+class DepthwiseConvInt8 : public KernelLite<TARGET(kHIP), PRECISION(kInt8)>, public PairLaunch {
  public:
   using param_t = operators::ConvParam;
   ~DepthwiseConvInt8() override {
@@ -83,6 +84,24 @@ class DepthwiseConvInt8 : public KernelLite<TARGET(kHIP), PRECISION(kInt8)> {
     const int rc = pl_dwconv3x3_run(handle_, static_cast<const int8_t*>(param.x->raw_data()), out, static_cast<int32_t>(xd[0]), static_cast<int32_t>(xd[2]), static_cast<int32_t>(xd[3]),
                                     this->ctx_->template As<HIPContext>().stream());
     if (rc != PL_OK) LOG(FATAL) << "pl_dwconv3x3_run failed (" << rc << "): " << pl_last_error();
+  }
+
+  // Second end of a pair launch (pair_launch.h): only the int8 -> int8 kernel can be one.
+  PairLaunch::Role pair_role() const override { return PairLaunch::kSecond; }
+  bool pair_endpoint(PairEndpoint* e) override {
+    if (handle_ == nullptr || O != PRECISION(kInt8)) return false;
+    auto& param = this->template Param<param_t>();
+    if (param.x->target() != TargetType::kHIP) return false;
+    const DDim& xd = param.x->dims();
+    if (xd.size() != 4) return false;
+    e->handle = handle_;
+    e->x = param.x->raw_data();
+    e->out = param.output->template mutable_data<int8_t>(TargetType::kHIP);
+    e->batch = static_cast<int>(xd[0]);
+    e->h = static_cast<int>(xd[2]);
+    e->w = static_cast<int>(xd[3]);
+    e->stream = this->ctx_->template As<HIPContext>().stream();
+    return true;
   }
 
  private:

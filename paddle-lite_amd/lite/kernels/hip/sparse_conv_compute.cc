@@ -171,6 +171,24 @@ void SparseConvCompute<P, O>::Run() {
 }
 
 template <PrecisionType P, PrecisionType O>
+bool SparseConvCompute<P, O>::pair_endpoint(PairEndpoint* e) {
+  if (handle_ == nullptr || P != PRECISION(kInt8) || O != PRECISION(kInt8)) return false;
+  auto& param = this->template Param<param_t>();
+  if (param.x->target() != TargetType::kHIP) return false;
+  CheckGeometry(param);
+  const DDim& xd = param.x->dims();
+  if (xd.size() != 4 || xd[1] != ic_) return false;
+  e->handle = handle_;
+  e->x = param.x->raw_data();
+  e->out = param.output->template mutable_data<int8_t>(TargetType::kHIP);
+  e->batch = static_cast<int>(xd[0]);
+  e->h = static_cast<int>(xd[2]);
+  e->w = static_cast<int>(xd[3]);
+  e->stream = this->ctx_->template As<HIPContext>().stream();
+  return true;
+}
+
+template <PrecisionType P, PrecisionType O>
 std::string SparseConvCompute<P, O>::kernel_func_name() const {
   if (handle_ == nullptr || last_batch_ < 0) return "NotImplForSparseConv";
   static const char* const kAlgo[] = {"auto", "row_walk", "block_mfma", "image_mfma"};

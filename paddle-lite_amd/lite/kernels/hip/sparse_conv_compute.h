@@ -8,6 +8,7 @@
 
 #include "lite/core/kernel.h"
 #include "lite/core/profile/profiler.h"
+#include "lite/kernels/hip/pair_launch.h"
 #include "lite/operators/op_params.h"
 
 struct pl_sparse_conv_handle;
@@ -18,7 +19,7 @@ namespace kernels {
 namespace hip {
 
 template <PrecisionType Ptype, PrecisionType OutType>
-class SparseConvCompute : public KernelLite<TARGET(kHIP), Ptype> {
+class SparseConvCompute : public KernelLite<TARGET(kHIP), Ptype>, public PairLaunch {
  public:
   using param_t = operators::SparseConvParam;
   ~SparseConvCompute() override;
@@ -30,6 +31,10 @@ class SparseConvCompute : public KernelLite<TARGET(kHIP), Ptype> {
   void Run() override;
 
   const std::vector<float>& merged_scales() const { return w_scale_; }
+
+  // First end of a pair launch (pair_launch.h): only the int8 -> int8 kernel can be one.
+  PairLaunch::Role pair_role() const override { return PairLaunch::kFirst; }
+  bool pair_endpoint(PairEndpoint* e) override;
 
   // The math entry point and algorithm of the last Run(), for the profiler
   // (the ARM class reports "sparse_conv_fp32_pipelined" etc. through

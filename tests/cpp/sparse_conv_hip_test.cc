@@ -1245,6 +1245,126 @@ static void MobileNetBlocks(bool run_on_device) {
   EXPECT(got->memory_size() == want.size() * 4 && std::memcmp(want.data(), got->raw_data(), want.size() * 4) == 0);
 }
 
+// Pair launches of mir::HipProgram: pointwise (128 -> 128, int8 out) -> depthwise (stride 2 and stride 1, int8 out)
+// -> pointwise (fp32 out) on 14 x 14 maps.  With pair launches on, a pointwise step and the depthwise step that
+// alone reads its output run as one launch where the library says it pays (stride 2: at any batch; stride 1: not
+// at a batch of two); the fetched output must not change by a bit.  A depthwise output with a second reader is
+// never joined.
+static void PairLaunches(bool run_on_device) {
+  std::printf("pair launches\n");
+  std::fflush(stdout);
+  for (int stride = 1; stride <= 2; ++stride) {
+    for (int second_reader = 0; second_reader <= 1; ++second_reader) {
+      const int batch = 2, size = 14, c = 128;
+      const int out_size = (size + 2 - 3) / stride + 1;
+      Scope scope;
+      std::mt19937 gen(500 + stride);
+      std::uniform_real_distribution<float> uni(0.f, 1.f);
+      Tensor* a0 = scope.NewTensor("p0");
+      a0->Resize({batch, c, size, size});
+      float* a0d = a0->mutable_data<float>(TargetType::kHost);
+      for (int64_t i = 0; i < a0->numel(); ++i) a0d[i] = uni(gen) * 2.f - 1.f;
+      std::vector<OpInfo> ops;
+      auto pointwise = [&](const std::string& n, const std::string& in, const std::string& out, int oc, float in_scale) {
+        Tensor* w = scope.NewTensor("ppw_w" + n);
+        w->Resize({oc, c, 1, 1});
+        int8_t* wd = w->mutable_data<int8_t>(TargetType::kHost);
+        for (int64_t i = 0; i < w->numel(); ++i) {
+          int v = static_cast<int>(uni(gen) * 127.f) + 1;
+          if (uni(gen) < 0.5f) v = -v;
+          wd[i] = uni(gen) >= 0.8f ? static_cast<int8_t>(v) : 0;
+        }
+        Tensor* b = scope.NewTensor("ppw_b" + n);
+        b->Resize({oc});
+        float* bd = b->mutable_data<float>(TargetType::kHost);
+        for (int i = 0; i < oc; ++i) bd[i] = (uni(gen) - 0.5f) * 0.2f;
+        std::vector<float> ws(oc);
+        for (float& v : ws) v = 0.001f + 0.004f * uni(gen);
+        OpInfo conv("conv2d");
+        conv.SetInput("Input", {in});
+        conv.SetInput("Filter", {"ppw_w" + n});
+        conv.SetInput("Bias", {"ppw_b" + n});
+        conv.SetOutput("Output", {out});
+        conv.SetAttr<std::vector<int>>("strides", {1, 1});
+        conv.SetAttr<std::vector<int>>("paddings", {0, 0});
+        conv.SetAttr<std::vector<int>>("dilations", {1, 1});
+        conv.SetAttr<int>("groups", 1);
+        conv.SetAttr<bool>("with_act", true);
+        conv.SetAttr<std::string>("act_type", "relu");
+        conv.SetAttr<bool>("enable_int8", true);
+        conv.SetInputScale("Input0_scale", {in_scale}, true);
+        conv.SetInputScale("Filter0_scale", ws, true);
+        conv.SetOutputScale("Output0_scale", {1.f}, true);
+        ops.push_back(conv);
+      };
+      pointwise("1", "p0", "p1", c, 0.02f);
+      scope.NewTensor("p1")->Resize({batch, c, size, size});
+      {
+        Tensor* f = scope.NewTensor("pdw_w");
+        f->Resize({c, 1, 3, 3});
+        int8_t* fd = f->mutable_data<int8_t>(TargetType::kHost);
+        for (int64_t i = 0; i < f->numel(); ++i) fd[i] = static_cast<int8_t>(static_cast<int>(uni(gen) * 255.f) - 127);
+        Tensor* b = scope.NewTensor("pdw_b");
+        b->Resize({c});
+        float* bd = b->mutable_data<float>(TargetType::kHost);
+        for (int i = 0; i < c; ++i) bd[i] = uni(gen) - 0.5f;
+        std::vector<float> ws(c);
+        for (float& v : ws) v = 0.0005f + 0.001f * uni(gen);
+        OpInfo dw("depthwise_conv2d");
+        dw.SetInput("Input", {"p1"});
+        dw.SetInput("Filter", {"pdw_w"});
+        dw.SetInput("Bias", {"pdw_b"});
+        dw.SetOutput("Output", {"p2"});
+        dw.SetAttr<std::vector<int>>("strides", {stride, stride});
+        dw.SetAttr<std::vector<int>>("paddings", {1, 1});
+        dw.SetAttr<std::vector<int>>("dilations", {1, 1});
+        dw.SetAttr<int>("groups", c);
+        dw.SetAttr<bool>("with_act", true);
+        dw.SetAttr<std::string>("act_type", "relu");
+        dw.SetAttr<bool>("enable_int8", true);
+        dw.SetInputScale("Input0_scale", {0.03f}, true);
+        dw.SetInputScale("Filter0_scale", ws, true);
+        dw.SetOutputScale("Output0_scale", {1.f}, true);
+        ops.push_back(dw);
+      }
+      scope.NewTensor("p2")->Resize({batch, c, out_size, out_size});
+      pointwise("2", "p2", "p3", 256, 0.025f);
+      scope.NewTensor("p3");
+      // a second reader of the pointwise output p1: it must then be written, so the pair is not joined
+      if (second_reader) {
+        pointwise("3", "p1", "p4", 128, 0.03f);
+        scope.NewTensor("p4");
+      }
+      mir::SparseConvDetectPass detect;
+      detect.SetSparseThreshold(0.5f);
+      EXPECT(detect.Apply(&ops, &scope) == (second_reader ? 3 : 2));
+      mir::Int8ChainPass chain;
+      std::vector<std::string> fetches = {"p3"};
+      if (second_reader) fetches.push_back("p4");
+      std::vector<mir::ProgramStep> steps = chain.Apply(ops, {"p0"}, fetches, &scope);
+      EXPECT(steps.size() >= 6);
+      if (!run_on_device || steps.size() < 6) continue;
+      mir::HipProgram program(steps, &scope);
+      program.Run();
+      EXPECT(program.pairs_joined_last_enqueue() == 0);
+      const Tensor* got = scope.FindMutableTensor("p3/host");
+      EXPECT(got != nullptr);
+      if (!got) continue;
+      std::vector<char> two_launches(static_cast<const char*>(got->raw_data()), static_cast<const char*>(got->raw_data()) + got->memory_size());
+      program.set_pair_launch(true);
+      program.Run();
+      // stride 2 pays at any batch, stride 1 only when the launch fills the chip
+      const size_t expect_pairs = (stride == 2 && !second_reader) ? 1 : 0;
+      EXPECT(program.pairs_joined_last_enqueue() == expect_pairs);
+      EXPECT(got->memory_size() == two_launches.size() && std::memcmp(got->raw_data(), two_launches.data(), two_launches.size()) == 0);
+      program.set_pair_launch(false);
+      program.Run();
+      EXPECT(program.pairs_joined_last_enqueue() == 0);
+      EXPECT(std::memcmp(got->raw_data(), two_launches.data(), two_launches.size()) == 0);
+    }
+  }
+}
+
 int main(int argc, char** argv) {
   const bool gpu = argc > 1 && std::string(argv[1]) == "--gpu";
   RegistryAndErrorPaths();
@@ -1271,6 +1391,7 @@ int main(int argc, char** argv) {
   ModelFile(gpu);
   Depthwise(gpu);
   MobileNetBlocks(gpu);
+  PairLaunches(gpu);
   std::printf("%s: %d failure(s)\n", gpu ? "gpu" : "cpu", g_failures);
   return g_failures ? 1 : 0;
 }

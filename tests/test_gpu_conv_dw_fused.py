@@ -1,0 +1,149 @@
+"""sparse_conv2d (int8 -> int8) followed by the int8 depthwise 3x3 convolution as ONE launch
+(pl_sparse_conv_dwconv3x3_run), through the C ABI: equal, bit for bit, to the two launches it replaces and to
+the oracle's two functions applied one after the other.  14 x 14 maps, depthwise stride 1 and 2, the channel
+counts of the image kernel (128 / 256 / 512 in, multiples of 128 out), the activations of both layers, batches
+that do and do not fill the chip; pairs that cannot run as one launch are refused with a reason."""
+import importlib
+
+import numpy as np
+import pytest
+
+from helpers import capi, make_kernel, merged_for_oracle, oracle_pack, workloads
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+pla = importlib.import_module("paddle-lite_amd")
+dwmod = importlib.import_module("paddle-lite_amd.depthwise_conv")
+
+ACTS = {
+    "none": lambda: pla.ActivationParam(),
+    "relu": lambda: pla.ActivationParam("relu"),
+    "relu6": lambda: pla.ActivationParam("relu6", Relu_clipped_coef=6.0),
+    "leaky": lambda: pla.ActivationParam("leaky_relu", Leaky_relu_alpha=0.12),
+    "hswish": lambda: pla.ActivationParam("hard_swish", hard_swish_scale=1.0 / 6.0, hard_swish_offset=3.0, hard_swish_threshold=6.0),
+}
+
+
+def oracle_act(ap):
+    a = O.Act()
+    a.type = ap.active_type if ap.has_active else 0
+    a.relu6_coef = ap.Relu_clipped_coef
+    a.leaky_alpha = ap.Leaky_relu_alpha
+    a.hs_scale = ap.hard_swish_scale
+    a.hs_offset = ap.hard_swish_offset
+    a.hs_threshold = ap.hard_swish_threshold
+    return a
+
+
+def make_pair(batch, ic, oc, stride, act_pw, act_dw, seed, size=14, pad=1, sparsity=0.85):
+    case = workloads.make_int8("fused", batch, ic, oc, size, size, sparsity, False, ACTS[act_pw](), out_int8=True, seed=seed)
+    # an output scale that keeps most of the pointwise outputs inside the int8 range and saturates some
+    sigma_acc = np.sqrt(ic * (1.0 - sparsity)) * 73.3 * 73.3
+    case.output_scale = float(2.0 * sigma_acc * float(np.mean(case.weight_scale)) * case.input_scale / 127.0)
+    conv, _ = make_kernel(case)
+    rng = np.random.RandomState(seed + 1000)
+    filt = rng.randint(-127, 128, size=(oc, 1, 3, 3)).astype(np.int8)
+    ws = rng.uniform(0.002, 0.02, size=oc).astype(np.float32)
+    b = (rng.standard_normal(oc) * 0.5).astype(np.float32)
+    param = pla.ConvParam(filt, b, strides=(stride, stride), paddings=(pad, pad, pad, pad), activation_param=ACTS[act_dw](), input_scale=0.02, weight_scale=ws, output_scale=0.11)
+    dw = pla.DepthwiseConv(param, out_precision="int8")
+    dw.PrepareForRun()
+    return case, conv, dw, filt
+
+
+def check_pair(batch, ic, oc, stride, act_pw="relu", act_dw="relu", seed=0, with_oracle=False, guard=64):
+    import torch
+
+    case, conv, dw, filt = make_pair(batch, ic, oc, stride, act_pw, act_dw, seed)
+    assert dwmod.conv_dw_fits(conv, dw, 14, 14)
+    x = torch.from_numpy(case.x).cuda()
+    mid = conv.Run(x)
+    want = dw.Run(mid)
+    shape = tuple(want.shape)
+    numel = int(np.prod(shape))
+    buf = torch.full((numel + 2 * guard,), 77, dtype=torch.int8, device="cuda")
+    got = dwmod.run_conv_dw(conv, dw, x, buf[guard:guard + numel].view(shape))
+    torch.cuda.synchronize()
+    host = buf.cpu().numpy()
+    assert (host[:guard] == 77).all() and (host[guard + numel:] == 77).all(), "wrote outside the output"
+    g, w = got.cpu().numpy(), want.cpu().numpy()
+    if not np.array_equal(g, w):
+        bad = np.argwhere(g != w)
+        raise AssertionError("%d of %d outputs differ from the two launches, first at %s: got %d want %d" % (len(bad), g.size, tuple(bad[0]), g[tuple(bad[0])], w[tuple(bad[0])]))
+    if with_oracle:
+        scale, bias, act = merged_for_oracle(case)
+        mid_o = O.sparse_conv_int8(oracle_pack(case), case.x, scale, bias, act, out_int8=True)
+        assert np.array_equal(mid.cpu().numpy(), mid_o)
+        want_o = O.dwconv3x3_int8(mid_o, filt[:, 0], dw.w_scale_, dw.bias_, oracle_act(dw.merged_act), out="int8", stride=stride, pad=1)
+        assert np.array_equal(g, want_o)
+
+
+@pytest.mark.parametrize("stride", [1, 2])
+@pytest.mark.parametrize("ic,oc", [(128, 128), (256, 512), (512, 512), (512, 256)])
+def test_channel_counts_against_the_oracle(ic, oc, stride):
+    check_pair(2, ic, oc, stride, seed=ic + oc + stride, with_oracle=True)
+
+
+@pytest.mark.parametrize("stride", [1, 2])
+@pytest.mark.parametrize("act_pw,act_dw", [("none", "none"), ("relu6", "relu"), ("leaky", "relu6"), ("hswish", "leaky"), ("relu", "hswish")])
+def test_activations(act_pw, act_dw, stride):
+    check_pair(3, 256, 128, stride, act_pw, act_dw, seed=7, with_oracle=True)
+
+
+@pytest.mark.parametrize("batch", [1, 5, 64, 67])
+@pytest.mark.parametrize("stride", [1, 2])
+def test_batches(batch, stride):
+    check_pair(batch, 512, 512, stride, seed=batch)
+
+
+def test_two_calls_in_a_row_reuse_nothing():
+    """The planes in LDS are rebuilt by every launch: a second call with other inputs is as exact as the first."""
+    check_pair(8, 512, 512, 1, seed=1)
+    check_pair(8, 512, 512, 2, seed=2)
+    check_pair(4, 256, 256, 1, seed=3)
+
+
+def test_pairs_that_do_not_fit_are_refused():
+    import torch
+
+    case, conv, dw, _ = make_pair(2, 256, 128, 1, "relu", "relu", 11)
+    # other map sizes
+    assert not dwmod.conv_dw_fits(conv, dw, 7, 7)
+    assert not dwmod.conv_dw_fits(conv, dw, 28, 28)
+    x = torch.zeros((2, 256, 28, 28), dtype=torch.int8, device="cuda")
+    with pytest.raises(RuntimeError, match="14 x 14"):
+        dwmod.run_conv_dw(conv, dw, x)
+    # a depthwise layer without padding
+    rng = np.random.RandomState(0)
+    filt = rng.randint(-127, 128, size=(128, 1, 3, 3)).astype(np.int8)
+    param = pla.ConvParam(filt, None, strides=(1, 1), paddings=(0, 0, 0, 0), activation_param=pla.ActivationParam(), input_scale=0.02, weight_scale=np.full(128, 0.01, np.float32), output_scale=0.1)
+    dw0 = pla.DepthwiseConv(param, out_precision="int8")
+    dw0.PrepareForRun()
+    assert not dwmod.conv_dw_fits(conv, dw0, 14, 14)
+    # channel counts that do not match
+    _, conv2, _, _ = make_pair(1, 128, 256, 1, "relu", "relu", 12)
+    assert not dwmod.conv_dw_fits(conv2, dw, 14, 14)
+    # a pointwise layer with fp32 output
+    case_f = workloads.make_int8("f", 1, 256, 128, 14, 14, 0.85, False, pla.ActivationParam("relu"), out_int8=False, seed=3)
+    conv_f, _ = make_kernel(case_f)
+    assert not dwmod.conv_dw_fits(conv_f, dw, 14, 14)
+    # a pointwise layer tied to another algorithm
+    conv_w, _ = make_kernel(case, algo=capi.ALGO_ROW_WALK)
+    assert not dwmod.conv_dw_fits(conv_w, dw, 14, 14)
+
+
+def test_when_the_one_launch_pays():
+    """pl_sparse_conv_dwconv3x3_pays: stride 2 at any batch; stride 1 only when the launch has about as many
+    workgroups (batch * oc / 128) as the device has CUs."""
+    L = capi.lib()
+    _, conv, dw1, _ = make_pair(1, 512, 512, 1, "relu", "relu", 21)
+    _, _, dw2, _ = make_pair(1, 512, 512, 2, "relu", "relu", 22)
+    cus = 256
+    assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw2._handle, 1, 14, 14) == 1
+    assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw2._handle, 64, 14, 14) == 1
+    assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw1._handle, 1, 14, 14) == 0
+    assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw1._handle, 8, 14, 14) == 0
+    assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw1._handle, cus // 4, 14, 14) == 1  # 512 / 128 = 4 workgroups per image
+    assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw1._handle, 2 * cus, 14, 14) == 1
+    assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw1._handle, 64, 7, 7) == 0  # does not fit
+    assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw1._handle, 0, 14, 14) == 0
