@@ -344,7 +344,7 @@ int pl_sparse_conv_dwconv3x3_fits(const pl_sparse_conv_handle* conv, const pl_dw
                                   int32_t h, int32_t w);
 /* 1 when the pair fits and the one launch is expected to be faster than the
  * two at this batch: always for stride 2; for stride 1 when the launch has
- * at least 7/8 as many workgroups (batch * oc / 128) as the device has CUs -
+ * at least half as many workgroups (batch * oc / 128) as the device has CUs -
  * the one launch keeps the depthwise work of a workgroup's 128 planes on its
  * CU, which loses to the depthwise kernel's spread at small batches. */
 int pl_sparse_conv_dwconv3x3_pays(const pl_sparse_conv_handle* conv, const pl_dwconv_handle* dw,

@@ -27,15 +27,18 @@ struct DwRowStage {
 // column -pad are read from LDS, shifted into place (v_alignbyte_b32), masked outside the row once, and the byte
 // windows of the NOUT outputs slid out of them.  int8 outputs are written byte by byte to dst_i8 (LDS), fp32
 // outputs stored to p.out directly.  Lanes that are not `live` compute nothing and store nothing.
-template <int STRIDE, int NOUT, int OUT, int ACT>
+template <int STRIDE, int NOUT, int OUT, int ACT, int FIXED = 0>
 __device__ __forceinline__ void DwRowItemWith(const DwConvParams& p, const DwRowStage& st, uint32_t plane, const uint32_t (&wrow)[3], float s, float b, int oy, bool live, char* dst_i8) {
+  // FIXED: planes of FIXED x FIXED with padding 1, known at compile time (masks and row bounds become constants)
+  const int h = FIXED ? FIXED : p.h, w = FIXED ? FIXED : p.w, pad = FIXED ? 1 : p.pad;
+  const int oh = FIXED ? (FIXED - 1) / STRIDE + 1 : p.oh, ow = FIXED ? (FIXED - 1) / STRIDE + 1 : p.ow;
   // byte b of a window is column b - pad
   uint32_t mask[4];
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
     uint32_t m = 0xffffffffu;
-    const int below = p.pad - 4 * k;          // bytes of the dword in front of column 0
-    const int inside = p.pad + p.w - 4 * k;   // bytes of the dword, from its first, up to the end of the row
+    const int below = pad - 4 * k;          // bytes of the dword in front of column 0
+    const int inside = pad + w - 4 * k;   // bytes of the dword, from its first, up to the end of the row
     if (below > 0) m &= 0xffffffffu << (8 * below);
     m = inside <= 0 ? 0u : (inside < 4 ? m & (0xffffffffu >> (8 * (4 - inside))) : m);
     mask[k] = m;
@@ -44,13 +47,13 @@ __device__ __forceinline__ void DwRowItemWith(const DwConvParams& p, const DwRow
 #pragma unroll
   for (int j = 0; j < NOUT; ++j) acc[j] = 0;
   if (live) {
-    const int iy0 = STRIDE * oy - p.pad;
-    const int64_t plane_at = (int64_t)plane * (uint32_t)(p.h * p.w) - st.in_base + 16;  // LDS offset of the plane's first byte
+    const int iy0 = STRIDE * oy - pad;
+    const int64_t plane_at = (int64_t)plane * (uint32_t)(h * w) - st.in_base + 16;  // LDS offset of the plane's first byte
     uint32_t D[3][4];
 #pragma unroll
     for (int r = 0; r < 3; ++r) {
       // a row outside [0, h) is zero padding: it reads its neighbour and meets a zero filter row below
-      const uint32_t at = (uint32_t)(plane_at + (uint32_t)(min(max(iy0 + r, 0), p.h - 1) * p.w) - p.pad);
+      const uint32_t at = (uint32_t)(plane_at + (uint32_t)(min(max(iy0 + r, 0), h - 1) * w) - pad);
       const uint32_t* words = reinterpret_cast<const uint32_t*>(st.lds_in + (at & ~3u));
       uint32_t e[5];
 #pragma unroll
@@ -61,7 +64,7 @@ __device__ __forceinline__ void DwRowItemWith(const DwConvParams& p, const DwRow
 #pragma unroll
     for (int r = 0; r < 3; ++r) {
       const int iy = iy0 + r;
-      const int wr = (int)(wrow[r] & ((iy >= 0 && iy < p.h) ? 0xffffffffu : 0u));
+      const int wr = (int)(wrow[r] & ((iy >= 0 && iy < h) ? 0xffffffffu : 0u));
       uint32_t d[4];
 #pragma unroll
       for (int k = 0; k < 4; ++k) d[k] = D[r][k] & mask[k];
@@ -78,14 +81,14 @@ __device__ __forceinline__ void DwRowItemWith(const DwConvParams& p, const DwRow
     if (live) {
 #pragma unroll
       for (int j = 0; j < NOUT; ++j)
-        if (j < p.ow) dst_i8[j] = (char)static_cast<int>(ActQuantF<ACT>(__builtin_fmaf((float)acc[j], s, b), p.act));
+        if (j < ow) dst_i8[j] = (char)static_cast<int>(ActQuantF<ACT>(__builtin_fmaf((float)acc[j], s, b), p.act));
     }
   } else if (live) {
-    float* dst = static_cast<float*>(p.out) + ((size_t)plane * (uint32_t)p.oh + (uint32_t)oy) * (uint32_t)p.ow;
+    float* dst = static_cast<float*>(p.out) + ((size_t)plane * (uint32_t)oh + (uint32_t)oy) * (uint32_t)ow;
     constexpr int NG = (NOUT + 3) / 4;
 #pragma unroll
     for (int q4 = 0; q4 < NG; ++q4) {
-      const int n_out = min(4, p.ow - 4 * q4);
+      const int n_out = min(4, ow - 4 * q4);
       if (n_out <= 0) break;
       float v[4];
 #pragma unroll

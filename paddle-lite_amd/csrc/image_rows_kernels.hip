@@ -161,7 +161,7 @@ __device__ __forceinline__ void DwStage(const DwConvParams& d, char* planes_in, 
       const bool live = item < items;
       const int it = live ? item : items - 1;
       const int m = it / oh, oy = it - m * oh;
-      dwrow::DwRowItemWith<STRIDE, NOUT, kOutI8, ACT>(d, st, (uint32_t)m, wrow[t], sc[t], bi[t], oy, live, planes_out + it * ow);
+      dwrow::DwRowItemWith<STRIDE, NOUT, kOutI8, ACT, 14>(d, st, (uint32_t)m, wrow[t], sc[t], bi[t], oy, live, planes_out + it * ow);
     }
   });
   const int plane_bytes = oh * ow;

@@ -1420,13 +1420,14 @@ int pl_sparse_conv_dwconv3x3_fits(const pl_sparse_conv_handle* conv, const pl_dw
 
 int pl_sparse_conv_dwconv3x3_pays(const pl_sparse_conv_handle* conv, const pl_dwconv_handle* dw, int32_t batch, int32_t height, int32_t width) {
   if (!pl_sparse_conv_dwconv3x3_fits(conv, dw, height, width) || batch <= 0) return 0;
-  // Measured on 512 -> 512 @14x14 (us, two launches against one): stride 2: 9.3 / 8.6 at one image, 11.6 / 9.0 at 64;
-  // stride 1: 9.5 / 11.4 at one image, 9.8 / 11.6 at 8, 13.5 / 12.4 at 64.  The one launch does the depthwise work of
-  // 128 planes on the CU that made them, whatever the batch; the depthwise kernel spreads a small batch over the chip.
+  // Measured on 512 -> 512 @14x14 (us, two launches against one, at 1 / 16 / 32 / 48 / 64 images): stride 2: 9.3 / 8.2,
+  // 9.8 / 8.4, 10.3 / 8.5, 11.0 / 8.6, 11.9 / 8.8; stride 1: 9.6 / 10.7, 10.4 / 11.1, 11.4 / 11.3, 12.7 / 11.5, 13.8 / 11.8.
+  // The one launch does the depthwise work of 128 planes on the CU that made them, whatever the batch; the
+  // depthwise kernel spreads a small batch over the chip.
   if (dw->stride == 2) return 1;
   const int64_t workgroups = static_cast<int64_t>(batch) * (conv->oc / 128);
   const int cus = std::max(1, conv->wg_slots_default / 2);
-  return workgroups * 8 >= static_cast<int64_t>(cus) * 7 ? 1 : 0;
+  return workgroups * 2 >= static_cast<int64_t>(cus) ? 1 : 0;
 }
 
 int pl_sparse_conv_dwconv3x3_run(pl_sparse_conv_handle* conv, pl_dwconv_handle* dw, const void* x_dev, void* out_dev, int32_t batch, int32_t height, int32_t width, void* stream) {

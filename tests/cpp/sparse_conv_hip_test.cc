@@ -1248,7 +1248,7 @@ static void MobileNetBlocks(bool run_on_device) {
 // Pair launches of mir::HipProgram: pointwise (128 -> 128, int8 out) -> depthwise (stride 2 and stride 1, int8 out)
 // -> pointwise (fp32 out) on 14 x 14 maps.  With pair launches on, a pointwise step and the depthwise step that
 // alone reads its output run as one launch where the library says it pays (stride 2: at any batch; stride 1: not
-// at a batch of two); the fetched output must not change by a bit.  A depthwise output with a second reader is
+// at a batch of two, which leaves most of the chip idle); the fetched output must not change by a bit.  A depthwise output with a second reader is
 // never joined.
 static void PairLaunches(bool run_on_device) {
   std::printf("pair launches\n");

@@ -133,8 +133,8 @@ def test_pairs_that_do_not_fit_are_refused():
 
 
 def test_when_the_one_launch_pays():
-    """pl_sparse_conv_dwconv3x3_pays: stride 2 at any batch; stride 1 only when the launch has about as many
-    workgroups (batch * oc / 128) as the device has CUs."""
+    """pl_sparse_conv_dwconv3x3_pays: stride 2 at any batch; stride 1 only when the launch has at least as many
+    workgroups (batch * oc / 128) as half the device's CUs."""
     L = capi.lib()
     _, conv, dw1, _ = make_pair(1, 512, 512, 1, "relu", "relu", 21)
     _, _, dw2, _ = make_pair(1, 512, 512, 2, "relu", "relu", 22)
@@ -143,7 +143,8 @@ def test_when_the_one_launch_pays():
     assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw2._handle, 64, 14, 14) == 1
     assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw1._handle, 1, 14, 14) == 0
     assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw1._handle, 8, 14, 14) == 0
-    assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw1._handle, cus // 4, 14, 14) == 1  # 512 / 128 = 4 workgroups per image
+    assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw1._handle, cus // 16, 14, 14) == 0
+    assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw1._handle, cus // 8, 14, 14) == 1  # 512 / 128 = 4 workgroups per image: half the CUs
     assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw1._handle, 2 * cus, 14, 14) == 1
     assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw1._handle, 64, 7, 7) == 0  # does not fit
     assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw1._handle, 0, 14, 14) == 0
