@@ -6,7 +6,7 @@
 //   * The image goes through registers, not through an LDS landing area.  A lane loads the dword (four
 //     positions) of one position quad for each of 16 consecutive channels, transposes the 16 x 4 bytes with
 //     two stages of v_perm_b32 and writes four cells.  LDS then takes the image once (writes run at about
-//     72 bytes per clock per CU, half the read rate); landing it by direct loads and regrouping it in place
+//     71 bytes per clock per CU, a third of the read rate); landing it by direct loads and regrouping it in place
 //     writes it twice and was 0.3 us slower.  The weight tiles of two k-steps are requested behind every
 //     regrouped channel group, so that they queue up behind the image and arrive in the order the
 //     multiplication uses them.
@@ -24,6 +24,12 @@
 // Wavefront w starts with window w mod (windows per row) and goes round from there, so that at any time all
 // parts of the rows are being written rather than one column of the output (all wavefronts ascending 9.9 - 10.4 us,
 // the upper four descending 9.23, going round 9.09 in one run).
+//
+// A second kernel (ImageRowsDwKernel) runs the int8 depthwise 3 x 3 layer that follows such a pointwise layer in
+// a MobileNet in the same launch: the tile of a wavefront is 16 output channels times all positions, i.e. 16 whole
+// planes of the depthwise layer.  With int8 output the epilogue writes them to the wavefront's own LDS instead of
+// global memory, and behind its last window the wavefront computes the depthwise layer on them (DwStage, no
+// barrier: the planes are private to the wavefront).  14 x 14 maps, padding 1, stride 1 or 2.
 //
 // Reference semantics: out = act(fmaf(float(acc), scale, bias)) per output, int32 accumulation over all
 // channels (sparse_conv_impl.cc:1661-1685 computes the same sum over the nonzeros only; zeros add nothing to
