@@ -77,11 +77,14 @@ enum {
  *                     (image, 128 output rows) keeps the whole image in LDS
  *                     and multiplies it with dense 16x64 weight tiles; also
  *                     7 x 7 maps with ic = 256 / 512 / 1024 (two images per
- *                     workgroup)
+ *                     workgroup), and larger maps of a multiple of 196
+ *                     positions (28 x 28, 56 x 56, 112 x 112) in slabs of 196
+ *                     positions
  * With PL_ALGO_AUTO an int8 handle holds every form its shape allows and
- * chooses per call by batch and H*W (the image kernels where they apply, else
- * the row walk for at most 256 positions in all, else the block kernel): see
- * pl_sparse_conv_algo_for(). */
+ * chooses per call by batch and H*W (the image kernels where the whole map
+ * fits, or in slabs while batch * slabs * oc / 128 is at most half the CU
+ * count; else the row walk for at most 256 positions in all;
+ * else the block kernel): see pl_sparse_conv_algo_for(). */
 enum { PL_ALGO_AUTO = 0, PL_ALGO_ROW_WALK = 1, PL_ALGO_BLOCK_MFMA = 2, PL_ALGO_IMAGE_MFMA = 3 };
 
 /* Activation constants, used as given (replaces the fields of

@@ -60,13 +60,13 @@ typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 PL_IN_HEAD(ImageMfmaParams, x);
 PL_IN_HEAD(ImageMfmaParams, out);
 PL_IN_HEAD(ImageMfmaParams, wtiles);
-PL_IN_HEAD(ImageMfmaParams, M);
 PL_IN_HEAD(ImageMfmaParams, K);
 PL_IN_HEAD(ImageMfmaParams, hw);
 PL_IN_HEAD(ImageMfmaParams, items);
 PL_IN_HEAD(ImageMfmaParams, per_xcd);
 PL_IN_HEAD(ImageMfmaParams, row_groups);
-PL_IN_HEAD(ImageMfmaParams, qpi);
+PL_IN_HEAD(ImageMfmaParams, pitch);
+PL_IN_HEAD(ImageMfmaParams, slabs);
 
 constexpr int kRowStride = 8;  // rows of a tile: w + 8 m
 // Output kind of the kernel that runs the following depthwise layer itself: int8 like kOutI8, written to the
@@ -114,12 +114,12 @@ __device__ __forceinline__ u4 Finish4(int a0, int a1, int a2, int a3, float s, f
 // Row 4 kq + i of a window's results (positions 4 q .. 4 q + 3 per lane): epilogue and store.  `partial`: the
 // lane's line is shared with the end of the previous output row and merges in L2 (plain store).
 template <int OUT, int ACT>
-__device__ __forceinline__ void StoreRow(const v4i (&acc)[4], int i, float sc, float bi, const DevAct& act, char* __restrict__ orow, int hw, int q, bool partial, Lane ln) {
+__device__ __forceinline__ void StoreRow(const v4i (&acc)[4], int i, float sc, float bi, const DevAct& act, char* __restrict__ orow, int pitch, int q, bool partial, Lane ln) {
   constexpr int kElem = (OUT == kOutI8 || OUT == kOutPlanes) ? 1 : 4;
   const u4 v = Finish4<OUT, ACT>(acc[0][i], acc[1][i], acc[2][i], acc[3][i], sc, bi, act);
   // at most 128 rows of at most 256 four-byte positions behind orow: the offset fits 32 bits; it is negative only
   // for the quads in front of a row, which are not stored
-  const int off = ((kPlaneStride<OUT> * (4 * ln.kq + i)) * hw + 4 * q) * kElem;
+  const int off = ((kPlaneStride<OUT> * (4 * ln.kq + i)) * pitch + 4 * q) * kElem;
   if (OUT == kOutPlanes) {
     if (q >= 0) StoreLds(v.x, orow + off);
   } else if (OUT == kOutI8) {
@@ -191,7 +191,7 @@ __device__ __forceinline__ void DwStage(const DwConvParams& d, char* planes_in, 
 // k-steps (all of them behind the last k-step when KS < 4).  The operand cells of two k-steps are in flight.
 template <int KS, int OUT, int ACT, bool EPI>
 __device__ __forceinline__ void Window(const uint4* __restrict__ xt, int kgs, int cps, int q0, const v4i (&a)[KS], v4i (&acc)[4], const v4i (&accp)[4], int qp, bool partialp, const float (&sc)[4],
-                                       const float (&bi)[4], const DevAct& act, char* __restrict__ orow, int hw, Lane ln) {
+                                       const float (&bi)[4], const DevAct& act, char* __restrict__ orow, int pitch, Lane ln) {
   const uint4* bbase = xt + ln.kq * kgs + (q0 + ln.n);  // + ks * 4 * kgs + c * cps
 #pragma unroll
   for (int c = 0; c < 4; ++c) acc[c] = v4i{0, 0, 0, 0};
@@ -218,13 +218,13 @@ __device__ __forceinline__ void Window(const uint4* __restrict__ xt, int kgs, in
     }
     if (EPI && ks % kStepsPerRow == 0 && ks / kStepsPerRow < 4) {
       const int i = ks / kStepsPerRow;
-      StoreRow<OUT, ACT>(accp, i, sc[i], bi[i], act, orow, hw, qp + ln.n, partialp && ln.n < kRowStride, ln);
+      StoreRow<OUT, ACT>(accp, i, sc[i], bi[i], act, orow, pitch, qp + ln.n, partialp && ln.n < kRowStride, ln);
     }
     __builtin_amdgcn_sched_barrier(0);
   }
   if (EPI && KS < 4) {
 #pragma unroll
-    for (int i = KS; i < 4; ++i) StoreRow<OUT, ACT>(accp, i, sc[i], bi[i], act, orow, hw, qp + ln.n, partialp && ln.n < kRowStride, ln);
+    for (int i = KS; i < 4; ++i) StoreRow<OUT, ACT>(accp, i, sc[i], bi[i], act, orow, pitch, qp + ln.n, partialp && ln.n < kRowStride, ln);
   }
 }
 
@@ -236,7 +236,10 @@ __device__ __forceinline__ void Window(const uint4* __restrict__ xt, int kgs, in
 //
 // dw (kOutPlanes only): the depthwise layer that follows; the wavefront then keeps its 16 output planes in LDS
 // and runs that layer on them (DwStage below).
-template <int KS, int OUT, int QPI, int DW_STRIDE = 0>
+//
+// SLAB: a work item takes one slab of hw positions of a larger map (p.pitch positions per channel, p.slabs slabs
+// per image): the channel rows of the input and the rows of the output are then p.pitch apart, not hw.
+template <int KS, int OUT, int QPI, int DW_STRIDE = 0, bool SLAB = false>
 __device__ __forceinline__ void RowsBody(const ImageMfmaParams& p, uint4* lds_raw, const DwConvParams* dw) {
   // shifted windows read up to seven cells in front of a row of cells
   uint4* xt = lds_raw + 16;
@@ -244,8 +247,10 @@ __device__ __forceinline__ void RowsBody(const ImageMfmaParams& p, uint4* lds_ra
   // a contiguous range of work items per XCD, the row groups of one image next to each other
   const int item = (int)(blockIdx.x & 7u) * p.per_xcd + (int)(blockIdx.x >> 3);
   if (item >= p.items) return;
-  const int n = item / p.row_groups, rg = item - n * p.row_groups;
-  const int qpi = QPI ? QPI : p.qpi, kgs = QPI ? (4 * QPI + 15) / 16 * 16 : p.kgs, hw = p.hw;
+  const int ns = item / p.row_groups, rg = item - ns * p.row_groups;
+  const int n = SLAB ? ns / p.slabs : ns, slab = SLAB ? ns - n * p.slabs : 0;
+  const int hw = p.hw, pitch = SLAB ? p.pitch : hw;
+  const int qpi = QPI ? QPI : hw >> 2, kgs = QPI ? (4 * QPI + 15) / 16 * 16 : ((hw + 15) >> 4) << 4;
   const int cps = qpi;  // cells of position c of every quad lie qpi cells apart
   constexpr int NKG = 4 * KS, BPW = NKG / 8;
   static_assert(NKG % 8 == 0, "channel groups are dealt evenly to the eight wavefronts");
@@ -254,8 +259,8 @@ __device__ __forceinline__ void RowsBody(const ImageMfmaParams& p, uint4* lds_ra
   uint32_t r[BPW][16];
   {
     // one address per channel group, the channel's offset in the instruction (16 rows of at most 256 bytes)
-    const char* ximg = reinterpret_cast<const char*>(p.x) + (size_t)n * p.K * hw + lane * 4;
-    const int row_bytes = QPI ? 4 * QPI : hw;
+    const char* ximg = reinterpret_cast<const char*>(p.x) + (size_t)n * p.K * pitch + slab * hw + lane * 4;
+    const int row_bytes = SLAB ? pitch : (QPI ? 4 * QPI : hw);
     if (lane < qpi) {
 #pragma unroll
       for (int u = 0; u < BPW; ++u) {
@@ -318,14 +323,14 @@ __device__ __forceinline__ void RowsBody(const ImageMfmaParams& p, uint4* lds_ra
 
   // windows shifted left by sh quads so that fp32 / int32 row pieces start on 128-byte boundaries: output row
   // r starts r * qpi quads into the tensor
-  const int sh = p.align ? ((row0 * qpi) & (kRowStride - 1)) : 0;
+  const int sh = p.align ? ((row0 * (pitch >> 2) + slab * qpi) & (kRowStride - 1)) : 0;
   const int nqt = (qpi + sh) >> 4;       // full windows
   const int left = qpi + sh - 16 * nqt;  // quads after the last window
   const int ntail = (left + 3) >> 2;
   constexpr int kElem = (OUT == kOutI8 || OUT == kOutPlanes) ? 1 : 4;
   // kOutPlanes: the wavefront's planes behind the image's cells, 16 bytes of slack in front of them
   char* planes = reinterpret_cast<char*>(lds_raw) + 256 + (size_t)NKG * kgs * 16 + wave * kPlaneBufBytes;
-  char* orow = OUT == kOutPlanes ? planes + 16 : Uniform(static_cast<char*>(p.out) + ((size_t)n * p.M + row0) * hw * kElem);
+  char* orow = OUT == kOutPlanes ? planes + 16 : Uniform(static_cast<char*>(p.out) + (((size_t)n * p.M + row0) * pitch + slab * hw) * kElem);
   DispatchAct(OUT == kOutAcc32 ? 0 : epilogue::LeakyAsMax(p.act), [&](auto act_c) {
     constexpr int ACT = decltype(act_c)::value;
     if (nqt > 0) {
@@ -334,20 +339,20 @@ __device__ __forceinline__ void RowsBody(const ImageMfmaParams& p, uint4* lds_ra
       // the first line of window 0 holds the end of the previous output row when the window is shifted
       auto partial = [&](int t) { return win(t) == 0 && sh > 0; };
       v4i acc_a[4], acc_b[4];
-      Window<KS, OUT, ACT, false>(xt, kgs, cps, 16 * win(0) - sh, a, acc_a, acc_a, 0, false, sc, bi, p.act, orow, hw, ln);
+      Window<KS, OUT, ACT, false>(xt, kgs, cps, 16 * win(0) - sh, a, acc_a, acc_a, 0, false, sc, bi, p.act, orow, pitch, ln);
       int t = 1;
       // two windows per round so that the accumulator sets alternate without copies
       for (; t + 1 < nqt; t += 2) {
-        Window<KS, OUT, ACT, true>(xt, kgs, cps, 16 * win(t) - sh, a, acc_b, acc_a, 16 * win(t - 1) - sh, partial(t - 1), sc, bi, p.act, orow, hw, ln);
-        Window<KS, OUT, ACT, true>(xt, kgs, cps, 16 * win(t + 1) - sh, a, acc_a, acc_b, 16 * win(t) - sh, partial(t), sc, bi, p.act, orow, hw, ln);
+        Window<KS, OUT, ACT, true>(xt, kgs, cps, 16 * win(t) - sh, a, acc_b, acc_a, 16 * win(t - 1) - sh, partial(t - 1), sc, bi, p.act, orow, pitch, ln);
+        Window<KS, OUT, ACT, true>(xt, kgs, cps, 16 * win(t + 1) - sh, a, acc_a, acc_b, 16 * win(t) - sh, partial(t), sc, bi, p.act, orow, pitch, ln);
       }
       if (t < nqt) {
-        Window<KS, OUT, ACT, true>(xt, kgs, cps, 16 * win(t) - sh, a, acc_b, acc_a, 16 * win(t - 1) - sh, partial(t - 1), sc, bi, p.act, orow, hw, ln);
+        Window<KS, OUT, ACT, true>(xt, kgs, cps, 16 * win(t) - sh, a, acc_b, acc_a, 16 * win(t - 1) - sh, partial(t - 1), sc, bi, p.act, orow, pitch, ln);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) StoreRow<OUT, ACT>(acc_b, i, sc[i], bi[i], p.act, orow, hw, 16 * win(t) - sh + ln.n, partial(t) && ln.n < kRowStride, ln);
+        for (int i = 0; i < 4; ++i) StoreRow<OUT, ACT>(acc_b, i, sc[i], bi[i], p.act, orow, pitch, 16 * win(t) - sh + ln.n, partial(t) && ln.n < kRowStride, ln);
       } else {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) StoreRow<OUT, ACT>(acc_a, i, sc[i], bi[i], p.act, orow, hw, 16 * win(t - 1) - sh + ln.n, partial(t - 1) && ln.n < kRowStride, ln);
+        for (int i = 0; i < 4; ++i) StoreRow<OUT, ACT>(acc_a, i, sc[i], bi[i], p.act, orow, pitch, 16 * win(t - 1) - sh + ln.n, partial(t - 1) && ln.n < kRowStride, ln);
       }
     }
     // The quads the windows leave over, four at a time, operands swapped: rows of the product are positions
@@ -368,7 +373,7 @@ __device__ __forceinline__ void RowsBody(const ImageMfmaParams& p, uint4* lds_ra
       const int q = q0 + ln.kq;
       if (q >= 0 && q < qpi) {
         const u4 v = Finish4<OUT, ACT>(acc[0], acc[1], acc[2], acc[3], sct, bit, p.act);
-        char* ptr = orow + ((size_t)(kPlaneStride<OUT> * ln.n) * hw + 4 * q) * kElem;
+        char* ptr = orow + ((size_t)(kPlaneStride<OUT> * ln.n) * pitch + 4 * q) * kElem;
         if (OUT == kOutPlanes) StoreLds(v.x, ptr); else if (OUT == kOutI8) StorePlain(v.x, ptr); else StorePlain(v, ptr);
       }
     }
@@ -376,11 +381,11 @@ __device__ __forceinline__ void RowsBody(const ImageMfmaParams& p, uint4* lds_ra
   if constexpr (OUT == kOutPlanes) DwStage<DW_STRIDE>(*dw, planes + 16, planes + kPlaneInBytes, n, p.M, row0, lane);
 }
 
-template <int KS, int OUT, int QPI>
+template <int KS, int OUT, int QPI, bool SLAB = false>
 __global__ void __launch_bounds__(512) ImageRowsMfmaKernel(PL_HEAD_PARAMS, const ImageMfmaParams block) {
   const ImageMfmaParams p = WithHead(block, PL_HEAD_ARGS);
   extern __shared__ uint4 lds_raw[];
-  RowsBody<KS, OUT, QPI>(p, lds_raw, nullptr);
+  RowsBody<KS, OUT, QPI, 0, SLAB>(p, lds_raw, nullptr);
 }
 
 // The same followed by the depthwise 3 x 3 layer (14 x 14 planes, padding 1, stride DW_STRIDE, int8 output) on
@@ -395,6 +400,18 @@ __global__ void __launch_bounds__(512) ImageRowsDwKernel(PL_HEAD_PARAMS, const I
 template <int OUT>
 hipError_t ByKs(const ImageMfmaParams& q, dim3 grid, size_t lds, hipStream_t s) {
   const dim3 block(512);
+  if (q.slabs > 1) {  // slabs of 196 positions
+    switch (q.K / 64) {
+      case 2:
+        return LaunchWithHead(ImageRowsMfmaKernel<2, OUT, 49, true>, grid, block, lds, s, q);
+      case 4:
+        return LaunchWithHead(ImageRowsMfmaKernel<4, OUT, 49, true>, grid, block, lds, s, q);
+      case 8:
+        return LaunchWithHead(ImageRowsMfmaKernel<8, OUT, 49, true>, grid, block, lds, s, q);
+      default:
+        return hipErrorInvalidValue;
+    }
+  }
   if (q.qpi == 49) {
     switch (q.K / 64) {
       case 2:
@@ -429,16 +446,26 @@ bool ImageRowsMfmaFits(int M, int K, int hw) {
   return 256 + (size_t)(K / 16) * kgs * 16 <= (size_t)kMaxLdsBytes;
 }
 
+constexpr int kSlab = 196;  // positions of a slab of a larger map (49 quads: the kernel's compile-time row length)
+
+bool ImageRowsSlabFits(int M, int K, int hw) { return hw > 256 && hw % kSlab == 0 && ImageRowsMfmaFits(M, K, kSlab); }
+
+// p.hw: positions of the whole map; it is taken whole where it fits, else in slabs of 196 positions.
 hipError_t LaunchImageRowsMfma(int out_kind, const ImageMfmaParams& p, hipStream_t stream) {
   if (p.batch <= 0) return hipSuccess;
-  if (!ImageRowsMfmaFits(p.M, p.K, p.hw)) return hipErrorInvalidValue;
+  const bool whole = ImageRowsMfmaFits(p.M, p.K, p.hw);
+  if (!whole && !ImageRowsSlabFits(p.M, p.K, p.hw)) return hipErrorInvalidValue;
   // the image is read as dwords, the output written as 16-byte pieces
   if (reinterpret_cast<uintptr_t>(p.x) % 4 != 0 || reinterpret_cast<uintptr_t>(p.out) % 16 != 0) return hipErrorInvalidValue;
   ImageMfmaParams q = p;
-  q.qpi = p.hw / 4;
+  q.pitch = p.hw;
+  q.slabs = whole ? 1 : p.hw / kSlab;
+  q.hw = whole ? p.hw : kSlab;
+  q.qpi = q.hw / 4;
   q.kgs = (4 * q.qpi + 15) / 16 * 16;  // a channel group's cells start on a 256-byte boundary: conflict-free operand reads
   q.row_groups = p.M / 128;
-  const int64_t items = (int64_t)p.batch * q.row_groups;
+  if ((int64_t)p.batch * p.K * p.hw >= (1ll << 40)) return hipErrorInvalidValue;
+  const int64_t items = (int64_t)p.batch * q.slabs * q.row_groups;
   if (items > (1 << 28)) return hipErrorInvalidValue;
   q.items = (int)items;
   q.per_xcd = (q.items + 7) / 8;
@@ -471,6 +498,8 @@ hipError_t LaunchImageRowsDw(const ImageMfmaParams& p, const DwConvParams& d, in
   // the image is read as dwords; planes of 196 bytes are stored as dwords, planes of 49 bytes byte by byte
   if (reinterpret_cast<uintptr_t>(p.x) % 4 != 0 || (stride == 1 && reinterpret_cast<uintptr_t>(d.out) % 4 != 0)) return hipErrorInvalidValue;
   ImageMfmaParams q = p;
+  q.pitch = p.hw;
+  q.slabs = 1;
   q.qpi = 49;
   q.kgs = 208;
   q.row_groups = p.M / 128;

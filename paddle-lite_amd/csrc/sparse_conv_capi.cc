@@ -689,6 +689,7 @@ pl::WalkConfig ChooseWalk(const pl_sparse_conv_handle* h, uint32_t P) {
 //  * the image kernels wherever their shape conditions hold: they tie with or beat the block kernel at every
 //    batch (by 2x on 7 x 7 maps, where the block kernel has too few tiles for the chip), and stay within 10 % of
 //    the row walk on a single 14 x 14 image of 512 channels, the one case where the walk is ahead;
+//  * the image kernel with one row tile per wavefront on slabs of larger maps while the slabs are few (below);
 //  * else the row walk for at most 256 positions in all (it spreads the output rows over the chip where the
 //    block kernel would have one or two tiles);
 //  * else the block kernel.
@@ -698,6 +699,14 @@ int AlgoForCall(const pl_sparse_conv_handle* h, int batch, int im_size, bool ali
   // work items: (image, row group), for 7 x 7 maps (pair of images, row group)
   const int64_t image_items = static_cast<int64_t>(im_size == 49 ? (batch + 1) / 2 : batch) * (h->oc / 128);
   if (h->wtiles.ptr && aligned16 && pl::ImageMfmaFits(h->oc, h->ic, im_size) && image_items >= h->image_min_items) return PL_ALGO_IMAGE_MFMA;
+  // Larger maps in slabs of 196 positions: ahead of the block kernel while the slabs are few (128 -> 256 @28x28: 4.0
+  // against 4.6 us at 4 images, 4.5 against 5.1 at 16, equal at 64; 256 -> 256 @28x28: 5.3 against 6.0 at 16, 12.7
+  // against 10.1 at 64; 128 -> 128 @56x56: 4.3 against 4.7 at 4, 5.9 against 5.5 at 16): every work item pays the
+  // kernel's whole load-multiply-store chain, and a CU holds one or two at a time.
+  if (h->wtiles_rows.ptr && aligned16 && (h->image_kernel == 0 || h->image_kernel == 3) && pl::ImageRowsSlabFits(h->oc, h->ic, im_size)) {
+    const int64_t slab_items = static_cast<int64_t>(batch) * (im_size / 196) * (h->oc / 128);
+    if (slab_items >= h->image_min_items && slab_items * 2 <= h->wg_slots_default / 2) return PL_ALGO_IMAGE_MFMA;
+  }
   if (h->auto_walk && static_cast<int64_t>(batch) * im_size <= 256) return PL_ALGO_ROW_WALK;
   return h->algo;
 }
@@ -941,7 +950,10 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.slices = CeilDiv(h->n_groups, p.groups_per_slice);
     e = pl::LaunchHalfWalk(h->semi ? 2 : 1, tp, threads, p, s);
   } else if (call_algo == PL_ALGO_IMAGE_MFMA) {
-    if (!pl::ImageMfmaFits(h->oc, h->ic, im_size)) return Fail(PL_ERR_UNSUPPORTED, "the image MFMA algorithm needs H*W = 49 or a multiple of 4 in [16, 256] that fits LDS with %d channels (H*W = %d)", h->ic, im_size);
+    // larger maps of a multiple of 196 positions are taken slab by slab by the kernel with one row tile per wavefront
+    const bool slabs = h->wtiles_rows.ptr != nullptr && (h->image_kernel == 0 || h->image_kernel == 3) && pl::ImageRowsSlabFits(h->oc, h->ic, im_size);
+    if (!slabs && !pl::ImageMfmaFits(h->oc, h->ic, im_size))
+      return Fail(PL_ERR_UNSUPPORTED, "the image MFMA algorithm needs H*W = 49, a multiple of 4 in [16, 256] or a multiple of 196 (its slabs) that fits LDS with %d channels (H*W = %d)", h->ic, im_size);
     if (reinterpret_cast<uintptr_t>(x_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(out_dev) % 16 != 0) return Fail(PL_ERR_UNSUPPORTED, "the image MFMA algorithm needs 16-byte aligned tensors");
     pl::ImageMfmaParams p{};
     p.x = static_cast<const int8_t*>(x_dev);
@@ -958,7 +970,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     const bool tr_fits = h->wtiles_tr.ptr != nullptr && pl::ImageTrMfmaFits(h->oc, h->ic, im_size);
     // One row tile per wavefront and the image through registers: the rule wherever it applies (every shape of
     // the image algorithm but the 7 x 7 maps).
-    const bool rows_fits = h->wtiles_rows.ptr != nullptr && pl::ImageRowsMfmaFits(h->oc, h->ic, im_size);
+    const bool rows_fits = h->wtiles_rows.ptr != nullptr && (slabs || pl::ImageRowsMfmaFits(h->oc, h->ic, im_size));
     if (h->image_kernel == 3 && !rows_fits) return Fail(PL_ERR_UNSUPPORTED, "the image kernel with one row tile per wavefront takes no 7 x 7 maps (H*W = %d, ic = %d)", im_size, h->ic);
     if (h->image_kernel == 2 && !tr_fits) return Fail(PL_ERR_UNSUPPORTED, "the image kernel with transposing LDS reads needs H*W = 4 (mod 8) from 20 on, ic = 128, 256 or 512 and an image that leaves 41 KB of LDS free (H*W = %d, ic = %d)", im_size, h->ic);
     if (tr_fits && h->image_kernel == 2) {

@@ -248,14 +248,17 @@ struct ImageMfmaParams {
   // [row group of 128][class rho = 0..3][tile j = 0..1][k-step][64 lanes][16 bytes];
   // lane l of tile (rho, j) holds row rho + 4 (16 j + l % 16), channels 64 ks + 16 (l / 16) .. + 15
   const void* wtiles;
-  int M, K;
-  int hw;
-  int batch;
+  int K;
+  int hw;              // positions a work item takes: the whole map (H * W), or one slab of it (image_rows_kernels.hip)
   // filled in by the launcher
-  int items, per_xcd;  // work items (image, row group) in all and per XCD
+  int pitch;           // positions of the whole map = bytes between the channel rows of x and elements between output rows
+  int slabs;           // slabs per image (1: the whole map is one item)
+  int items, per_xcd;  // work items (image, slab, row group) in all and per XCD
   int row_groups;      // M / 128
-  int qpi;             // position quads per image = hw / 4
+  int batch;
   // behind the head
+  int M;
+  int qpi;             // position quads per item = hw / 4
   const float* scale;  // output-row order, at least M entries
   const float* bias;   // likewise (zeros when the op has no bias)
   DevAct act;
@@ -290,6 +293,9 @@ hipError_t LaunchImageMfma(int out_kind, const ImageMfmaParams& p, hipStream_t s
 // holds row w + 8 (l % 16), channels 64 ks + 16 (l / 16) .. + 15.  M a multiple of 128, K = 128, 256 or 512, hw a
 // multiple of 4 in [16, 256] and the image's cells within the LDS of a CU; x 4-byte and out 16-byte aligned.
 bool ImageRowsMfmaFits(int M, int K, int hw);
+// Larger maps of a multiple of 196 positions (28 x 28, 56 x 56, 112 x 112): the same kernel on slabs of 196
+// positions, one work item per (image, slab, 128 output rows).
+bool ImageRowsSlabFits(int M, int K, int hw);
 hipError_t LaunchImageRowsMfma(int out_kind, const ImageMfmaParams& p, hipStream_t stream);
 
 bool ImageTrMfmaFits(int M, int K, int hw);

@@ -303,3 +303,60 @@ def test_mixed_empty_sparse_and_dense_blocks_all_algorithms(kind):
     kernel, _ = make_kernel(case, capi.ALGO_BLOCK_MFMA)
     info = kernel.info()
     assert info["mfma_blocks"] == int(np.count_nonzero([[mask[32 * i:32 * i + 32, 32 * j:32 * j + 32].any() for j in range(8)] for i in range(8)])) < info["mfma_blocks_total"] == 64
+
+
+# Larger maps of a multiple of 196 positions, taken in slabs of 196 by the kernel with one row tile per wavefront:
+# (batch, ic, oc, h, w); 28 x 28 = 4 slabs, 56 x 56 = 16, 14 x 42 = 3, 112 x 7 = 4 (rows of any shape: only H*W counts)
+SLAB_SHAPES = [(2, 128, 256, 28, 28), (3, 256, 256, 28, 28), (1, 128, 128, 56, 56), (2, 512, 128, 14, 42), (5, 256, 384, 112, 7)]
+
+
+@pytest.mark.parametrize("kind", sorted(KINDS))
+@pytest.mark.parametrize("shape", SLAB_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_image_rows_slabs_bit_exact(shape, kind):
+    announce("image slabs", shape, kind)
+    batch, ic, oc, h, w = shape
+    k = KINDS[kind]
+    for act, paired in ((("none", False),) if kind == "acc32" else (("leaky", False), ("hswish", True), ("relu6", False))):
+        case = case_for(k, batch, ic, oc, h, w, 0.85, paired, ACTS[act], seed=ic + 3 * oc + h * w)
+        want = run_oracle(case, oracle_pack(case))
+        got = run_hip(case, capi.ALGO_IMAGE_MFMA)
+        assert_same(case, got, want, "image slabs %s %s %s" % (kind, act, shape))
+        # the automatic choice takes the slabs for these few work items and gives the same bits
+        kernel, _ = make_kernel(case, capi.ALGO_AUTO)
+        assert capi.lib().pl_sparse_conv_algo_for(kernel._handle, batch, h * w) == capi.ALGO_IMAGE_MFMA
+        assert np.array_equal(run_hip(case, kernel=kernel), got)
+        # and the block kernel agrees
+        assert np.array_equal(run_hip(case, capi.ALGO_BLOCK_MFMA), got)
+
+
+def test_image_rows_slabs_rule_and_surroundings():
+    """Slabs are taken while batch * slabs * oc / 128 is at most half the CU count; the kernel writes nothing
+    outside its output and reads nothing it must not (the tensor sits inside a larger buffer)."""
+    import torch
+
+    L = capi.lib()
+    case = case_for(capi.KIND_INT8_INT8, 4, 128, 256, 28, 28, 0.85, False, ACTS["relu"], seed=5)
+    kernel, _ = make_kernel(case, capi.ALGO_AUTO)
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 16, 784) == capi.ALGO_IMAGE_MFMA   # 16 * 4 * 2 = 128 work items
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 17, 784) == capi.ALGO_BLOCK_MFMA
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 64, 784) == capi.ALGO_BLOCK_MFMA
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 4, 3136) == capi.ALGO_IMAGE_MFMA   # 4 * 16 * 2 = 128
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 5, 3136) == capi.ALGO_BLOCK_MFMA
+    assert L.pl_sparse_conv_algo_for(kernel._handle, 1, 4 * 197) == capi.ALGO_BLOCK_MFMA  # not a multiple of 196
+    regroup, _ = make_kernel(case, capi.ALGO_AUTO, tuning=REGROUP)                      # the other image kernels take no slabs
+    assert L.pl_sparse_conv_algo_for(regroup._handle, 4, 784) == capi.ALGO_BLOCK_MFMA
+    guard = 4096
+    x = torch.from_numpy(case.x).cuda()
+    xin = torch.randint(-127, 128, (x.numel() + 2 * guard,), dtype=torch.int8, device="cuda")
+    xin[guard:guard + x.numel()] = x.reshape(-1)
+    numel = 4 * 256 * 784
+    buf = torch.full((numel + 2 * guard,), 77, dtype=torch.int8, device="cuda")
+    kernel.Run(xin[guard:guard + x.numel()].view(x.shape), buf[guard:guard + numel].view(4, 256, 28, 28))
+    torch.cuda.synchronize()
+    host = buf.cpu().numpy()
+    assert (host[:guard] == 77).all() and (host[guard + numel:] == 77).all()
+    assert np.array_equal(host[guard:guard + numel].reshape(4, 256, 28, 28), run_oracle(case))
+    with pytest.raises(capi.SparseConvError) as e:  # asked for explicitly on a map that has no slabs of 196
+        forced, _ = make_kernel(case, capi.ALGO_IMAGE_MFMA)
+        forced.Run(torch.zeros((1, 128, 20, 20), dtype=torch.int8, device="cuda"))
+    assert e.value.code == capi.PL_ERR_UNSUPPORTED
