@@ -134,7 +134,9 @@ typedef struct pl_sparse_conv_tuning {
                                 done by transposing LDS reads where that exists
                                 (ic = 512, 14 x 14 maps); NEVER = by the vector
                                 ALU everywhere                                 */
-  int32_t reserved;          /* must be 0                                      */
+  int32_t walk_pairs;        /* (switch) that walk with two row groups per
+                                wavefront instruction: lanes 0 - 31 walk one,
+                                lanes 32 - 63 the other, four positions per lane */
 } pl_sparse_conv_tuning;
 
 /* Everything PrepareForRun() knows.  All pointers are HOST pointers and are

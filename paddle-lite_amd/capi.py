@@ -69,7 +69,7 @@ class Tuning(C.Structure):
         ("walk_threads", C.c_int32),
         ("walk_slices", C.c_int32),
         ("image_tr_regroup", C.c_int32),
-        ("reserved", C.c_int32),
+        ("walk_pairs", C.c_int32),
     ]
 
 
@@ -77,7 +77,7 @@ def tuning(**fields):
     """A Tuning with the named fields set (the rest stay 0 = by rule)."""
     t = Tuning()
     for name, value in fields.items():
-        if name not in dict(Tuning._fields_) or name == "reserved":
+        if name not in dict(Tuning._fields_):
             raise ValueError("no tuning field %r" % name)
         setattr(t, name, int(value))
     return t

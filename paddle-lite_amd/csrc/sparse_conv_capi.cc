@@ -154,6 +154,7 @@ struct pl_sparse_conv_handle {
   int64_t tw_stream_work = 0;  // work units (entry batches + 2 per row group) of the fullest of the sixteen unsplit streams
   int walk_split = -1;          // sixteenths of the row groups' work dealt to the CUs without a tile: -1 by rule, 0 never, 1 .. 8 forced
   int walk_tiled = 1;            // 0 never, 1 when the problem suits it, 2 whenever the shape allows
+  bool walk_pairs = true;        // the tile walk's streams hold pairs of row groups (two per wavefront instruction)
   int cw_groups = 8;  // row groups per wavefront of the fp32 walk over channel chunks: 8, or 4 on request
   int walk_chunked = 1;  // 0 never, 1 when the problem is large enough, 2 whenever the shape allows
   bool walk_plain_fits = true;  // false: more channels than the plain walk's LDS tile holds, only the chunked walk can run
@@ -390,26 +391,47 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
   std::vector<int> order(n_groups);
   for (int g = 0; g < n_groups; ++g) order[g] = g;
   std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return L.groups[a].count > L.groups[b].count; });
-  auto work = [&](int g) { return static_cast<int64_t>((L.groups[g].count + 3) / 4 + 2); };  // batches, plus the group's epilogue
+  // A unit is what one wavefront instruction walks: one row group, or (walk_pairs) two of about the same
+  // length - neighbours in the order by length - of which the shorter is padded with entries of weight zero that
+  // point at the tile's zero row; a last group without a partner gets an empty one (no rows).
+  const bool pairs = h->walk_pairs;
+  struct Unit {
+    int a, b;        // row groups (b = -1: none)
+    uint32_t count;  // entries walked
+  };
+  std::vector<Unit> units;
+  if (pairs) {
+    for (int i = 0; i < n_groups; i += 2) {
+      const int a = order[i], b = i + 1 < n_groups ? order[i + 1] : -1;
+      units.push_back({a, b, L.groups[a].count});  // sorted: a is the longer one
+    }
+  } else {
+    for (int g : order) units.push_back({g, -1, L.groups[g].count});
+  }
+  const int n_units = static_cast<int>(units.size());
+  std::vector<int> unit_order(n_units);
+  for (int u = 0; u < n_units; ++u) unit_order[u] = u;
+  auto work = [&](int u) { return static_cast<int64_t>((units[u].count + 3) / 4 + 2); };  // batches, plus the unit's epilogue
   const uint32_t rec_words = 4 + 4 * nr;
+  const uint32_t unit_words = pairs ? 2 * rec_words : rec_words;  // a double record per step of a pair
   const uint32_t chunk_words = pl::kTileWalkChunkBytes / 4;
-  const uint32_t recs_per_chunk = chunk_words / rec_words;
+  const uint32_t recs_per_chunk = chunk_words / unit_words;
   const uint32_t zero_row = static_cast<uint32_t>(L.ic) * pl::kTileWalkTile * 4;
   std::vector<uint32_t>& stream = h->tw_host_stream;
   stream.clear();
   h->tw_bias_slots.clear();
   std::vector<uint32_t> first, counts;
-  // Streams for the given row groups (largest first): each group goes to the stream with the least work so far.
+  // Streams for the given units (largest first): each unit goes to the stream with the least work so far.
   // Sixteen streams make one part.  Returns the work of the fullest stream.
   auto emit = [&](const std::vector<int>& part, int n_streams) {
     std::vector<std::vector<int>> members(n_streams);
     std::vector<int64_t> load(n_streams, 0);
-    for (int g : part) {
+    for (int u : part) {
       int best = 0;
       for (int s2 = 1; s2 < n_streams; ++s2)
         if (load[s2] < load[best]) best = s2;
-      members[best].push_back(g);
-      load[best] += work(g);
+      members[best].push_back(u);
+      load[best] += work(u);
     }
     for (int s2 = 0; s2 < n_streams; ++s2) {
       first.push_back(static_cast<uint32_t>(stream.size() / chunk_words));
@@ -423,26 +445,38 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
           pad_chunk();
           recs = 0;
         }
-        stream.insert(stream.end(), rec, rec + rec_words);
+        stream.insert(stream.end(), rec, rec + unit_words);
         ++recs;
       };
-      for (int g : members[s2]) {
-        const pl::RowGroup& rg = L.groups[g];
-        uint32_t rec[12] = {0};
-        rec[0] = static_cast<uint32_t>(rg.row0) | (static_cast<uint32_t>(rg.nrows) << 24);
-        rec[1] = rg.count;
-        if (bias) {
-          std::memcpy(&rec[2], &bias[rg.row0], 4);
-          if (rg.nrows == 2) std::memcpy(&rec[3], &bias[rg.row0 + 1], 4);
+      for (int u : members[s2]) {
+        const Unit& un = units[u];
+        uint32_t rec[24] = {0};
+        const int side_groups[2] = {un.a, un.b};
+        const int sides = pairs ? 2 : 1;
+        for (int side = 0; side < sides; ++side) {
+          uint32_t* r = rec + side * rec_words;
+          r[1] = un.count;
+          if (side_groups[side] < 0) continue;  // no partner: no rows
+          const pl::RowGroup& rg = L.groups[side_groups[side]];
+          r[0] = static_cast<uint32_t>(rg.row0) | (static_cast<uint32_t>(rg.nrows) << 24);
+          if (bias) {
+            std::memcpy(&r[2], &bias[rg.row0], 4);
+            if (rg.nrows == 2) std::memcpy(&r[3], &bias[rg.row0 + 1], 4);
+          }
         }
         put(rec);
-        h->tw_bias_slots.emplace_back(static_cast<uint32_t>(stream.size() - rec_words + 2), rec[0]);
-        for (uint32_t e0 = 0; e0 < rg.count; e0 += 4) {
-          for (uint32_t e = 0; e < 4; ++e) {
-            const bool real = e0 + e < rg.count;
-            rec[e] = real ? L.ic_index[rg.first + e0 + e] * pl::kTileWalkTile * 4 : zero_row;
-            rec[4 + e * nr] = real ? L.w0[rg.first + e0 + e] : 0u;
-            if (nr == 2) rec[4 + e * nr + 1] = real ? L.w1[rg.first + e0 + e] : 0u;
+        for (int side = 0; side < sides; ++side)
+          if (side_groups[side] >= 0) h->tw_bias_slots.emplace_back(static_cast<uint32_t>(stream.size() - unit_words + side * rec_words + 2), rec[side * rec_words]);
+        for (uint32_t e0 = 0; e0 < un.count; e0 += 4) {
+          for (int side = 0; side < sides; ++side) {
+            uint32_t* r = rec + side * rec_words;
+            const pl::RowGroup* rg = side_groups[side] >= 0 ? &L.groups[side_groups[side]] : nullptr;
+            for (uint32_t e = 0; e < 4; ++e) {
+              const bool real = rg != nullptr && e0 + e < rg->count;
+              r[e] = real ? L.ic_index[rg->first + e0 + e] * pl::kTileWalkTile * 4 : zero_row;
+              r[4 + e * nr] = real ? L.w0[rg->first + e0 + e] : 0u;
+              if (nr == 2) r[4 + e * nr + 1] = real ? L.w1[rg->first + e0 + e] : 0u;
+            }
           }
           put(rec);
         }
@@ -452,29 +486,29 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
     }
     return *std::max_element(load.begin(), load.end());
   };
-  // Set 0: all row groups in one part.  Sets 1 .. kTileWalkSplits: a spare part with about s / 16 of the work
-  // (a mix of sizes: going through the groups from the largest, a group joins the spare part whenever that
+  // Set 0: all units in one part.  Sets 1 .. kTileWalkSplits: a spare part with about s / 16 of the work
+  // (a mix of sizes: going through the units from the largest, a unit joins the spare part whenever that
   // keeps the part at or below its share), the rest in the main part.
-  h->tw_stream_work = emit(order, streams);
+  h->tw_stream_work = emit(unit_order, streams);
   for (int s16 = 1; s16 <= kTileWalkSplits; ++s16) {
     std::vector<int> main_part, spare_part;
     int64_t all_w = 0, spare_w = 0;
-    for (int g : order) {
-      const int64_t w = work(g);
+    for (int u : unit_order) {
+      const int64_t w = work(u);
       all_w += w;
       if ((spare_w + w) * 16 <= static_cast<int64_t>(s16) * all_w) {
-        spare_part.push_back(g);
+        spare_part.push_back(u);
         spare_w += w;
       } else {
-        main_part.push_back(g);
+        main_part.push_back(u);
       }
     }
     emit(main_part, streams);
     emit(spare_part, streams);
   }
   // Equal parts for problems with at most half as many tiles as CUs: n workgroups per tile, each with a
-  // sixteenth-of-n share of the row groups.
-  for (int n : kTileWalkEqualParts) emit(order, streams * n);
+  // sixteenth-of-n share of the units.
+  for (int n : kTileWalkEqualParts) emit(unit_order, streams * n);
   hipError_t e = h->tw_stream.Upload(stream.data(), stream.size() * sizeof(uint32_t));
   if (e == hipSuccess) e = h->tw_first.Upload(first.data(), first.size() * sizeof(uint32_t));
   if (e == hipSuccess) e = h->tw_desc.Upload(counts.data(), counts.size() * sizeof(uint32_t));
@@ -740,8 +774,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
     return Fail(PL_ERR_BAD_ARG, "pl_sparse_conv_desc size mismatch (%u vs %zu)", desc->struct_size, sizeof(pl_sparse_conv_desc));
   pl_sparse_conv_tuning tune{};
   if (desc->struct_size == sizeof(pl_sparse_conv_desc)) tune = desc->tuning;
-  if (tune.reserved != 0) return Fail(PL_ERR_BAD_ARG, "pl_sparse_conv_tuning.reserved must be 0");
-  for (int32_t sw : {tune.mfma_stream, tune.mfma_sub_tiles, tune.walk_tiled, tune.walk_chunked, tune.image_tr_regroup})
+  for (int32_t sw : {tune.mfma_stream, tune.mfma_sub_tiles, tune.walk_tiled, tune.walk_chunked, tune.image_tr_regroup, tune.walk_pairs})
     if (sw < PL_TUNE_RULE || sw > PL_TUNE_ALWAYS) return Fail(PL_ERR_BAD_ARG, "a tuning switch is not PL_TUNE_RULE, PL_TUNE_NEVER or PL_TUNE_ALWAYS");
   if (tune.image_kernel < 0 || tune.image_kernel > 3) return Fail(PL_ERR_BAD_ARG, "tuning.image_kernel must be 0, 1, 2 or 3");
   if (desc->kind < PL_KIND_FP32 || desc->kind > PL_KIND_FP16) return Fail(PL_ERR_BAD_ARG, "unknown kind %d", desc->kind);
@@ -785,6 +818,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   h->mfma_stream = sw(tune.mfma_stream);
   h->mfma_sub_tiles = sw(tune.mfma_sub_tiles);
   h->walk_tiled = sw(tune.walk_tiled);
+  h->walk_pairs = sw(tune.walk_pairs) != 0;  // the rule: pairs
   h->walk_chunked = sw(tune.walk_chunked);
   h->mfma_i8_wide = tune.mfma_narrow_i8_stores == 0;
   if (tune.walk_split > 0) h->walk_split = std::min(kTileWalkSplits, tune.walk_split - 1);
@@ -1070,6 +1104,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.stream_groups = static_cast<const uint32_t*>(h->tw_desc.ptr) + table;
     p.split = equal_parts != 0 ? 2 : (s16 != 0 ? 1 : 0);
     p.parts = equal_parts;
+    p.pairs = h->walk_pairs ? 1 : 0;
     p.split_slots = cus / 8;
     p.n_groups = h->n_groups;
     p.M = h->oc;

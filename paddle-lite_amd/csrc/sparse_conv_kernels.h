@@ -126,7 +126,10 @@ struct TileWalkParams {
   // an XCD must not exceed split_slots); the stream tables then hold
   // parts x kTileWalkWaves entries.
   int16_t split;
-  int16_t parts;
+  int8_t parts;
+  // 1: the streams hold pairs of row groups, padded to one length, as double records (first group's record, second
+  // group's record): lanes 0 - 31 walk the first group, lanes 32 - 63 the second, four positions per lane
+  int8_t pairs;
   // The first 56 bytes (kernarg_head.h) end behind act.type: what selects the tile, picks the activation and
   // addresses the first loads.
   DevAct act;

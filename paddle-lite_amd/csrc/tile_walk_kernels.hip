@@ -17,6 +17,11 @@
 // spread over the whole walk.  The order of the fused multiply-adds of one
 // output is the index order and the accumulator starts at the bias, as in the
 // other walks (same bits).
+// With pairs (TileWalkParams::pairs) a wavefront instruction walks two row groups of about the same length at
+// once: lanes 0 - 31 the first, lanes 32 - 63 the second, four positions per lane, the records of the two
+// groups side by side in the stream.  The activations are then read 16 bytes per lane (LDS delivers those at
+// twice the rate of 8-byte reads) and every LDS instruction, address add and loop step serves two row groups;
+// the shorter group of a pair is padded with entries of weight zero at the tile's zero row.
 // With fewer tiles than CUs, the row groups can be dealt into a main and a
 // spare part (two sets of sixteen streams): the tile's own workgroup walks the
 // main part, and the workgroups on the CUs that have no tile of their own walk
@@ -36,6 +41,7 @@ namespace pl {
 namespace {
 
 typedef float v2f __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 typedef uint32_t u2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 typedef const __attribute__((address_space(4))) uint32_t* ConstWords;
@@ -51,6 +57,7 @@ PL_IN_HEAD(TileWalkParams, P);
 PL_IN_HEAD(TileWalkParams, tiles);
 PL_IN_HEAD(TileWalkParams, split);
 PL_IN_HEAD(TileWalkParams, parts);
+PL_IN_HEAD(TileWalkParams, pairs);
 static_assert(offsetof(TileWalkParams, act) + sizeof(int) <= kHeadWords * 8, "act.type must lie in the first 56 bytes of TileWalkParams");
 
 using epilogue::ActivateT;
@@ -61,10 +68,12 @@ constexpr int kWaves = kTileWalkWaves;  // wavefronts per workgroup = list strea
 constexpr int kChunkBytes = kTileWalkChunkBytes;
 
 // One tile: stage it, then walk the streams of one part (0 main, 1 spare).
-template <int NR, int ACT>
+template <int NR, int ACT, bool PAIR>
 __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile, int tile_id, int part) {
   constexpr int kRecBytes = NR == 2 ? 48 : 32;  // four byte offsets, then 4 * NR weights
-  constexpr int kRecs = kChunkBytes / kRecBytes;
+  constexpr int kStepBytes = PAIR ? 2 * kRecBytes : kRecBytes;  // what one step of the walk reads: one record per row group
+  constexpr int kRecs = kChunkBytes / kStepBytes;
+  constexpr int PPL = PAIR ? 4 : 2;  // positions per lane
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int sidx = part * kWaves + wave;
@@ -104,8 +113,10 @@ __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile
   }
   __syncthreads();
 
-  const uint32_t lane8 = 8u * (uint32_t)lane;
-  const uint32_t gpos = tile0 + 2u * (uint32_t)lane;
+  // pairs: the half of the wavefront a lane belongs to picks the record, its place in the half the positions
+  const int half = PAIR ? lane >> 5 : 0;
+  const uint32_t lane8 = PAIR ? 16u * (uint32_t)(lane & 31) : 8u * (uint32_t)lane;
+  const uint32_t gpos = tile0 + (PAIR ? 4u * (uint32_t)(lane & 31) : 2u * (uint32_t)lane);
   const bool store_on = gpos < p.P;
   const uint32_t on = store_on ? gpos / (uint32_t)p.hw : 0u, opp = store_on ? gpos % (uint32_t)p.hw : 0u;
   float* obase = p.out + (size_t)on * p.M * p.hw + opp;
@@ -125,24 +136,29 @@ __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile
       pb = *reinterpret_cast<const u2*>(np + 1024 + 8 * lane);
       rec = 0;
     }
-    return lbuf + (rec++) * kRecBytes;
+    return lbuf + (rec++) * kStepBytes + half * kRecBytes;
   };
   const int n_groups = (int)((ConstWords)p.stream_groups)[sidx];
   for (int j = 0; j < n_groups; ++j) {
-    // header record of the row group: first row | rows << 24, entries, bias bits of its rows
+    // header record of the row group: first row | rows << 24, entries, bias bits of its rows (pairs: one per half,
+    // the same number of entries in both)
     const u4 hdr = *reinterpret_cast<const u4*>(next());
-    const int row0 = __builtin_amdgcn_readfirstlane((int)(hdr.x & 0xffffffu)), nrows = __builtin_amdgcn_readfirstlane((int)(hdr.x >> 24));
+    const int row0 = PAIR ? (int)(hdr.x & 0xffffffu) : __builtin_amdgcn_readfirstlane((int)(hdr.x & 0xffffffu));
+    const int nrows = PAIR ? (int)(hdr.x >> 24) : __builtin_amdgcn_readfirstlane((int)(hdr.x >> 24));
     const uint32_t entries = (uint32_t)__builtin_amdgcn_readfirstlane((int)hdr.y);
-    float acc[NR][2];
-    acc[0][0] = acc[0][1] = __uint_as_float(hdr.z);
-    if (NR == 2) acc[NR - 1][0] = acc[NR - 1][1] = __uint_as_float(hdr.w);
+    float acc[NR][PPL];
+#pragma unroll
+    for (int q = 0; q < PPL; ++q) {
+      acc[0][q] = __uint_as_float(hdr.z);
+      if (NR == 2) acc[NR - 1][q] = __uint_as_float(hdr.w);
+    }
+    typedef float vx __attribute__((ext_vector_type(PPL)));
     auto entry = [&](uint32_t off, float w0, float w1) {
-      const v2f x = *reinterpret_cast<const v2f*>(tile_bytes + (off + lane8));
-      acc[0][0] = __builtin_fmaf(x[0], w0, acc[0][0]);
-      acc[0][1] = __builtin_fmaf(x[1], w0, acc[0][1]);
-      if (NR == 2) {
-        acc[NR - 1][0] = __builtin_fmaf(x[0], w1, acc[NR - 1][0]);
-        acc[NR - 1][1] = __builtin_fmaf(x[1], w1, acc[NR - 1][1]);
+      const vx x = *reinterpret_cast<const vx*>(tile_bytes + (off + lane8));
+#pragma unroll
+      for (int q = 0; q < PPL; ++q) {
+        acc[0][q] = __builtin_fmaf(x[q], w0, acc[0][q]);
+        if (NR == 2) acc[NR - 1][q] = __builtin_fmaf(x[q], w1, acc[NR - 1][q]);
       }
     };
     auto weights = [&](const char* r, float (&w)[4 * NR]) {
@@ -159,16 +175,15 @@ __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile
       const u4 off = *reinterpret_cast<const u4*>(r);
       float w[4 * NR];
       weights(r, w);
-      v2f x[4];
+      vx x[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) x[e] = *reinterpret_cast<const v2f*>(tile_bytes + (off[e] + lane8));
+      for (int e = 0; e < 4; ++e) x[e] = *reinterpret_cast<const vx*>(tile_bytes + (off[e] + lane8));
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        acc[0][0] = __builtin_fmaf(x[e][0], w[e * NR], acc[0][0]);
-        acc[0][1] = __builtin_fmaf(x[e][1], w[e * NR], acc[0][1]);
-        if (NR == 2) {
-          acc[NR - 1][0] = __builtin_fmaf(x[e][0], w[e * NR + NR - 1], acc[NR - 1][0]);
-          acc[NR - 1][1] = __builtin_fmaf(x[e][1], w[e * NR + NR - 1], acc[NR - 1][1]);
+#pragma unroll
+        for (int q = 0; q < PPL; ++q) {
+          acc[0][q] = __builtin_fmaf(x[e][q], w[e * NR], acc[0][q]);
+          if (NR == 2) acc[NR - 1][q] = __builtin_fmaf(x[e][q], w[e * NR + NR - 1], acc[NR - 1][q]);
         }
       }
     }
@@ -185,8 +200,10 @@ __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile
 #pragma unroll
       for (int rr = 0; rr < NR; ++rr) {
         if (rr < nrows) {
-          const v2f o = {ActivateT<ACT>(acc[rr][0], p.act), ActivateT<ACT>(acc[rr][1], p.act)};
-          __builtin_nontemporal_store(o, reinterpret_cast<v2f*>(obase + (size_t)(row0 + rr) * p.hw));
+          vx o;
+#pragma unroll
+          for (int q = 0; q < PPL; ++q) o[q] = ActivateT<ACT>(acc[rr][q], p.act);
+          __builtin_nontemporal_store(o, reinterpret_cast<vx*>(obase + (size_t)(row0 + rr) * p.hw));
         }
       }
     }
@@ -196,7 +213,7 @@ __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile
 // Workgroup id -> tiles: each XCD (linear id mod 8) owns a contiguous range of
 // tiles.  Its first workgroups take one tile each (main part); with a spare
 // part, the workgroups behind them share the range's tiles among themselves.
-template <int NR, int ACT>
+template <int NR, int ACT, bool PAIR>
 __device__ __forceinline__ void TileWalkBody(const TileWalkParams& p, float* tile) {
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int first = (xcd * p.tiles) >> 3, last = ((xcd + 1) * p.tiles) >> 3;
@@ -204,17 +221,17 @@ __device__ __forceinline__ void TileWalkBody(const TileWalkParams& p, float* til
   if (p.split == 2) {
     // equal parts: part = slot / count of tile slot % count
     const int part = count > 0 ? slot / count : p.parts;
-    if (part < p.parts) WalkOneTile<NR, ACT>(p, tile, first + (slot - part * count), part);
+    if (part < p.parts) WalkOneTile<NR, ACT, PAIR>(p, tile, first + (slot - part * count), part);
     return;
   }
   if (slot < count) {
-    WalkOneTile<NR, ACT>(p, tile, first + slot, 0);
+    WalkOneTile<NR, ACT, PAIR>(p, tile, first + slot, 0);
     return;
   }
   if (p.split == 0) return;
   const int n_spare = (int)(gridDim.x >> 3) - count;
   for (int t = first + (slot - count); t < last; t += n_spare) {
-    WalkOneTile<NR, ACT>(p, tile, t, 1);
+    WalkOneTile<NR, ACT, PAIR>(p, tile, t, 1);
     __syncthreads();  // every wavefront has left the tile before the next one is staged
   }
 }
@@ -225,7 +242,11 @@ __global__ void __launch_bounds__(64 * kTileWalkWaves) TileWalkKernel(PL_HEAD_PA
   extern __shared__ float tile_lds[];
   DispatchAct(p.act.type, [&](auto act_c) {
     constexpr int ACT = decltype(act_c)::value;
-    TileWalkBody<NR, ACT>(p, tile_lds);
+    if (p.pairs) {
+      TileWalkBody<NR, ACT, true>(p, tile_lds);
+    } else {
+      TileWalkBody<NR, ACT, false>(p, tile_lds);
+    }
   });
 }
 

@@ -199,6 +199,9 @@ def test_fp32_tiled_walk(shape, paired, act):
     # run above took the share the library computes): the same bits
     for split in (0, 3, 8):  # the field holds 1 + sixteenths
         assert np.array_equal(got, run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired, tuning=capi.tuning(walk_tiled=capi.TUNE_ALWAYS, walk_split=1 + split))), "split %s" % split
+    # one row group per wavefront instruction (two positions per lane) instead of a pair of them (four): the same bits
+    assert np.array_equal(got, run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired, tuning=capi.tuning(walk_tiled=capi.TUNE_ALWAYS, walk_pairs=capi.TUNE_NEVER))), "single row groups"
+    assert np.array_equal(got, run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired, tuning=capi.tuning(walk_tiled=capi.TUNE_ALWAYS, walk_pairs=capi.TUNE_NEVER, walk_split=4))), "single row groups, split"
     # and the plain walk gives the same bits (same order of fused multiply-adds)
     plain = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired, tuning=capi.tuning(walk_tiled=capi.TUNE_NEVER, walk_chunked=capi.TUNE_NEVER))
     assert np.array_equal(got, plain)
