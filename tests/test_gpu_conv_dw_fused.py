@@ -148,3 +148,27 @@ def test_when_the_one_launch_pays():
     assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw1._handle, 2 * cus, 14, 14) == 1
     assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw1._handle, 64, 7, 7) == 0  # does not fit
     assert L.pl_sparse_conv_dwconv3x3_pays(conv._handle, dw1._handle, 0, 14, 14) == 0
+
+
+def test_bad_arguments_are_refused():
+    import ctypes as C
+
+    import torch
+
+    L = capi.lib()
+    _, conv, dw, _ = make_pair(1, 128, 128, 2, "relu", "relu", 31)
+    x = torch.zeros((1, 128, 14, 14), dtype=torch.int8, device="cuda")
+    out = torch.full((128 * 49 + 64,), 77, dtype=torch.int8, device="cuda")
+    s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    run = L.pl_sparse_conv_dwconv3x3_run
+    assert run(None, dw._handle, C.c_void_p(x.data_ptr()), C.c_void_p(out.data_ptr()), 1, 14, 14, s) == capi.PL_ERR_BAD_ARG
+    assert run(conv._handle, None, C.c_void_p(x.data_ptr()), C.c_void_p(out.data_ptr()), 1, 14, 14, s) == capi.PL_ERR_BAD_ARG
+    assert run(conv._handle, dw._handle, C.c_void_p(x.data_ptr()), C.c_void_p(out.data_ptr()), -1, 14, 14, s) == capi.PL_ERR_BAD_ARG
+    assert run(conv._handle, dw._handle, None, C.c_void_p(out.data_ptr()), 1, 14, 14, s) == capi.PL_ERR_BAD_ARG
+    assert run(conv._handle, dw._handle, None, None, 0, 14, 14, s) == capi.PL_OK  # an empty batch is no work
+    # tensors that are not 4-byte aligned
+    assert run(conv._handle, dw._handle, C.c_void_p(x.data_ptr()), C.c_void_p(out.data_ptr() + 1), 1, 14, 14, s) == capi.PL_ERR_UNSUPPORTED
+    assert L.pl_sparse_conv_dwconv3x3_fits(None, dw._handle, 14, 14) == 0
+    assert L.pl_sparse_conv_dwconv3x3_fits(conv._handle, dw._handle, 0, 14) == 0
+    torch.cuda.synchronize()
+    assert bool((out == 77).all())  # none of the refused calls wrote anything
