@@ -188,14 +188,16 @@ __device__ __forceinline__ void DwStage(const DwConvParams& d, char* planes_in, 
 
 // One window of 16 position quads times the wavefront's row tile.  When EPI, the four rows of the previous
 // window (accumulators accp, first quad qp) are finished and stored between the k-steps, one row per KS / 4
-// k-steps (all of them behind the last k-step when KS < 4).  The operand cells of two k-steps are in flight.
+// k-steps (all of them behind the last k-step when KS < 4).
 template <int KS, int OUT, int ACT, bool EPI>
 __device__ __forceinline__ void Window(const uint4* __restrict__ xt, int kgs, int cps, int q0, const v4i (&a)[KS], v4i (&acc)[4], const v4i (&accp)[4], int qp, bool partialp, const float (&sc)[4],
                                        const float (&bi)[4], const DevAct& act, char* __restrict__ orow, int pitch, Lane ln) {
   const uint4* bbase = xt + ln.kq * kgs + (q0 + ln.n);  // + ks * 4 * kgs + c * cps
 #pragma unroll
   for (int c = 0; c < 4; ++c) acc[c] = v4i{0, 0, 0, 0};
-  constexpr int PF = 2;
+  // operand cells in flight ahead of the multiply: two k-steps where the multiply is what the wavefront waits for
+  // (int8 output), one where it hides behind the stores (8.13 against 8.17 us on the metric shape; three: 8.27)
+  constexpr int PF = (OUT == kOutI8 || OUT == kOutPlanes) ? 2 : 1;
   constexpr int kStepsPerRow = KS >= 4 ? KS / 4 : 1;
   uint4 bq[PF + 1][4];
 #pragma unroll
