@@ -122,7 +122,7 @@ typedef struct pl_sparse_conv_tuning {
   int32_t mfma_tile_quads;   /* block kernel: position quads per tile, 8 .. 32 */
   int32_t mfma_narrow_i8_stores; /* 1 = 4-byte int8 stores in the block kernel */
   int32_t wg_slots;          /* workgroups taken as resident at once           */
-  int32_t walk_tiled;        /* (switch) fp32 walk with tile and lists in LDS  */
+  int32_t walk_tiled;        /* (switch) fp32 / fp16 walk with tile and lists in LDS */
   int32_t walk_split;        /* that walk: 1 = row groups not divided between
                                 CUs, 1 + k = k sixteenths to the spare CUs     */
   int32_t walk_chunked;      /* (switch) fp32 / fp16 walk over channel chunks  */

@@ -11,6 +11,7 @@
 
 #include <cstdint>
 
+#include "kernarg_head.h"
 #include "launch_lds.h"
 #include "sparse_conv_kernels.h"
 
@@ -335,6 +336,217 @@ __global__ void __launch_bounds__(64 * kChunkWalkWaves, 2) HalfChunkWalkKernel(c
   }
 }
 
+// Walk with the whole tile and the index lists in LDS (the structure of the fp32 tile walk with pairs of row
+// groups): a workgroup of sixteen wavefronts keeps all channels of 256 positions in LDS, 512 bytes per channel
+// row, and every wavefront streams the double records of its pairs of row groups through a private LDS buffer.
+// Lanes 0 - 31 walk the first row group of a pair, lanes 32 - 63 the second, eight positions per lane: per
+// entry one 16-byte LDS read and four v_pk_fma_f16 per row.  Weights and biases arrive in the stream as
+// binary16 values doubled into a dword, so they need no splat.  The accumulator of an output starts at its
+// bias and takes its entries in index order, one rounding per entry, as in the other half-precision walks
+// (same bits).
+PL_IN_HEAD(HalfTileWalkParams, x);
+PL_IN_HEAD(HalfTileWalkParams, stream);
+PL_IN_HEAD(HalfTileWalkParams, stream_first);
+PL_IN_HEAD(HalfTileWalkParams, K);
+PL_IN_HEAD(HalfTileWalkParams, hw);
+PL_IN_HEAD(HalfTileWalkParams, P);
+PL_IN_HEAD(HalfTileWalkParams, tiles);
+PL_IN_HEAD(HalfTileWalkParams, split);
+PL_IN_HEAD(HalfTileWalkParams, parts);
+static_assert(offsetof(HalfTileWalkParams, act) + sizeof(int) <= kHeadWords * 8, "act.type must lie in the first 56 bytes of HalfTileWalkParams");
+
+typedef uint32_t u2w __attribute__((ext_vector_type(2)));
+typedef uint32_t u4w __attribute__((ext_vector_type(4)));
+constexpr int kTwTile = kHalfTileWalkTile;
+constexpr int kTwRowBytes = kTwTile * 2;
+constexpr int kTwWaves = kTileWalkWaves;
+constexpr int kTwChunkBytes = kTileWalkChunkBytes;
+static_assert(kTwRowBytes == kTileWalkTile * 4, "the list streams hold byte offsets of 512-byte channel rows");
+
+// One tile: stage it, then walk the streams of one part (0 main, 1 spare).
+template <int NR, int ACT>
+__device__ __forceinline__ void HalfWalkOneTile(const HalfTileWalkParams& p, char* tile_bytes, int tile_id, int part) {
+  constexpr int kRecBytes = NR == 2 ? 48 : 32;  // four byte offsets, then 4 * NR doubled weights
+  constexpr int kStepBytes = 2 * kRecBytes;     // one record per row group of the pair
+  constexpr int kRecs = kTwChunkBytes / kStepBytes;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int sidx = part * kTwWaves + wave;
+  const uint32_t tile0 = (uint32_t)tile_id * (uint32_t)kTwTile;
+  char* lbuf = tile_bytes + (size_t)(p.K + 1) * kTwRowBytes + wave * kTwChunkBytes;
+
+  // the wavefront's list stream: chunks of kTwChunkBytes, lane i holds bytes [16 i, 16 i + 16) and
+  // [1024 + 8 i, 1024 + 8 i + 8) of a chunk
+  const char* sp = reinterpret_cast<const char*>(p.stream) + (size_t)((ConstWords)p.stream_first)[sidx] * kTwChunkBytes;
+  u4w pa = *reinterpret_cast<const u4w*>(sp + 16 * lane);
+  u2w pb = *reinterpret_cast<const u2w*>(sp + 1024 + 8 * lane);
+
+  // staging: 32 threads per channel row (eight positions each), 32 rows per pass
+  {
+    const int c8 = tid & 31, r0 = tid >> 5;
+    const uint32_t gpos = tile0 + 8u * (uint32_t)c8;
+    const bool live = gpos < p.P;
+    const uint32_t n = live ? gpos / (uint32_t)p.hw : 0u;
+    const uint32_t pp = live ? gpos % (uint32_t)p.hw : 0u;
+    const uint16_t* xcol = p.x + (size_t)n * p.K * p.hw + pp;
+    for (int k0 = 0; k0 < p.K; k0 += 128) {
+      uint4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int k = min(k0 + r0 + 32 * u, p.K - 1);
+        v[u] = *reinterpret_cast<const uint4*>(xcol + (size_t)k * p.hw);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int k = k0 + r0 + 32 * u;
+        if (k < p.K) *reinterpret_cast<uint4*>(tile_bytes + (size_t)k * kTwRowBytes + 16 * c8) = live ? v[u] : make_uint4(0, 0, 0, 0);
+      }
+    }
+    // row K is all zero: the target of list padding entries
+    if (tid < kTwRowBytes / 16) *reinterpret_cast<uint4*>(tile_bytes + (size_t)p.K * kTwRowBytes + 16 * tid) = make_uint4(0, 0, 0, 0);
+  }
+  __syncthreads();
+
+  const int half = lane >> 5;
+  const uint32_t lane16 = 16u * (uint32_t)(lane & 31);
+  const uint32_t gpos = tile0 + 8u * (uint32_t)(lane & 31);
+  const bool store_on = gpos < p.P;
+  const uint32_t on = store_on ? gpos / (uint32_t)p.hw : 0u, opp = store_on ? gpos % (uint32_t)p.hw : 0u;
+  uint16_t* obase = p.out + (size_t)on * p.M * p.hw + opp;
+
+  int rec = kRecs;  // records of the current chunk already walked: the first chunk is still in registers
+  int chunk = 0;
+  // next double record of the stream; at the end of a chunk the prefetched one becomes the current one (only
+  // this wavefront reads the buffer, and its LDS operations execute in order) and the one after it is requested
+  auto next = [&]() -> const char* {
+    if (rec == kRecs) {
+      *reinterpret_cast<u4w*>(lbuf + 16 * lane) = pa;
+      *reinterpret_cast<u2w*>(lbuf + 1024 + 8 * lane) = pb;
+      ++chunk;
+      const char* np = sp + (size_t)chunk * kTwChunkBytes;  // the stream ends with one spare chunk
+      pa = *reinterpret_cast<const u4w*>(np + 16 * lane);
+      pb = *reinterpret_cast<const u2w*>(np + 1024 + 8 * lane);
+      rec = 0;
+    }
+    return lbuf + (rec++) * kStepBytes + half * kRecBytes;
+  };
+  const int n_groups = (int)((ConstWords)p.stream_groups)[sidx];
+  for (int j = 0; j < n_groups; ++j) {
+    // header record of a row group: first row | rows << 24, entries (the same in both halves), doubled bias
+    // of its rows
+    const u4w hdr = *reinterpret_cast<const u4w*>(next());
+    const int row0 = (int)(hdr.x & 0xffffffu);
+    const int nrows = (int)(hdr.x >> 24);
+    const uint32_t entries = (uint32_t)__builtin_amdgcn_readfirstlane((int)hdr.y);
+    // (bit casts take scalars: applied to an element of a vector they read its first element)
+    const uint32_t bias0 = hdr.z, bias1 = hdr.w;
+    h2 acc[NR][4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      acc[0][q] = __builtin_bit_cast(h2, bias0);
+      if (NR == 2) acc[NR - 1][q] = __builtin_bit_cast(h2, bias1);
+    }
+    auto entry = [&](const u4w& x, uint32_t w0, uint32_t w1) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint32_t xq = x[q];
+        const h2 x2 = __builtin_bit_cast(h2, xq);
+        acc[0][q] = __builtin_elementwise_fma(x2, __builtin_bit_cast(h2, w0), acc[0][q]);
+        if (NR == 2) acc[NR - 1][q] = __builtin_elementwise_fma(x2, __builtin_bit_cast(h2, w1), acc[NR - 1][q]);
+      }
+    };
+    auto weights = [&](const char* r, uint32_t (&w)[4 * NR]) {
+      const u4w wa = *reinterpret_cast<const u4w*>(r + 16);
+      w[0] = wa.x, w[1] = wa.y, w[2] = wa.z, w[3] = wa.w;
+      if (NR == 2) {
+        const u4w wb = *reinterpret_cast<const u4w*>(r + (NR == 2 ? 32 : 16));
+        w[4 * NR - 4] = wb.x, w[4 * NR - 3] = wb.y, w[4 * NR - 2] = wb.z, w[4 * NR - 1] = wb.w;
+      }
+    };
+    const uint32_t batches = entries >> 2, rem = entries & 3u;
+    for (uint32_t b = 0; b < batches; ++b) {
+      const char* r = next();
+      const u4w off = *reinterpret_cast<const u4w*>(r);
+      uint32_t w[4 * NR];
+      weights(r, w);
+      u4w x[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[e] = *reinterpret_cast<const u4w*>(tile_bytes + (off[e] + lane16));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) entry(x[e], w[e * NR], w[e * NR + NR - 1]);
+    }
+    if (rem != 0) {  // the last, partly filled batch: only its real entries
+      const char* r = next();
+      const u4w off = *reinterpret_cast<const u4w*>(r);
+      uint32_t w[4 * NR];
+      weights(r, w);
+      entry(*reinterpret_cast<const u4w*>(tile_bytes + (off[0] + lane16)), w[0], w[NR - 1]);
+      if (rem > 1) entry(*reinterpret_cast<const u4w*>(tile_bytes + (off[1] + lane16)), w[NR], w[NR + NR - 1]);
+      if (rem > 2) entry(*reinterpret_cast<const u4w*>(tile_bytes + (off[2] + lane16)), w[2 * NR], w[2 * NR + NR - 1]);
+    }
+    if (store_on) {
+#pragma unroll
+      for (int rr = 0; rr < NR; ++rr) {
+        if (rr < nrows) {
+          u4w o;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) o[q] = __builtin_bit_cast(uint32_t, ActivateH<ACT>(acc[rr][q], p.act));
+          __builtin_nontemporal_store(o, reinterpret_cast<u4w*>(obase + (size_t)(row0 + rr) * p.hw));
+        }
+      }
+    }
+  }
+}
+
+// Workgroup id -> tiles, as in the fp32 tile walk: each XCD (linear id mod 8) owns a contiguous range of tiles;
+// its first workgroups take one tile each (main part), with a spare part the workgroups behind them share the
+// range's tiles among themselves, with equal parts `parts` workgroups share every tile.
+template <int NR, int ACT>
+__device__ __forceinline__ void HalfTileWalkBody(const HalfTileWalkParams& p, char* tile) {
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int first = (xcd * p.tiles) >> 3, last = ((xcd + 1) * p.tiles) >> 3;
+  const int count = last - first;
+  if (p.split == 2) {
+    const int part = count > 0 ? slot / count : p.parts;
+    if (part < p.parts) HalfWalkOneTile<NR, ACT>(p, tile, first + (slot - part * count), part);
+    return;
+  }
+  if (slot < count) {
+    HalfWalkOneTile<NR, ACT>(p, tile, first + slot, 0);
+    return;
+  }
+  if (p.split == 0) return;
+  const int n_spare = (int)(gridDim.x >> 3) - count;
+  for (int t = first + (slot - count); t < last; t += n_spare) {
+    HalfWalkOneTile<NR, ACT>(p, tile, t, 1);
+    __syncthreads();  // every wavefront has left the tile before the next one is staged
+  }
+}
+
+template <int NR>
+__global__ void __launch_bounds__(64 * kTileWalkWaves) HalfTileWalkKernel(PL_HEAD_PARAMS, const HalfTileWalkParams block) {
+  const HalfTileWalkParams p = WithHead(block, PL_HEAD_ARGS);
+  extern __shared__ uint32_t tile32[];
+  char* tile = reinterpret_cast<char*>(tile32);
+  switch (p.act.type) {
+    case 1:
+      HalfTileWalkBody<NR, 1>(p, tile);
+      break;
+    case 2:
+      HalfTileWalkBody<NR, 2>(p, tile);
+      break;
+    case 4:
+      HalfTileWalkBody<NR, 4>(p, tile);
+      break;
+    case 10:
+      HalfTileWalkBody<NR, 10>(p, tile);
+      break;
+    default:
+      HalfTileWalkBody<NR, 0>(p, tile);
+      break;
+  }
+}
+
 template <typename K>
 hipError_t LaunchBig(K kernel, dim3 grid, dim3 block, size_t lds, hipStream_t s, const HalfWalkParams& p) {
   return LaunchWithLds(kernel, grid, block, lds, s, p);
@@ -386,6 +598,27 @@ hipError_t LaunchHalfChunkWalk(int nrows, const HalfChunkWalkParams& p, hipStrea
   if (p.P == 0 || p.n_groups == 0) return hipSuccess;
   if (p.hw % 4 != 0 || p.n_chunks < 1 || p.slices < 1) return hipErrorInvalidValue;
   return nrows == 2 ? HalfChunkLaunch<2, 4>(p, stream) : HalfChunkLaunch<1, 4>(p, stream);
+}
+
+// Needs hw % 8 == 0 and 16-byte aligned x / out (a lane's eight positions are one 16-byte piece of one image).
+hipError_t LaunchHalfTileWalk(int nrows, const HalfTileWalkParams& p, hipStream_t stream) {
+  if (p.P == 0 || p.n_groups == 0) return hipSuccess;
+  if (p.hw % 8 != 0) return hipErrorInvalidValue;
+  const size_t lds = TileWalkLdsBytes(p.K);
+  if (lds > (size_t)kMaxLdsBytes) return hipErrorInvalidValue;
+  HalfTileWalkParams q = p;
+  q.tiles = (int)((p.P + kTwTile - 1) / kTwTile);
+  uint32_t slots = ((uint32_t)q.tiles + 7) / 8;  // workgroups per XCD
+  if (q.split == 2) {
+    if (q.parts < 2 || (int64_t)q.parts * slots > q.split_slots) return hipErrorInvalidValue;
+    slots *= (uint32_t)q.parts;
+  } else if (q.split != 0) {
+    if (q.split_slots < (int)slots + 1) return hipErrorInvalidValue;  // every XCD needs a spare workgroup
+    slots = (uint32_t)q.split_slots;
+  }
+  dim3 grid(8u * slots), block(64 * kTwWaves);
+  if (nrows == 2) return LaunchWithHead(HalfTileWalkKernel<2>, grid, block, lds, stream, q);
+  return LaunchWithHead(HalfTileWalkKernel<1>, grid, block, lds, stream, q);
 }
 
 }  // namespace pl

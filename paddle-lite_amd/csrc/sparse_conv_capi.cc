@@ -373,16 +373,24 @@ int BuildChunkWalk(const pl::DecodedLayout& L, pl_sparse_conv_handle* h, bool ha
   return PL_OK;
 }
 
-// Device-side form for the fp32 tile walk: the row groups are dealt to
+// Device-side form for the tile walks (fp32 and half precision): the row groups are dealt to
 // kTileWalkWaves list streams (longest list first, each to the stream with the
 // least work so far); a stream is the concatenation of its groups' batches of
-// four entries as records of byte offsets and weights.
+// four entries as records of byte offsets and weights.  In half precision a weight or bias word is the
+// binary16 value doubled (value | value << 16) and the streams always hold pairs.
 // Main / spare divisions of the tile walk's row groups that are prepared: spare shares of 1/16 .. 8/16.
 constexpr int kTileWalkSplits = 8;
 // Equal divisions that are prepared (two equal parts are the 8/16 division above).
 constexpr int kTileWalkEqualParts[] = {3, 4, 5, 6, 8, 10};
 
-int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_handle* h) {
+uint32_t DoubledHalf(uint32_t float_bits) {
+  float v;
+  std::memcpy(&v, &float_bits, 4);
+  const uint32_t b = HalfBits(v);
+  return b | (b << 16);
+}
+
+int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_handle* h, bool half = false) {
   h->tw_built = 0;
   if (pl::TileWalkLdsBytes(L.ic) > static_cast<size_t>(pl::kMaxLdsBytes)) return PL_OK;  // too many channels for one tile: other walks
   const int nr = L.semi ? 2 : 1;
@@ -394,7 +402,8 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
   // A unit is what one wavefront instruction walks: one row group, or (walk_pairs) two of about the same
   // length - neighbours in the order by length - of which the shorter is padded with entries of weight zero that
   // point at the tile's zero row; a last group without a partner gets an empty one (no rows).
-  const bool pairs = h->walk_pairs;
+  const bool pairs = half || h->walk_pairs;
+  auto word = [&](uint32_t float_bits) { return half ? DoubledHalf(float_bits) : float_bits; };
   struct Unit {
     int a, b;        // row groups (b = -1: none)
     uint32_t count;  // entries walked
@@ -460,8 +469,11 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
           const pl::RowGroup& rg = L.groups[side_groups[side]];
           r[0] = static_cast<uint32_t>(rg.row0) | (static_cast<uint32_t>(rg.nrows) << 24);
           if (bias) {
-            std::memcpy(&r[2], &bias[rg.row0], 4);
-            if (rg.nrows == 2) std::memcpy(&r[3], &bias[rg.row0 + 1], 4);
+            uint32_t b0 = 0, b1 = 0;
+            std::memcpy(&b0, &bias[rg.row0], 4);
+            if (rg.nrows == 2) std::memcpy(&b1, &bias[rg.row0 + 1], 4);
+            r[2] = word(b0);
+            if (rg.nrows == 2) r[3] = word(b1);
           }
         }
         put(rec);
@@ -474,8 +486,8 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
             for (uint32_t e = 0; e < 4; ++e) {
               const bool real = rg != nullptr && e0 + e < rg->count;
               r[e] = real ? L.ic_index[rg->first + e0 + e] * pl::kTileWalkTile * 4 : zero_row;
-              r[4 + e * nr] = real ? L.w0[rg->first + e0 + e] : 0u;
-              if (nr == 2) r[4 + e * nr + 1] = real ? L.w1[rg->first + e0 + e] : 0u;
+              r[4 + e * nr] = real ? word(L.w0[rg->first + e0 + e]) : 0u;
+              if (nr == 2) r[4 + e * nr + 1] = real ? word(L.w1[rg->first + e0 + e]) : 0u;
             }
           }
           put(rec);
@@ -856,6 +868,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
     h->algo = PL_ALGO_ROW_WALK;
     int hrc = BuildHalfWalk(L, h);
     if (hrc == PL_OK) hrc = BuildChunkWalk(L, h, true);
+    if (hrc == PL_OK) hrc = BuildTileWalk(L, desc->bias, h, true);
     if (hrc == PL_OK) hrc = UploadHalfBias(h, desc->bias);
     if (hrc != PL_OK) {
       delete h;
@@ -918,6 +931,55 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   return PL_OK;
 }
 
+// How a tile walk of `tiles` tiles is divided over the CUs, and where the stream tables of that division start.
+// With fewer tiles than CUs, the CUs without a tile take a share of the row groups of several tiles each
+// (one after the other, each staged anew).  The share that evens out the two kinds of workgroup: a main
+// workgroup spends S + (1 - f) W, a spare one r (S + f W) for its r tiles, with S the staging time of a tile
+// and W the walk of all row groups, so f = (1 - (r - 1) S / W) / (r + 1).  S and W in cycles, fitted to
+// measurements (a tile of 256 channels costs a spare workgroup about 5.6 K cycles besides its walk; 355
+// cycles per work unit of the fullest stream).  Rounded down: a share above the balance point costs r
+// times what one below it costs.
+struct TileWalkDivision {
+  int split = 0;    // 0 none, 1 main + spare part, 2 equal parts
+  int parts = 0;    // equal parts
+  int split_slots = 0;
+  size_t table = 0;  // first entry of the division's stream tables
+};
+
+TileWalkDivision DivideTileWalk(const pl_sparse_conv_handle* h, int tiles) {
+  TileWalkDivision d;
+  const int cus = std::max(8, h->wg_slots_default / 2) / 8 * 8;
+  int s16 = 0, equal_parts = 0;
+  if (tiles < cus && h->walk_split != 0) {
+    const int per_xcd = CeilDiv(tiles, 8), spare = cus / 8 - per_xcd;
+    if (h->walk_split < 0 && per_xcd * 3 <= cus / 8) {
+      // at most a third as many tiles as CUs: n workgroups per tile, equal shares
+      const int room = (cus / 8) / per_xcd;
+      for (int n : kTileWalkEqualParts)
+        if (n <= room) equal_parts = n;
+    } else if (spare >= 1) {
+      const int r = CeilDiv(per_xcd, spare);
+      const double sw = (2000.0 + 14.0 * h->ic) / (355.0 * static_cast<double>(std::max<int64_t>(1, h->tw_stream_work)));
+      const double f = (1.0 - (r - 1) * sw) / (r + 1);
+      s16 = h->walk_split > 0 ? h->walk_split : static_cast<int>(f * 16.0 + 0.3);
+      s16 = std::max(0, std::min(kTileWalkSplits, s16));
+    }
+  }
+  // stream tables: set 0 has one part, sets 1 .. 8 two, then the equal divisions
+  d.table = s16 == 0 ? 0 : static_cast<size_t>(pl::kTileWalkWaves) * (2 * s16 - 1);
+  if (equal_parts != 0) {
+    d.table = static_cast<size_t>(pl::kTileWalkWaves) * (1 + 2 * kTileWalkSplits);
+    for (int n : kTileWalkEqualParts) {
+      if (n == equal_parts) break;
+      d.table += static_cast<size_t>(pl::kTileWalkWaves) * n;
+    }
+  }
+  d.split = equal_parts != 0 ? 2 : (s16 != 0 ? 1 : 0);
+  d.parts = equal_parts;
+  d.split_slots = cus / 8;
+  return d;
+}
+
 int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_dev, int32_t batch, int32_t im_size, void* stream) {
   if (!h) return Fail(PL_ERR_BAD_ARG, "null handle");
   if (batch < 0 || im_size <= 0) return Fail(PL_ERR_BAD_ARG, "batch must be >= 0 and im_size > 0");
@@ -933,7 +995,29 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipError_t e;
   const int call_algo = AlgoForCall(h, batch, im_size, aligned16);
-  if (h->half && (im_size % 4 == 0) && (reinterpret_cast<uintptr_t>(x_dev) % 8 == 0) && (reinterpret_cast<uintptr_t>(out_dev) % 8 == 0) && h->walk_chunked > 0 && h->cw_chunks > 0 &&
+  if (h->half && h->tw_built != 0 && h->walk_tiled > 0 && im_size % 8 == 0 && aligned16 &&
+      (h->walk_tiled == 2 || (h->semi ? 42 : 84) * static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kHalfTileWalkTile)) >= h->wg_slots_default)) {
+    // The walk with the tile and the lists in LDS, from 7 tiles of 256 positions on (13 with row pairs, whose
+    // plain walk is twice as efficient per list entry) on 256 CUs: measured against the other half-precision
+    // walks at 1 - 784 tiles, it is 1.3 - 2.5 times as fast from there on and slower below.
+    const TileWalkDivision d = DivideTileWalk(h, CeilDiv(static_cast<int>(P), pl::kHalfTileWalkTile));
+    pl::HalfTileWalkParams p{};
+    p.x = static_cast<const uint16_t*>(x_dev);
+    p.out = static_cast<uint16_t*>(out_dev);
+    p.stream = h->tw_stream.ptr;
+    p.stream_first = static_cast<const uint32_t*>(h->tw_first.ptr) + d.table;
+    p.stream_groups = static_cast<const uint32_t*>(h->tw_desc.ptr) + d.table;
+    p.split = static_cast<int16_t>(d.split);
+    p.parts = static_cast<int8_t>(d.parts);
+    p.split_slots = d.split_slots;
+    p.n_groups = h->n_groups;
+    p.M = h->oc;
+    p.K = h->ic;
+    p.hw = im_size;
+    p.P = P;
+    p.act = h->act_h;
+    e = pl::LaunchHalfTileWalk(h->semi ? 2 : 1, p, s);
+  } else if (h->half && (im_size % 4 == 0) && (reinterpret_cast<uintptr_t>(x_dev) % 8 == 0) && (reinterpret_cast<uintptr_t>(out_dev) % 8 == 0) && h->walk_chunked > 0 && h->cw_chunks > 0 &&
       (h->walk_chunked == 2 || (h->ic > 128 && static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kChunkWalkTile)) * h->cw_slices >= 256))) {
     // many channels and enough work for every CU: walk over channel chunks
     pl::HalfChunkWalkParams p{};
@@ -1066,46 +1150,13 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.x = static_cast<const float*>(x_dev);
     p.out = static_cast<float*>(out_dev);
     p.stream = h->tw_stream.ptr;
-    // With fewer tiles than CUs, the CUs without a tile take a share of the row groups of several tiles each
-    // (one after the other, each staged anew).  The share that evens out the two kinds of workgroup: a main
-    // workgroup spends S + (1 - f) W, a spare one r (S + f W) for its r tiles, with S the staging time of a tile
-    // and W the walk of all row groups, so f = (1 - (r - 1) S / W) / (r + 1).  S and W in cycles, fitted to
-    // measurements (a tile of 256 channels costs a spare workgroup about 5.6 K cycles besides its walk; 355
-    // cycles per work unit of the fullest stream).  Rounded down: a share above the balance point costs r
-    // times what one below it costs.
-    const int tiles = CeilDiv(static_cast<int>(P), pl::kTileWalkTile);
-    const int cus = std::max(8, h->wg_slots_default / 2) / 8 * 8;
-    int s16 = 0, equal_parts = 0;
-    if (tiles < cus && h->walk_split != 0) {
-      const int per_xcd = CeilDiv(tiles, 8), spare = cus / 8 - per_xcd;
-      if (h->walk_split < 0 && per_xcd * 3 <= cus / 8) {
-        // at most a third as many tiles as CUs: n workgroups per tile, equal shares
-        const int room = (cus / 8) / per_xcd;
-        for (int n : kTileWalkEqualParts)
-          if (n <= room) equal_parts = n;
-      } else if (spare >= 1) {
-        const int r = CeilDiv(per_xcd, spare);
-        const double sw = (2000.0 + 14.0 * h->ic) / (355.0 * static_cast<double>(std::max<int64_t>(1, h->tw_stream_work)));
-        const double f = (1.0 - (r - 1) * sw) / (r + 1);
-        s16 = h->walk_split > 0 ? h->walk_split : static_cast<int>(f * 16.0 + 0.3);
-        s16 = std::max(0, std::min(kTileWalkSplits, s16));
-      }
-    }
-    // stream tables: set 0 has one part, sets 1 .. 8 two, then the equal divisions
-    size_t table = s16 == 0 ? 0 : static_cast<size_t>(pl::kTileWalkWaves) * (2 * s16 - 1);
-    if (equal_parts != 0) {
-      table = static_cast<size_t>(pl::kTileWalkWaves) * (1 + 2 * kTileWalkSplits);
-      for (int n : kTileWalkEqualParts) {
-        if (n == equal_parts) break;
-        table += static_cast<size_t>(pl::kTileWalkWaves) * n;
-      }
-    }
-    p.stream_first = static_cast<const uint32_t*>(h->tw_first.ptr) + table;
-    p.stream_groups = static_cast<const uint32_t*>(h->tw_desc.ptr) + table;
-    p.split = equal_parts != 0 ? 2 : (s16 != 0 ? 1 : 0);
-    p.parts = equal_parts;
+    const TileWalkDivision d = DivideTileWalk(h, CeilDiv(static_cast<int>(P), pl::kTileWalkTile));
+    p.stream_first = static_cast<const uint32_t*>(h->tw_first.ptr) + d.table;
+    p.stream_groups = static_cast<const uint32_t*>(h->tw_desc.ptr) + d.table;
+    p.split = static_cast<int16_t>(d.split);
+    p.parts = static_cast<int8_t>(d.parts);
     p.pairs = h->walk_pairs ? 1 : 0;
-    p.split_slots = cus / 8;
+    p.split_slots = d.split_slots;
     p.n_groups = h->n_groups;
     p.M = h->oc;
     p.K = h->ic;
@@ -1220,8 +1271,11 @@ int pl_sparse_conv_set_epilogue(pl_sparse_conv_handle* h, const float* scale, co
     // the tile walk starts its accumulators from the bias in its header records
     for (const auto& slot : h->tw_bias_slots) {
       const uint32_t row0 = slot.second & 0xffffffu, nrows = slot.second >> 24;
-      std::memcpy(&h->tw_host_stream[slot.first], &bias[row0], 4);
-      if (nrows == 2) std::memcpy(&h->tw_host_stream[slot.first + 1], &bias[row0 + 1], 4);
+      uint32_t b0 = 0, b1 = 0;
+      std::memcpy(&b0, &bias[row0], 4);
+      if (nrows == 2) std::memcpy(&b1, &bias[row0 + 1], 4);
+      h->tw_host_stream[slot.first] = h->half ? DoubledHalf(b0) : b0;
+      if (nrows == 2) h->tw_host_stream[slot.first + 1] = h->half ? DoubledHalf(b1) : b1;
     }
     const hipError_t e = h->tw_stream.Upload(h->tw_host_stream.data(), h->tw_host_stream.size() * sizeof(uint32_t));
     if (e != hipSuccess) return FailHip(e, "uploading the tile-walk list streams");

@@ -176,6 +176,34 @@ struct HalfChunkWalkParams {
 // Needs hw % 4 == 0 and 8-byte aligned x / out.
 hipError_t LaunchHalfChunkWalk(int nrows, const HalfChunkWalkParams& p, hipStream_t stream);
 
+// Half-precision tile walk: the layout of TileWalkParams with pairs of row groups.  A tile holds 256 positions
+// (the same 512 bytes per channel row, so the byte offsets in the list streams are those of the fp32 walk), a
+// lane eight; weights and biases in the streams are binary16 values doubled into a dword (value | value << 16).
+constexpr int kHalfTileWalkTile = 256;
+
+struct HalfTileWalkParams {
+  const uint16_t* x;
+  uint16_t* out;
+  const void* stream;
+  const uint32_t* stream_first;
+  int K;
+  int hw;
+  uint32_t P;
+  int tiles;  // filled in by the launcher
+  int16_t split;
+  int8_t parts;
+  int8_t reserved;
+  // the first 56 bytes (kernarg_head.h) end behind act.type
+  DevActH act;
+  const uint32_t* stream_groups;
+  int n_groups;
+  int M;
+  int split_slots;
+};
+
+// Needs hw % 8 == 0 and 16-byte aligned x / out.
+hipError_t LaunchHalfTileWalk(int nrows, const HalfTileWalkParams& p, hipStream_t stream);
+
 struct HalfWalkParams {
   const uint16_t* x;
   uint16_t* out;

@@ -68,3 +68,50 @@ def test_fp16_chunked_walk(shape, paired, act):
     # the plain half-precision walk gives the same bits (same order of operations)
     plain = run_hip(case, capi.ALGO_AUTO, force_semi=paired, tuning=capi.tuning(walk_chunked=capi.TUNE_NEVER))
     assert np.array_equal(got.view(np.uint16), plain.view(np.uint16))
+
+
+# Half-precision walk with the whole tile (256 positions, all channels) and the list streams in LDS, two row
+# groups per wavefront instruction; forced here, the library picks it by itself from 8 tiles on.  Needs
+# H*W % 8 == 0 and at most 271 channels.  (batch, ic, oc, h, w): one tile shared by ten workgroups, a channel
+# count off the staging pass of 128, an odd number of row groups (a pair without partner), a tile that spans
+# images and ends inside one, a single row group.
+TILED_SHAPES = [(2, 64, 64, 4, 4), (1, 96, 48, 8, 6), (3, 130, 67, 4, 6), (5, 70, 33, 2, 4), (2, 257, 20, 12, 12), (3, 200, 1, 8, 8), (1, 271, 96, 16, 24)]
+
+
+@pytest.mark.parametrize("act", ["none", "relu", "relu6", "leaky", "hswish"])
+@pytest.mark.parametrize("shape", TILED_SHAPES, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
+def test_fp16_tile_walk(shape, paired, act):
+    batch, ic, oc, h, w = shape
+    case = half_case(batch, ic, oc, h, w, 0.75, paired, ACTS[act], seed=ic + 3 * oc)
+    want = run_oracle(case, oracle_pack(case, force_semi=paired))
+    got = run_hip(case, capi.ALGO_AUTO, force_semi=paired, tuning=capi.tuning(walk_tiled=capi.TUNE_ALWAYS))
+    assert_same(case, got, want, "fp16 tile walk %s %s" % (act, shape))
+
+
+@pytest.mark.parametrize("batch", [3, 24, 40, 64, 65])
+@pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
+def test_fp16_tile_walk_divisions(batch, paired):
+    """Tiles shared by several workgroups in equal parts, main and spare parts, one tile per workgroup and more
+    tiles than CUs: the bits of the plain half-precision walk (the oracle's, by the tests above) every time."""
+    case = half_case(batch, 256, 512, 28, 28, 0.85, paired, ACTS["relu"], seed=batch)
+    tiled = run_hip(case, capi.ALGO_AUTO, force_semi=paired, tuning=capi.tuning(walk_tiled=capi.TUNE_ALWAYS))
+    plain = run_hip(case, capi.ALGO_AUTO, force_semi=paired, tuning=capi.tuning(walk_tiled=capi.TUNE_NEVER, walk_chunked=capi.TUNE_NEVER))
+    assert np.array_equal(tiled.view(np.uint16), plain.view(np.uint16))
+
+
+@pytest.mark.parametrize("had_bias", [True, False], ids=["bias", "no_bias"])
+def test_fp16_tile_walk_takes_a_new_bias(had_bias):
+    """set_epilogue rewrites the biases in the list streams (the accumulators start from them), also in a handle
+    that was prepared without one."""
+    from helpers import make_kernel
+
+    case = half_case(12, 128, 96, 16, 16, 0.8, False, ACTS["relu"], seed=9)
+    if not had_bias:
+        case.bias = None
+    kernel, _ = make_kernel(case, tuning=capi.tuning(walk_tiled=capi.TUNE_ALWAYS))
+    assert_same(case, run_hip(case, kernel=kernel), run_oracle(case), "fp16 tile walk, first bias")
+    new_bias = np.linspace(-0.7, 0.9, 96).astype(np.float32)
+    capi.check(capi.lib().pl_sparse_conv_set_epilogue(kernel._handle, None, new_bias.ctypes.data, None))
+    case.bias = new_bias
+    assert_same(case, run_hip(case, kernel=kernel), run_oracle(case), "fp16 tile walk, second bias")
