@@ -340,7 +340,9 @@ __global__ void __launch_bounds__(64 * kChunkWalkWaves, 2) HalfChunkWalkKernel(c
 // groups): a workgroup of sixteen wavefronts keeps all channels of 256 positions in LDS, 512 bytes per channel
 // row, and every wavefront streams the double records of its pairs of row groups through a private LDS buffer.
 // Lanes 0 - 31 walk the first row group of a pair, lanes 32 - 63 the second, eight positions per lane: per
-// entry one 16-byte LDS read and four v_pk_fma_f16 per row.  Weights and biases arrive in the stream as
+// entry one 16-byte LDS read and four v_pk_fma_f16 per row.  (PPL = 4: tiles of 128 positions, four per lane,
+// 8-byte reads and two v_pk_fma_f16 - for channel counts whose wide tile does not fit LDS and for maps whose size
+// is a multiple of 4 only.)  Weights and biases arrive in the stream as
 // binary16 values doubled into a dword, so they need no splat.  The accumulator of an output starts at its
 // bias and takes its entries in index order, one rounding per entry, as in the other half-precision walks
 // (same bits).
@@ -357,15 +359,28 @@ static_assert(offsetof(HalfTileWalkParams, act) + sizeof(int) <= kHeadWords * 8,
 
 typedef uint32_t u2w __attribute__((ext_vector_type(2)));
 typedef uint32_t u4w __attribute__((ext_vector_type(4)));
-constexpr int kTwTile = kHalfTileWalkTile;
-constexpr int kTwRowBytes = kTwTile * 2;
 constexpr int kTwWaves = kTileWalkWaves;
 constexpr int kTwChunkBytes = kTileWalkChunkBytes;
-static_assert(kTwRowBytes == kTileWalkTile * 4, "the list streams hold byte offsets of 512-byte channel rows");
+static_assert(kHalfTileWalkTile == 32 * 8 && kHalfTileWalkNarrowTile == 32 * 4, "32 lanes of a row group times the positions per lane");
+static_assert(kHalfTileWalkTile * 2 == kTileWalkTile * 4, "the wide tile's list streams hold the byte offsets of the fp32 walk's channel rows");
+
+// what a lane holds of a channel row: PPL positions
+template <int PPL>
+struct TwPiece;
+template <>
+struct TwPiece<8> {
+  typedef u4w type;
+};
+template <>
+struct TwPiece<4> {
+  typedef u2w type;
+};
 
 // One tile: stage it, then walk the streams of one part (0 main, 1 spare).
-template <int NR, int ACT>
+template <int NR, int PPL, int ACT>
 __device__ __forceinline__ void HalfWalkOneTile(const HalfTileWalkParams& p, char* tile_bytes, int tile_id, int part) {
+  typedef typename TwPiece<PPL>::type Piece;
+  constexpr int kTwTile = 32 * PPL, kTwRowBytes = kTwTile * 2, kPieceBytes = 2 * PPL, NW = PPL / 2;
   constexpr int kRecBytes = NR == 2 ? 48 : 32;  // four byte offsets, then 4 * NR doubled weights
   constexpr int kStepBytes = 2 * kRecBytes;     // one record per row group of the pair
   constexpr int kRecs = kTwChunkBytes / kStepBytes;
@@ -381,35 +396,37 @@ __device__ __forceinline__ void HalfWalkOneTile(const HalfTileWalkParams& p, cha
   u4w pa = *reinterpret_cast<const u4w*>(sp + 16 * lane);
   u2w pb = *reinterpret_cast<const u2w*>(sp + 1024 + 8 * lane);
 
-  // staging: 32 threads per channel row (eight positions each), 32 rows per pass
+  // staging: 32 threads per channel row (PPL positions each), 32 rows per pass
   {
     const int c8 = tid & 31, r0 = tid >> 5;
-    const uint32_t gpos = tile0 + 8u * (uint32_t)c8;
+    const uint32_t gpos = tile0 + (uint32_t)PPL * (uint32_t)c8;
     const bool live = gpos < p.P;
     const uint32_t n = live ? gpos / (uint32_t)p.hw : 0u;
     const uint32_t pp = live ? gpos % (uint32_t)p.hw : 0u;
     const uint16_t* xcol = p.x + (size_t)n * p.K * p.hw + pp;
+    Piece zero;
+    __builtin_memset(&zero, 0, sizeof(zero));
     for (int k0 = 0; k0 < p.K; k0 += 128) {
-      uint4 v[4];
+      Piece v[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const int k = min(k0 + r0 + 32 * u, p.K - 1);
-        v[u] = *reinterpret_cast<const uint4*>(xcol + (size_t)k * p.hw);
+        v[u] = *reinterpret_cast<const Piece*>(xcol + (size_t)k * p.hw);
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const int k = k0 + r0 + 32 * u;
-        if (k < p.K) *reinterpret_cast<uint4*>(tile_bytes + (size_t)k * kTwRowBytes + 16 * c8) = live ? v[u] : make_uint4(0, 0, 0, 0);
+        if (k < p.K) *reinterpret_cast<Piece*>(tile_bytes + (size_t)k * kTwRowBytes + kPieceBytes * c8) = live ? v[u] : zero;
       }
     }
     // row K is all zero: the target of list padding entries
-    if (tid < kTwRowBytes / 16) *reinterpret_cast<uint4*>(tile_bytes + (size_t)p.K * kTwRowBytes + 16 * tid) = make_uint4(0, 0, 0, 0);
+    if (tid < 32) *reinterpret_cast<Piece*>(tile_bytes + (size_t)p.K * kTwRowBytes + kPieceBytes * tid) = zero;
   }
   __syncthreads();
 
   const int half = lane >> 5;
-  const uint32_t lane16 = 16u * (uint32_t)(lane & 31);
-  const uint32_t gpos = tile0 + 8u * (uint32_t)(lane & 31);
+  const uint32_t lane16 = (uint32_t)kPieceBytes * (uint32_t)(lane & 31);
+  const uint32_t gpos = tile0 + (uint32_t)PPL * (uint32_t)(lane & 31);
   const bool store_on = gpos < p.P;
   const uint32_t on = store_on ? gpos / (uint32_t)p.hw : 0u, opp = store_on ? gpos % (uint32_t)p.hw : 0u;
   uint16_t* obase = p.out + (size_t)on * p.M * p.hw + opp;
@@ -440,15 +457,15 @@ __device__ __forceinline__ void HalfWalkOneTile(const HalfTileWalkParams& p, cha
     const uint32_t entries = (uint32_t)__builtin_amdgcn_readfirstlane((int)hdr.y);
     // (bit casts take scalars: applied to an element of a vector they read its first element)
     const uint32_t bias0 = hdr.z, bias1 = hdr.w;
-    h2 acc[NR][4];
+    h2 acc[NR][NW];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
+    for (int q = 0; q < NW; ++q) {
       acc[0][q] = __builtin_bit_cast(h2, bias0);
       if (NR == 2) acc[NR - 1][q] = __builtin_bit_cast(h2, bias1);
     }
-    auto entry = [&](const u4w& x, uint32_t w0, uint32_t w1) {
+    auto entry = [&](const Piece& x, uint32_t w0, uint32_t w1) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
+      for (int q = 0; q < NW; ++q) {
         const uint32_t xq = x[q];
         const h2 x2 = __builtin_bit_cast(h2, xq);
         acc[0][q] = __builtin_elementwise_fma(x2, __builtin_bit_cast(h2, w0), acc[0][q]);
@@ -469,9 +486,9 @@ __device__ __forceinline__ void HalfWalkOneTile(const HalfTileWalkParams& p, cha
       const u4w off = *reinterpret_cast<const u4w*>(r);
       uint32_t w[4 * NR];
       weights(r, w);
-      u4w x[4];
+      Piece x[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) x[e] = *reinterpret_cast<const u4w*>(tile_bytes + (off[e] + lane16));
+      for (int e = 0; e < 4; ++e) x[e] = *reinterpret_cast<const Piece*>(tile_bytes + (off[e] + lane16));
 #pragma unroll
       for (int e = 0; e < 4; ++e) entry(x[e], w[e * NR], w[e * NR + NR - 1]);
     }
@@ -480,18 +497,18 @@ __device__ __forceinline__ void HalfWalkOneTile(const HalfTileWalkParams& p, cha
       const u4w off = *reinterpret_cast<const u4w*>(r);
       uint32_t w[4 * NR];
       weights(r, w);
-      entry(*reinterpret_cast<const u4w*>(tile_bytes + (off[0] + lane16)), w[0], w[NR - 1]);
-      if (rem > 1) entry(*reinterpret_cast<const u4w*>(tile_bytes + (off[1] + lane16)), w[NR], w[NR + NR - 1]);
-      if (rem > 2) entry(*reinterpret_cast<const u4w*>(tile_bytes + (off[2] + lane16)), w[2 * NR], w[2 * NR + NR - 1]);
+      entry(*reinterpret_cast<const Piece*>(tile_bytes + (off[0] + lane16)), w[0], w[NR - 1]);
+      if (rem > 1) entry(*reinterpret_cast<const Piece*>(tile_bytes + (off[1] + lane16)), w[NR], w[NR + NR - 1]);
+      if (rem > 2) entry(*reinterpret_cast<const Piece*>(tile_bytes + (off[2] + lane16)), w[2 * NR], w[2 * NR + NR - 1]);
     }
     if (store_on) {
 #pragma unroll
       for (int rr = 0; rr < NR; ++rr) {
         if (rr < nrows) {
-          u4w o;
+          Piece o;
 #pragma unroll
-          for (int q = 0; q < 4; ++q) o[q] = __builtin_bit_cast(uint32_t, ActivateH<ACT>(acc[rr][q], p.act));
-          __builtin_nontemporal_store(o, reinterpret_cast<u4w*>(obase + (size_t)(row0 + rr) * p.hw));
+          for (int q = 0; q < NW; ++q) o[q] = __builtin_bit_cast(uint32_t, ActivateH<ACT>(acc[rr][q], p.act));
+          __builtin_nontemporal_store(o, reinterpret_cast<Piece*>(obase + (size_t)(row0 + rr) * p.hw));
         }
       }
     }
@@ -501,48 +518,48 @@ __device__ __forceinline__ void HalfWalkOneTile(const HalfTileWalkParams& p, cha
 // Workgroup id -> tiles, as in the fp32 tile walk: each XCD (linear id mod 8) owns a contiguous range of tiles;
 // its first workgroups take one tile each (main part), with a spare part the workgroups behind them share the
 // range's tiles among themselves, with equal parts `parts` workgroups share every tile.
-template <int NR, int ACT>
+template <int NR, int PPL, int ACT>
 __device__ __forceinline__ void HalfTileWalkBody(const HalfTileWalkParams& p, char* tile) {
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int first = (xcd * p.tiles) >> 3, last = ((xcd + 1) * p.tiles) >> 3;
   const int count = last - first;
   if (p.split == 2) {
     const int part = count > 0 ? slot / count : p.parts;
-    if (part < p.parts) HalfWalkOneTile<NR, ACT>(p, tile, first + (slot - part * count), part);
+    if (part < p.parts) HalfWalkOneTile<NR, PPL, ACT>(p, tile, first + (slot - part * count), part);
     return;
   }
   if (slot < count) {
-    HalfWalkOneTile<NR, ACT>(p, tile, first + slot, 0);
+    HalfWalkOneTile<NR, PPL, ACT>(p, tile, first + slot, 0);
     return;
   }
   if (p.split == 0) return;
   const int n_spare = (int)(gridDim.x >> 3) - count;
   for (int t = first + (slot - count); t < last; t += n_spare) {
-    HalfWalkOneTile<NR, ACT>(p, tile, t, 1);
+    HalfWalkOneTile<NR, PPL, ACT>(p, tile, t, 1);
     __syncthreads();  // every wavefront has left the tile before the next one is staged
   }
 }
 
-template <int NR>
+template <int NR, int PPL>
 __global__ void __launch_bounds__(64 * kTileWalkWaves) HalfTileWalkKernel(PL_HEAD_PARAMS, const HalfTileWalkParams block) {
   const HalfTileWalkParams p = WithHead(block, PL_HEAD_ARGS);
   extern __shared__ uint32_t tile32[];
   char* tile = reinterpret_cast<char*>(tile32);
   switch (p.act.type) {
     case 1:
-      HalfTileWalkBody<NR, 1>(p, tile);
+      HalfTileWalkBody<NR, PPL, 1>(p, tile);
       break;
     case 2:
-      HalfTileWalkBody<NR, 2>(p, tile);
+      HalfTileWalkBody<NR, PPL, 2>(p, tile);
       break;
     case 4:
-      HalfTileWalkBody<NR, 4>(p, tile);
+      HalfTileWalkBody<NR, PPL, 4>(p, tile);
       break;
     case 10:
-      HalfTileWalkBody<NR, 10>(p, tile);
+      HalfTileWalkBody<NR, PPL, 10>(p, tile);
       break;
     default:
-      HalfTileWalkBody<NR, 0>(p, tile);
+      HalfTileWalkBody<NR, PPL, 0>(p, tile);
       break;
   }
 }
@@ -600,14 +617,16 @@ hipError_t LaunchHalfChunkWalk(int nrows, const HalfChunkWalkParams& p, hipStrea
   return nrows == 2 ? HalfChunkLaunch<2, 4>(p, stream) : HalfChunkLaunch<1, 4>(p, stream);
 }
 
-// Needs hw % 8 == 0 and 16-byte aligned x / out (a lane's eight positions are one 16-byte piece of one image).
-hipError_t LaunchHalfTileWalk(int nrows, const HalfTileWalkParams& p, hipStream_t stream) {
+// A lane's positions are one piece of one image: tile 256 needs hw % 8 == 0 and 16-byte aligned x / out, tile 128
+// hw % 4 == 0 and 8-byte alignment.
+hipError_t LaunchHalfTileWalk(int nrows, int tile, const HalfTileWalkParams& p, hipStream_t stream) {
   if (p.P == 0 || p.n_groups == 0) return hipSuccess;
-  if (p.hw % 8 != 0) return hipErrorInvalidValue;
-  const size_t lds = TileWalkLdsBytes(p.K);
+  if (tile != kHalfTileWalkTile && tile != kHalfTileWalkNarrowTile) return hipErrorInvalidValue;
+  if (p.hw % (tile / 32) != 0) return hipErrorInvalidValue;
+  const size_t lds = TileWalkLdsBytes(p.K, tile * 2);
   if (lds > (size_t)kMaxLdsBytes) return hipErrorInvalidValue;
   HalfTileWalkParams q = p;
-  q.tiles = (int)((p.P + kTwTile - 1) / kTwTile);
+  q.tiles = (int)((p.P + (uint32_t)tile - 1) / (uint32_t)tile);
   uint32_t slots = ((uint32_t)q.tiles + 7) / 8;  // workgroups per XCD
   if (q.split == 2) {
     if (q.parts < 2 || (int64_t)q.parts * slots > q.split_slots) return hipErrorInvalidValue;
@@ -617,8 +636,12 @@ hipError_t LaunchHalfTileWalk(int nrows, const HalfTileWalkParams& p, hipStream_
     slots = (uint32_t)q.split_slots;
   }
   dim3 grid(8u * slots), block(64 * kTwWaves);
-  if (nrows == 2) return LaunchWithHead(HalfTileWalkKernel<2>, grid, block, lds, stream, q);
-  return LaunchWithHead(HalfTileWalkKernel<1>, grid, block, lds, stream, q);
+  if (tile == kHalfTileWalkTile) {
+    if (nrows == 2) return LaunchWithHead(HalfTileWalkKernel<2, 8>, grid, block, lds, stream, q);
+    return LaunchWithHead(HalfTileWalkKernel<1, 8>, grid, block, lds, stream, q);
+  }
+  if (nrows == 2) return LaunchWithHead(HalfTileWalkKernel<2, 4>, grid, block, lds, stream, q);
+  return LaunchWithHead(HalfTileWalkKernel<1, 4>, grid, block, lds, stream, q);
 }
 
 }  // namespace pl

@@ -126,6 +126,19 @@ pl::DevActH ToDevActH(const pl_activation& a) {
 
 }  // namespace
 
+// List streams of a tile walk (fp32, or half precision with a given number of bytes per channel row of the tile).
+struct TileWalkStreams {
+  DevBuf stream, first, desc;
+  int built = 0;  // uploaded
+  int row_bytes = 0;  // bytes per channel row of the LDS tile the byte offsets in the records are made for
+  // host copy of the streams and, per header record, (word index of its bias, first row | rows << 24):
+  // the headers carry the bias, so a new bias is patched in here and the streams are uploaded again
+  std::vector<uint32_t> host_stream;
+  std::vector<std::pair<uint32_t, uint32_t>> bias_slots;
+  int64_t stream_work = 0;  // work units (entry batches + 2 per row group) of the fullest of the sixteen unsplit streams
+  size_t DeviceBytes() const { return stream.bytes + first.bytes + desc.bytes; }
+};
+
 struct pl_sparse_conv_handle {
   int device = 0;
   int kind = PL_KIND_FP32;
@@ -144,14 +157,10 @@ struct pl_sparse_conv_handle {
   // fp32 row walk over channel chunks (built beside the plain form)
   DevBuf cw_desc, cw_idx, cw_wts;
   int cw_chunks = 0, cw_slices = 0;
-  // fp32 tile walk (whole tile and lists in LDS)
-  DevBuf tw_stream, tw_first, tw_desc;
-  int tw_built = 0;  // list streams of the tile walk uploaded
-  // host copy of the streams and, per header record, (word index of its bias, first row | rows << 24):
-  // the headers carry the bias, so a new bias is patched in here and the streams are uploaded again
-  std::vector<uint32_t> tw_host_stream;
-  std::vector<std::pair<uint32_t, uint32_t>> tw_bias_slots;
-  int64_t tw_stream_work = 0;  // work units (entry batches + 2 per row group) of the fullest of the sixteen unsplit streams
+  // tile walk (whole tile and lists in LDS): fp32 with 128 positions per tile, half precision with 256; tw_narrow:
+  // half precision with 128 positions per tile (256-byte channel rows), for more channels and for maps whose
+  // size is a multiple of 4 but not of 8
+  TileWalkStreams tw, tw_narrow;
   int walk_split = -1;          // sixteenths of the row groups' work dealt to the CUs without a tile: -1 by rule, 0 never, 1 .. 8 forced
   int walk_tiled = 1;            // 0 never, 1 when the problem suits it, 2 whenever the shape allows
   bool walk_pairs = true;        // the tile walk's streams hold pairs of row groups (two per wavefront instruction)
@@ -190,7 +199,7 @@ struct pl_sparse_conv_handle {
   int padded_rows = 0;
 
   int64_t DeviceBytes() const {
-    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + cw_desc.bytes + cw_idx.bytes + cw_wts.bytes + hw_kidx.bytes + hw_wts.bytes + hw_bias.bytes + wblocks.bytes + kmask.bytes + wtiles.bytes + wtiles_rg.bytes + wtiles_tr.bytes + wtiles_rows.bytes + tw_stream.bytes + tw_first.bytes + tw_desc.bytes + scale.bytes + bias.bytes);
+    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + cw_desc.bytes + cw_idx.bytes + cw_wts.bytes + hw_kidx.bytes + hw_wts.bytes + hw_bias.bytes + wblocks.bytes + kmask.bytes + wtiles.bytes + wtiles_rg.bytes + wtiles_tr.bytes + wtiles_rows.bytes + tw.DeviceBytes() + tw_narrow.DeviceBytes() + scale.bytes + bias.bytes);
   }
 };
 
@@ -390,9 +399,10 @@ uint32_t DoubledHalf(uint32_t float_bits) {
   return b | (b << 16);
 }
 
-int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_handle* h, bool half = false) {
-  h->tw_built = 0;
-  if (pl::TileWalkLdsBytes(L.ic) > static_cast<size_t>(pl::kMaxLdsBytes)) return PL_OK;  // too many channels for one tile: other walks
+int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_handle* h, TileWalkStreams* tw, bool half = false, int row_bytes = pl::kTileWalkTile * 4) {
+  tw->built = 0;
+  tw->row_bytes = row_bytes;
+  if (pl::TileWalkLdsBytes(L.ic, row_bytes) > static_cast<size_t>(pl::kMaxLdsBytes)) return PL_OK;  // too many channels for one tile: other walks
   const int nr = L.semi ? 2 : 1;
   const int streams = pl::kTileWalkWaves;
   const int n_groups = static_cast<int>(L.groups.size());
@@ -425,10 +435,10 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
   const uint32_t unit_words = pairs ? 2 * rec_words : rec_words;  // a double record per step of a pair
   const uint32_t chunk_words = pl::kTileWalkChunkBytes / 4;
   const uint32_t recs_per_chunk = chunk_words / unit_words;
-  const uint32_t zero_row = static_cast<uint32_t>(L.ic) * pl::kTileWalkTile * 4;
-  std::vector<uint32_t>& stream = h->tw_host_stream;
+  const uint32_t zero_row = static_cast<uint32_t>(L.ic) * static_cast<uint32_t>(row_bytes);
+  std::vector<uint32_t>& stream = tw->host_stream;
   stream.clear();
-  h->tw_bias_slots.clear();
+  tw->bias_slots.clear();
   std::vector<uint32_t> first, counts;
   // Streams for the given units (largest first): each unit goes to the stream with the least work so far.
   // Sixteen streams make one part.  Returns the work of the fullest stream.
@@ -478,14 +488,14 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
         }
         put(rec);
         for (int side = 0; side < sides; ++side)
-          if (side_groups[side] >= 0) h->tw_bias_slots.emplace_back(static_cast<uint32_t>(stream.size() - unit_words + side * rec_words + 2), rec[side * rec_words]);
+          if (side_groups[side] >= 0) tw->bias_slots.emplace_back(static_cast<uint32_t>(stream.size() - unit_words + side * rec_words + 2), rec[side * rec_words]);
         for (uint32_t e0 = 0; e0 < un.count; e0 += 4) {
           for (int side = 0; side < sides; ++side) {
             uint32_t* r = rec + side * rec_words;
             const pl::RowGroup* rg = side_groups[side] >= 0 ? &L.groups[side_groups[side]] : nullptr;
             for (uint32_t e = 0; e < 4; ++e) {
               const bool real = rg != nullptr && e0 + e < rg->count;
-              r[e] = real ? L.ic_index[rg->first + e0 + e] * pl::kTileWalkTile * 4 : zero_row;
+              r[e] = real ? L.ic_index[rg->first + e0 + e] * static_cast<uint32_t>(row_bytes) : zero_row;
               r[4 + e * nr] = real ? word(L.w0[rg->first + e0 + e]) : 0u;
               if (nr == 2) r[4 + e * nr + 1] = real ? word(L.w1[rg->first + e0 + e]) : 0u;
             }
@@ -501,7 +511,7 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
   // Set 0: all units in one part.  Sets 1 .. kTileWalkSplits: a spare part with about s / 16 of the work
   // (a mix of sizes: going through the units from the largest, a unit joins the spare part whenever that
   // keeps the part at or below its share), the rest in the main part.
-  h->tw_stream_work = emit(unit_order, streams);
+  tw->stream_work = emit(unit_order, streams);
   for (int s16 = 1; s16 <= kTileWalkSplits; ++s16) {
     std::vector<int> main_part, spare_part;
     int64_t all_w = 0, spare_w = 0;
@@ -521,11 +531,11 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
   // Equal parts for problems with at most half as many tiles as CUs: n workgroups per tile, each with a
   // sixteenth-of-n share of the units.
   for (int n : kTileWalkEqualParts) emit(unit_order, streams * n);
-  hipError_t e = h->tw_stream.Upload(stream.data(), stream.size() * sizeof(uint32_t));
-  if (e == hipSuccess) e = h->tw_first.Upload(first.data(), first.size() * sizeof(uint32_t));
-  if (e == hipSuccess) e = h->tw_desc.Upload(counts.data(), counts.size() * sizeof(uint32_t));
+  hipError_t e = tw->stream.Upload(stream.data(), stream.size() * sizeof(uint32_t));
+  if (e == hipSuccess) e = tw->first.Upload(first.data(), first.size() * sizeof(uint32_t));
+  if (e == hipSuccess) e = tw->desc.Upload(counts.data(), counts.size() * sizeof(uint32_t));
   if (e != hipSuccess) return FailHip(e, "uploading the tile-walk list streams");
-  h->tw_built = 1;
+  tw->built = 1;
   return PL_OK;
 }
 
@@ -868,7 +878,8 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
     h->algo = PL_ALGO_ROW_WALK;
     int hrc = BuildHalfWalk(L, h);
     if (hrc == PL_OK) hrc = BuildChunkWalk(L, h, true);
-    if (hrc == PL_OK) hrc = BuildTileWalk(L, desc->bias, h, true);
+    if (hrc == PL_OK) hrc = BuildTileWalk(L, desc->bias, h, &h->tw, true);
+    if (hrc == PL_OK) hrc = BuildTileWalk(L, desc->bias, h, &h->tw_narrow, true, pl::kHalfTileWalkNarrowTile * 2);
     if (hrc == PL_OK) hrc = UploadHalfBias(h, desc->bias);
     if (hrc != PL_OK) {
       delete h;
@@ -905,7 +916,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   if (rc == PL_OK && h->wtiles.ptr && pl::ImageMfmaRegroupsByTransposingReads(desc->ic, 196)) rc = BuildImageMfmaTrRegroup(L, h);
   if (rc == PL_OK && h->wtiles.ptr && pl::ImageRowsMfmaFits(desc->oc, desc->ic, 16)) rc = BuildImageRowsMfma(L, h);
   if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8) rc = BuildChunkWalk(L, h);
-  if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8 && !half) rc = BuildTileWalk(L, desc->bias, h);
+  if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8 && !half) rc = BuildTileWalk(L, desc->bias, h, &h->tw);
   if (rc == PL_OK) {
     // the MFMA epilogues always read a bias; give them zeros when the op has none
     std::vector<float> zeros;
@@ -946,7 +957,7 @@ struct TileWalkDivision {
   size_t table = 0;  // first entry of the division's stream tables
 };
 
-TileWalkDivision DivideTileWalk(const pl_sparse_conv_handle* h, int tiles) {
+TileWalkDivision DivideTileWalk(const pl_sparse_conv_handle* h, const TileWalkStreams& tw, int tiles) {
   TileWalkDivision d;
   const int cus = std::max(8, h->wg_slots_default / 2) / 8 * 8;
   int s16 = 0, equal_parts = 0;
@@ -959,7 +970,7 @@ TileWalkDivision DivideTileWalk(const pl_sparse_conv_handle* h, int tiles) {
         if (n <= room) equal_parts = n;
     } else if (spare >= 1) {
       const int r = CeilDiv(per_xcd, spare);
-      const double sw = (2000.0 + 14.0 * h->ic) / (355.0 * static_cast<double>(std::max<int64_t>(1, h->tw_stream_work)));
+      const double sw = (2000.0 + 14.0 * h->ic) / (355.0 * static_cast<double>(std::max<int64_t>(1, tw.stream_work)));
       const double f = (1.0 - (r - 1) * sw) / (r + 1);
       s16 = h->walk_split > 0 ? h->walk_split : static_cast<int>(f * 16.0 + 0.3);
       s16 = std::max(0, std::min(kTileWalkSplits, s16));
@@ -995,18 +1006,31 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipError_t e;
   const int call_algo = AlgoForCall(h, batch, im_size, aligned16);
-  if (h->half && h->tw_built != 0 && h->walk_tiled > 0 && im_size % 8 == 0 && aligned16 &&
-      (h->walk_tiled == 2 || (h->semi ? 42 : 84) * static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kHalfTileWalkTile)) >= h->wg_slots_default)) {
-    // The walk with the tile and the lists in LDS, from 7 tiles of 256 positions on (13 with row pairs, whose
-    // plain walk is twice as efficient per list entry) on 256 CUs: measured against the other half-precision
-    // walks at 1 - 784 tiles, it is 1.3 - 2.5 times as fast from there on and slower below.
-    const TileWalkDivision d = DivideTileWalk(h, CeilDiv(static_cast<int>(P), pl::kHalfTileWalkTile));
+  // Half precision: the walk with the tile and the lists in LDS, from 7 tiles on (13 with row pairs, whose plain
+  // walk is twice as efficient per list entry) on 256 CUs: measured against the other half-precision walks at
+  // 1 - 784 tiles, it is 1.3 - 2.5 times as fast from there on and slower below.  Tiles of 256 positions where
+  // the channels fit and the map size is a multiple of 8, else tiles of 128.
+  const bool aligned8 = reinterpret_cast<uintptr_t>(x_dev) % 8 == 0 && reinterpret_cast<uintptr_t>(out_dev) % 8 == 0;
+  const TileWalkStreams* half_tw = nullptr;
+  int half_tile = 0;
+  if (h->half && h->walk_tiled > 0) {
+    if (h->tw.built != 0 && im_size % 8 == 0 && aligned16) {
+      half_tw = &h->tw;
+      half_tile = pl::kHalfTileWalkTile;
+    } else if (h->tw_narrow.built != 0 && im_size % 4 == 0 && aligned8) {
+      half_tw = &h->tw_narrow;
+      half_tile = pl::kHalfTileWalkNarrowTile;
+    }
+    if (half_tw && h->walk_tiled != 2 && (h->semi ? 42 : 84) * static_cast<int64_t>(CeilDiv(static_cast<int>(P), half_tile)) < h->wg_slots_default) half_tw = nullptr;
+  }
+  if (half_tw) {
+    const TileWalkDivision d = DivideTileWalk(h, *half_tw, CeilDiv(static_cast<int>(P), half_tile));
     pl::HalfTileWalkParams p{};
     p.x = static_cast<const uint16_t*>(x_dev);
     p.out = static_cast<uint16_t*>(out_dev);
-    p.stream = h->tw_stream.ptr;
-    p.stream_first = static_cast<const uint32_t*>(h->tw_first.ptr) + d.table;
-    p.stream_groups = static_cast<const uint32_t*>(h->tw_desc.ptr) + d.table;
+    p.stream = half_tw->stream.ptr;
+    p.stream_first = static_cast<const uint32_t*>(half_tw->first.ptr) + d.table;
+    p.stream_groups = static_cast<const uint32_t*>(half_tw->desc.ptr) + d.table;
     p.split = static_cast<int16_t>(d.split);
     p.parts = static_cast<int8_t>(d.parts);
     p.split_slots = d.split_slots;
@@ -1016,7 +1040,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.hw = im_size;
     p.P = P;
     p.act = h->act_h;
-    e = pl::LaunchHalfTileWalk(h->semi ? 2 : 1, p, s);
+    e = pl::LaunchHalfTileWalk(h->semi ? 2 : 1, half_tile, p, s);
   } else if (h->half && (im_size % 4 == 0) && (reinterpret_cast<uintptr_t>(x_dev) % 8 == 0) && (reinterpret_cast<uintptr_t>(out_dev) % 8 == 0) && h->walk_chunked > 0 && h->cw_chunks > 0 &&
       (h->walk_chunked == 2 || (h->ic > 128 && static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kChunkWalkTile)) * h->cw_slices >= 256))) {
     // many channels and enough work for every CU: walk over channel chunks
@@ -1140,7 +1164,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     c.sub_tiles = h->mfma_sub_tiles;
     if (h->mfma_tile_quads > 0) c.tile_quads = h->mfma_tile_quads;
     e = pl::LaunchBlockMfma(c, p, s);
-  } else if (!h->int8 && !h->half && vec && h->tw_built != 0 && h->walk_tiled > 0 &&
+  } else if (!h->int8 && !h->half && vec && h->tw.built != 0 && h->walk_tiled > 0 &&
              (h->walk_tiled == 2 || 32 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kTileWalkTile)) >= h->wg_slots_default)) {
     // fp32 with 128-position tiles for at least a sixteenth of the CUs (the
     // row groups of a tile are shared between up to ten CUs; measured
@@ -1149,10 +1173,10 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     pl::TileWalkParams p{};
     p.x = static_cast<const float*>(x_dev);
     p.out = static_cast<float*>(out_dev);
-    p.stream = h->tw_stream.ptr;
-    const TileWalkDivision d = DivideTileWalk(h, CeilDiv(static_cast<int>(P), pl::kTileWalkTile));
-    p.stream_first = static_cast<const uint32_t*>(h->tw_first.ptr) + d.table;
-    p.stream_groups = static_cast<const uint32_t*>(h->tw_desc.ptr) + d.table;
+    p.stream = h->tw.stream.ptr;
+    const TileWalkDivision d = DivideTileWalk(h, h->tw, CeilDiv(static_cast<int>(P), pl::kTileWalkTile));
+    p.stream_first = static_cast<const uint32_t*>(h->tw.first.ptr) + d.table;
+    p.stream_groups = static_cast<const uint32_t*>(h->tw.desc.ptr) + d.table;
     p.split = static_cast<int16_t>(d.split);
     p.parts = static_cast<int8_t>(d.parts);
     p.pairs = h->walk_pairs ? 1 : 0;
@@ -1267,17 +1291,18 @@ int pl_sparse_conv_set_epilogue(pl_sparse_conv_handle* h, const float* scale, co
   if (scale && !h->int8) return Fail(PL_ERR_BAD_ARG, "floating-point kernels take no scales");
   int rc = h->half ? UploadHalfBias(h, bias) : UploadEpilogue(h, scale, bias);
   if (rc != PL_OK) return rc;
-  if (bias && h->tw_built) {
+  for (TileWalkStreams* tw : {&h->tw, &h->tw_narrow}) {
+    if (!bias || !tw->built) continue;
     // the tile walk starts its accumulators from the bias in its header records
-    for (const auto& slot : h->tw_bias_slots) {
+    for (const auto& slot : tw->bias_slots) {
       const uint32_t row0 = slot.second & 0xffffffu, nrows = slot.second >> 24;
       uint32_t b0 = 0, b1 = 0;
       std::memcpy(&b0, &bias[row0], 4);
       if (nrows == 2) std::memcpy(&b1, &bias[row0 + 1], 4);
-      h->tw_host_stream[slot.first] = h->half ? DoubledHalf(b0) : b0;
-      if (nrows == 2) h->tw_host_stream[slot.first + 1] = h->half ? DoubledHalf(b1) : b1;
+      tw->host_stream[slot.first] = h->half ? DoubledHalf(b0) : b0;
+      if (nrows == 2) tw->host_stream[slot.first + 1] = h->half ? DoubledHalf(b1) : b1;
     }
-    const hipError_t e = h->tw_stream.Upload(h->tw_host_stream.data(), h->tw_host_stream.size() * sizeof(uint32_t));
+    const hipError_t e = tw->stream.Upload(tw->host_stream.data(), tw->host_stream.size() * sizeof(uint32_t));
     if (e != hipSuccess) return FailHip(e, "uploading the tile-walk list streams");
   }
   if (act) {

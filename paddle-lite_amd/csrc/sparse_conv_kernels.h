@@ -140,7 +140,7 @@ struct TileWalkParams {
 };
 
 // LDS the kernel needs for K input channels.
-size_t TileWalkLdsBytes(int K);
+size_t TileWalkLdsBytes(int K, int row_bytes = kTileWalkTile * 4);  // row_bytes: bytes per channel row of the tile
 // Needs hw % 4 == 0 and 16-byte aligned x / out.
 hipError_t LaunchTileWalk(int nrows, const TileWalkParams& p, hipStream_t stream);
 
@@ -178,8 +178,11 @@ hipError_t LaunchHalfChunkWalk(int nrows, const HalfChunkWalkParams& p, hipStrea
 
 // Half-precision tile walk: the layout of TileWalkParams with pairs of row groups.  A tile holds 256 positions
 // (the same 512 bytes per channel row, so the byte offsets in the list streams are those of the fp32 walk), a
-// lane eight; weights and biases in the streams are binary16 values doubled into a dword (value | value << 16).
+// lane eight; or 128 positions (256 bytes per channel row, streams made for that), a lane four: twice the
+// channels fit, and a map size that is a multiple of 4 is enough.  Weights and biases in the streams are binary16
+// values doubled into a dword (value | value << 16).
 constexpr int kHalfTileWalkTile = 256;
+constexpr int kHalfTileWalkNarrowTile = 128;
 
 struct HalfTileWalkParams {
   const uint16_t* x;
@@ -201,8 +204,9 @@ struct HalfTileWalkParams {
   int split_slots;
 };
 
-// Needs hw % 8 == 0 and 16-byte aligned x / out.
-hipError_t LaunchHalfTileWalk(int nrows, const HalfTileWalkParams& p, hipStream_t stream);
+// tile: kHalfTileWalkTile (needs hw % 8 == 0 and 16-byte aligned x / out) or kHalfTileWalkNarrowTile (hw % 4 == 0,
+// 8-byte aligned); the streams must be made for that tile's channel rows.
+hipError_t LaunchHalfTileWalk(int nrows, int tile, const HalfTileWalkParams& p, hipStream_t stream);
 
 struct HalfWalkParams {
   const uint16_t* x;

@@ -252,7 +252,7 @@ __global__ void __launch_bounds__(64 * kTileWalkWaves) TileWalkKernel(PL_HEAD_PA
 
 }  // namespace
 
-size_t TileWalkLdsBytes(int K) { return (size_t)(K + 1) * kTP * 4 + (size_t)kWaves * kChunkBytes; }
+size_t TileWalkLdsBytes(int K, int row_bytes) { return (size_t)(K + 1) * (size_t)row_bytes + (size_t)kWaves * kChunkBytes; }
 
 hipError_t LaunchTileWalk(int nrows, const TileWalkParams& p, hipStream_t stream) {
   if (p.P == 0 || p.n_groups == 0) return hipSuccess;

@@ -71,11 +71,15 @@ def test_fp16_chunked_walk(shape, paired, act):
 
 
 # Half-precision walk with the whole tile (256 positions, all channels) and the list streams in LDS, two row
-# groups per wavefront instruction; forced here, the library picks it by itself from 8 tiles on.  Needs
+# groups per wavefront instruction; forced here, the library picks it by itself from 7 tiles on.  Needs
 # H*W % 8 == 0 and at most 271 channels.  (batch, ic, oc, h, w): one tile shared by ten workgroups, a channel
 # count off the staging pass of 128, an odd number of row groups (a pair without partner), a tile that spans
 # images and ends inside one, a single row group.
 TILED_SHAPES = [(2, 64, 64, 4, 4), (1, 96, 48, 8, 6), (3, 130, 67, 4, 6), (5, 70, 33, 2, 4), (2, 257, 20, 12, 12), (3, 200, 1, 8, 8), (1, 271, 96, 16, 24)]
+# Tiles of 128 positions (four per lane) serve maps whose size is a multiple of 4 only and up to 543 channels:
+# 14 x 14 and 2 x 2 maps, a tile that ends inside an image, channel counts above the wide tile's limit on maps of
+# both kinds, the largest channel count.
+TILED_SHAPES += [(3, 64, 48, 14, 14), (7, 40, 33, 2, 2), (2, 257, 20, 6, 6), (1, 300, 150, 16, 16), (2, 512, 64, 14, 14), (1, 543, 40, 4, 4)]
 
 
 @pytest.mark.parametrize("act", ["none", "relu", "relu6", "leaky", "hswish"])
@@ -90,23 +94,26 @@ def test_fp16_tile_walk(shape, paired, act):
 
 
 @pytest.mark.parametrize("batch", [3, 24, 40, 64, 65])
+@pytest.mark.parametrize("ic,size", [(256, 28), (512, 14)], ids=["wide_tiles", "narrow_tiles"])
 @pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
-def test_fp16_tile_walk_divisions(batch, paired):
+def test_fp16_tile_walk_divisions(batch, paired, ic, size):
     """Tiles shared by several workgroups in equal parts, main and spare parts, one tile per workgroup and more
     tiles than CUs: the bits of the plain half-precision walk (the oracle's, by the tests above) every time."""
-    case = half_case(batch, 256, 512, 28, 28, 0.85, paired, ACTS["relu"], seed=batch)
+    batch = batch if size == 28 else 4 * batch
+    case = half_case(batch, ic, 512, size, size, 0.85, paired, ACTS["relu"], seed=batch)
     tiled = run_hip(case, capi.ALGO_AUTO, force_semi=paired, tuning=capi.tuning(walk_tiled=capi.TUNE_ALWAYS))
     plain = run_hip(case, capi.ALGO_AUTO, force_semi=paired, tuning=capi.tuning(walk_tiled=capi.TUNE_NEVER, walk_chunked=capi.TUNE_NEVER))
     assert np.array_equal(tiled.view(np.uint16), plain.view(np.uint16))
 
 
+@pytest.mark.parametrize("size", [16, 14], ids=["wide_tiles", "narrow_tiles"])
 @pytest.mark.parametrize("had_bias", [True, False], ids=["bias", "no_bias"])
-def test_fp16_tile_walk_takes_a_new_bias(had_bias):
+def test_fp16_tile_walk_takes_a_new_bias(had_bias, size):
     """set_epilogue rewrites the biases in the list streams (the accumulators start from them), also in a handle
     that was prepared without one."""
     from helpers import make_kernel
 
-    case = half_case(12, 128, 96, 16, 16, 0.8, False, ACTS["relu"], seed=9)
+    case = half_case(12, 128, 96, size, size, 0.8, False, ACTS["relu"], seed=9)
     if not had_bias:
         case.bias = None
     kernel, _ = make_kernel(case, tuning=capi.tuning(walk_tiled=capi.TUNE_ALWAYS))
