@@ -158,8 +158,9 @@ struct pl_sparse_conv_handle {
   DevBuf cw_desc, cw_idx, cw_wts;
   int cw_chunks = 0, cw_slices = 0;
   // tile walk (whole tile and lists in LDS): fp32 with 128 positions per tile, half precision with 256; tw_narrow:
-  // half precision with 128 positions per tile (256-byte channel rows), for more channels and for maps whose
-  // size is a multiple of 4 but not of 8
+  // 256-byte channel rows - half precision with 128 positions per tile, for more channels and for maps whose
+  // size is a multiple of 4 but not of 8; fp32 with 64 positions per tile (pairs only), built when the channels do
+  // not fit the wide tile
   TileWalkStreams tw, tw_narrow;
   int walk_split = -1;          // sixteenths of the row groups' work dealt to the CUs without a tile: -1 by rule, 0 never, 1 .. 8 forced
   int walk_tiled = 1;            // 0 never, 1 when the problem suits it, 2 whenever the shape allows
@@ -917,6 +918,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   if (rc == PL_OK && h->wtiles.ptr && pl::ImageRowsMfmaFits(desc->oc, desc->ic, 16)) rc = BuildImageRowsMfma(L, h);
   if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8) rc = BuildChunkWalk(L, h);
   if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8 && !half) rc = BuildTileWalk(L, desc->bias, h, &h->tw);
+  if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8 && !half && !h->tw.built && h->walk_pairs) rc = BuildTileWalk(L, desc->bias, h, &h->tw_narrow, false, pl::kTileWalkNarrowTile * 4);
   if (rc == PL_OK) {
     // the MFMA epilogues always read a bias; give them zeros when the op has none
     std::vector<float> zeros;
@@ -1164,22 +1166,25 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     c.sub_tiles = h->mfma_sub_tiles;
     if (h->mfma_tile_quads > 0) c.tile_quads = h->mfma_tile_quads;
     e = pl::LaunchBlockMfma(c, p, s);
-  } else if (!h->int8 && !h->half && vec && h->tw.built != 0 && h->walk_tiled > 0 &&
-             (h->walk_tiled == 2 || 32 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kTileWalkTile)) >= h->wg_slots_default)) {
-    // fp32 with 128-position tiles for at least a sixteenth of the CUs (the
+  } else if (!h->int8 && !h->half && vec && (h->tw.built != 0 || h->tw_narrow.built != 0) && h->walk_tiled > 0 &&
+             (h->walk_tiled == 2 || 32 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), h->tw.built ? pl::kTileWalkTile : pl::kTileWalkNarrowTile)) >= h->wg_slots_default)) {
+    // fp32 with tiles for at least a sixteenth of the CUs (the
     // row groups of a tile are shared between up to ten CUs; measured
     // crossover against the other walks between 13 and 25 tiles on 256 CUs):
-    // the walk with the tile and the lists in LDS
+    // the walk with the tile and the lists in LDS - tiles of 128 positions, of 64 where
+    // only those fit LDS with all channels
+    const TileWalkStreams& tw = h->tw.built ? h->tw : h->tw_narrow;
+    const int tile = h->tw.built ? pl::kTileWalkTile : pl::kTileWalkNarrowTile;
     pl::TileWalkParams p{};
     p.x = static_cast<const float*>(x_dev);
     p.out = static_cast<float*>(out_dev);
-    p.stream = h->tw.stream.ptr;
-    const TileWalkDivision d = DivideTileWalk(h, h->tw, CeilDiv(static_cast<int>(P), pl::kTileWalkTile));
-    p.stream_first = static_cast<const uint32_t*>(h->tw.first.ptr) + d.table;
-    p.stream_groups = static_cast<const uint32_t*>(h->tw.desc.ptr) + d.table;
+    p.stream = tw.stream.ptr;
+    const TileWalkDivision d = DivideTileWalk(h, tw, CeilDiv(static_cast<int>(P), tile));
+    p.stream_first = static_cast<const uint32_t*>(tw.first.ptr) + d.table;
+    p.stream_groups = static_cast<const uint32_t*>(tw.desc.ptr) + d.table;
     p.split = static_cast<int16_t>(d.split);
     p.parts = static_cast<int8_t>(d.parts);
-    p.pairs = h->walk_pairs ? 1 : 0;
+    p.pairs = h->tw.built ? (h->walk_pairs ? 1 : 0) : 2;
     p.split_slots = d.split_slots;
     p.n_groups = h->n_groups;
     p.M = h->oc;

@@ -101,6 +101,7 @@ hipError_t LaunchChunkWalk(int nrows, const ChunkWalkParams& p, hipStream_t stre
 // kTileWalkTile positions with all input channels; wavefront s walks the row
 // groups of list stream s.
 constexpr int kTileWalkTile = 128;
+constexpr int kTileWalkNarrowTile = 64;  // for channel counts whose 128-position tile does not fit LDS (pairs only)
 constexpr int kTileWalkWaves = 16;
 constexpr int kTileWalkChunkBytes = 1536;  // piece of a list stream held in LDS per wavefront
 
@@ -129,6 +130,7 @@ struct TileWalkParams {
   int8_t parts;
   // 1: the streams hold pairs of row groups, padded to one length, as double records (first group's record, second
   // group's record): lanes 0 - 31 walk the first group, lanes 32 - 63 the second, four positions per lane
+  // 2: pairs on tiles of kTileWalkNarrowTile positions, two per lane (streams made for 256-byte channel rows)
   int8_t pairs;
   // The first 56 bytes (kernarg_head.h) end behind act.type: what selects the tile, picks the activation and
   // addresses the first loads.

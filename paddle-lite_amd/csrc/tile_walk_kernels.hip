@@ -22,6 +22,8 @@
 // groups side by side in the stream.  The activations are then read 16 bytes per lane (LDS delivers those at
 // twice the rate of 8-byte reads) and every LDS instruction, address add and loop step serves two row groups;
 // the shorter group of a pair is padded with entries of weight zero at the tile's zero row.
+// With more channels than a tile of 128 positions holds in LDS, the pairs walk tiles of 64 positions, two per
+// lane (NARROW; channel rows of 256 bytes, list streams made for those).
 // With fewer tiles than CUs, the row groups can be dealt into a main and a
 // spare part (two sets of sixteen streams): the tile's own workgroup walks the
 // main part, and the workgroups on the CUs that have no tile of their own walk
@@ -63,17 +65,18 @@ static_assert(offsetof(TileWalkParams, act) + sizeof(int) <= kHeadWords * 8, "ac
 using epilogue::ActivateT;
 using epilogue::DispatchAct;
 
-constexpr int kTP = kTileWalkTile;      // positions per workgroup
 constexpr int kWaves = kTileWalkWaves;  // wavefronts per workgroup = list streams
 constexpr int kChunkBytes = kTileWalkChunkBytes;
 
 // One tile: stage it, then walk the streams of one part (0 main, 1 spare).
-template <int NR, int ACT, bool PAIR>
+template <int NR, int ACT, bool PAIR, bool NARROW>
 __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile, int tile_id, int part) {
+  static_assert(PAIR || !NARROW, "narrow tiles are walked in pairs");
   constexpr int kRecBytes = NR == 2 ? 48 : 32;  // four byte offsets, then 4 * NR weights
   constexpr int kStepBytes = PAIR ? 2 * kRecBytes : kRecBytes;  // what one step of the walk reads: one record per row group
   constexpr int kRecs = kChunkBytes / kStepBytes;
-  constexpr int PPL = PAIR ? 4 : 2;  // positions per lane
+  constexpr int PPL = PAIR && !NARROW ? 4 : 2;  // positions per lane
+  constexpr int kTP = NARROW ? kTileWalkNarrowTile : kTileWalkTile;  // positions per workgroup
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int sidx = part * kWaves + wave;
@@ -87,24 +90,25 @@ __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile
   u4 pa = *reinterpret_cast<const u4*>(sp + 16 * lane);
   u2 pb = *reinterpret_cast<const u2*>(sp + 1024 + 8 * lane);
 
-  // staging: 32 threads per channel row (four positions each), 32 rows per pass
+  // staging: kTP / 4 threads per channel row (four positions each), 32 or 64 rows per pass
   {
-    const int c4 = tid & 31, r0 = tid >> 5;
+    constexpr int kRowThreads = kTP / 4, kPassRows = 64 * kWaves / kRowThreads;
+    const int c4 = tid & (kRowThreads - 1), r0 = tid / kRowThreads;
     const uint32_t gpos = tile0 + 4u * (uint32_t)c4;
     const bool live = gpos < p.P;
     const uint32_t n = live ? gpos / (uint32_t)p.hw : 0u;
     const uint32_t pp = live ? gpos % (uint32_t)p.hw : 0u;
     const float* xcol = p.x + (size_t)n * p.K * p.hw + pp;
-    for (int k0 = 0; k0 < p.K; k0 += 128) {
+    for (int k0 = 0; k0 < p.K; k0 += 4 * kPassRows) {
       uint4 v[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int k = min(k0 + r0 + 32 * u, p.K - 1);
+        const int k = min(k0 + r0 + kPassRows * u, p.K - 1);
         v[u] = *reinterpret_cast<const uint4*>(xcol + (size_t)k * p.hw);
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int k = k0 + r0 + 32 * u;
+        const int k = k0 + r0 + kPassRows * u;
         if (k < p.K) *reinterpret_cast<uint4*>(tile_bytes + ((size_t)k * kTP + 4 * c4) * 4) = live ? v[u] : make_uint4(0, 0, 0, 0);
       }
     }
@@ -115,8 +119,8 @@ __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile
 
   // pairs: the half of the wavefront a lane belongs to picks the record, its place in the half the positions
   const int half = PAIR ? lane >> 5 : 0;
-  const uint32_t lane8 = PAIR ? 16u * (uint32_t)(lane & 31) : 8u * (uint32_t)lane;
-  const uint32_t gpos = tile0 + (PAIR ? 4u * (uint32_t)(lane & 31) : 2u * (uint32_t)lane);
+  const uint32_t lane8 = PAIR ? 4u * PPL * (uint32_t)(lane & 31) : 8u * (uint32_t)lane;
+  const uint32_t gpos = tile0 + (PAIR ? (uint32_t)PPL * (uint32_t)(lane & 31) : 2u * (uint32_t)lane);
   const bool store_on = gpos < p.P;
   const uint32_t on = store_on ? gpos / (uint32_t)p.hw : 0u, opp = store_on ? gpos % (uint32_t)p.hw : 0u;
   float* obase = p.out + (size_t)on * p.M * p.hw + opp;
@@ -213,7 +217,7 @@ __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile
 // Workgroup id -> tiles: each XCD (linear id mod 8) owns a contiguous range of
 // tiles.  Its first workgroups take one tile each (main part); with a spare
 // part, the workgroups behind them share the range's tiles among themselves.
-template <int NR, int ACT, bool PAIR>
+template <int NR, int ACT, bool PAIR, bool NARROW>
 __device__ __forceinline__ void TileWalkBody(const TileWalkParams& p, float* tile) {
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int first = (xcd * p.tiles) >> 3, last = ((xcd + 1) * p.tiles) >> 3;
@@ -221,17 +225,17 @@ __device__ __forceinline__ void TileWalkBody(const TileWalkParams& p, float* til
   if (p.split == 2) {
     // equal parts: part = slot / count of tile slot % count
     const int part = count > 0 ? slot / count : p.parts;
-    if (part < p.parts) WalkOneTile<NR, ACT, PAIR>(p, tile, first + (slot - part * count), part);
+    if (part < p.parts) WalkOneTile<NR, ACT, PAIR, NARROW>(p, tile, first + (slot - part * count), part);
     return;
   }
   if (slot < count) {
-    WalkOneTile<NR, ACT, PAIR>(p, tile, first + slot, 0);
+    WalkOneTile<NR, ACT, PAIR, NARROW>(p, tile, first + slot, 0);
     return;
   }
   if (p.split == 0) return;
   const int n_spare = (int)(gridDim.x >> 3) - count;
   for (int t = first + (slot - count); t < last; t += n_spare) {
-    WalkOneTile<NR, ACT, PAIR>(p, tile, t, 1);
+    WalkOneTile<NR, ACT, PAIR, NARROW>(p, tile, t, 1);
     __syncthreads();  // every wavefront has left the tile before the next one is staged
   }
 }
@@ -242,10 +246,12 @@ __global__ void __launch_bounds__(64 * kTileWalkWaves) TileWalkKernel(PL_HEAD_PA
   extern __shared__ float tile_lds[];
   DispatchAct(p.act.type, [&](auto act_c) {
     constexpr int ACT = decltype(act_c)::value;
-    if (p.pairs) {
-      TileWalkBody<NR, ACT, true>(p, tile_lds);
+    if (p.pairs == 2) {
+      TileWalkBody<NR, ACT, true, true>(p, tile_lds);
+    } else if (p.pairs) {
+      TileWalkBody<NR, ACT, true, false>(p, tile_lds);
     } else {
-      TileWalkBody<NR, ACT, false>(p, tile_lds);
+      TileWalkBody<NR, ACT, false, false>(p, tile_lds);
     }
   });
 }
@@ -257,10 +263,11 @@ size_t TileWalkLdsBytes(int K, int row_bytes) { return (size_t)(K + 1) * (size_t
 hipError_t LaunchTileWalk(int nrows, const TileWalkParams& p, hipStream_t stream) {
   if (p.P == 0 || p.n_groups == 0) return hipSuccess;
   if (p.hw % 4 != 0) return hipErrorInvalidValue;
-  const size_t lds = TileWalkLdsBytes(p.K);
+  const int tile = p.pairs == 2 ? kTileWalkNarrowTile : kTileWalkTile;
+  const size_t lds = TileWalkLdsBytes(p.K, tile * 4);
   if (lds > (size_t)kMaxLdsBytes) return hipErrorInvalidValue;
   TileWalkParams q = p;
-  q.tiles = (int)((p.P + kTP - 1) / kTP);
+  q.tiles = (int)((p.P + (uint32_t)tile - 1) / (uint32_t)tile);
   uint32_t slots = ((uint32_t)q.tiles + 7) / 8;  // workgroups per XCD
   if (q.split == 2) {
     if (q.parts < 2 || (int64_t)q.parts * slots > q.split_slots) return hipErrorInvalidValue;

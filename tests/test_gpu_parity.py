@@ -176,11 +176,14 @@ def test_fp32_chunked_walk(shape, paired, act):
 
 # fp32 walk with the whole tile and the index lists in LDS (128 positions and
 # sixteen list streams per workgroup); forced here, the library picks it by
-# itself for large problems.  Needs H*W % 4 == 0 and at most 264 channels.
+# itself for large problems.  Needs H*W % 4 == 0 and at most 271 channels;
+# with 272 - 543 channels the tiles have 64 positions (pairs of row groups only).
 # (batch, ic, oc, h, w): fewer row groups than streams, more, an odd row
 # count, a tile that spans images, a last tile that is not full, the largest
-# channel count, lists longer than one LDS piece.
-TILED_SHAPES = [(2, 64, 8, 4, 4), (1, 96, 48, 8, 6), (3, 130, 67, 4, 5), (1, 264, 150, 16, 16), (5, 70, 33, 2, 2), (2, 257, 20, 12, 12), (3, 256, 96, 10, 10)]
+# channel count, lists longer than one LDS piece; then tiles of 64: the
+# smallest and the largest channel count, tiles that span and end inside images.
+TILED_SHAPES = [(2, 64, 8, 4, 4), (1, 96, 48, 8, 6), (3, 130, 67, 4, 5), (1, 271, 150, 16, 16), (5, 70, 33, 2, 2), (2, 257, 20, 12, 12), (3, 256, 96, 10, 10),
+                (3, 272, 33, 2, 2), (1, 300, 150, 16, 16), (2, 512, 40, 6, 6), (1, 543, 20, 4, 4)]
 
 
 @pytest.mark.parametrize("act", ["none", "relu6", "hswish"])
