@@ -1166,13 +1166,18 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     c.sub_tiles = h->mfma_sub_tiles;
     if (h->mfma_tile_quads > 0) c.tile_quads = h->mfma_tile_quads;
     e = pl::LaunchBlockMfma(c, p, s);
-  } else if (!h->int8 && !h->half && vec && (h->tw.built != 0 || h->tw_narrow.built != 0) && h->walk_tiled > 0 &&
-             (h->walk_tiled == 2 || 32 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), h->tw.built ? pl::kTileWalkTile : pl::kTileWalkNarrowTile)) >= h->wg_slots_default)) {
+  } else if (!h->int8 && !h->half && (vec || (h->walk_pairs && reinterpret_cast<uintptr_t>(x_dev) % 4 == 0 && reinterpret_cast<uintptr_t>(out_dev) % 4 == 0)) &&
+             (h->tw.built != 0 || h->tw_narrow.built != 0) && h->walk_tiled > 0 &&
+             (h->walk_tiled == 2 || (vec ? 32 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), h->tw.built ? pl::kTileWalkTile : pl::kTileWalkNarrowTile)) >= h->wg_slots_default
+                                         // the other walks move such tensors element by element too and lose earlier: measured
+                                         // crossover at 400 - 700 positions with row pairs, 50 - 200 without (256 CUs)
+                                         : (h->semi ? 4 : 14) * static_cast<int64_t>(P) >= 5 * static_cast<int64_t>(h->wg_slots_default)))) {
     // fp32 with tiles for at least a sixteenth of the CUs (the
     // row groups of a tile are shared between up to ten CUs; measured
     // crossover against the other walks between 13 and 25 tiles on 256 CUs):
     // the walk with the tile and the lists in LDS - tiles of 128 positions, of 64 where
-    // only those fit LDS with all channels
+    // only those fit LDS with all channels; element by element in and out of the tile where the map size is
+    // not a multiple of 4 or the tensors are not 16-byte aligned
     const TileWalkStreams& tw = h->tw.built ? h->tw : h->tw_narrow;
     const int tile = h->tw.built ? pl::kTileWalkTile : pl::kTileWalkNarrowTile;
     pl::TileWalkParams p{};
@@ -1184,7 +1189,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.stream_groups = static_cast<const uint32_t*>(tw.desc.ptr) + d.table;
     p.split = static_cast<int16_t>(d.split);
     p.parts = static_cast<int8_t>(d.parts);
-    p.pairs = h->tw.built ? (h->walk_pairs ? 1 : 0) : 2;
+    p.pairs = static_cast<int8_t>((h->tw.built ? (h->walk_pairs ? 1 : 0) : 2) | (vec ? 0 : pl::kTileWalkRagged));
     p.split_slots = d.split_slots;
     p.n_groups = h->n_groups;
     p.M = h->oc;

@@ -101,6 +101,7 @@ hipError_t LaunchChunkWalk(int nrows, const ChunkWalkParams& p, hipStream_t stre
 // kTileWalkTile positions with all input channels; wavefront s walks the row
 // groups of list stream s.
 constexpr int kTileWalkTile = 128;
+constexpr int kTileWalkRagged = 4;      // flag in TileWalkParams::pairs
 constexpr int kTileWalkNarrowTile = 64;  // for channel counts whose 128-position tile does not fit LDS (pairs only)
 constexpr int kTileWalkWaves = 16;
 constexpr int kTileWalkChunkBytes = 1536;  // piece of a list stream held in LDS per wavefront
@@ -131,6 +132,7 @@ struct TileWalkParams {
   // 1: the streams hold pairs of row groups, padded to one length, as double records (first group's record, second
   // group's record): lanes 0 - 31 walk the first group, lanes 32 - 63 the second, four positions per lane
   // 2: pairs on tiles of kTileWalkNarrowTile positions, two per lane (streams made for 256-byte channel rows)
+  // + kTileWalkRagged (with 1 or 2): hw is not a multiple of 4; tile and outputs are moved element by element
   int8_t pairs;
   // The first 56 bytes (kernarg_head.h) end behind act.type: what selects the tile, picks the activation and
   // addresses the first loads.
@@ -143,7 +145,7 @@ struct TileWalkParams {
 
 // LDS the kernel needs for K input channels.
 size_t TileWalkLdsBytes(int K, int row_bytes = kTileWalkTile * 4);  // row_bytes: bytes per channel row of the tile
-// Needs hw % 4 == 0 and 16-byte aligned x / out.
+// Needs hw % 4 == 0 and 16-byte aligned x / out, or the ragged form.
 hipError_t LaunchTileWalk(int nrows, const TileWalkParams& p, hipStream_t stream);
 
 // Half-precision row walk (fp16_walk_kernels.hip).  Activation constants as

@@ -24,6 +24,10 @@
 // the shorter group of a pair is padded with entries of weight zero at the tile's zero row.
 // With more channels than a tile of 128 positions holds in LDS, the pairs walk tiles of 64 positions, two per
 // lane (NARROW; channel rows of 256 bytes, list streams made for those).
+// Maps whose size is not a multiple of 4 (RAGGED, pairs only): neighbouring positions of a tile may lie in
+// different images, so the tile is staged and the outputs are stored element by element (a thread stages the
+// positions c, c + 32, ... of a channel row, a lane stores each of its positions through its own address); the
+// walk between the two is the same.
 // With fewer tiles than CUs, the row groups can be dealt into a main and a
 // spare part (two sets of sixteen streams): the tile's own workgroup walks the
 // main part, and the workgroups on the CUs that have no tile of their own walk
@@ -69,9 +73,10 @@ constexpr int kWaves = kTileWalkWaves;  // wavefronts per workgroup = list strea
 constexpr int kChunkBytes = kTileWalkChunkBytes;
 
 // One tile: stage it, then walk the streams of one part (0 main, 1 spare).
-template <int NR, int ACT, bool PAIR, bool NARROW>
+template <int NR, int ACT, bool PAIR, bool NARROW, bool RAGGED>
 __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile, int tile_id, int part) {
   static_assert(PAIR || !NARROW, "narrow tiles are walked in pairs");
+  static_assert(PAIR || !RAGGED, "maps of any size are walked in pairs");
   constexpr int kRecBytes = NR == 2 ? 48 : 32;  // four byte offsets, then 4 * NR weights
   constexpr int kStepBytes = PAIR ? 2 * kRecBytes : kRecBytes;  // what one step of the walk reads: one record per row group
   constexpr int kRecs = kChunkBytes / kStepBytes;
@@ -91,7 +96,39 @@ __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile
   u2 pb = *reinterpret_cast<const u2*>(sp + 1024 + 8 * lane);
 
   // staging: kTP / 4 threads per channel row (four positions each), 32 or 64 rows per pass
-  {
+  if (RAGGED) {
+    constexpr int kRowThreads = kTP / 4, kPassRows = 64 * kWaves / kRowThreads;
+    const int c = tid & (kRowThreads - 1), r0 = tid / kRowThreads;
+    // the thread's positions c + kRowThreads * e of the tile: offset of each in channel 0 of its image
+    size_t eoff[4];
+    bool elive[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t pos = tile0 + (uint32_t)(c + kRowThreads * e);
+      elive[e] = pos < p.P;
+      const uint32_t n = elive[e] ? pos / (uint32_t)p.hw : 0u;
+      const uint32_t pp = elive[e] ? pos % (uint32_t)p.hw : 0u;
+      eoff[e] = (size_t)n * p.K * p.hw + pp;
+    }
+    for (int k0 = 0; k0 < p.K; k0 += 4 * kPassRows) {
+      float v[4][4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int k = min(k0 + r0 + kPassRows * u, p.K - 1);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[u][e] = p.x[eoff[e] + (size_t)k * p.hw];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int k = k0 + r0 + kPassRows * u;
+        if (k < p.K) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) tile[(size_t)k * kTP + c + kRowThreads * e] = elive[e] ? v[u][e] : 0.0f;
+        }
+      }
+    }
+    if (tid < kTP / 4) *reinterpret_cast<uint4*>(tile_bytes + ((size_t)p.K * kTP + 4 * tid) * 4) = make_uint4(0, 0, 0, 0);
+  } else {
     constexpr int kRowThreads = kTP / 4, kPassRows = 64 * kWaves / kRowThreads;
     const int c4 = tid & (kRowThreads - 1), r0 = tid / kRowThreads;
     const uint32_t gpos = tile0 + 4u * (uint32_t)c4;
@@ -124,6 +161,18 @@ __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile
   const bool store_on = gpos < p.P;
   const uint32_t on = store_on ? gpos / (uint32_t)p.hw : 0u, opp = store_on ? gpos % (uint32_t)p.hw : 0u;
   float* obase = p.out + (size_t)on * p.M * p.hw + opp;
+  // RAGGED: every position of the lane through its own address (row 0 of its image)
+  [[maybe_unused]] float* qbase[RAGGED ? PPL : 1];
+  [[maybe_unused]] bool qlive[RAGGED ? PPL : 1];
+  if (RAGGED) {
+#pragma unroll
+    for (int q = 0; q < PPL; ++q) {
+      const uint32_t pos = gpos + (uint32_t)q;
+      qlive[q] = pos < p.P;
+      const uint32_t n = qlive[q] ? pos / (uint32_t)p.hw : 0u, pp = qlive[q] ? pos % (uint32_t)p.hw : 0u;
+      qbase[q] = p.out + (size_t)n * p.M * p.hw + pp;
+    }
+  }
 
   int rec = kRecs;  // records of the current chunk already walked: the first chunk is still in registers
   int chunk = 0;
@@ -200,7 +249,17 @@ __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile
       if (rem > 1) entry(off[1], w[NR], w[NR + NR - 1]);
       if (rem > 2) entry(off[2], w[2 * NR], w[2 * NR + NR - 1]);
     }
-    if (store_on) {
+    if (RAGGED) {
+#pragma unroll
+      for (int rr = 0; rr < NR; ++rr) {
+        if (rr < nrows) {
+          const size_t at = (size_t)(row0 + rr) * p.hw;
+#pragma unroll
+          for (int q = 0; q < PPL; ++q)
+            if (qlive[q]) qbase[q][at] = ActivateT<ACT>(acc[rr][q], p.act);
+        }
+      }
+    } else if (store_on) {
 #pragma unroll
       for (int rr = 0; rr < NR; ++rr) {
         if (rr < nrows) {
@@ -217,7 +276,7 @@ __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile
 // Workgroup id -> tiles: each XCD (linear id mod 8) owns a contiguous range of
 // tiles.  Its first workgroups take one tile each (main part); with a spare
 // part, the workgroups behind them share the range's tiles among themselves.
-template <int NR, int ACT, bool PAIR, bool NARROW>
+template <int NR, int ACT, bool PAIR, bool NARROW, bool RAGGED>
 __device__ __forceinline__ void TileWalkBody(const TileWalkParams& p, float* tile) {
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int first = (xcd * p.tiles) >> 3, last = ((xcd + 1) * p.tiles) >> 3;
@@ -225,17 +284,17 @@ __device__ __forceinline__ void TileWalkBody(const TileWalkParams& p, float* til
   if (p.split == 2) {
     // equal parts: part = slot / count of tile slot % count
     const int part = count > 0 ? slot / count : p.parts;
-    if (part < p.parts) WalkOneTile<NR, ACT, PAIR, NARROW>(p, tile, first + (slot - part * count), part);
+    if (part < p.parts) WalkOneTile<NR, ACT, PAIR, NARROW, RAGGED>(p, tile, first + (slot - part * count), part);
     return;
   }
   if (slot < count) {
-    WalkOneTile<NR, ACT, PAIR, NARROW>(p, tile, first + slot, 0);
+    WalkOneTile<NR, ACT, PAIR, NARROW, RAGGED>(p, tile, first + slot, 0);
     return;
   }
   if (p.split == 0) return;
   const int n_spare = (int)(gridDim.x >> 3) - count;
   for (int t = first + (slot - count); t < last; t += n_spare) {
-    WalkOneTile<NR, ACT, PAIR, NARROW>(p, tile, t, 1);
+    WalkOneTile<NR, ACT, PAIR, NARROW, RAGGED>(p, tile, t, 1);
     __syncthreads();  // every wavefront has left the tile before the next one is staged
   }
 }
@@ -246,12 +305,22 @@ __global__ void __launch_bounds__(64 * kTileWalkWaves) TileWalkKernel(PL_HEAD_PA
   extern __shared__ float tile_lds[];
   DispatchAct(p.act.type, [&](auto act_c) {
     constexpr int ACT = decltype(act_c)::value;
-    if (p.pairs == 2) {
-      TileWalkBody<NR, ACT, true, true>(p, tile_lds);
-    } else if (p.pairs) {
-      TileWalkBody<NR, ACT, true, false>(p, tile_lds);
-    } else {
-      TileWalkBody<NR, ACT, false, false>(p, tile_lds);
+    switch (p.pairs) {
+      case 0:
+        TileWalkBody<NR, ACT, false, false, false>(p, tile_lds);
+        break;
+      case 1:
+        TileWalkBody<NR, ACT, true, false, false>(p, tile_lds);
+        break;
+      case 2:
+        TileWalkBody<NR, ACT, true, true, false>(p, tile_lds);
+        break;
+      case 1 | kTileWalkRagged:
+        TileWalkBody<NR, ACT, true, false, true>(p, tile_lds);
+        break;
+      default:  // 2 | kTileWalkRagged
+        TileWalkBody<NR, ACT, true, true, true>(p, tile_lds);
+        break;
     }
   });
 }
@@ -262,8 +331,10 @@ size_t TileWalkLdsBytes(int K, int row_bytes) { return (size_t)(K + 1) * (size_t
 
 hipError_t LaunchTileWalk(int nrows, const TileWalkParams& p, hipStream_t stream) {
   if (p.P == 0 || p.n_groups == 0) return hipSuccess;
-  if (p.hw % 4 != 0) return hipErrorInvalidValue;
-  const int tile = p.pairs == 2 ? kTileWalkNarrowTile : kTileWalkTile;
+  const int form = p.pairs & 3;
+  const bool ragged = (p.pairs & kTileWalkRagged) != 0;
+  if (form > 2 || (ragged && form == 0) || (!ragged && p.hw % 4 != 0)) return hipErrorInvalidValue;
+  const int tile = form == 2 ? kTileWalkNarrowTile : kTileWalkTile;
   const size_t lds = TileWalkLdsBytes(p.K, tile * 4);
   if (lds > (size_t)kMaxLdsBytes) return hipErrorInvalidValue;
   TileWalkParams q = p;

@@ -184,6 +184,9 @@ def test_fp32_chunked_walk(shape, paired, act):
 # smallest and the largest channel count, tiles that span and end inside images.
 TILED_SHAPES = [(2, 64, 8, 4, 4), (1, 96, 48, 8, 6), (3, 130, 67, 4, 5), (1, 271, 150, 16, 16), (5, 70, 33, 2, 2), (2, 257, 20, 12, 12), (3, 256, 96, 10, 10),
                 (3, 272, 33, 2, 2), (1, 300, 150, 16, 16), (2, 512, 40, 6, 6), (1, 543, 20, 4, 4)]
+# map sizes that are not a multiple of 4 (the tile is staged and stored element by element): 7 x 7, single
+# pixels (four neighbouring positions in four images), 3 x 5 and 13 x 13, on tiles of 128 and of 64 positions
+TILED_SHAPES += [(3, 64, 48, 7, 7), (9, 96, 33, 1, 1), (2, 130, 67, 3, 5), (4, 256, 96, 9, 9), (2, 300, 40, 7, 7), (1, 512, 64, 13, 13)]
 
 
 @pytest.mark.parametrize("act", ["none", "relu6", "hswish"])
@@ -208,6 +211,30 @@ def test_fp32_tiled_walk(shape, paired, act):
     # and the plain walk gives the same bits (same order of fused multiply-adds)
     plain = run_hip(case, capi.ALGO_ROW_WALK, force_semi=paired, tuning=capi.tuning(walk_tiled=capi.TUNE_NEVER, walk_chunked=capi.TUNE_NEVER))
     assert np.array_equal(got, plain)
+
+
+@pytest.mark.parametrize("ic", [96, 300], ids=["tiles_of_128", "tiles_of_64"])
+def test_fp32_tiled_walk_with_tensors_off_the_16_byte_grid(ic):
+    """Tensors that start 4 bytes behind a 16-byte boundary take the element-wise form of the tile walk: the same
+    bits as the aligned call, nothing written outside the output."""
+    import torch
+
+    announce("fp32 tiled, unaligned", ic)
+    case = small_case(capi.KIND_FP32, 3, ic, 40, 6, 6, 0.75, False, ACTS["relu6"], seed=ic)
+    kernel, _ = make_kernel(case, capi.ALGO_ROW_WALK, tuning=capi.tuning(walk_tiled=capi.TUNE_ALWAYS))
+    want = run_hip(case, kernel=kernel)
+    assert_same(case, want, run_oracle(case), "aligned")
+    flat_x = torch.zeros(case.x.size + 8, dtype=torch.float32, device="cuda")
+    x = flat_x[1:1 + case.x.size].view(case.x.shape)
+    x.copy_(torch.from_numpy(case.x))
+    flat_o = torch.full((want.size + 8,), 77.0, dtype=torch.float32, device="cuda")
+    out = flat_o[1:1 + want.size].view(want.shape)
+    assert x.data_ptr() % 16 == 4 and out.data_ptr() % 16 == 4
+    kernel.Run(x, out)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), want)
+    host = flat_o.cpu().numpy()
+    assert host[0] == 77.0 and (host[1 + want.size:] == 77.0).all()
 
 
 def test_no_bias_and_single_scale():
