@@ -377,7 +377,9 @@ struct TwPiece<4> {
 };
 
 // One tile: stage it, then walk the streams of one part (0 main, 1 spare).
-template <int NR, int PPL, int ACT>
+// RAGGED: the map size is not a multiple of the lane's piece (or the tensors are not aligned to it), so the tile is
+// staged and the outputs are stored one binary16 value at a time, each through its own address.
+template <int NR, int PPL, int ACT, bool RAGGED>
 __device__ __forceinline__ void HalfWalkOneTile(const HalfTileWalkParams& p, char* tile_bytes, int tile_id, int part) {
   typedef typename TwPiece<PPL>::type Piece;
   constexpr int kTwTile = 32 * PPL, kTwRowBytes = kTwTile * 2, kPieceBytes = 2 * PPL, NW = PPL / 2;
@@ -397,7 +399,41 @@ __device__ __forceinline__ void HalfWalkOneTile(const HalfTileWalkParams& p, cha
   u2w pb = *reinterpret_cast<const u2w*>(sp + 1024 + 8 * lane);
 
   // staging: 32 threads per channel row (PPL positions each), 32 rows per pass
-  {
+  if (RAGGED) {
+    const int c = tid & 31, r0 = tid >> 5;
+    // the thread's positions c + 32 e of the tile: offset of each in channel 0 of its image
+    size_t eoff[PPL];
+    bool elive[PPL];
+#pragma unroll
+    for (int e = 0; e < PPL; ++e) {
+      const uint32_t pos = tile0 + (uint32_t)(c + 32 * e);
+      elive[e] = pos < p.P;
+      const uint32_t n = elive[e] ? pos / (uint32_t)p.hw : 0u;
+      const uint32_t pp = elive[e] ? pos % (uint32_t)p.hw : 0u;
+      eoff[e] = (size_t)n * p.K * p.hw + pp;
+    }
+    uint16_t* tile16 = reinterpret_cast<uint16_t*>(tile_bytes);
+    for (int k0 = 0; k0 < p.K; k0 += 128) {
+      uint16_t v[4][PPL];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int k = min(k0 + r0 + 32 * u, p.K - 1);
+#pragma unroll
+        for (int e = 0; e < PPL; ++e) v[u][e] = p.x[eoff[e] + (size_t)k * p.hw];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int k = k0 + r0 + 32 * u;
+        if (k < p.K) {
+#pragma unroll
+          for (int e = 0; e < PPL; ++e) tile16[(size_t)k * kTwTile + c + 32 * e] = elive[e] ? v[u][e] : (uint16_t)0;
+        }
+      }
+    }
+    Piece zero;
+    __builtin_memset(&zero, 0, sizeof(zero));
+    if (tid < 32) *reinterpret_cast<Piece*>(tile_bytes + (size_t)p.K * kTwRowBytes + kPieceBytes * tid) = zero;
+  } else {
     const int c8 = tid & 31, r0 = tid >> 5;
     const uint32_t gpos = tile0 + (uint32_t)PPL * (uint32_t)c8;
     const bool live = gpos < p.P;
@@ -430,6 +466,18 @@ __device__ __forceinline__ void HalfWalkOneTile(const HalfTileWalkParams& p, cha
   const bool store_on = gpos < p.P;
   const uint32_t on = store_on ? gpos / (uint32_t)p.hw : 0u, opp = store_on ? gpos % (uint32_t)p.hw : 0u;
   uint16_t* obase = p.out + (size_t)on * p.M * p.hw + opp;
+  // RAGGED: every position of the lane through its own address (row 0 of its image)
+  [[maybe_unused]] uint16_t* qbase[RAGGED ? PPL : 1];
+  [[maybe_unused]] bool qlive[RAGGED ? PPL : 1];
+  if (RAGGED) {
+#pragma unroll
+    for (int q = 0; q < PPL; ++q) {
+      const uint32_t pos = gpos + (uint32_t)q;
+      qlive[q] = pos < p.P;
+      const uint32_t n = qlive[q] ? pos / (uint32_t)p.hw : 0u, pp = qlive[q] ? pos % (uint32_t)p.hw : 0u;
+      qbase[q] = p.out + (size_t)n * p.M * p.hw + pp;
+    }
+  }
 
   int rec = kRecs;  // records of the current chunk already walked: the first chunk is still in registers
   int chunk = 0;
@@ -501,7 +549,20 @@ __device__ __forceinline__ void HalfWalkOneTile(const HalfTileWalkParams& p, cha
       if (rem > 1) entry(*reinterpret_cast<const Piece*>(tile_bytes + (off[1] + lane16)), w[NR], w[NR + NR - 1]);
       if (rem > 2) entry(*reinterpret_cast<const Piece*>(tile_bytes + (off[2] + lane16)), w[2 * NR], w[2 * NR + NR - 1]);
     }
-    if (store_on) {
+    if (RAGGED) {
+#pragma unroll
+      for (int rr = 0; rr < NR; ++rr) {
+        if (rr < nrows) {
+          const size_t at = (size_t)(row0 + rr) * p.hw;
+#pragma unroll
+          for (int q = 0; q < NW; ++q) {
+            const h2 o = ActivateH<ACT>(acc[rr][q], p.act);
+            if (qlive[2 * q]) qbase[2 * q][at] = BitsOf(o.x);
+            if (qlive[2 * q + 1]) qbase[2 * q + 1][at] = BitsOf(o.y);
+          }
+        }
+      }
+    } else if (store_on) {
 #pragma unroll
       for (int rr = 0; rr < NR; ++rr) {
         if (rr < nrows) {
@@ -518,24 +579,24 @@ __device__ __forceinline__ void HalfWalkOneTile(const HalfTileWalkParams& p, cha
 // Workgroup id -> tiles, as in the fp32 tile walk: each XCD (linear id mod 8) owns a contiguous range of tiles;
 // its first workgroups take one tile each (main part), with a spare part the workgroups behind them share the
 // range's tiles among themselves, with equal parts `parts` workgroups share every tile.
-template <int NR, int PPL, int ACT>
+template <int NR, int PPL, int ACT, bool RAGGED>
 __device__ __forceinline__ void HalfTileWalkBody(const HalfTileWalkParams& p, char* tile) {
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int first = (xcd * p.tiles) >> 3, last = ((xcd + 1) * p.tiles) >> 3;
   const int count = last - first;
   if (p.split == 2) {
     const int part = count > 0 ? slot / count : p.parts;
-    if (part < p.parts) HalfWalkOneTile<NR, PPL, ACT>(p, tile, first + (slot - part * count), part);
+    if (part < p.parts) HalfWalkOneTile<NR, PPL, ACT, RAGGED>(p, tile, first + (slot - part * count), part);
     return;
   }
   if (slot < count) {
-    HalfWalkOneTile<NR, PPL, ACT>(p, tile, first + slot, 0);
+    HalfWalkOneTile<NR, PPL, ACT, RAGGED>(p, tile, first + slot, 0);
     return;
   }
   if (p.split == 0) return;
   const int n_spare = (int)(gridDim.x >> 3) - count;
   for (int t = first + (slot - count); t < last; t += n_spare) {
-    HalfWalkOneTile<NR, PPL, ACT>(p, tile, t, 1);
+    HalfWalkOneTile<NR, PPL, ACT, RAGGED>(p, tile, t, 1);
     __syncthreads();  // every wavefront has left the tile before the next one is staged
   }
 }
@@ -547,19 +608,39 @@ __global__ void __launch_bounds__(64 * kTileWalkWaves) HalfTileWalkKernel(PL_HEA
   char* tile = reinterpret_cast<char*>(tile32);
   switch (p.act.type) {
     case 1:
-      HalfTileWalkBody<NR, PPL, 1>(p, tile);
+      if (p.ragged) {
+        HalfTileWalkBody<NR, PPL, 1, true>(p, tile);
+      } else {
+        HalfTileWalkBody<NR, PPL, 1, false>(p, tile);
+      }
       break;
     case 2:
-      HalfTileWalkBody<NR, PPL, 2>(p, tile);
+      if (p.ragged) {
+        HalfTileWalkBody<NR, PPL, 2, true>(p, tile);
+      } else {
+        HalfTileWalkBody<NR, PPL, 2, false>(p, tile);
+      }
       break;
     case 4:
-      HalfTileWalkBody<NR, PPL, 4>(p, tile);
+      if (p.ragged) {
+        HalfTileWalkBody<NR, PPL, 4, true>(p, tile);
+      } else {
+        HalfTileWalkBody<NR, PPL, 4, false>(p, tile);
+      }
       break;
     case 10:
-      HalfTileWalkBody<NR, PPL, 10>(p, tile);
+      if (p.ragged) {
+        HalfTileWalkBody<NR, PPL, 10, true>(p, tile);
+      } else {
+        HalfTileWalkBody<NR, PPL, 10, false>(p, tile);
+      }
       break;
     default:
-      HalfTileWalkBody<NR, PPL, 0>(p, tile);
+      if (p.ragged) {
+        HalfTileWalkBody<NR, PPL, 0, true>(p, tile);
+      } else {
+        HalfTileWalkBody<NR, PPL, 0, false>(p, tile);
+      }
       break;
   }
 }
@@ -618,11 +699,11 @@ hipError_t LaunchHalfChunkWalk(int nrows, const HalfChunkWalkParams& p, hipStrea
 }
 
 // A lane's positions are one piece of one image: tile 256 needs hw % 8 == 0 and 16-byte aligned x / out, tile 128
-// hw % 4 == 0 and 8-byte alignment.
+// hw % 4 == 0 and 8-byte alignment; the ragged form (HalfTileWalkParams::ragged) takes any map size.
 hipError_t LaunchHalfTileWalk(int nrows, int tile, const HalfTileWalkParams& p, hipStream_t stream) {
   if (p.P == 0 || p.n_groups == 0) return hipSuccess;
   if (tile != kHalfTileWalkTile && tile != kHalfTileWalkNarrowTile) return hipErrorInvalidValue;
-  if (p.hw % (tile / 32) != 0) return hipErrorInvalidValue;
+  if (!p.ragged && p.hw % (tile / 32) != 0) return hipErrorInvalidValue;
   const size_t lds = TileWalkLdsBytes(p.K, tile * 2);
   if (lds > (size_t)kMaxLdsBytes) return hipErrorInvalidValue;
   HalfTileWalkParams q = p;

@@ -1015,6 +1015,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
   const bool aligned8 = reinterpret_cast<uintptr_t>(x_dev) % 8 == 0 && reinterpret_cast<uintptr_t>(out_dev) % 8 == 0;
   const TileWalkStreams* half_tw = nullptr;
   int half_tile = 0;
+  bool half_ragged = false;
   if (h->half && h->walk_tiled > 0) {
     if (h->tw.built != 0 && im_size % 8 == 0 && aligned16) {
       half_tw = &h->tw;
@@ -1022,6 +1023,11 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     } else if (h->tw_narrow.built != 0 && im_size % 4 == 0 && aligned8) {
       half_tw = &h->tw_narrow;
       half_tile = pl::kHalfTileWalkNarrowTile;
+    } else if (reinterpret_cast<uintptr_t>(x_dev) % 2 == 0 && reinterpret_cast<uintptr_t>(out_dev) % 2 == 0 && (h->tw.built != 0 || h->tw_narrow.built != 0)) {
+      // any other map size or alignment: value by value in and out of the tile
+      half_tw = h->tw.built != 0 ? &h->tw : &h->tw_narrow;
+      half_tile = h->tw.built != 0 ? pl::kHalfTileWalkTile : pl::kHalfTileWalkNarrowTile;
+      half_ragged = true;
     }
     if (half_tw && h->walk_tiled != 2 && (h->semi ? 42 : 84) * static_cast<int64_t>(CeilDiv(static_cast<int>(P), half_tile)) < h->wg_slots_default) half_tw = nullptr;
   }
@@ -1035,6 +1041,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.stream_groups = static_cast<const uint32_t*>(half_tw->desc.ptr) + d.table;
     p.split = static_cast<int16_t>(d.split);
     p.parts = static_cast<int8_t>(d.parts);
+    p.ragged = half_ragged ? 1 : 0;
     p.split_slots = d.split_slots;
     p.n_groups = h->n_groups;
     p.M = h->oc;

@@ -199,7 +199,7 @@ struct HalfTileWalkParams {
   int tiles;  // filled in by the launcher
   int16_t split;
   int8_t parts;
-  int8_t reserved;
+  int8_t ragged;  // 1: the tile is staged and the outputs are stored value by value (any map size and alignment)
   // the first 56 bytes (kernarg_head.h) end behind act.type
   DevActH act;
   const uint32_t* stream_groups;

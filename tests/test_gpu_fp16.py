@@ -80,6 +80,9 @@ TILED_SHAPES = [(2, 64, 64, 4, 4), (1, 96, 48, 8, 6), (3, 130, 67, 4, 6), (5, 70
 # 14 x 14 and 2 x 2 maps, a tile that ends inside an image, channel counts above the wide tile's limit on maps of
 # both kinds, the largest channel count.
 TILED_SHAPES += [(3, 64, 48, 14, 14), (7, 40, 33, 2, 2), (2, 257, 20, 6, 6), (1, 300, 150, 16, 16), (2, 512, 64, 14, 14), (1, 543, 40, 4, 4)]
+# Any other map size goes in and out of the tile value by value: 7 x 7, single pixels (neighbouring positions in
+# different images), 3 x 5, 9 x 9, 13 x 13, a map of 2 x 3, on tiles of 256 and of 128 positions.
+TILED_SHAPES += [(3, 64, 48, 7, 7), (9, 96, 33, 1, 1), (2, 130, 67, 3, 5), (4, 256, 96, 9, 9), (2, 300, 40, 7, 7), (1, 512, 64, 13, 13), (5, 48, 20, 2, 3)]
 
 
 @pytest.mark.parametrize("act", ["none", "relu", "relu6", "leaky", "hswish"])
@@ -122,3 +125,27 @@ def test_fp16_tile_walk_takes_a_new_bias(had_bias, size):
     capi.check(capi.lib().pl_sparse_conv_set_epilogue(kernel._handle, None, new_bias.ctypes.data, None))
     case.bias = new_bias
     assert_same(case, run_hip(case, kernel=kernel), run_oracle(case), "fp16 tile walk, second bias")
+
+
+def test_fp16_tile_walk_with_tensors_off_the_16_byte_grid():
+    """Tensors that start 2 bytes behind a 16-byte boundary take the value-by-value form of the tile walk: the same
+    bits as the aligned call, nothing written outside the output."""
+    import torch
+
+    from helpers import make_kernel
+
+    case = half_case(3, 96, 40, 8, 8, 0.75, False, ACTS["relu6"], seed=4)
+    kernel, _ = make_kernel(case, tuning=capi.tuning(walk_tiled=capi.TUNE_ALWAYS))
+    want = run_hip(case, kernel=kernel)
+    assert_same(case, want, run_oracle(case), "aligned")
+    flat_x = torch.zeros(case.x.size + 16, dtype=torch.float16, device="cuda")
+    x = flat_x[1:1 + case.x.size].view(case.x.shape)
+    x.copy_(torch.from_numpy(case.x))
+    flat_o = torch.full((want.size + 16,), 77.0, dtype=torch.float16, device="cuda")
+    out = flat_o[1:1 + want.size].view(want.shape)
+    assert x.data_ptr() % 16 == 2 and out.data_ptr() % 16 == 2
+    kernel.Run(x, out)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    host = flat_o.cpu().numpy()
+    assert host[0] == 77.0 and (host[1 + want.size:] == 77.0).all()
