@@ -161,7 +161,8 @@ struct pl_sparse_conv_handle {
   // 256-byte channel rows - half precision with 128 positions per tile, for more channels and for maps whose
   // size is a multiple of 4 but not of 8; fp32 with 64 positions per tile (pairs only), built when the channels do
   // not fit the wide tile
-  TileWalkStreams tw, tw_narrow;
+  // tw_slim: fp32 with 32 positions per tile (128-byte channel rows), built when the narrow tile does not fit either
+  TileWalkStreams tw, tw_narrow, tw_slim;
   int walk_split = -1;          // sixteenths of the row groups' work dealt to the CUs without a tile: -1 by rule, 0 never, 1 .. 8 forced
   int walk_tiled = 1;            // 0 never, 1 when the problem suits it, 2 whenever the shape allows
   bool walk_pairs = true;        // the tile walk's streams hold pairs of row groups (two per wavefront instruction)
@@ -200,7 +201,7 @@ struct pl_sparse_conv_handle {
   int padded_rows = 0;
 
   int64_t DeviceBytes() const {
-    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + cw_desc.bytes + cw_idx.bytes + cw_wts.bytes + hw_kidx.bytes + hw_wts.bytes + hw_bias.bytes + wblocks.bytes + kmask.bytes + wtiles.bytes + wtiles_rg.bytes + wtiles_tr.bytes + wtiles_rows.bytes + tw.DeviceBytes() + tw_narrow.DeviceBytes() + scale.bytes + bias.bytes);
+    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + cw_desc.bytes + cw_idx.bytes + cw_wts.bytes + hw_kidx.bytes + hw_wts.bytes + hw_bias.bytes + wblocks.bytes + kmask.bytes + wtiles.bytes + wtiles_rg.bytes + wtiles_tr.bytes + wtiles_rows.bytes + tw.DeviceBytes() + tw_narrow.DeviceBytes() + tw_slim.DeviceBytes() + scale.bytes + bias.bytes);
   }
 };
 
@@ -919,6 +920,7 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8) rc = BuildChunkWalk(L, h);
   if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8 && !half) rc = BuildTileWalk(L, desc->bias, h, &h->tw);
   if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8 && !half && !h->tw.built && h->walk_pairs) rc = BuildTileWalk(L, desc->bias, h, &h->tw_narrow, false, pl::kTileWalkNarrowTile * 4);
+  if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8 && !half && !h->tw.built && !h->tw_narrow.built && h->walk_pairs) rc = BuildTileWalk(L, desc->bias, h, &h->tw_slim, false, pl::kTileWalkSlimTile * 4);
   if (rc == PL_OK) {
     // the MFMA epilogues always read a bias; give them zeros when the op has none
     std::vector<float> zeros;
@@ -1174,8 +1176,8 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     if (h->mfma_tile_quads > 0) c.tile_quads = h->mfma_tile_quads;
     e = pl::LaunchBlockMfma(c, p, s);
   } else if (!h->int8 && !h->half && (vec || (h->walk_pairs && reinterpret_cast<uintptr_t>(x_dev) % 4 == 0 && reinterpret_cast<uintptr_t>(out_dev) % 4 == 0)) &&
-             (h->tw.built != 0 || h->tw_narrow.built != 0) && h->walk_tiled > 0 &&
-             (h->walk_tiled == 2 || (vec ? 32 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), h->tw.built ? pl::kTileWalkTile : pl::kTileWalkNarrowTile)) >= h->wg_slots_default
+             (h->tw.built != 0 || h->tw_narrow.built != 0 || h->tw_slim.built != 0) && h->walk_tiled > 0 &&
+             (h->walk_tiled == 2 || (vec ? 32 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), h->tw.built ? pl::kTileWalkTile : h->tw_narrow.built ? pl::kTileWalkNarrowTile : pl::kTileWalkSlimTile)) >= h->wg_slots_default
                                          // the other walks move such tensors element by element too and lose earlier: measured
                                          // crossover at 400 - 700 positions with row pairs, 50 - 200 without (256 CUs)
                                          : (h->semi ? 4 : 14) * static_cast<int64_t>(P) >= 5 * static_cast<int64_t>(h->wg_slots_default)))) {
@@ -1185,8 +1187,8 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     // the walk with the tile and the lists in LDS - tiles of 128 positions, of 64 where
     // only those fit LDS with all channels; element by element in and out of the tile where the map size is
     // not a multiple of 4 or the tensors are not 16-byte aligned
-    const TileWalkStreams& tw = h->tw.built ? h->tw : h->tw_narrow;
-    const int tile = h->tw.built ? pl::kTileWalkTile : pl::kTileWalkNarrowTile;
+    const TileWalkStreams& tw = h->tw.built ? h->tw : h->tw_narrow.built ? h->tw_narrow : h->tw_slim;
+    const int tile = h->tw.built ? pl::kTileWalkTile : h->tw_narrow.built ? pl::kTileWalkNarrowTile : pl::kTileWalkSlimTile;
     pl::TileWalkParams p{};
     p.x = static_cast<const float*>(x_dev);
     p.out = static_cast<float*>(out_dev);
@@ -1196,7 +1198,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.stream_groups = static_cast<const uint32_t*>(tw.desc.ptr) + d.table;
     p.split = static_cast<int16_t>(d.split);
     p.parts = static_cast<int8_t>(d.parts);
-    p.pairs = static_cast<int8_t>((h->tw.built ? (h->walk_pairs ? 1 : 0) : 2) | (vec ? 0 : pl::kTileWalkRagged));
+    p.pairs = static_cast<int8_t>((h->tw.built ? (h->walk_pairs ? 1 : 0) : h->tw_narrow.built ? 2 : 3) | (vec ? 0 : pl::kTileWalkRagged));
     p.split_slots = d.split_slots;
     p.n_groups = h->n_groups;
     p.M = h->oc;
@@ -1308,7 +1310,7 @@ int pl_sparse_conv_set_epilogue(pl_sparse_conv_handle* h, const float* scale, co
   if (scale && !h->int8) return Fail(PL_ERR_BAD_ARG, "floating-point kernels take no scales");
   int rc = h->half ? UploadHalfBias(h, bias) : UploadEpilogue(h, scale, bias);
   if (rc != PL_OK) return rc;
-  for (TileWalkStreams* tw : {&h->tw, &h->tw_narrow}) {
+  for (TileWalkStreams* tw : {&h->tw, &h->tw_narrow, &h->tw_slim}) {
     if (!bias || !tw->built) continue;
     // the tile walk starts its accumulators from the bias in its header records
     for (const auto& slot : tw->bias_slots) {

@@ -102,7 +102,8 @@ hipError_t LaunchChunkWalk(int nrows, const ChunkWalkParams& p, hipStream_t stre
 // groups of list stream s.
 constexpr int kTileWalkTile = 128;
 constexpr int kTileWalkRagged = 4;      // flag in TileWalkParams::pairs
-constexpr int kTileWalkNarrowTile = 64;  // for channel counts whose 128-position tile does not fit LDS (pairs only)
+constexpr int kTileWalkNarrowTile = 64;
+constexpr int kTileWalkSlimTile = 32;    // one position per lane: up to 1087 channels  // for channel counts whose 128-position tile does not fit LDS (pairs only)
 constexpr int kTileWalkWaves = 16;
 constexpr int kTileWalkChunkBytes = 1536;  // piece of a list stream held in LDS per wavefront
 
@@ -132,7 +133,8 @@ struct TileWalkParams {
   // 1: the streams hold pairs of row groups, padded to one length, as double records (first group's record, second
   // group's record): lanes 0 - 31 walk the first group, lanes 32 - 63 the second, four positions per lane
   // 2: pairs on tiles of kTileWalkNarrowTile positions, two per lane (streams made for 256-byte channel rows)
-  // + kTileWalkRagged (with 1 or 2): hw is not a multiple of 4; tile and outputs are moved element by element
+  // 3: pairs on tiles of kTileWalkSlimTile positions, one per lane (streams made for 128-byte channel rows)
+  // + kTileWalkRagged (with 1, 2 or 3): hw is not a multiple of 4; tile and outputs are moved element by element
   int8_t pairs;
   // The first 56 bytes (kernarg_head.h) end behind act.type: what selects the tile, picks the activation and
   // addresses the first loads.

@@ -23,7 +23,8 @@
 // twice the rate of 8-byte reads) and every LDS instruction, address add and loop step serves two row groups;
 // the shorter group of a pair is padded with entries of weight zero at the tile's zero row.
 // With more channels than a tile of 128 positions holds in LDS, the pairs walk tiles of 64 positions, two per
-// lane (NARROW; channel rows of 256 bytes, list streams made for those).
+// lane (TILE = 64; channel rows of 256 bytes, list streams made for those), and tiles of 32 positions, one per lane,
+// beyond that (TILE = 32, up to 1087 channels).
 // Maps whose size is not a multiple of 4 (RAGGED, pairs only): neighbouring positions of a tile may lie in
 // different images, so the tile is staged and the outputs are stored element by element (a thread stages the
 // positions c, c + 32, ... of a channel row, a lane stores each of its positions through its own address); the
@@ -73,15 +74,15 @@ constexpr int kWaves = kTileWalkWaves;  // wavefronts per workgroup = list strea
 constexpr int kChunkBytes = kTileWalkChunkBytes;
 
 // One tile: stage it, then walk the streams of one part (0 main, 1 spare).
-template <int NR, int ACT, bool PAIR, bool NARROW, bool RAGGED>
+template <int NR, int ACT, bool PAIR, int TILE, bool RAGGED>
 __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile, int tile_id, int part) {
-  static_assert(PAIR || !NARROW, "narrow tiles are walked in pairs");
+  static_assert(PAIR || TILE == kTileWalkTile, "narrow tiles are walked in pairs");
   static_assert(PAIR || !RAGGED, "maps of any size are walked in pairs");
   constexpr int kRecBytes = NR == 2 ? 48 : 32;  // four byte offsets, then 4 * NR weights
   constexpr int kStepBytes = PAIR ? 2 * kRecBytes : kRecBytes;  // what one step of the walk reads: one record per row group
   constexpr int kRecs = kChunkBytes / kStepBytes;
-  constexpr int PPL = PAIR && !NARROW ? 4 : 2;  // positions per lane
-  constexpr int kTP = NARROW ? kTileWalkNarrowTile : kTileWalkTile;  // positions per workgroup
+  constexpr int PPL = PAIR ? TILE / 32 : 2;  // positions per lane
+  constexpr int kTP = TILE;                  // positions per workgroup
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int sidx = part * kWaves + wave;
@@ -276,7 +277,7 @@ __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile
 // Workgroup id -> tiles: each XCD (linear id mod 8) owns a contiguous range of
 // tiles.  Its first workgroups take one tile each (main part); with a spare
 // part, the workgroups behind them share the range's tiles among themselves.
-template <int NR, int ACT, bool PAIR, bool NARROW, bool RAGGED>
+template <int NR, int ACT, bool PAIR, int TILE, bool RAGGED>
 __device__ __forceinline__ void TileWalkBody(const TileWalkParams& p, float* tile) {
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int first = (xcd * p.tiles) >> 3, last = ((xcd + 1) * p.tiles) >> 3;
@@ -284,17 +285,17 @@ __device__ __forceinline__ void TileWalkBody(const TileWalkParams& p, float* til
   if (p.split == 2) {
     // equal parts: part = slot / count of tile slot % count
     const int part = count > 0 ? slot / count : p.parts;
-    if (part < p.parts) WalkOneTile<NR, ACT, PAIR, NARROW, RAGGED>(p, tile, first + (slot - part * count), part);
+    if (part < p.parts) WalkOneTile<NR, ACT, PAIR, TILE, RAGGED>(p, tile, first + (slot - part * count), part);
     return;
   }
   if (slot < count) {
-    WalkOneTile<NR, ACT, PAIR, NARROW, RAGGED>(p, tile, first + slot, 0);
+    WalkOneTile<NR, ACT, PAIR, TILE, RAGGED>(p, tile, first + slot, 0);
     return;
   }
   if (p.split == 0) return;
   const int n_spare = (int)(gridDim.x >> 3) - count;
   for (int t = first + (slot - count); t < last; t += n_spare) {
-    WalkOneTile<NR, ACT, PAIR, NARROW, RAGGED>(p, tile, t, 1);
+    WalkOneTile<NR, ACT, PAIR, TILE, RAGGED>(p, tile, t, 1);
     __syncthreads();  // every wavefront has left the tile before the next one is staged
   }
 }
@@ -307,19 +308,25 @@ __global__ void __launch_bounds__(64 * kTileWalkWaves) TileWalkKernel(PL_HEAD_PA
     constexpr int ACT = decltype(act_c)::value;
     switch (p.pairs) {
       case 0:
-        TileWalkBody<NR, ACT, false, false, false>(p, tile_lds);
+        TileWalkBody<NR, ACT, false, kTileWalkTile, false>(p, tile_lds);
         break;
       case 1:
-        TileWalkBody<NR, ACT, true, false, false>(p, tile_lds);
+        TileWalkBody<NR, ACT, true, kTileWalkTile, false>(p, tile_lds);
         break;
       case 2:
-        TileWalkBody<NR, ACT, true, true, false>(p, tile_lds);
+        TileWalkBody<NR, ACT, true, kTileWalkNarrowTile, false>(p, tile_lds);
+        break;
+      case 3:
+        TileWalkBody<NR, ACT, true, kTileWalkSlimTile, false>(p, tile_lds);
         break;
       case 1 | kTileWalkRagged:
-        TileWalkBody<NR, ACT, true, false, true>(p, tile_lds);
+        TileWalkBody<NR, ACT, true, kTileWalkTile, true>(p, tile_lds);
         break;
-      default:  // 2 | kTileWalkRagged
-        TileWalkBody<NR, ACT, true, true, true>(p, tile_lds);
+      case 2 | kTileWalkRagged:
+        TileWalkBody<NR, ACT, true, kTileWalkNarrowTile, true>(p, tile_lds);
+        break;
+      default:  // 3 | kTileWalkRagged
+        TileWalkBody<NR, ACT, true, kTileWalkSlimTile, true>(p, tile_lds);
         break;
     }
   });
@@ -333,8 +340,8 @@ hipError_t LaunchTileWalk(int nrows, const TileWalkParams& p, hipStream_t stream
   if (p.P == 0 || p.n_groups == 0) return hipSuccess;
   const int form = p.pairs & 3;
   const bool ragged = (p.pairs & kTileWalkRagged) != 0;
-  if (form > 2 || (ragged && form == 0) || (!ragged && p.hw % 4 != 0)) return hipErrorInvalidValue;
-  const int tile = form == 2 ? kTileWalkNarrowTile : kTileWalkTile;
+  if ((ragged && form == 0) || (!ragged && p.hw % 4 != 0)) return hipErrorInvalidValue;
+  const int tile = form == 3 ? kTileWalkSlimTile : form == 2 ? kTileWalkNarrowTile : kTileWalkTile;
   const size_t lds = TileWalkLdsBytes(p.K, tile * 4);
   if (lds > (size_t)kMaxLdsBytes) return hipErrorInvalidValue;
   TileWalkParams q = p;

@@ -187,6 +187,8 @@ TILED_SHAPES = [(2, 64, 8, 4, 4), (1, 96, 48, 8, 6), (3, 130, 67, 4, 5), (1, 271
 # map sizes that are not a multiple of 4 (the tile is staged and stored element by element): 7 x 7, single
 # pixels (four neighbouring positions in four images), 3 x 5 and 13 x 13, on tiles of 128 and of 64 positions
 TILED_SHAPES += [(3, 64, 48, 7, 7), (9, 96, 33, 1, 1), (2, 130, 67, 3, 5), (4, 256, 96, 9, 9), (2, 300, 40, 7, 7), (1, 512, 64, 13, 13)]
+# 544 - 1087 channels: tiles of 32 positions, one per lane; aligned maps and a 7 x 7 one
+TILED_SHAPES += [(2, 544, 20, 4, 4), (1, 1024, 48, 6, 6), (2, 1087, 9, 2, 2), (3, 800, 33, 7, 7)]
 
 
 @pytest.mark.parametrize("act", ["none", "relu6", "hswish"])
