@@ -131,6 +131,8 @@ struct TileWalkStreams {
   DevBuf stream, first, desc;
   int built = 0;  // uploaded
   int row_bytes = 0;  // bytes per channel row of the LDS tile the byte offsets in the records are made for
+  int groups = 1;     // row groups per step of a stream (records side by side)
+  int form = 0;       // fp32: TileWalkParams::pairs without flags
   // host copy of the streams and, per header record, (word index of its bias, first row | rows << 24):
   // the headers carry the bias, so a new bias is patched in here and the streams are uploaded again
   std::vector<uint32_t> host_stream;
@@ -157,12 +159,11 @@ struct pl_sparse_conv_handle {
   // fp32 row walk over channel chunks (built beside the plain form)
   DevBuf cw_desc, cw_idx, cw_wts;
   int cw_chunks = 0, cw_slices = 0;
-  // tile walk (whole tile and lists in LDS): fp32 with 128 positions per tile, half precision with 256; tw_narrow:
-  // 256-byte channel rows - half precision with 128 positions per tile, for more channels and for maps whose
-  // size is a multiple of 4 but not of 8; fp32 with 64 positions per tile (pairs only), built when the channels do
-  // not fit the wide tile
-  // tw_slim: fp32 with 32 positions per tile (128-byte channel rows), built when the narrow tile does not fit either
-  TileWalkStreams tw, tw_narrow, tw_slim;
+  // tile walk (whole tile and lists in LDS).  tw: fp32 in the form with the largest tile that holds all channels
+  // (128 positions, or 64 / 32 / 16 with 4 / 8 / 16 row groups per step); half precision with 256 positions per
+  // tile.  tw_narrow: half precision with 128 positions per tile (256-byte channel rows), for more channels and for
+  // maps whose size is a multiple of 4 but not of 8.
+  TileWalkStreams tw, tw_narrow;
   int walk_split = -1;          // sixteenths of the row groups' work dealt to the CUs without a tile: -1 by rule, 0 never, 1 .. 8 forced
   int walk_tiled = 1;            // 0 never, 1 when the problem suits it, 2 whenever the shape allows
   bool walk_pairs = true;        // the tile walk's streams hold pairs of row groups (two per wavefront instruction)
@@ -201,7 +202,7 @@ struct pl_sparse_conv_handle {
   int padded_rows = 0;
 
   int64_t DeviceBytes() const {
-    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + cw_desc.bytes + cw_idx.bytes + cw_wts.bytes + hw_kidx.bytes + hw_wts.bytes + hw_bias.bytes + wblocks.bytes + kmask.bytes + wtiles.bytes + wtiles_rg.bytes + wtiles_tr.bytes + wtiles_rows.bytes + tw.DeviceBytes() + tw_narrow.DeviceBytes() + tw_slim.DeviceBytes() + scale.bytes + bias.bytes);
+    return static_cast<int64_t>(groups.bytes + kidx.bytes + wts.bytes + cw_desc.bytes + cw_idx.bytes + cw_wts.bytes + hw_kidx.bytes + hw_wts.bytes + hw_bias.bytes + wblocks.bytes + kmask.bytes + wtiles.bytes + wtiles_rg.bytes + wtiles_tr.bytes + wtiles_rows.bytes + tw.DeviceBytes() + tw_narrow.DeviceBytes() + scale.bytes + bias.bytes);
   }
 };
 
@@ -401,9 +402,10 @@ uint32_t DoubledHalf(uint32_t float_bits) {
   return b | (b << 16);
 }
 
-int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_handle* h, TileWalkStreams* tw, bool half = false, int row_bytes = pl::kTileWalkTile * 4) {
+int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_handle* h, TileWalkStreams* tw, bool half, int row_bytes, int groups_per_step) {
   tw->built = 0;
   tw->row_bytes = row_bytes;
+  tw->groups = groups_per_step;
   if (pl::TileWalkLdsBytes(L.ic, row_bytes) > static_cast<size_t>(pl::kMaxLdsBytes)) return PL_OK;  // too many channels for one tile: other walks
   const int nr = L.semi ? 2 : 1;
   const int streams = pl::kTileWalkWaves;
@@ -411,30 +413,30 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
   std::vector<int> order(n_groups);
   for (int g = 0; g < n_groups; ++g) order[g] = g;
   std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return L.groups[a].count > L.groups[b].count; });
-  // A unit is what one wavefront instruction walks: one row group, or (walk_pairs) two of about the same
-  // length - neighbours in the order by length - of which the shorter is padded with entries of weight zero that
-  // point at the tile's zero row; a last group without a partner gets an empty one (no rows).
-  const bool pairs = half || h->walk_pairs;
+  // A unit is what one wavefront instruction walks: one row group, or G of about the same length - neighbours
+  // in the order by length - of which the shorter ones are padded with entries of weight zero that point at the
+  // tile's zero row; a last unit without enough groups gets empty ones (no rows).
+  constexpr int kMaxG = 16;
+  const int G = groups_per_step;
+  if (G < 1 || G > kMaxG) return Fail(PL_ERR_BAD_ARG, "bad number of row groups per step");
   auto word = [&](uint32_t float_bits) { return half ? DoubledHalf(float_bits) : float_bits; };
   struct Unit {
-    int a, b;        // row groups (b = -1: none)
+    int g[kMaxG];    // row groups (-1: none)
     uint32_t count;  // entries walked
   };
   std::vector<Unit> units;
-  if (pairs) {
-    for (int i = 0; i < n_groups; i += 2) {
-      const int a = order[i], b = i + 1 < n_groups ? order[i + 1] : -1;
-      units.push_back({a, b, L.groups[a].count});  // sorted: a is the longer one
-    }
-  } else {
-    for (int g : order) units.push_back({g, -1, L.groups[g].count});
+  for (int i = 0; i < n_groups; i += G) {
+    Unit un;
+    for (int k = 0; k < kMaxG; ++k) un.g[k] = k < G && i + k < n_groups ? order[i + k] : -1;
+    un.count = L.groups[un.g[0]].count;  // sorted: the first is the longest
+    units.push_back(un);
   }
   const int n_units = static_cast<int>(units.size());
   std::vector<int> unit_order(n_units);
   for (int u = 0; u < n_units; ++u) unit_order[u] = u;
   auto work = [&](int u) { return static_cast<int64_t>((units[u].count + 3) / 4 + 2); };  // batches, plus the unit's epilogue
   const uint32_t rec_words = 4 + 4 * nr;
-  const uint32_t unit_words = pairs ? 2 * rec_words : rec_words;  // a double record per step of a pair
+  const uint32_t unit_words = static_cast<uint32_t>(G) * rec_words;  // the records of a step side by side
   const uint32_t chunk_words = pl::kTileWalkChunkBytes / 4;
   const uint32_t recs_per_chunk = chunk_words / unit_words;
   const uint32_t zero_row = static_cast<uint32_t>(L.ic) * static_cast<uint32_t>(row_bytes);
@@ -471,9 +473,9 @@ int BuildTileWalk(const pl::DecodedLayout& L, const float* bias, pl_sparse_conv_
       };
       for (int u : members[s2]) {
         const Unit& un = units[u];
-        uint32_t rec[24] = {0};
-        const int side_groups[2] = {un.a, un.b};
-        const int sides = pairs ? 2 : 1;
+        uint32_t rec[kMaxG * 12] = {0};
+        const int* side_groups = un.g;
+        const int sides = G;
         for (int side = 0; side < sides; ++side) {
           uint32_t* r = rec + side * rec_words;
           r[1] = un.count;
@@ -880,8 +882,8 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
     h->algo = PL_ALGO_ROW_WALK;
     int hrc = BuildHalfWalk(L, h);
     if (hrc == PL_OK) hrc = BuildChunkWalk(L, h, true);
-    if (hrc == PL_OK) hrc = BuildTileWalk(L, desc->bias, h, &h->tw, true);
-    if (hrc == PL_OK) hrc = BuildTileWalk(L, desc->bias, h, &h->tw_narrow, true, pl::kHalfTileWalkNarrowTile * 2);
+    if (hrc == PL_OK) hrc = BuildTileWalk(L, desc->bias, h, &h->tw, true, pl::kHalfTileWalkTile * 2, 2);
+    if (hrc == PL_OK) hrc = BuildTileWalk(L, desc->bias, h, &h->tw_narrow, true, pl::kHalfTileWalkNarrowTile * 2, 2);
     if (hrc == PL_OK) hrc = UploadHalfBias(h, desc->bias);
     if (hrc != PL_OK) {
       delete h;
@@ -918,9 +920,16 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   if (rc == PL_OK && h->wtiles.ptr && pl::ImageMfmaRegroupsByTransposingReads(desc->ic, 196)) rc = BuildImageMfmaTrRegroup(L, h);
   if (rc == PL_OK && h->wtiles.ptr && pl::ImageRowsMfmaFits(desc->oc, desc->ic, 16)) rc = BuildImageRowsMfma(L, h);
   if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8) rc = BuildChunkWalk(L, h);
-  if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8 && !half) rc = BuildTileWalk(L, desc->bias, h, &h->tw);
-  if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8 && !half && !h->tw.built && h->walk_pairs) rc = BuildTileWalk(L, desc->bias, h, &h->tw_narrow, false, pl::kTileWalkNarrowTile * 4);
-  if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8 && !half && !h->tw.built && !h->tw_narrow.built && h->walk_pairs) rc = BuildTileWalk(L, desc->bias, h, &h->tw_slim, false, pl::kTileWalkSlimTile * 4);
+  if (rc == PL_OK && algo == PL_ALGO_ROW_WALK && !int8 && !half) {
+    // the form with the largest tile that holds all channels in LDS: 128 positions (pairs of row groups, or single
+    // ones on request), else 64 / 32 / 16 positions with 4 / 8 / 16 row groups per step
+    for (int form = h->walk_pairs ? 1 : 0; form < (h->walk_pairs ? pl::kTileWalkForms : 1); ++form) {
+      if (pl::TileWalkLdsBytes(desc->ic, pl::TileWalkTileOf(form) * 4) > static_cast<size_t>(pl::kMaxLdsBytes)) continue;
+      h->tw.form = form;
+      rc = BuildTileWalk(L, desc->bias, h, &h->tw, false, pl::TileWalkTileOf(form) * 4, pl::TileWalkGroupsOf(form));
+      break;
+    }
+  }
   if (rc == PL_OK) {
     // the MFMA epilogues always read a bias; give them zeros when the op has none
     std::vector<float> zeros;
@@ -1175,20 +1184,20 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     c.sub_tiles = h->mfma_sub_tiles;
     if (h->mfma_tile_quads > 0) c.tile_quads = h->mfma_tile_quads;
     e = pl::LaunchBlockMfma(c, p, s);
-  } else if (!h->int8 && !h->half && (vec || (h->walk_pairs && reinterpret_cast<uintptr_t>(x_dev) % 4 == 0 && reinterpret_cast<uintptr_t>(out_dev) % 4 == 0)) &&
-             (h->tw.built != 0 || h->tw_narrow.built != 0 || h->tw_slim.built != 0) && h->walk_tiled > 0 &&
-             (h->walk_tiled == 2 || (vec ? 32 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), h->tw.built ? pl::kTileWalkTile : h->tw_narrow.built ? pl::kTileWalkNarrowTile : pl::kTileWalkSlimTile)) >= h->wg_slots_default
+  } else if (!h->int8 && !h->half && h->tw.built != 0 && h->walk_tiled > 0 &&
+             (vec || (h->tw.form != 0 && reinterpret_cast<uintptr_t>(x_dev) % 4 == 0 && reinterpret_cast<uintptr_t>(out_dev) % 4 == 0)) &&
+             (h->walk_tiled == 2 || (vec ? 32 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::TileWalkTileOf(h->tw.form))) >= h->wg_slots_default
                                          // the other walks move such tensors element by element too and lose earlier: measured
                                          // crossover at 400 - 700 positions with row pairs, 50 - 200 without (256 CUs)
                                          : (h->semi ? 4 : 14) * static_cast<int64_t>(P) >= 5 * static_cast<int64_t>(h->wg_slots_default)))) {
     // fp32 with tiles for at least a sixteenth of the CUs (the
     // row groups of a tile are shared between up to ten CUs; measured
     // crossover against the other walks between 13 and 25 tiles on 256 CUs):
-    // the walk with the tile and the lists in LDS - tiles of 128 positions, of 64 where
-    // only those fit LDS with all channels; element by element in and out of the tile where the map size is
-    // not a multiple of 4 or the tensors are not 16-byte aligned
-    const TileWalkStreams& tw = h->tw.built ? h->tw : h->tw_narrow.built ? h->tw_narrow : h->tw_slim;
-    const int tile = h->tw.built ? pl::kTileWalkTile : h->tw_narrow.built ? pl::kTileWalkNarrowTile : pl::kTileWalkSlimTile;
+    // the walk with the tile and the lists in LDS, in the form the streams were made for (tiles of 128 positions, or
+    // smaller ones where only those hold all channels); element by element in and out of the tile where the map
+    // size is not a multiple of 4 or the tensors are not 16-byte aligned
+    const TileWalkStreams& tw = h->tw;
+    const int tile = pl::TileWalkTileOf(tw.form);
     pl::TileWalkParams p{};
     p.x = static_cast<const float*>(x_dev);
     p.out = static_cast<float*>(out_dev);
@@ -1198,7 +1207,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.stream_groups = static_cast<const uint32_t*>(tw.desc.ptr) + d.table;
     p.split = static_cast<int16_t>(d.split);
     p.parts = static_cast<int8_t>(d.parts);
-    p.pairs = static_cast<int8_t>((h->tw.built ? (h->walk_pairs ? 1 : 0) : h->tw_narrow.built ? 2 : 3) | (vec ? 0 : pl::kTileWalkRagged));
+    p.pairs = static_cast<int8_t>(tw.form | (vec ? 0 : pl::kTileWalkRagged));
     p.split_slots = d.split_slots;
     p.n_groups = h->n_groups;
     p.M = h->oc;
@@ -1310,7 +1319,7 @@ int pl_sparse_conv_set_epilogue(pl_sparse_conv_handle* h, const float* scale, co
   if (scale && !h->int8) return Fail(PL_ERR_BAD_ARG, "floating-point kernels take no scales");
   int rc = h->half ? UploadHalfBias(h, bias) : UploadEpilogue(h, scale, bias);
   if (rc != PL_OK) return rc;
-  for (TileWalkStreams* tw : {&h->tw, &h->tw_narrow, &h->tw_slim}) {
+  for (TileWalkStreams* tw : {&h->tw, &h->tw_narrow}) {
     if (!bias || !tw->built) continue;
     // the tile walk starts its accumulators from the bias in its header records
     for (const auto& slot : tw->bias_slots) {

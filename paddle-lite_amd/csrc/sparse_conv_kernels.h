@@ -101,9 +101,12 @@ hipError_t LaunchChunkWalk(int nrows, const ChunkWalkParams& p, hipStream_t stre
 // kTileWalkTile positions with all input channels; wavefront s walks the row
 // groups of list stream s.
 constexpr int kTileWalkTile = 128;
-constexpr int kTileWalkRagged = 4;      // flag in TileWalkParams::pairs
-constexpr int kTileWalkNarrowTile = 64;
-constexpr int kTileWalkSlimTile = 32;    // one position per lane: up to 1087 channels  // for channel counts whose 128-position tile does not fit LDS (pairs only)
+constexpr int kTileWalkRagged = 8;      // flag in TileWalkParams::pairs
+// TileWalkParams::pairs without the flag: the form.  0: one row group per wavefront instruction, 1: two (tiles of
+// 128 positions both), 2: four on tiles of 64 positions, 3: eight on tiles of 32, 4: sixteen on tiles of 16.
+constexpr int kTileWalkForms = 5;
+constexpr int TileWalkGroupsOf(int form) { return 1 << form; }
+constexpr int TileWalkTileOf(int form) { return form <= 1 ? kTileWalkTile : 256 >> form; }  // for channel counts whose 128-position tile does not fit LDS (pairs only)
 constexpr int kTileWalkWaves = 16;
 constexpr int kTileWalkChunkBytes = 1536;  // piece of a list stream held in LDS per wavefront
 
@@ -130,11 +133,10 @@ struct TileWalkParams {
   // parts x kTileWalkWaves entries.
   int16_t split;
   int8_t parts;
-  // 1: the streams hold pairs of row groups, padded to one length, as double records (first group's record, second
-  // group's record): lanes 0 - 31 walk the first group, lanes 32 - 63 the second, four positions per lane
-  // 2: pairs on tiles of kTileWalkNarrowTile positions, two per lane (streams made for 256-byte channel rows)
-  // 3: pairs on tiles of kTileWalkSlimTile positions, one per lane (streams made for 128-byte channel rows)
-  // + kTileWalkRagged (with 1, 2 or 3): hw is not a multiple of 4; tile and outputs are moved element by element
+  // The form (above).  From 1 on the streams hold 2, 4, 8 or 16 row groups per step, padded to one length, their
+  // records side by side: lanes [0, 64 / groups) walk the first group, the next 64 / groups lanes the second, ...,
+  // four positions per lane; the byte offsets in the records are made for channel rows of the form's tile.
+  // + kTileWalkRagged (not with form 0): hw is not a multiple of 4; tile and outputs are moved element by element
   int8_t pairs;
   // The first 56 bytes (kernarg_head.h) end behind act.type: what selects the tile, picks the activation and
   // addresses the first loads.

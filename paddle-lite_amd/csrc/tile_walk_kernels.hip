@@ -22,10 +22,11 @@
 // groups side by side in the stream.  The activations are then read 16 bytes per lane (LDS delivers those at
 // twice the rate of 8-byte reads) and every LDS instruction, address add and loop step serves two row groups;
 // the shorter group of a pair is padded with entries of weight zero at the tile's zero row.
-// With more channels than a tile of 128 positions holds in LDS, the pairs walk tiles of 64 positions, two per
-// lane (TILE = 64; channel rows of 256 bytes, list streams made for those), and tiles of 32 positions, one per lane,
-// beyond that (TILE = 32, up to 1087 channels).
-// Maps whose size is not a multiple of 4 (RAGGED, pairs only): neighbouring positions of a tile may lie in
+// With more channels than a tile of 128 positions holds in LDS, the tile shrinks and a wavefront instruction walks
+// more row groups, always four positions per lane: four groups on tiles of 64 positions (16 lanes each, up to 543
+// channels), eight on tiles of 32 (1087), sixteen on tiles of 16 (2175).  The records of a step's groups lie side
+// by side in the stream, padded to the longest list among them; the streams are made for the tile's channel rows.
+// Maps whose size is not a multiple of 4 (RAGGED, not with single row groups): neighbouring positions of a tile may lie in
 // different images, so the tile is staged and the outputs are stored element by element (a thread stages the
 // positions c, c + 32, ... of a channel row, a lane stores each of its positions through its own address); the
 // walk between the two is the same.
@@ -74,14 +75,17 @@ constexpr int kWaves = kTileWalkWaves;  // wavefronts per workgroup = list strea
 constexpr int kChunkBytes = kTileWalkChunkBytes;
 
 // One tile: stage it, then walk the streams of one part (0 main, 1 spare).
-template <int NR, int ACT, bool PAIR, int TILE, bool RAGGED>
+template <int NR, int ACT, int G, bool RAGGED>
 __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile, int tile_id, int part) {
-  static_assert(PAIR || TILE == kTileWalkTile, "narrow tiles are walked in pairs");
-  static_assert(PAIR || !RAGGED, "maps of any size are walked in pairs");
+  // G row groups per wavefront instruction, LG lanes each
+  constexpr bool PAIR = G > 1;
+  constexpr int LG = 64 / G;
+  constexpr int TILE = G == 1 ? kTileWalkTile : 4 * LG;
+  static_assert(PAIR || !RAGGED, "maps of any size are not walked with single row groups");
   constexpr int kRecBytes = NR == 2 ? 48 : 32;  // four byte offsets, then 4 * NR weights
-  constexpr int kStepBytes = PAIR ? 2 * kRecBytes : kRecBytes;  // what one step of the walk reads: one record per row group
+  constexpr int kStepBytes = G * kRecBytes;  // what one step of the walk reads: one record per row group
   constexpr int kRecs = kChunkBytes / kStepBytes;
-  constexpr int PPL = PAIR ? TILE / 32 : 2;  // positions per lane
+  constexpr int PPL = PAIR ? 4 : 2;  // positions per lane
   constexpr int kTP = TILE;                  // positions per workgroup
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -155,10 +159,10 @@ __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile
   }
   __syncthreads();
 
-  // pairs: the half of the wavefront a lane belongs to picks the record, its place in the half the positions
-  const int half = PAIR ? lane >> 5 : 0;
-  const uint32_t lane8 = PAIR ? 4u * PPL * (uint32_t)(lane & 31) : 8u * (uint32_t)lane;
-  const uint32_t gpos = tile0 + (PAIR ? (uint32_t)PPL * (uint32_t)(lane & 31) : 2u * (uint32_t)lane);
+  // the part of the wavefront a lane belongs to picks the record, its place in the part the positions
+  const int half = lane / LG;
+  const uint32_t lane8 = 4u * PPL * (uint32_t)(lane & (LG - 1));
+  const uint32_t gpos = tile0 + (uint32_t)PPL * (uint32_t)(lane & (LG - 1));
   const bool store_on = gpos < p.P;
   const uint32_t on = store_on ? gpos / (uint32_t)p.hw : 0u, opp = store_on ? gpos % (uint32_t)p.hw : 0u;
   float* obase = p.out + (size_t)on * p.M * p.hw + opp;
@@ -277,7 +281,7 @@ __device__ __forceinline__ void WalkOneTile(const TileWalkParams& p, float* tile
 // Workgroup id -> tiles: each XCD (linear id mod 8) owns a contiguous range of
 // tiles.  Its first workgroups take one tile each (main part); with a spare
 // part, the workgroups behind them share the range's tiles among themselves.
-template <int NR, int ACT, bool PAIR, int TILE, bool RAGGED>
+template <int NR, int ACT, int G, bool RAGGED>
 __device__ __forceinline__ void TileWalkBody(const TileWalkParams& p, float* tile) {
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int first = (xcd * p.tiles) >> 3, last = ((xcd + 1) * p.tiles) >> 3;
@@ -285,17 +289,17 @@ __device__ __forceinline__ void TileWalkBody(const TileWalkParams& p, float* til
   if (p.split == 2) {
     // equal parts: part = slot / count of tile slot % count
     const int part = count > 0 ? slot / count : p.parts;
-    if (part < p.parts) WalkOneTile<NR, ACT, PAIR, TILE, RAGGED>(p, tile, first + (slot - part * count), part);
+    if (part < p.parts) WalkOneTile<NR, ACT, G, RAGGED>(p, tile, first + (slot - part * count), part);
     return;
   }
   if (slot < count) {
-    WalkOneTile<NR, ACT, PAIR, TILE, RAGGED>(p, tile, first + slot, 0);
+    WalkOneTile<NR, ACT, G, RAGGED>(p, tile, first + slot, 0);
     return;
   }
   if (p.split == 0) return;
   const int n_spare = (int)(gridDim.x >> 3) - count;
   for (int t = first + (slot - count); t < last; t += n_spare) {
-    WalkOneTile<NR, ACT, PAIR, TILE, RAGGED>(p, tile, t, 1);
+    WalkOneTile<NR, ACT, G, RAGGED>(p, tile, t, 1);
     __syncthreads();  // every wavefront has left the tile before the next one is staged
   }
 }
@@ -308,25 +312,31 @@ __global__ void __launch_bounds__(64 * kTileWalkWaves) TileWalkKernel(PL_HEAD_PA
     constexpr int ACT = decltype(act_c)::value;
     switch (p.pairs) {
       case 0:
-        TileWalkBody<NR, ACT, false, kTileWalkTile, false>(p, tile_lds);
+        TileWalkBody<NR, ACT, 1, false>(p, tile_lds);
         break;
       case 1:
-        TileWalkBody<NR, ACT, true, kTileWalkTile, false>(p, tile_lds);
+        TileWalkBody<NR, ACT, 2, false>(p, tile_lds);
         break;
       case 2:
-        TileWalkBody<NR, ACT, true, kTileWalkNarrowTile, false>(p, tile_lds);
+        TileWalkBody<NR, ACT, 4, false>(p, tile_lds);
         break;
       case 3:
-        TileWalkBody<NR, ACT, true, kTileWalkSlimTile, false>(p, tile_lds);
+        TileWalkBody<NR, ACT, 8, false>(p, tile_lds);
+        break;
+      case 4:
+        TileWalkBody<NR, ACT, 16, false>(p, tile_lds);
         break;
       case 1 | kTileWalkRagged:
-        TileWalkBody<NR, ACT, true, kTileWalkTile, true>(p, tile_lds);
+        TileWalkBody<NR, ACT, 2, true>(p, tile_lds);
         break;
       case 2 | kTileWalkRagged:
-        TileWalkBody<NR, ACT, true, kTileWalkNarrowTile, true>(p, tile_lds);
+        TileWalkBody<NR, ACT, 4, true>(p, tile_lds);
         break;
-      default:  // 3 | kTileWalkRagged
-        TileWalkBody<NR, ACT, true, kTileWalkSlimTile, true>(p, tile_lds);
+      case 3 | kTileWalkRagged:
+        TileWalkBody<NR, ACT, 8, true>(p, tile_lds);
+        break;
+      default:  // 4 | kTileWalkRagged
+        TileWalkBody<NR, ACT, 16, true>(p, tile_lds);
         break;
     }
   });
@@ -338,10 +348,10 @@ size_t TileWalkLdsBytes(int K, int row_bytes) { return (size_t)(K + 1) * (size_t
 
 hipError_t LaunchTileWalk(int nrows, const TileWalkParams& p, hipStream_t stream) {
   if (p.P == 0 || p.n_groups == 0) return hipSuccess;
-  const int form = p.pairs & 3;
+  const int form = p.pairs & (kTileWalkRagged - 1);
   const bool ragged = (p.pairs & kTileWalkRagged) != 0;
-  if ((ragged && form == 0) || (!ragged && p.hw % 4 != 0)) return hipErrorInvalidValue;
-  const int tile = form == 3 ? kTileWalkSlimTile : form == 2 ? kTileWalkNarrowTile : kTileWalkTile;
+  if (form > 4 || (ragged && form == 0) || (!ragged && p.hw % 4 != 0)) return hipErrorInvalidValue;
+  const int tile = TileWalkTileOf(form);
   const size_t lds = TileWalkLdsBytes(p.K, tile * 4);
   if (lds > (size_t)kMaxLdsBytes) return hipErrorInvalidValue;
   TileWalkParams q = p;

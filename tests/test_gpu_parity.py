@@ -176,8 +176,8 @@ def test_fp32_chunked_walk(shape, paired, act):
 
 # fp32 walk with the whole tile and the index lists in LDS (128 positions and
 # sixteen list streams per workgroup); forced here, the library picks it by
-# itself for large problems.  Needs H*W % 4 == 0 and at most 271 channels;
-# with 272 - 543 channels the tiles have 64 positions (pairs of row groups only).
+# itself for large problems.  At most 271 channels; with 272 - 543 channels
+# the tiles have 64 positions and a wavefront instruction walks four row groups.
 # (batch, ic, oc, h, w): fewer row groups than streams, more, an odd row
 # count, a tile that spans images, a last tile that is not full, the largest
 # channel count, lists longer than one LDS piece; then tiles of 64: the
@@ -187,8 +187,9 @@ TILED_SHAPES = [(2, 64, 8, 4, 4), (1, 96, 48, 8, 6), (3, 130, 67, 4, 5), (1, 271
 # map sizes that are not a multiple of 4 (the tile is staged and stored element by element): 7 x 7, single
 # pixels (four neighbouring positions in four images), 3 x 5 and 13 x 13, on tiles of 128 and of 64 positions
 TILED_SHAPES += [(3, 64, 48, 7, 7), (9, 96, 33, 1, 1), (2, 130, 67, 3, 5), (4, 256, 96, 9, 9), (2, 300, 40, 7, 7), (1, 512, 64, 13, 13)]
-# 544 - 1087 channels: tiles of 32 positions, one per lane; aligned maps and a 7 x 7 one
-TILED_SHAPES += [(2, 544, 20, 4, 4), (1, 1024, 48, 6, 6), (2, 1087, 9, 2, 2), (3, 800, 33, 7, 7)]
+# 544 - 1087 channels: tiles of 32 positions, eight row groups per wavefront instruction; 1088 - 2175: tiles of 16,
+# sixteen row groups; aligned maps and 7 x 7 / 3 x 3 ones, fewer row groups than a step holds
+TILED_SHAPES += [(2, 544, 20, 4, 4), (1, 1024, 48, 6, 6), (2, 1087, 9, 2, 2), (3, 800, 33, 7, 7), (1, 2048, 40, 4, 4), (2, 2175, 9, 2, 2), (2, 1500, 70, 3, 3)]
 
 
 @pytest.mark.parametrize("act", ["none", "relu6", "hswish"])
