@@ -361,7 +361,6 @@ typedef uint32_t u2w __attribute__((ext_vector_type(2)));
 typedef uint32_t u4w __attribute__((ext_vector_type(4)));
 constexpr int kTwWaves = kTileWalkWaves;
 constexpr int kTwChunkBytes = kTileWalkChunkBytes;
-static_assert(kHalfTileWalkTile == 32 * 8 && kHalfTileWalkNarrowTile == 32 * 4, "32 lanes of a row group times the positions per lane");
 static_assert(kHalfTileWalkTile * 2 == kTileWalkTile * 4, "the wide tile's list streams hold the byte offsets of the fp32 walk's channel rows");
 
 // what a lane holds of a channel row: PPL positions
@@ -379,12 +378,14 @@ struct TwPiece<4> {
 // One tile: stage it, then walk the streams of one part (0 main, 1 spare).
 // RAGGED: the map size is not a multiple of the lane's piece (or the tensors are not aligned to it), so the tile is
 // staged and the outputs are stored one binary16 value at a time, each through its own address.
-template <int NR, int PPL, int ACT, bool RAGGED>
+// G row groups per wavefront instruction (LG = 64 / G lanes each) on tiles of LG * PPL positions.
+template <int NR, int G, int PPL, int ACT, bool RAGGED>
 __device__ __forceinline__ void HalfWalkOneTile(const HalfTileWalkParams& p, char* tile_bytes, int tile_id, int part) {
   typedef typename TwPiece<PPL>::type Piece;
-  constexpr int kTwTile = 32 * PPL, kTwRowBytes = kTwTile * 2, kPieceBytes = 2 * PPL, NW = PPL / 2;
+  constexpr int LG = 64 / G, kPassRows = 64 * kTwWaves / LG;
+  constexpr int kTwTile = LG * PPL, kTwRowBytes = kTwTile * 2, kPieceBytes = 2 * PPL, NW = PPL / 2;
   constexpr int kRecBytes = NR == 2 ? 48 : 32;  // four byte offsets, then 4 * NR doubled weights
-  constexpr int kStepBytes = 2 * kRecBytes;     // one record per row group of the pair
+  constexpr int kStepBytes = G * kRecBytes;     // one record per row group of the step
   constexpr int kRecs = kTwChunkBytes / kStepBytes;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -398,43 +399,43 @@ __device__ __forceinline__ void HalfWalkOneTile(const HalfTileWalkParams& p, cha
   u4w pa = *reinterpret_cast<const u4w*>(sp + 16 * lane);
   u2w pb = *reinterpret_cast<const u2w*>(sp + 1024 + 8 * lane);
 
-  // staging: 32 threads per channel row (PPL positions each), 32 rows per pass
+  // staging: LG threads per channel row (PPL positions each), kPassRows rows per pass
   if (RAGGED) {
-    const int c = tid & 31, r0 = tid >> 5;
-    // the thread's positions c + 32 e of the tile: offset of each in channel 0 of its image
+    const int c = tid & (LG - 1), r0 = tid / LG;
+    // the thread's positions c + LG e of the tile: offset of each in channel 0 of its image
     size_t eoff[PPL];
     bool elive[PPL];
 #pragma unroll
     for (int e = 0; e < PPL; ++e) {
-      const uint32_t pos = tile0 + (uint32_t)(c + 32 * e);
+      const uint32_t pos = tile0 + (uint32_t)(c + LG * e);
       elive[e] = pos < p.P;
       const uint32_t n = elive[e] ? pos / (uint32_t)p.hw : 0u;
       const uint32_t pp = elive[e] ? pos % (uint32_t)p.hw : 0u;
       eoff[e] = (size_t)n * p.K * p.hw + pp;
     }
     uint16_t* tile16 = reinterpret_cast<uint16_t*>(tile_bytes);
-    for (int k0 = 0; k0 < p.K; k0 += 128) {
+    for (int k0 = 0; k0 < p.K; k0 += 4 * kPassRows) {
       uint16_t v[4][PPL];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int k = min(k0 + r0 + 32 * u, p.K - 1);
+        const int k = min(k0 + r0 + kPassRows * u, p.K - 1);
 #pragma unroll
         for (int e = 0; e < PPL; ++e) v[u][e] = p.x[eoff[e] + (size_t)k * p.hw];
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int k = k0 + r0 + 32 * u;
+        const int k = k0 + r0 + kPassRows * u;
         if (k < p.K) {
 #pragma unroll
-          for (int e = 0; e < PPL; ++e) tile16[(size_t)k * kTwTile + c + 32 * e] = elive[e] ? v[u][e] : (uint16_t)0;
+          for (int e = 0; e < PPL; ++e) tile16[(size_t)k * kTwTile + c + LG * e] = elive[e] ? v[u][e] : (uint16_t)0;
         }
       }
     }
     Piece zero;
     __builtin_memset(&zero, 0, sizeof(zero));
-    if (tid < 32) *reinterpret_cast<Piece*>(tile_bytes + (size_t)p.K * kTwRowBytes + kPieceBytes * tid) = zero;
+    if (tid < LG) *reinterpret_cast<Piece*>(tile_bytes + (size_t)p.K * kTwRowBytes + kPieceBytes * tid) = zero;
   } else {
-    const int c8 = tid & 31, r0 = tid >> 5;
+    const int c8 = tid & (LG - 1), r0 = tid / LG;
     const uint32_t gpos = tile0 + (uint32_t)PPL * (uint32_t)c8;
     const bool live = gpos < p.P;
     const uint32_t n = live ? gpos / (uint32_t)p.hw : 0u;
@@ -442,27 +443,27 @@ __device__ __forceinline__ void HalfWalkOneTile(const HalfTileWalkParams& p, cha
     const uint16_t* xcol = p.x + (size_t)n * p.K * p.hw + pp;
     Piece zero;
     __builtin_memset(&zero, 0, sizeof(zero));
-    for (int k0 = 0; k0 < p.K; k0 += 128) {
+    for (int k0 = 0; k0 < p.K; k0 += 4 * kPassRows) {
       Piece v[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int k = min(k0 + r0 + 32 * u, p.K - 1);
+        const int k = min(k0 + r0 + kPassRows * u, p.K - 1);
         v[u] = *reinterpret_cast<const Piece*>(xcol + (size_t)k * p.hw);
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int k = k0 + r0 + 32 * u;
+        const int k = k0 + r0 + kPassRows * u;
         if (k < p.K) *reinterpret_cast<Piece*>(tile_bytes + (size_t)k * kTwRowBytes + kPieceBytes * c8) = live ? v[u] : zero;
       }
     }
     // row K is all zero: the target of list padding entries
-    if (tid < 32) *reinterpret_cast<Piece*>(tile_bytes + (size_t)p.K * kTwRowBytes + kPieceBytes * tid) = zero;
+    if (tid < LG) *reinterpret_cast<Piece*>(tile_bytes + (size_t)p.K * kTwRowBytes + kPieceBytes * tid) = zero;
   }
   __syncthreads();
 
-  const int half = lane >> 5;
-  const uint32_t lane16 = (uint32_t)kPieceBytes * (uint32_t)(lane & 31);
-  const uint32_t gpos = tile0 + (uint32_t)PPL * (uint32_t)(lane & 31);
+  const int half = lane / LG;
+  const uint32_t lane16 = (uint32_t)kPieceBytes * (uint32_t)(lane & (LG - 1));
+  const uint32_t gpos = tile0 + (uint32_t)PPL * (uint32_t)(lane & (LG - 1));
   const bool store_on = gpos < p.P;
   const uint32_t on = store_on ? gpos / (uint32_t)p.hw : 0u, opp = store_on ? gpos % (uint32_t)p.hw : 0u;
   uint16_t* obase = p.out + (size_t)on * p.M * p.hw + opp;
@@ -579,67 +580,67 @@ __device__ __forceinline__ void HalfWalkOneTile(const HalfTileWalkParams& p, cha
 // Workgroup id -> tiles, as in the fp32 tile walk: each XCD (linear id mod 8) owns a contiguous range of tiles;
 // its first workgroups take one tile each (main part), with a spare part the workgroups behind them share the
 // range's tiles among themselves, with equal parts `parts` workgroups share every tile.
-template <int NR, int PPL, int ACT, bool RAGGED>
+template <int NR, int G, int PPL, int ACT, bool RAGGED>
 __device__ __forceinline__ void HalfTileWalkBody(const HalfTileWalkParams& p, char* tile) {
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int first = (xcd * p.tiles) >> 3, last = ((xcd + 1) * p.tiles) >> 3;
   const int count = last - first;
   if (p.split == 2) {
     const int part = count > 0 ? slot / count : p.parts;
-    if (part < p.parts) HalfWalkOneTile<NR, PPL, ACT, RAGGED>(p, tile, first + (slot - part * count), part);
+    if (part < p.parts) HalfWalkOneTile<NR, G, PPL, ACT, RAGGED>(p, tile, first + (slot - part * count), part);
     return;
   }
   if (slot < count) {
-    HalfWalkOneTile<NR, PPL, ACT, RAGGED>(p, tile, first + slot, 0);
+    HalfWalkOneTile<NR, G, PPL, ACT, RAGGED>(p, tile, first + slot, 0);
     return;
   }
   if (p.split == 0) return;
   const int n_spare = (int)(gridDim.x >> 3) - count;
   for (int t = first + (slot - count); t < last; t += n_spare) {
-    HalfWalkOneTile<NR, PPL, ACT, RAGGED>(p, tile, t, 1);
+    HalfWalkOneTile<NR, G, PPL, ACT, RAGGED>(p, tile, t, 1);
     __syncthreads();  // every wavefront has left the tile before the next one is staged
   }
 }
 
-template <int NR, int PPL>
+template <int NR, int G, int PPL>
 __global__ void __launch_bounds__(64 * kTileWalkWaves) HalfTileWalkKernel(PL_HEAD_PARAMS, const HalfTileWalkParams block) {
   const HalfTileWalkParams p = WithHead(block, PL_HEAD_ARGS);
   extern __shared__ uint32_t tile32[];
   char* tile = reinterpret_cast<char*>(tile32);
   switch (p.act.type) {
     case 1:
-      if (p.ragged) {
-        HalfTileWalkBody<NR, PPL, 1, true>(p, tile);
+      if (p.form & kTileWalkRagged) {
+        HalfTileWalkBody<NR, G, PPL, 1, true>(p, tile);
       } else {
-        HalfTileWalkBody<NR, PPL, 1, false>(p, tile);
+        HalfTileWalkBody<NR, G, PPL, 1, false>(p, tile);
       }
       break;
     case 2:
-      if (p.ragged) {
-        HalfTileWalkBody<NR, PPL, 2, true>(p, tile);
+      if (p.form & kTileWalkRagged) {
+        HalfTileWalkBody<NR, G, PPL, 2, true>(p, tile);
       } else {
-        HalfTileWalkBody<NR, PPL, 2, false>(p, tile);
+        HalfTileWalkBody<NR, G, PPL, 2, false>(p, tile);
       }
       break;
     case 4:
-      if (p.ragged) {
-        HalfTileWalkBody<NR, PPL, 4, true>(p, tile);
+      if (p.form & kTileWalkRagged) {
+        HalfTileWalkBody<NR, G, PPL, 4, true>(p, tile);
       } else {
-        HalfTileWalkBody<NR, PPL, 4, false>(p, tile);
+        HalfTileWalkBody<NR, G, PPL, 4, false>(p, tile);
       }
       break;
     case 10:
-      if (p.ragged) {
-        HalfTileWalkBody<NR, PPL, 10, true>(p, tile);
+      if (p.form & kTileWalkRagged) {
+        HalfTileWalkBody<NR, G, PPL, 10, true>(p, tile);
       } else {
-        HalfTileWalkBody<NR, PPL, 10, false>(p, tile);
+        HalfTileWalkBody<NR, G, PPL, 10, false>(p, tile);
       }
       break;
     default:
-      if (p.ragged) {
-        HalfTileWalkBody<NR, PPL, 0, true>(p, tile);
+      if (p.form & kTileWalkRagged) {
+        HalfTileWalkBody<NR, G, PPL, 0, true>(p, tile);
       } else {
-        HalfTileWalkBody<NR, PPL, 0, false>(p, tile);
+        HalfTileWalkBody<NR, G, PPL, 0, false>(p, tile);
       }
       break;
   }
@@ -698,12 +699,15 @@ hipError_t LaunchHalfChunkWalk(int nrows, const HalfChunkWalkParams& p, hipStrea
   return nrows == 2 ? HalfChunkLaunch<2, 4>(p, stream) : HalfChunkLaunch<1, 4>(p, stream);
 }
 
-// A lane's positions are one piece of one image: tile 256 needs hw % 8 == 0 and 16-byte aligned x / out, tile 128
-// hw % 4 == 0 and 8-byte alignment; the ragged form (HalfTileWalkParams::ragged) takes any map size.
-hipError_t LaunchHalfTileWalk(int nrows, int tile, const HalfTileWalkParams& p, hipStream_t stream) {
+// A lane's positions are one piece of one image: eight positions per lane need hw % 8 == 0 and 16-byte aligned
+// x / out, four (the narrow form) hw % 4 == 0 and 8-byte alignment; with kTileWalkRagged any map size.
+hipError_t LaunchHalfTileWalk(int nrows, const HalfTileWalkParams& p, hipStream_t stream) {
   if (p.P == 0 || p.n_groups == 0) return hipSuccess;
-  if (tile != kHalfTileWalkTile && tile != kHalfTileWalkNarrowTile) return hipErrorInvalidValue;
-  if (!p.ragged && p.hw % (tile / 32) != 0) return hipErrorInvalidValue;
+  const int form = p.form & (kTileWalkRagged - 1);
+  const bool ragged = (p.form & kTileWalkRagged) != 0;
+  if (form >= kHalfTileWalkForms) return hipErrorInvalidValue;
+  const int tile = HalfTileWalkTileOf(form), ppl = form == kHalfTileWalkNarrowForm ? 4 : 8;
+  if (!ragged && p.hw % ppl != 0) return hipErrorInvalidValue;
   const size_t lds = TileWalkLdsBytes(p.K, tile * 2);
   if (lds > (size_t)kMaxLdsBytes) return hipErrorInvalidValue;
   HalfTileWalkParams q = p;
@@ -717,12 +721,19 @@ hipError_t LaunchHalfTileWalk(int nrows, int tile, const HalfTileWalkParams& p, 
     slots = (uint32_t)q.split_slots;
   }
   dim3 grid(8u * slots), block(64 * kTwWaves);
-  if (tile == kHalfTileWalkTile) {
-    if (nrows == 2) return LaunchWithHead(HalfTileWalkKernel<2, 8>, grid, block, lds, stream, q);
-    return LaunchWithHead(HalfTileWalkKernel<1, 8>, grid, block, lds, stream, q);
+  const bool two = nrows == 2;
+  switch (form) {
+    case 0:
+      return two ? LaunchWithHead(HalfTileWalkKernel<2, 2, 8>, grid, block, lds, stream, q) : LaunchWithHead(HalfTileWalkKernel<1, 2, 8>, grid, block, lds, stream, q);
+    case 1:
+      return two ? LaunchWithHead(HalfTileWalkKernel<2, 4, 8>, grid, block, lds, stream, q) : LaunchWithHead(HalfTileWalkKernel<1, 4, 8>, grid, block, lds, stream, q);
+    case 2:
+      return two ? LaunchWithHead(HalfTileWalkKernel<2, 8, 8>, grid, block, lds, stream, q) : LaunchWithHead(HalfTileWalkKernel<1, 8, 8>, grid, block, lds, stream, q);
+    case 3:
+      return two ? LaunchWithHead(HalfTileWalkKernel<2, 16, 8>, grid, block, lds, stream, q) : LaunchWithHead(HalfTileWalkKernel<1, 16, 8>, grid, block, lds, stream, q);
+    default:  // the narrow form
+      return two ? LaunchWithHead(HalfTileWalkKernel<2, 2, 4>, grid, block, lds, stream, q) : LaunchWithHead(HalfTileWalkKernel<1, 2, 4>, grid, block, lds, stream, q);
   }
-  if (nrows == 2) return LaunchWithHead(HalfTileWalkKernel<2, 4>, grid, block, lds, stream, q);
-  return LaunchWithHead(HalfTileWalkKernel<1, 4>, grid, block, lds, stream, q);
 }
 
 }  // namespace pl

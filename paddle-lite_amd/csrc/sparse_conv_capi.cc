@@ -882,7 +882,14 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
     h->algo = PL_ALGO_ROW_WALK;
     int hrc = BuildHalfWalk(L, h);
     if (hrc == PL_OK) hrc = BuildChunkWalk(L, h, true);
-    if (hrc == PL_OK) hrc = BuildTileWalk(L, desc->bias, h, &h->tw, true, pl::kHalfTileWalkTile * 2, 2);
+    // eight positions per lane in the form with the largest tile that holds all channels; the narrow form beside it
+    for (int form = 0; hrc == PL_OK && form < pl::kHalfTileWalkNarrowForm; ++form) {
+      if (pl::TileWalkLdsBytes(desc->ic, pl::HalfTileWalkTileOf(form) * 2) > static_cast<size_t>(pl::kMaxLdsBytes)) continue;
+      h->tw.form = form;
+      hrc = BuildTileWalk(L, desc->bias, h, &h->tw, true, pl::HalfTileWalkTileOf(form) * 2, pl::HalfTileWalkGroupsOf(form));
+      break;
+    }
+    h->tw_narrow.form = pl::kHalfTileWalkNarrowForm;
     if (hrc == PL_OK) hrc = BuildTileWalk(L, desc->bias, h, &h->tw_narrow, true, pl::kHalfTileWalkNarrowTile * 2, 2);
     if (hrc == PL_OK) hrc = UploadHalfBias(h, desc->bias);
     if (hrc != PL_OK) {
@@ -1030,17 +1037,16 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
   if (h->half && h->walk_tiled > 0) {
     if (h->tw.built != 0 && im_size % 8 == 0 && aligned16) {
       half_tw = &h->tw;
-      half_tile = pl::kHalfTileWalkTile;
     } else if (h->tw_narrow.built != 0 && im_size % 4 == 0 && aligned8) {
       half_tw = &h->tw_narrow;
-      half_tile = pl::kHalfTileWalkNarrowTile;
     } else if (reinterpret_cast<uintptr_t>(x_dev) % 2 == 0 && reinterpret_cast<uintptr_t>(out_dev) % 2 == 0 && (h->tw.built != 0 || h->tw_narrow.built != 0)) {
       // any other map size or alignment: value by value in and out of the tile
       half_tw = h->tw.built != 0 ? &h->tw : &h->tw_narrow;
-      half_tile = h->tw.built != 0 ? pl::kHalfTileWalkTile : pl::kHalfTileWalkNarrowTile;
       half_ragged = true;
     }
-    if (half_tw && h->walk_tiled != 2 && (h->semi ? 42 : 84) * static_cast<int64_t>(CeilDiv(static_cast<int>(P), half_tile)) < h->wg_slots_default) half_tw = nullptr;
+    if (half_tw) half_tile = pl::HalfTileWalkTileOf(half_tw->form);
+    // measured on tiles of 256 and 128 positions; smaller tiles count by positions
+    if (half_tw && h->walk_tiled != 2 && (h->semi ? 42 : 84) * static_cast<int64_t>(CeilDiv(static_cast<int>(P), std::max(half_tile, pl::kHalfTileWalkNarrowTile))) < h->wg_slots_default) half_tw = nullptr;
   }
   if (half_tw) {
     const TileWalkDivision d = DivideTileWalk(h, *half_tw, CeilDiv(static_cast<int>(P), half_tile));
@@ -1052,7 +1058,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.stream_groups = static_cast<const uint32_t*>(half_tw->desc.ptr) + d.table;
     p.split = static_cast<int16_t>(d.split);
     p.parts = static_cast<int8_t>(d.parts);
-    p.ragged = half_ragged ? 1 : 0;
+    p.form = static_cast<int8_t>(half_tw->form | (half_ragged ? pl::kTileWalkRagged : 0));
     p.split_slots = d.split_slots;
     p.n_groups = h->n_groups;
     p.M = h->oc;
@@ -1060,7 +1066,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     p.hw = im_size;
     p.P = P;
     p.act = h->act_h;
-    e = pl::LaunchHalfTileWalk(h->semi ? 2 : 1, half_tile, p, s);
+    e = pl::LaunchHalfTileWalk(h->semi ? 2 : 1, p, s);
   } else if (h->half && (im_size % 4 == 0) && (reinterpret_cast<uintptr_t>(x_dev) % 8 == 0) && (reinterpret_cast<uintptr_t>(out_dev) % 8 == 0) && h->walk_chunked > 0 && h->cw_chunks > 0 &&
       (h->walk_chunked == 2 || (h->ic > 128 && static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kChunkWalkTile)) * h->cw_slices >= 256))) {
     // many channels and enough work for every CU: walk over channel chunks

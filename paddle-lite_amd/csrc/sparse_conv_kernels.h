@@ -191,6 +191,13 @@ hipError_t LaunchHalfChunkWalk(int nrows, const HalfChunkWalkParams& p, hipStrea
 // values doubled into a dword (value | value << 16).
 constexpr int kHalfTileWalkTile = 256;
 constexpr int kHalfTileWalkNarrowTile = 128;
+// HalfTileWalkParams::form without the flag.  0 - 3: 2 / 4 / 8 / 16 row groups per wavefront instruction, eight
+// positions per lane, on tiles of 256 / 128 / 64 / 32 positions (up to 271 / 543 / 1087 / 2175 channels); 4: the narrow
+// form, pairs with four positions per lane on tiles of 128.
+constexpr int kHalfTileWalkForms = 5;
+constexpr int kHalfTileWalkNarrowForm = 4;
+constexpr int HalfTileWalkGroupsOf(int form) { return form == kHalfTileWalkNarrowForm ? 2 : 2 << form; }
+constexpr int HalfTileWalkTileOf(int form) { return form == kHalfTileWalkNarrowForm ? kHalfTileWalkNarrowTile : kHalfTileWalkTile >> form; }
 
 struct HalfTileWalkParams {
   const uint16_t* x;
@@ -203,7 +210,7 @@ struct HalfTileWalkParams {
   int tiles;  // filled in by the launcher
   int16_t split;
   int8_t parts;
-  int8_t ragged;  // 1: the tile is staged and the outputs are stored value by value (any map size and alignment)
+  int8_t form;  // the form (above); + kTileWalkRagged: the tile is staged and the outputs are stored value by value (any map size and alignment)
   // the first 56 bytes (kernarg_head.h) end behind act.type
   DevActH act;
   const uint32_t* stream_groups;
@@ -212,9 +219,9 @@ struct HalfTileWalkParams {
   int split_slots;
 };
 
-// tile: kHalfTileWalkTile (needs hw % 8 == 0 and 16-byte aligned x / out) or kHalfTileWalkNarrowTile (hw % 4 == 0,
-// 8-byte aligned); the streams must be made for that tile's channel rows.
-hipError_t LaunchHalfTileWalk(int nrows, int tile, const HalfTileWalkParams& p, hipStream_t stream);
+// Eight positions per lane need hw % 8 == 0 and 16-byte aligned x / out, the narrow form hw % 4 == 0 and 8-byte
+// alignment, the ragged flag lifts both; the streams must be made for the form's channel rows and groups per step.
+hipError_t LaunchHalfTileWalk(int nrows, const HalfTileWalkParams& p, hipStream_t stream);
 
 struct HalfWalkParams {
   const uint16_t* x;

@@ -83,6 +83,10 @@ TILED_SHAPES += [(3, 64, 48, 14, 14), (7, 40, 33, 2, 2), (2, 257, 20, 6, 6), (1,
 # Any other map size goes in and out of the tile value by value: 7 x 7, single pixels (neighbouring positions in
 # different images), 3 x 5, 9 x 9, 13 x 13, a map of 2 x 3, on tiles of 256 and of 128 positions.
 TILED_SHAPES += [(3, 64, 48, 7, 7), (9, 96, 33, 1, 1), (2, 130, 67, 3, 5), (4, 256, 96, 9, 9), (2, 300, 40, 7, 7), (1, 512, 64, 13, 13), (5, 48, 20, 2, 3)]
+# More channels on maps of a multiple of 8 positions: 4 / 8 / 16 row groups per wavefront instruction on tiles of
+# 128 / 64 / 32 positions (up to 543 / 1087 / 2175 channels); the same with odd maps and with a map of 36 positions
+# whose channels do not fit the narrow form; fewer row groups than a step holds.
+TILED_SHAPES += [(1, 300, 150, 8, 8), (2, 543, 20, 4, 4), (1, 1024, 48, 8, 8), (2, 1087, 9, 2, 4), (1, 2048, 40, 4, 4), (2, 2175, 9, 2, 4), (3, 800, 33, 7, 7), (2, 1500, 70, 3, 3), (2, 600, 20, 6, 6)]
 
 
 @pytest.mark.parametrize("act", ["none", "relu", "relu6", "leaky", "hswish"])
