@@ -67,7 +67,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib", "mobilenet", "density-sweep", "floors", "store-shapes", "device-rates", "custom", "small-batch"])
+    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "calib", "mobilenet", "density-sweep", "floors", "store-shapes", "device-rates", "custom", "small-batch", "float-layers"])
     ap.add_argument("--algo", default="auto", choices=["auto", "walk", "mfma", "image"])
     ap.add_argument("--image-kernel", default="rule", choices=["rule", "regroup", "transpose", "rows"], help="which image MFMA kernel a handle uses where both apply (pl_sparse_conv_tuning.image_kernel)")
     ap.add_argument("--image-regroup", default="rule", choices=["rule", "valu"], help="regrouping image kernel: by transposing LDS reads where that exists (rule) or by the vector ALU everywhere (pl_sparse_conv_tuning.image_tr_regroup)")
@@ -313,6 +313,72 @@ def run_density_sweep(args):
         torch.cuda.empty_cache()
     print(json.dumps({"metric": "int8 sparse 1x1 conv: kernel us per launch by algorithm, sparsity and zero structure", "unit": "us", "n_gpus": 1, "steps": steps, "data": "synthetic",
                       "config": {"workload": "density_sweep", "parity_checked": True}, "rows": rows}))
+    return 0
+
+
+# (batch, ic, oc, h, w): pointwise layers of MobileNet / ResNet / Inception kinds - channel counts on both sides of
+# the limits of the tile walk's forms (271 / 543 / 1087 / 2175), maps of a multiple of 8 positions, of 4 only, and odd.
+FLOAT_LAYERS = [(32, 256, 512, 28, 28), (64, 384, 384, 16, 16), (64, 512, 512, 16, 16), (64, 512, 512, 14, 14), (64, 1024, 1024, 8, 8), (64, 1024, 1024, 7, 7),
+                (32, 1024, 256, 14, 14), (32, 2048, 512, 8, 8), (32, 2048, 512, 7, 7), (32, 256, 512, 27, 27), (8, 128, 256, 55, 55), (64, 192, 384, 17, 17)]
+
+
+def run_float_layers(args):
+    """fp32 and fp16 sparse_conv2d on layers outside the headline configurations, through the three floating-point
+    walks: what the library picks (the walk with the tile and the lists in LDS on all of these), the walk over channel
+    chunks and the plain walk, each forced through pl_sparse_conv_tuning.  Device time per launch (HIP events over
+    400 launches, rotating buffer sets); row pairs at 70 % zeros and unstructured at 85 %.  The three walks must give
+    the same bits; fp32 is also compared with the oracle on one image.  Not the headline metric: its own JSON line."""
+    import numpy as np
+    import torch
+
+    import helpers
+
+    capi, wl, pla = helpers.capi, helpers.workloads, helpers.pla
+    L = capi.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    steps = max(50, min(args.steps, 400))
+    tunings = (("library_choice", None), ("chunk_walk", capi.tuning(walk_tiled=capi.TUNE_NEVER, walk_chunked=capi.TUNE_ALWAYS)),
+               ("plain_walk", capi.tuning(walk_tiled=capi.TUNE_NEVER, walk_chunked=capi.TUNE_NEVER)))
+    rows = []
+    for kind in ("fp32", "fp16"):
+        for paired in (True, False):
+            for batch, ic, oc, h, w in FLOAT_LAYERS:
+                case = wl.make_fp32("layer", batch, ic, oc, h, w, 0.7 if paired else 0.85, paired, pla.ActivationParam("relu"), seed=1)
+                esize, tdt = 4, torch.float32
+                if kind == "fp16":
+                    case.kind = capi.KIND_FP16
+                    case.x = case.x.astype(np.float16)
+                    esize, tdt = 2, torch.float16
+                set_bytes = batch * h * w * (ic + oc) * esize
+                n_sets = max(2, min(24, int(LLC_BYTES * 1.25 // set_bytes) + 1))
+                x0 = torch.from_numpy(case.x).cuda()
+                xs = [x0] + [x0.clone() for _ in range(n_sets - 1)]
+                outs = [torch.empty((batch, oc, h, w), dtype=tdt, device="cuda") for _ in range(n_sets)]
+                xp = (C.c_void_p * n_sets)(*[t.data_ptr() for t in xs])
+                op = (C.c_void_p * n_sets)(*[t.data_ptr() for t in outs])
+                row = {"kind": kind, "zeros": "row pairs, 70 %" if paired else "unstructured, 85 %", "shape": "N=%d %d->%d @%dx%d" % (batch, ic, oc, h, w), "kernel_us": {}}
+                first = None
+                for name, tune in tunings:
+                    kernel, _ = helpers.make_kernel(case, force_semi=paired, tuning=tune)
+                    capi.check(L.pl_sparse_conv_run_sequence(kernel._handle, xp, op, n_sets, batch, h * w, n_sets + 10, C.c_void_p(stream), None))
+                    torch.cuda.synchronize()
+                    got = outs[0].cpu().numpy()
+                    if first is None:
+                        first = got
+                        if kind == "fp32":
+                            want = helpers.run_oracle(case, helpers.oracle_pack(case, force_semi=paired), x=case.x[:1])
+                            helpers.assert_same(case, got[:1], want, "float-layers %s" % row["shape"])
+                    else:
+                        assert np.array_equal(got.view(np.uint8), first.view(np.uint8)), "%s differs from the library's choice at %s" % (name, row)
+                    settle(lambda: capi.check(L.pl_sparse_conv_run_sequence(kernel._handle, xp, op, n_sets, batch, h * w, 100, C.c_void_p(stream), None)), 0.03)
+                    ms = C.c_float(0.0)
+                    capi.check(L.pl_sparse_conv_run_sequence(kernel._handle, xp, op, n_sets, batch, h * w, steps, C.c_void_p(stream), C.byref(ms)))
+                    row["kernel_us"][name] = round(ms.value * 1e3 / steps, 2)
+                rows.append(row)
+                del xs, outs
+        torch.cuda.empty_cache()
+    print(json.dumps({"metric": "floating-point sparse 1x1 conv: kernel us per launch by walk on layers outside the headline configurations", "unit": "us", "n_gpus": 1,
+                      "steps": steps, "data": "synthetic", "config": {"workload": "float_layers", "parity_checked": True}, "rows": rows}))
     return 0
 
 
@@ -830,6 +896,8 @@ def main():
         return run_mobilenet(args)
     if args.config == "small-batch":
         return run_small_batch(args)
+    if args.config == "float-layers":
+        return run_float_layers(args)
     if args.config == "custom":
         case = custom_case(args)
         args.fp16 = args.fp16 or args.kind == "fp16"
