@@ -134,9 +134,14 @@ typedef struct pl_sparse_conv_tuning {
                                 done by transposing LDS reads where that exists
                                 (ic = 512, 14 x 14 maps); NEVER = by the vector
                                 ALU everywhere                                 */
-  int32_t walk_pairs;        /* (switch) that walk with two row groups per
-                                wavefront instruction: lanes 0 - 31 walk one,
-                                lanes 32 - 63 the other, four positions per lane */
+  int32_t walk_pairs;        /* (switch) the fp32 walk with tile and lists in LDS
+                                takes several row groups per wavefront
+                                instruction (two: lanes 0 - 31 walk one, lanes
+                                32 - 63 the other, four positions per lane; with
+                                more than 271 channels 4 / 8 / 16 on smaller
+                                tiles).  NEVER = one row group per instruction:
+                                that form exists up to 271 channels and for maps
+                                of a multiple of 4 positions only             */
 } pl_sparse_conv_tuning;
 
 /* Everything PrepareForRun() knows.  All pointers are HOST pointers and are
