@@ -962,6 +962,15 @@ int pl_sparse_conv_prepare(const pl_sparse_conv_desc* desc, pl_sparse_conv_handl
   return PL_OK;
 }
 
+// From how many positions on a tile walk on tiles of at most 64 positions (more than 271 channels in fp32, more than
+// 543 in half precision) is ahead of the plain walk, which loses ground as the channel count grows; measured at 49 -
+// 3136 positions on 256 CUs, scaled with the CU count.  Below it a step of 4 - 16 row groups leaves a wavefront too
+// few, too long units.
+bool SmallTilesPay(const pl_sparse_conv_handle* h, int tile, uint32_t P) {
+  const int64_t from = tile >= 64 ? (h->semi ? 1024 : 640) : (h->semi ? 784 : 392);
+  return static_cast<int64_t>(P) * 512 >= from * h->wg_slots_default;
+}
+
 // How a tile walk of `tiles` tiles is divided over the CUs, and where the stream tables of that division start.
 // With fewer tiles than CUs, the CUs without a tile take a share of the row groups of several tiles each
 // (one after the other, each staged anew).  The share that evens out the two kinds of workgroup: a main
@@ -1045,8 +1054,10 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
       half_ragged = true;
     }
     if (half_tw) half_tile = pl::HalfTileWalkTileOf(half_tw->form);
-    // measured on tiles of 256 and 128 positions; smaller tiles count by positions
-    if (half_tw && h->walk_tiled != 2 && (h->semi ? 42 : 84) * static_cast<int64_t>(CeilDiv(static_cast<int>(P), std::max(half_tile, pl::kHalfTileWalkNarrowTile))) < h->wg_slots_default) half_tw = nullptr;
+    if (half_tw && h->walk_tiled != 2) {
+      const bool pays = half_tile <= 64 ? SmallTilesPay(h, 32, P) : (h->semi ? 42 : 84) * static_cast<int64_t>(CeilDiv(static_cast<int>(P), half_tile)) >= h->wg_slots_default;
+      if (!pays) half_tw = nullptr;
+    }
   }
   if (half_tw) {
     const TileWalkDivision d = DivideTileWalk(h, *half_tw, CeilDiv(static_cast<int>(P), half_tile));
@@ -1192,7 +1203,7 @@ int pl_sparse_conv_run(pl_sparse_conv_handle* h, const void* x_dev, void* out_de
     e = pl::LaunchBlockMfma(c, p, s);
   } else if (!h->int8 && !h->half && h->tw.built != 0 && h->walk_tiled > 0 &&
              (vec || (h->tw.form != 0 && reinterpret_cast<uintptr_t>(x_dev) % 4 == 0 && reinterpret_cast<uintptr_t>(out_dev) % 4 == 0)) &&
-             (h->walk_tiled == 2 || (vec ? 32 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::TileWalkTileOf(h->tw.form))) >= h->wg_slots_default
+             (h->walk_tiled == 2 || (vec ? (h->tw.form >= 2 ? SmallTilesPay(h, pl::TileWalkTileOf(h->tw.form), P) : 32 * static_cast<int64_t>(CeilDiv(static_cast<int>(P), pl::kTileWalkTile)) >= h->wg_slots_default)
                                          // the other walks move such tensors element by element too and lose earlier: measured
                                          // crossover at 400 - 700 positions with row pairs, 50 - 200 without (256 CUs)
                                          : (h->semi ? 4 : 14) * static_cast<int64_t>(P) >= 5 * static_cast<int64_t>(h->wg_slots_default)))) {
