@@ -113,14 +113,15 @@ def test_fp16_tile_walk_divisions(batch, paired, ic, size):
     assert np.array_equal(tiled.view(np.uint16), plain.view(np.uint16))
 
 
+@pytest.mark.parametrize("ic", [128, 600], ids=["pairs", "eight_groups_per_step"])
 @pytest.mark.parametrize("size", [16, 14], ids=["wide_tiles", "narrow_tiles"])
 @pytest.mark.parametrize("had_bias", [True, False], ids=["bias", "no_bias"])
-def test_fp16_tile_walk_takes_a_new_bias(had_bias, size):
+def test_fp16_tile_walk_takes_a_new_bias(had_bias, size, ic):
     """set_epilogue rewrites the biases in the list streams (the accumulators start from them), also in a handle
     that was prepared without one."""
     from helpers import make_kernel
 
-    case = half_case(12, 128, 96, size, size, 0.8, False, ACTS["relu"], seed=9)
+    case = half_case(12 if ic == 128 else 3, ic, 96, size, size, 0.8, False, ACTS["relu"], seed=9)
     if not had_bias:
         case.bias = None
     kernel, _ = make_kernel(case, tuning=capi.tuning(walk_tiled=capi.TUNE_ALWAYS))

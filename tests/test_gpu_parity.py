@@ -299,13 +299,14 @@ def test_set_epilogue_replaces_scales():
 
 
 @pytest.mark.parametrize("paired", [False, True], ids=["unstructured", "semi"])
-def test_set_epilogue_replaces_the_bias_of_every_fp32_walk(paired):
+@pytest.mark.parametrize("ic", [130, 600, 1500], ids=["pairs", "eight_groups_per_step", "sixteen_groups_per_step"])
+def test_set_epilogue_replaces_the_bias_of_every_fp32_walk(paired, ic):
     """The walk with the tile and the lists in LDS starts its accumulators from
     the bias carried in its list headers: a new bias must reach those too, and
     a handle prepared without a bias must take one."""
-    announce("set_epilogue bias", paired)
+    announce("set_epilogue bias", paired, ic)
     for had_bias in (True, False):
-        case = small_case(capi.KIND_FP32, 3, 130, 67, 4, 5, 0.75, paired, ACTS["relu6"], seed=31)
+        case = small_case(capi.KIND_FP32, 3, ic, 67, 4, 5, 0.75, paired, ACTS["relu6"], seed=31)
         new_bias = np.linspace(-0.7, 0.9, 67).astype(np.float32)
         if not had_bias:
             case.bias = None
